@@ -1,0 +1,246 @@
+// Embedding gather, residual add + RMSNorm, per-head q/k norm + rotation + cache
+// write, SwiGLU.  Statistics, rotation and the residual sum are 32-bit whatever
+// the activation type is; a result is rounded once, when it is stored.
+#include "common.hpp"
+
+// ---------------------------------------------------------------------------
+// Embedding: out[t, :] = table[ids[t], :] as the 32-bit residual stream.
+// A negative id marks a padding row and gives zeros.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                             float* __restrict__ out, int H, int V) {
+    const int t = blockIdx.x;
+    const int id = ids[t];
+    float* o = out + static_cast<size_t>(t) * H;
+    if (id < 0 || id >= V) {
+        for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = 0.f;
+        return;
+    }
+    const T* row = table + static_cast<size_t>(id) * H;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_float(row[i]);
+}
+
+extern "C" int pl_embed(const int* ids, const void* table, int dtype, float* out, int n, int H,
+                        int V, hipStream_t stream) {
+    PL_REQUIRE(n >= 0 && H > 0 && V > 0, "embed: n %d, width %d, vocabulary %d", n, H, V);
+    if (n == 0) return 0;
+    const int threads = H >= 256 ? 256 : 64;
+    if (dtype == PL_DTYPE_F32)
+        embed_kernel<float><<<n, threads, 0, stream>>>(ids, static_cast<const float*>(table), out, H, V);
+    else if (dtype == PL_DTYPE_BF16)
+        embed_kernel<bf16_t><<<n, threads, 0, stream>>>(ids, static_cast<const bf16_t*>(table), out, H, V);
+    else
+        PL_REQUIRE(false, "embed: dtype code %d", dtype);
+    PL_CHECK_LAUNCH("embed");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Residual add + RMSNorm.
+//   x = resid[r] (+ delta[r]);  if write_resid: resid[r] = x
+//   out[i] = x / sqrt(mean(x^2) + eps) * gain
+// r = rows[i] when a row list is given (then nothing is written back), else i.
+// One workgroup per output row; the sum of squares is reduced in a fixed order.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restrict__ delta,
+                                   const void* __restrict__ gain, int gain_dtype, float eps,
+                                   T* __restrict__ out, const int* __restrict__ rows, int H,
+                                   int write_resid) {
+    __shared__ float scratch[16];
+    const int i = blockIdx.x;
+    const int r = rows ? rows[i] : i;
+    float* x = resid + static_cast<size_t>(r) * H;
+    const T* d = delta ? delta + static_cast<size_t>(r) * H : nullptr;
+    T* o = out + static_cast<size_t>(i) * H;
+
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        float v = x[c];
+        if (d) v += to_float(d[c]);
+        if (write_resid) x[c] = v;
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float denom = sqrtf(ss / static_cast<float>(H) + eps);
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        float v = x[c];
+        if (d && !write_resid) v += to_float(d[c]);
+        o[c] = from_float<T>(v / denom * load_as_float(gain, gain_dtype, c));
+    }
+}
+
+extern "C" int pl_add_rmsnorm(float* resid, const void* delta, const void* gain, int gain_dtype,
+                              float eps, void* out, int dtype, const int* rows, int n_out, int H,
+                              int write_resid, hipStream_t stream) {
+    PL_REQUIRE(n_out >= 0 && H > 0, "add_rmsnorm: rows %d, width %d", n_out, H);
+    PL_REQUIRE(!(rows && write_resid), "add_rmsnorm: a gathered call cannot write the residual back");
+    PL_REQUIRE(gain_dtype == PL_DTYPE_F32 || gain_dtype == PL_DTYPE_BF16, "add_rmsnorm: gain dtype code %d", gain_dtype);
+    if (n_out == 0) return 0;
+    const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 64);
+    if (dtype == PL_DTYPE_F32)
+        add_rmsnorm_kernel<float><<<n_out, threads, 0, stream>>>(
+            resid, static_cast<const float*>(delta), gain, gain_dtype, eps, static_cast<float*>(out), rows, H, write_resid);
+    else if (dtype == PL_DTYPE_BF16)
+        add_rmsnorm_kernel<bf16_t><<<n_out, threads, 0, stream>>>(
+            resid, static_cast<const bf16_t*>(delta), gain, gain_dtype, eps, static_cast<bf16_t*>(out), rows, H, write_resid);
+    else
+        PL_REQUIRE(false, "add_rmsnorm: dtype code %d", dtype);
+    PL_CHECK_LAUNCH("add_rmsnorm");
+    return 0;
+}
+
+// A plain residual add for blocks whose next step is not a norm: resid += delta.
+template <typename T>
+__global__ void residual_add_kernel(float* __restrict__ resid, const T* __restrict__ delta, size_t count) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < count) resid[i] += to_float(delta[i]);
+}
+
+extern "C" int pl_residual_add(float* resid, const void* delta, int dtype, int n, int H, hipStream_t stream) {
+    PL_REQUIRE(n >= 0 && H > 0, "residual_add: rows %d, width %d", n, H);
+    const size_t count = static_cast<size_t>(n) * H;
+    if (count == 0) return 0;
+    const int blocks = static_cast<int>((count + 255) / 256);
+    if (dtype == PL_DTYPE_F32)
+        residual_add_kernel<float><<<blocks, 256, 0, stream>>>(resid, static_cast<const float*>(delta), count);
+    else if (dtype == PL_DTYPE_BF16)
+        residual_add_kernel<bf16_t><<<blocks, 256, 0, stream>>>(resid, static_cast<const bf16_t*>(delta), count);
+    else
+        PL_REQUIRE(false, "residual_add: dtype code %d", dtype);
+    PL_CHECK_LAUNCH("residual_add");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Per-head RMSNorm on q and k, rotation of q and k, and the write of k and v
+// into their cache slots.  One wave per (token, head) over the nq + 2*nkv heads
+// of the fused projection row [q | k | v].  q is rewritten in place.
+//
+//   slot(t) = block_table[seq_of[t], pos / bs] * bs + pos % bs
+//
+// A token with a negative position is padding and is skipped.  The rotation
+// pairs element i with i + rot/2 (the two halves of the head) and uses 32-bit
+// cos/sin tables of [max_pos, rot/2].
+// ---------------------------------------------------------------------------
+#define PL_MAX_HEAD_DIM 256
+
+template <typename T>
+__global__ void qk_norm_rope_kv_write_kernel(
+    T* __restrict__ qkv, const void* __restrict__ q_gain, const void* __restrict__ k_gain,
+    int gain_dtype, float eps, const float* __restrict__ cos_table,
+    const float* __restrict__ sin_table, int rot, const int* __restrict__ positions,
+    const int* __restrict__ seq_of, const int* __restrict__ block_table, int max_blocks,
+    int block_size, T* __restrict__ k_pool, T* __restrict__ v_pool, int nq, int nkv, int d) {
+    __shared__ float head[PL_MAX_HEAD_DIM];
+    const int t = blockIdx.x;
+    const int h = blockIdx.y;
+    const int lane = threadIdx.x;
+    const int pos = positions[t];
+    if (pos < 0) return;
+
+    const int row_width = (nq + 2 * nkv) * d;
+    T* src = qkv + static_cast<size_t>(t) * row_width + static_cast<size_t>(h) * d;
+    const bool is_q = h < nq;
+    const bool is_k = !is_q && h < nq + nkv;
+
+    T* dst = src;
+    if (!is_q) {
+        const int blk = block_table[static_cast<size_t>(seq_of[t]) * max_blocks + pos / block_size];
+        if (blk < 0) return;  // the host refuses such a batch; never write through a hole
+        const size_t slot = static_cast<size_t>(blk) * block_size + pos % block_size;
+        const int kvh = is_k ? h - nq : h - nq - nkv;
+        dst = (is_k ? k_pool : v_pool) + (slot * nkv + kvh) * d;
+    }
+
+    if (!is_q && !is_k) {  // v: a copy
+        for (int i = lane; i < d; i += PL_WAVE) dst[i] = src[i];
+        return;
+    }
+
+    const void* gain = is_q ? q_gain : k_gain;
+    float ss = 0.f;
+    for (int i = lane; i < d; i += PL_WAVE) {
+        const float v = to_float(src[i]);
+        head[i] = v;
+        ss += v * v;
+    }
+    if (gain) {
+        ss = wave_sum(ss);
+        const float denom = sqrtf(ss / static_cast<float>(d) + eps);
+        __syncthreads();
+        for (int i = lane; i < d; i += PL_WAVE) head[i] = head[i] / denom * load_as_float(gain, gain_dtype, i);
+    }
+    __syncthreads();
+    const int half = rot / 2;
+    if (cos_table) {
+        const float* c = cos_table + static_cast<size_t>(pos) * half;
+        const float* s = sin_table + static_cast<size_t>(pos) * half;
+        for (int i = lane; i < half; i += PL_WAVE) {
+            const float x1 = head[i], x2 = head[i + half];
+            dst[i] = from_float<T>(x1 * c[i] - x2 * s[i]);
+            dst[i + half] = from_float<T>(x2 * c[i] + x1 * s[i]);
+        }
+        for (int i = rot + lane; i < d; i += PL_WAVE) dst[i] = from_float<T>(head[i]);
+    } else {
+        for (int i = lane; i < d; i += PL_WAVE) dst[i] = from_float<T>(head[i]);
+    }
+}
+
+extern "C" int pl_qk_norm_rope_kv_write(
+    void* qkv, const void* q_gain, const void* k_gain, int gain_dtype, float eps,
+    const float* cos_table, const float* sin_table, int rot, const int* positions,
+    const int* seq_of, const int* block_table, int max_blocks, int block_size, void* k_pool,
+    void* v_pool, int n, int nq, int nkv, int d, int write_kv, int dtype, hipStream_t stream) {
+    PL_REQUIRE(d > 0 && d <= PL_MAX_HEAD_DIM && d % 16 == 0,
+               "qk_norm_rope: head size %d, which has to be a multiple of 16 up to %d", d, PL_MAX_HEAD_DIM);
+    PL_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0, "qk_norm_rope: rotated width %d of a head of %d", rot, d);
+    PL_REQUIRE(nq > 0 && nkv > 0 && block_size > 0 && max_blocks > 0,
+               "qk_norm_rope: %d query heads, %d key heads, block size %d, %d blocks a row", nq, nkv, block_size, max_blocks);
+    PL_REQUIRE((q_gain == nullptr) == (k_gain == nullptr), "qk_norm_rope: one of the two gains is missing");
+    if (n <= 0) return 0;
+    // Without the cache write (a layer that reads another layer's pages) only the query heads run.
+    dim3 grid(n, write_kv ? nq + 2 * nkv : nq);
+    if (dtype == PL_DTYPE_F32)
+        qk_norm_rope_kv_write_kernel<float><<<grid, PL_WAVE, 0, stream>>>(
+            static_cast<float*>(qkv), q_gain, k_gain, gain_dtype, eps, cos_table, sin_table, rot, positions, seq_of,
+            block_table, max_blocks, block_size, static_cast<float*>(k_pool), static_cast<float*>(v_pool), nq, nkv, d);
+    else if (dtype == PL_DTYPE_BF16)
+        qk_norm_rope_kv_write_kernel<bf16_t><<<grid, PL_WAVE, 0, stream>>>(
+            static_cast<bf16_t*>(qkv), q_gain, k_gain, gain_dtype, eps, cos_table, sin_table, rot, positions, seq_of,
+            block_table, max_blocks, block_size, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), nq, nkv, d);
+    else
+        PL_REQUIRE(false, "qk_norm_rope: dtype code %d", dtype);
+    PL_CHECK_LAUNCH("qk_norm_rope_kv_write");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// SwiGLU on the fused projection row [gate | up]: out = silu(gate) * up.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t count) {
+    const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= count) return;
+    const size_t row = idx / I;
+    const int c = static_cast<int>(idx % I);
+    const float g = to_float(gu[row * 2 * I + c]);
+    const float u = to_float(gu[row * 2 * I + I + c]);
+    out[idx] = from_float<T>(g / (1.f + expf(-g)) * u);
+}
+
+extern "C" int pl_swiglu(const void* gu, void* out, int n, int I, int dtype, hipStream_t stream) {
+    PL_REQUIRE(n >= 0 && I > 0, "swiglu: rows %d, width %d", n, I);
+    const size_t count = static_cast<size_t>(n) * I;
+    if (count == 0) return 0;
+    const int blocks = static_cast<int>((count + 255) / 256);
+    if (dtype == PL_DTYPE_F32)
+        swiglu_kernel<float><<<blocks, 256, 0, stream>>>(static_cast<const float*>(gu), static_cast<float*>(out), I, count);
+    else if (dtype == PL_DTYPE_BF16)
+        swiglu_kernel<bf16_t><<<blocks, 256, 0, stream>>>(static_cast<const bf16_t*>(gu), static_cast<bf16_t*>(out), I, count);
+    else
+        PL_REQUIRE(false, "swiglu: dtype code %d", dtype);
+    PL_CHECK_LAUNCH("swiglu");
+    return 0;
+}

@@ -1,0 +1,135 @@
+"""The descriptor of one step: a ragged batch of (request, its next tokens).
+
+Portions of prompts stand beside single decoded tokens, cut anywhere.  Per token
+the batch carries its id, its position and the index of its request; per request
+the first row, the number of rows, the context length after the step, the state
+slot and, for every cache group, the row of the block table.  Everything goes to
+the device in one copy.  (Reference: batch.rs:67-275, which pads a rectangle and
+builds a mask on the host instead.)
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+from ..errors import ConfigError
+
+
+@dataclass
+class StepEntry:
+    """The next tokens of one request.  ``start`` is the position of the first;
+    ``want`` lists the places among these tokens whose logits are asked for."""
+    seq_id: int
+    tokens: list
+    start: int
+    want: list = field(default_factory=list)
+    state_slot: int = -1
+    fresh_state: bool = False
+
+
+class StepBatch:
+    """Device tensors of one step (all int32)."""
+
+    def __init__(self, packed: torch.Tensor, layout: dict, num_tokens: int, num_seqs: int, max_blocks: list,
+                 num_logit_rows: int, max_q_len: int, max_ctx_len: int, seq_ids: list):
+        self.packed = packed
+        self.num_tokens = num_tokens
+        self.num_seqs = num_seqs
+        self.num_logit_rows = num_logit_rows
+        self.max_q_len = max_q_len
+        self.max_ctx_len = max_ctx_len
+        self.seq_ids = seq_ids
+
+        def view(name, *shape):
+            begin, count = layout[name]
+            return packed[begin:begin + count].view(*shape)
+
+        self.token_ids = view("token_ids", num_tokens)
+        self.positions = view("positions", num_tokens)
+        self.seq_of = view("seq_of", num_tokens)
+        self.q_start = view("q_start", num_seqs)
+        self.q_len = view("q_len", num_seqs)
+        self.ctx_len = view("ctx_len", num_seqs)
+        self.state_slots = view("state_slots", num_seqs)
+        self.logit_rows = view("logit_rows", num_logit_rows)
+        self.block_tables = [view(f"block_table_{g}", num_seqs, mb) for g, mb in enumerate(max_blocks)]
+
+
+def build_batch(entries, manager, num_groups: int, vocab_size: int, max_positions: int, device,
+                check_start: bool = True) -> StepBatch:
+    """Validate the entries against the cache manager and lay the step out for the device.
+
+    Refused with ConfigError: an empty step, an entry without tokens, a token id
+    outside the vocabulary, a position with no page or past the longest position
+    the model knows, a wanted place outside the entry, a request that appears
+    twice, and (with ``check_start``) an entry that does not start where the
+    cache says the request has got to."""
+    entries = list(entries)
+    if not entries:
+        raise ConfigError("an empty batch")
+    seen = set()
+    n = sum(len(e.tokens) for e in entries)
+    S = len(entries)
+    token_ids = np.empty(n, np.int32)
+    positions = np.empty(n, np.int32)
+    seq_of = np.empty(n, np.int32)
+    q_start = np.empty(S, np.int32)
+    q_len = np.empty(S, np.int32)
+    ctx_len = np.empty(S, np.int32)
+    state_slots = np.empty(S, np.int32)
+    logit_rows: list = []
+    tables = [[] for _ in range(num_groups)]
+    at = 0
+    for s, e in enumerate(entries):
+        count = len(e.tokens)
+        if count == 0:
+            raise ConfigError(f"request {e.seq_id} brings no tokens to the step")
+        if e.seq_id in seen:
+            raise ConfigError(f"request {e.seq_id} appears twice in one step")
+        seen.add(e.seq_id)
+        toks = np.asarray(e.tokens, dtype=np.int64)
+        if toks.min() < 0 or toks.max() >= vocab_size:
+            raise ConfigError(f"request {e.seq_id}: token id outside the vocabulary of {vocab_size}")
+        written = manager.tokens(e.seq_id)
+        if check_start and e.start != written:
+            raise ConfigError(f"request {e.seq_id}: tokens start at position {e.start}, the cache holds {written}")
+        if e.start + count > manager.capacity(e.seq_id):
+            raise ConfigError(f"request {e.seq_id} has no block for position {e.start + count - 1}")
+        if max_positions and e.start + count > max_positions:
+            raise ConfigError(f"request {e.seq_id}: position {e.start + count - 1} is past the model's {max_positions}")
+        for w in e.want:
+            if not 0 <= w < count:
+                raise ConfigError(f"request {e.seq_id}: logits wanted at place {w} of {count} tokens")
+            logit_rows.append(at + w)
+        token_ids[at:at + count] = toks
+        positions[at:at + count] = np.arange(e.start, e.start + count, dtype=np.int32)
+        seq_of[at:at + count] = s
+        q_start[s], q_len[s], ctx_len[s], state_slots[s] = at, count, e.start + count, e.state_slot
+        for g in range(num_groups):
+            tables[g].append(manager.table(e.seq_id, g))
+        at += count
+
+    max_blocks = [max(1, max(len(t) for t in tables[g])) for g in range(num_groups)]
+    pieces = [("token_ids", token_ids), ("positions", positions), ("seq_of", seq_of), ("q_start", q_start),
+              ("q_len", q_len), ("ctx_len", ctx_len), ("state_slots", state_slots),
+              ("logit_rows", np.asarray(logit_rows, dtype=np.int32))]
+    for g in range(num_groups):
+        bt = np.full((S, max_blocks[g]), -1, np.int32)
+        for s, t in enumerate(tables[g]):
+            bt[s, :len(t)] = t
+        pieces.append((f"block_table_{g}", bt.reshape(-1)))
+    layout = {}
+    offset = 0
+    for name, arr in pieces:
+        layout[name] = (offset, arr.size)
+        offset += (arr.size + 3) // 4 * 4      # keep every piece 16-byte aligned
+    host = np.zeros(max(offset, 4), np.int32)
+    for name, arr in pieces:
+        begin, count = layout[name]
+        host[begin:begin + count] = arr
+    packed = torch.from_numpy(host).to(device)
+    return StepBatch(packed, layout, n, S, max_blocks, len(logit_rows), int(q_len.max()), int(ctx_len.max()),
+                     [e.seq_id for e in entries])

@@ -1,0 +1,250 @@
+"""The hand-written gfx950 kernels, as functions over torch tensors.
+
+Every function checks on the host that shapes, types and strides are what the
+kernel and its launch assume, then launches on torch's current stream.  There is
+no fallback: without the compiled library, or on a tensor that is not on the
+GPU, these functions raise.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_void_p
+
+import torch
+
+from . import build
+from .errors import TensorError
+
+F32, BF16 = 0, 1
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+
+_lib = None
+
+
+def _signatures(lib) -> None:
+    p, i, f = c_void_p, c_int, c_float
+    lib.pl_last_error.restype = ctypes.c_char_p
+    lib.pl_abi_version.restype = c_int
+    table = {
+        "pl_embed": [p, p, i, p, i, i, i, p],
+        "pl_add_rmsnorm": [p, p, p, i, f, p, i, p, i, i, i, p],
+        "pl_residual_add": [p, p, i, i, i, p],
+        "pl_qk_norm_rope_kv_write": [p, p, p, i, f, p, p, i, p, p, p, i, i, p, p, i, i, i, i, i, i, p],
+        "pl_swiglu": [p, p, i, i, i, p],
+        "pl_gemm_plain": [p, p, p, i, i, i, i, i, i, i, p],
+        "pl_paged_attention_plain": [p, i, p, p, p, p, i, i, p, p, i, i, i, i, f, i, i, p],
+        "pl_argmax": [p, p, i, i, p],
+    }
+    for name, argtypes in table.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = c_int
+
+
+def library():
+    """The kernel library, compiled at its first use when nothing is built."""
+    global _lib
+    if _lib is None:
+        lib = build.load("hip")
+        _signatures(lib)
+        _lib = lib
+    return _lib
+
+
+def _check(code: int) -> None:
+    if code != 0:
+        raise TensorError(library().pl_last_error().decode())
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _code(t: torch.Tensor, what: str) -> int:
+    if t.dtype not in _CODES:
+        raise TensorError(f"{what} is {t.dtype}, the kernels take float32 and bfloat16")
+    return _CODES[t.dtype]
+
+
+def _need(t: torch.Tensor, what: str, shape=None, dtype=None) -> torch.Tensor:
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise TensorError(f"{what} is not a tensor on the GPU")
+    if not t.is_contiguous():
+        raise TensorError(f"{what} is not contiguous (strides {t.stride()} for shape {tuple(t.shape)})")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise TensorError(f"{what} has shape {tuple(t.shape)}, expected {tuple(shape)}")
+    if dtype is not None and t.dtype != dtype:
+        raise TensorError(f"{what} is {t.dtype}, expected {dtype}")
+    return t
+
+
+def _ptr(t) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+# ---------------------------------------------------------------------------
+
+def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t] = table[ids[t]] as the 32-bit residual stream; a negative id gives zeros."""
+    n = ids.numel()
+    V, H = table.shape
+    _need(ids, "token ids", (n,), torch.int32)
+    _need(table, "embedding table")
+    if out is None:
+        out = torch.empty((n, H), dtype=torch.float32, device=table.device)
+    _need(out, "embedding output", (n, H), torch.float32)
+    _check(library().pl_embed(ids.data_ptr(), table.data_ptr(), _code(table, "embedding table"),
+                              out.data_ptr(), n, H, V, _stream()))
+    return out
+
+
+def add_rmsnorm(resid: torch.Tensor, delta, gain: torch.Tensor, eps: float, out: torch.Tensor,
+                rows: torch.Tensor | None = None, write_resid: bool = True) -> torch.Tensor:
+    """x = resid (+ delta); resid = x when ``write_resid``; out = rmsnorm(x) * gain.
+    With ``rows`` the i-th output row is computed from row rows[i] and nothing is written back."""
+    n, H = resid.shape
+    _need(resid, "residual stream", None, torch.float32)
+    n_out = n if rows is None else rows.numel()
+    _need(out, "norm output", (n_out, H))
+    if delta is not None:
+        _need(delta, "residual delta", (n, H), out.dtype)
+    _need(gain, "norm gain", (H,))
+    if rows is not None:
+        _need(rows, "row list", (n_out,), torch.int32)
+        write_resid = False
+    _check(library().pl_add_rmsnorm(resid.data_ptr(), _ptr(delta), gain.data_ptr(), _code(gain, "norm gain"),
+                                    float(eps), out.data_ptr(), _code(out, "norm output"), _ptr(rows),
+                                    n_out, H, 1 if write_resid else 0, _stream()))
+    return out
+
+
+def residual_add(resid: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
+    n, H = resid.shape
+    _need(resid, "residual stream", None, torch.float32)
+    _need(delta, "residual delta", (n, H))
+    _check(library().pl_residual_add(resid.data_ptr(), delta.data_ptr(), _code(delta, "residual delta"), n, H, _stream()))
+    return resid
+
+
+def qk_norm_rope_kv_write(qkv: torch.Tensor, q_gain, k_gain, eps: float, cos, sin, rot: int,
+                          positions: torch.Tensor, seq_of: torch.Tensor, block_table: torch.Tensor,
+                          block_size: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                          nq: int, nkv: int, d: int, write_kv: bool = True) -> None:
+    """Per-head norm of q and k, rotation of q and k at each token's position, and
+    the write of k and v into their pages.  q is rewritten in place inside ``qkv``."""
+    n = qkv.shape[0]
+    _need(qkv, "fused q/k/v projection", (n, (nq + 2 * nkv) * d))
+    _need(positions, "positions", (n,), torch.int32)
+    _need(seq_of, "request index of each token", (n,), torch.int32)
+    _need(block_table, "block table", None, torch.int32)
+    if block_table.dim() != 2:
+        raise TensorError(f"block table has shape {tuple(block_table.shape)}, expected [requests, pages]")
+    for pool, what in ((k_pool, "key pool"), (v_pool, "value pool")):
+        _need(pool, what, None, qkv.dtype)
+        if pool.dim() != 2 or pool.shape[1] != nkv * d or pool.shape[0] % block_size != 0:
+            raise TensorError(f"{what} has shape {tuple(pool.shape)}, expected [pages*{block_size}, {nkv * d}]")
+    if k_pool.shape != v_pool.shape:
+        raise TensorError("key and value pools differ in shape")
+    if k_pool.shape[0] >= 2 ** 31:
+        raise TensorError("a pool of 2^31 slots or more is not addressed by these kernels")
+    gain_code = F32
+    if q_gain is not None:
+        _need(q_gain, "query norm gain", (d,))
+        _need(k_gain, "key norm gain", (d,), q_gain.dtype)
+        gain_code = _code(q_gain, "query norm gain")
+    if cos is not None:
+        _need(cos, "cosine table", None, torch.float32)
+        _need(sin, "sine table", tuple(cos.shape), torch.float32)
+        if cos.dim() != 2 or cos.shape[1] != rot // 2:
+            raise TensorError(f"rotary tables have shape {tuple(cos.shape)}, expected [positions, {rot // 2}]")
+    _check(library().pl_qk_norm_rope_kv_write(
+        qkv.data_ptr(), _ptr(q_gain), _ptr(k_gain), gain_code, float(eps), _ptr(cos), _ptr(sin), rot,
+        positions.data_ptr(), seq_of.data_ptr(), block_table.data_ptr(), block_table.shape[1], block_size,
+        k_pool.data_ptr(), v_pool.data_ptr(), n, nq, nkv, d, 1 if write_kv else 0,
+        _code(qkv, "fused q/k/v projection"), _stream()))
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """silu(gate) * up on rows laid out [gate | up]."""
+    n, two_i = gate_up.shape
+    _need(gate_up, "fused gate/up projection")
+    if two_i % 2:
+        raise TensorError(f"fused gate/up projection has odd width {two_i}")
+    inter = two_i // 2
+    if out is None:
+        out = torch.empty((n, inter), dtype=gate_up.dtype, device=gate_up.device)
+    _need(out, "feed-forward activation", (n, inter), gate_up.dtype)
+    _check(library().pl_swiglu(gate_up.data_ptr(), out.data_ptr(), n, inter, _code(gate_up, "gate/up"), _stream()))
+    return out
+
+
+def gemm_plain(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor | None = None,
+               out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """y = x . w^T with 32-bit multiply-add on the vector units (no matrix-core mode)."""
+    n, K = x.shape
+    N = w.shape[0]
+    _need(x, "matrix product input")
+    _need(w, "weight", (N, K), x.dtype)
+    out_dtype = out_dtype or x.dtype
+    if out is None:
+        out = torch.empty((n, N), dtype=out_dtype, device=x.device)
+    _need(out, "matrix product output", (n, N), out_dtype)
+    if out_dtype not in (x.dtype, torch.float32):
+        raise TensorError(f"matrix product output {out_dtype} from input {x.dtype}")
+    _check(library().pl_gemm_plain(x.data_ptr(), w.data_ptr(), out.data_ptr(), n, N, K, K, N,
+                                   _code(x, "matrix product input"), 1 if out_dtype == torch.float32 else 0, _stream()))
+    return out
+
+
+def paged_attention_plain(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, positions: torch.Tensor,
+                          seq_of: torch.Tensor, block_table: torch.Tensor, block_size: int,
+                          k_pool: torch.Tensor, v_pool: torch.Tensor, nq: int, nkv: int, d: int,
+                          scale: float, window: int = 0) -> torch.Tensor:
+    """Attention of every token over the keys 0..position of its request, read
+    through the block table.  ``q`` is the fused projection buffer whose rows begin
+    with the nq*d query values."""
+    n = positions.numel()
+    _need(q, "query buffer")
+    if q.dim() != 2 or q.shape[0] != n or q.shape[1] != q_row_stride or q_row_stride < nq * d:
+        raise TensorError(f"query buffer has shape {tuple(q.shape)} for {n} tokens and row stride {q_row_stride}")
+    _need(out, "attention output", (n, nq * d), q.dtype)
+    _need(positions, "positions", (n,), torch.int32)
+    _need(seq_of, "request index of each token", (n,), torch.int32)
+    _need(block_table, "block table", None, torch.int32)
+    for pool, what in ((k_pool, "key pool"), (v_pool, "value pool")):
+        _need(pool, what, None, q.dtype)
+        if pool.dim() != 2 or pool.shape[1] != nkv * d or pool.shape[0] % block_size != 0:
+            raise TensorError(f"{what} has shape {tuple(pool.shape)}, expected [pages*{block_size}, {nkv * d}]")
+    _check(library().pl_paged_attention_plain(
+        q.data_ptr(), q_row_stride, out.data_ptr(), positions.data_ptr(), seq_of.data_ptr(),
+        block_table.data_ptr(), block_table.shape[1], block_size, k_pool.data_ptr(), v_pool.data_ptr(),
+        n, nq, nkv, d, float(scale), int(window or 0), _code(q, "query buffer"), _stream()))
+    return out
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """The index of the largest logit of each row; the first maximum wins."""
+    m, V = logits.shape
+    _need(logits, "logits", None, torch.float32)
+    if out is None:
+        out = torch.empty((m,), dtype=torch.int32, device=logits.device)
+    _need(out, "chosen tokens", (m,), torch.int32)
+    _check(library().pl_argmax(logits.data_ptr(), out.data_ptr(), m, V, _stream()))
+    return out
+
+
+def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nkv: int, d: int,
+                    scale: float, window: int = 0) -> torch.Tensor:
+    """Attention for every token of a step.  ``qkv`` rows begin with the rotated queries."""
+    return paged_attention_plain(qkv, qkv.shape[1], out, batch.positions, batch.seq_of, kv.block_table,
+                                 kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window)
+
+
+def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """y = x . w^T for bfloat16 operands with 32-bit accumulation."""
+    _need(x, "matrix product input", None, torch.bfloat16)
+    _need(w, "weight", None, torch.bfloat16)
+    if out_dtype == torch.float32:
+        return gemm_plain(x, w, out_dtype=torch.float32)
+    return torch.mm(x, w.t())

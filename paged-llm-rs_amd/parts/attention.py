@@ -1,0 +1,82 @@
+"""Grouped-query attention over a paged cache (reference: model/attention.rs).
+
+Order of operations, which cannot be guessed from a Llama-shaped model: project,
+split into heads, normalise q and k over one head's width (when the spec asks
+for it), rotate q and k, write k and v into the pages, then attend.  The write
+precedes the read inside the layer, so a token attends to itself and the later
+tokens of a portion read the earlier ones through the cache.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from .. import kernels
+from ..cache.layout import KVCacheSpec
+from ..errors import UnsupportedError
+from ..weights.loader import ParamDecl
+from .linear import Linear
+from .registry import register_mixer
+from .rotary import rotary_tables
+
+
+class PagedAttention:
+    @staticmethod
+    def declare(spec, hidden: int) -> list:
+        q, kv = spec.num_heads * spec.head_dim, spec.num_kv_heads * spec.head_dim
+        decls = [
+            ParamDecl("q_proj.weight", (q, hidden)), ParamDecl("k_proj.weight", (kv, hidden)),
+            ParamDecl("v_proj.weight", (kv, hidden)), ParamDecl("o_proj.weight", (hidden, q)),
+        ]
+        if spec.qk_norm is not None:
+            decls += [ParamDecl("q_norm.weight", (spec.head_dim,), "gain"),
+                      ParamDecl("k_norm.weight", (spec.head_dim,), "gain")]
+        return decls
+
+    def __init__(self, spec, hidden: int, params: dict, dtype, device, shared: dict):
+        if spec.num_heads % spec.num_kv_heads:
+            raise UnsupportedError(f"{spec.num_heads} query heads over {spec.num_kv_heads} key heads, "
+                                   "which do not group evenly")
+        if spec.head_dim % 16 or not 16 <= spec.head_dim <= 256:
+            raise UnsupportedError(f"head size {spec.head_dim}: the kernels take multiples of 16 up to 256")
+        if spec.qk_norm is not None and spec.qk_norm.kind != "rms_norm":
+            raise UnsupportedError(f"q/k norm {spec.qk_norm.kind!r}, only rms_norm is implemented")
+        self.spec = spec
+        self.nq, self.nkv, self.d = spec.num_heads, spec.num_kv_heads, spec.head_dim
+        self.scale = spec.scale if spec.scale is not None else 1.0 / math.sqrt(spec.head_dim)
+        self.window = int(spec.window or 0)
+        # one product for q, k and v: the output row is [q | k | v]
+        self.qkv_proj = Linear.fused([params["q_proj.weight"], params["k_proj.weight"], params["v_proj.weight"]])
+        self.o_proj = Linear(params["o_proj.weight"])
+        self.q_gain = params.get("q_norm.weight")
+        self.k_gain = params.get("k_norm.weight")
+        self.eps = float(spec.qk_norm.eps) if spec.qk_norm is not None else 0.0
+        self.rotary = rotary_tables(spec.position, device, shared) if spec.position is not None else None
+        if self.rotary is not None and self.rotary.dim > self.d:
+            raise UnsupportedError(f"a rotation over {self.rotary.dim} values of a head of {self.d}")
+
+    def cache_spec(self):
+        return KVCacheSpec(self.nkv, self.d, self.window or None)
+
+    def state_spec(self):
+        return None
+
+    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        batch = ctx.batch
+        kv = ctx.kv()
+        qkv = self.qkv_proj.forward(x)
+        cos = self.rotary.cos if self.rotary is not None else None
+        sin = self.rotary.sin if self.rotary is not None else None
+        rot = self.rotary.dim if self.rotary is not None else 0
+        kernels.qk_norm_rope_kv_write(
+            qkv, self.q_gain, self.k_gain, self.eps, cos, sin, rot, batch.positions, batch.seq_of,
+            kv.block_table, kv.block_size, kv.k_pool, kv.v_pool, self.nq, self.nkv, self.d,
+            write_kv=ctx.writes_cache)
+        out = torch.empty((x.shape[0], self.nq * self.d), dtype=x.dtype, device=x.device)
+        kernels.paged_attention(qkv, out, batch, kv, self.nq, self.nkv, self.d, self.scale, self.window)
+        return self.o_proj.forward(out)
+
+
+register_mixer("paged_attention", PagedAttention)

@@ -1,0 +1,48 @@
+"""The pre-norm arrangement of a layer: norm, mixer, residual, norm,
+feed-forward, residual (reference: model/mod.rs:84-136).
+
+The residual stream is 32-bit.  A block receives the stream and the previous
+block's output that has not been added yet, adds it inside its first norm, and
+returns its own feed-forward output unadded, so that every residual sum is
+fused with the norm that follows it.
+"""
+
+from __future__ import annotations
+
+from .registry import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, lookup, prefixed, register_block, scoped)
+
+
+class PreNormBlock:
+    NAMES = {"norm1": "input_layernorm", "mixer": "self_attn", "norm2": "post_attention_layernorm",
+             "feed_forward": "mlp"}
+
+    @classmethod
+    def declare(cls, layer, hidden: int) -> list:
+        norm = lookup(NORMS, layer.norm.kind, "norm")
+        mixer = lookup(MIXERS, layer.mixer.kind, "mixer")
+        ffn = lookup(FEED_FORWARDS, layer.feed_forward.kind, "feed-forward")
+        n = cls.NAMES
+        return (prefixed(norm.declare(layer.norm, hidden), n["norm1"])
+                + prefixed(mixer.declare(layer.mixer, hidden), n["mixer"])
+                + prefixed(norm.declare(layer.norm, hidden), n["norm2"])
+                + prefixed(ffn.declare(layer.feed_forward, hidden), n["feed_forward"]))
+
+    def __init__(self, layer, hidden: int, params: dict, dtype, device, shared: dict):
+        n = self.NAMES
+        norm = lookup(NORMS, layer.norm.kind, "norm")
+        self.dtype = dtype
+        self.norm1 = norm(layer.norm, hidden, scoped(params, n["norm1"]), dtype, device)
+        self.mixer = lookup(MIXERS, layer.mixer.kind, "mixer")(
+            layer.mixer, hidden, scoped(params, n["mixer"]), dtype, device, shared)
+        self.norm2 = norm(layer.norm, hidden, scoped(params, n["norm2"]), dtype, device)
+        self.feed_forward = lookup(FEED_FORWARDS, layer.feed_forward.kind, "feed-forward")(
+            layer.feed_forward, hidden, scoped(params, n["feed_forward"]), dtype, device, shared)
+
+    def forward(self, resid, delta, ctx):
+        normed = self.norm1.apply(resid, delta, self.dtype)
+        mixed = self.mixer.forward(normed, ctx)
+        normed = self.norm2.apply(resid, mixed, self.dtype)
+        return self.feed_forward.forward(normed)
+
+
+register_block("pre_norm", PreNormBlock)

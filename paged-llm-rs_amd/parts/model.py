@@ -1,0 +1,124 @@
+"""The generic decoder: embedding, the layers in the order the schedule gives,
+final norm on the wanted rows, output projection (reference: model/mod.rs).
+
+The model is put together from a ModelSpec alone.  Which architecture the spec
+came from is not known here.
+"""
+
+from __future__ import annotations
+
+from pathlib import Path
+
+import torch
+
+from .. import kernels
+from ..cache.layout import CacheLayout
+from ..config import load_config
+from ..errors import ConfigError, UnsupportedError, WeightError
+from ..weights.loader import ParamDecl, load_weights
+from . import attention, block, mlp, norm  # noqa: F401  (register the built-in parts)
+from .linear import Linear
+from .registry import BLOCKS, NORMS, lookup, prefixed, scoped
+
+DTYPES = {"float32": torch.float32, "f32": torch.float32, "bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
+          torch.float32: torch.float32, torch.bfloat16: torch.bfloat16}
+
+
+def declare_parameters(spec) -> list:
+    """Every tensor the model needs, by checkpoint name (reference: model/mod.rs:178-227)."""
+    decls = [ParamDecl(spec.embed_name, (spec.vocab_size, spec.hidden_size), "embedding")]
+    for layer in spec.layers:
+        cls = lookup(BLOCKS, layer.block, "block")
+        decls += prefixed(cls.declare(layer, spec.hidden_size), layer.weight_prefix)
+    final = lookup(NORMS, spec.final_norm.kind, "norm")
+    stem = spec.final_norm_name.rsplit(".", 1)[0]
+    decls += prefixed(final.declare(spec.final_norm, spec.hidden_size), stem)
+    # A tied checkpoint may still store the output projection; the stored tensor wins.
+    decls.append(ParamDecl(spec.head_name, (spec.vocab_size, spec.hidden_size), "matrix", optional=True))
+    return decls
+
+
+class LayerContext:
+    """What one run of one layer sees of the step: the batch, its own pages (or
+    the pages of the layer it reads from) and its state slots."""
+
+    __slots__ = ("batch", "cache", "layer", "cache_layer", "writes_cache")
+
+    def __init__(self, batch, cache, layer: int, cache_layer: int, writes_cache: bool):
+        self.batch = batch
+        self.cache = cache
+        self.layer = layer
+        self.cache_layer = cache_layer
+        self.writes_cache = writes_cache
+
+    def kv(self):
+        return self.cache.layer_view(self.cache_layer, self.batch)
+
+    def state(self):
+        """[slots, ...] state tensor of this layer; ``batch.state_slots`` says which slot each request has."""
+        return self.cache.layer_state(self.layer)
+
+
+class DecoderModel:
+    def __init__(self, spec, params: dict, dtype: torch.dtype, device):
+        self.spec = spec
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.shared: dict = {}
+        self.embed_tokens = params[spec.embed_name]
+        self.blocks = []
+        for layer in spec.layers:
+            cls = lookup(BLOCKS, layer.block, "block")
+            self.blocks.append(cls(layer, spec.hidden_size, scoped(params, layer.weight_prefix), dtype,
+                                   self.device, self.shared))
+        stem = spec.final_norm_name.rsplit(".", 1)[0]
+        self.norm = lookup(NORMS, spec.final_norm.kind, "norm")(
+            spec.final_norm, spec.hidden_size, scoped(params, stem), dtype, self.device)
+        if spec.head_name in params:
+            head = params[spec.head_name]
+        elif spec.tie_word_embeddings:
+            head = self.embed_tokens
+        else:
+            raise WeightError(f"no {spec.head_name}, and the config does not tie the embeddings")
+        self.lm_head = Linear(head)
+        for entry in spec.schedule:
+            if not 0 <= entry.layer < len(self.blocks):
+                raise ConfigError(f"the schedule names layer {entry.layer} of {len(self.blocks)}")
+            if entry.cache_from is not None and not 0 <= entry.cache_from < len(self.blocks):
+                raise ConfigError(f"the schedule reads the cache of layer {entry.cache_from} of {len(self.blocks)}")
+        self.cache_layout = CacheLayout.from_blocks(self.blocks, spec.schedule)
+
+    # -- the forward pass of one step -------------------------------------------------
+
+    def forward(self, batch, cache) -> torch.Tensor:
+        """Run the tokens of ``batch`` from ``cache`` and return 32-bit logits
+        [wanted rows, vocabulary].  Pages are written; no length is moved."""
+        resid = kernels.embed(batch.token_ids, self.embed_tokens)
+        delta = None
+        for entry in self.spec.schedule:
+            own = entry.cache_from is None
+            ctx = LayerContext(batch, cache, entry.layer, entry.layer if own else entry.cache_from, own)
+            delta = self.blocks[entry.layer].forward(resid, delta, ctx)
+        m = batch.num_logit_rows
+        if m == 0:
+            # A portion in the middle of a prompt runs only to fill the cache.
+            # Nothing further is launched for it.
+            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
+        normed = self.norm.apply(resid, delta, self.dtype, rows=batch.logit_rows)
+        return self.lm_head.forward(normed, out_dtype=torch.float32)
+
+
+def build_model(config, params: dict, dtype, device) -> DecoderModel:
+    return DecoderModel(config.model_spec(), params, DTYPES[dtype], device)
+
+
+def load_model(model_dir, dtype="bfloat16", device="cuda:0"):
+    """(typed configuration, model) from a folder with config.json and model.safetensors.
+    The model class is chosen by config.json through the architecture registry."""
+    if dtype not in DTYPES:
+        raise ConfigError(f"dtype {dtype!r}, which is neither bfloat16 nor float32")
+    model_dir = Path(model_dir)
+    config = load_config(model_dir)
+    spec = config.model_spec()
+    params = load_weights(model_dir, declare_parameters(spec), DTYPES[dtype], device)
+    return config, DecoderModel(spec, params, DTYPES[dtype], device)

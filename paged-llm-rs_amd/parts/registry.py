@@ -1,0 +1,63 @@
+"""Registries of parts.  A spec's ``kind`` names the class that implements it.
+
+A part is built from its own spec and the width of the residual stream, asks
+for its tensors by local name, and never learns which model it is in.  New
+parts are added by registering a class; no file of the package has to change.
+
+Interfaces
+----------
+mixer         ``declare(spec, hidden) -> [ParamDecl]`` (local names);
+              ``__init__(spec, hidden, params, dtype, device, shared)``;
+              ``cache_spec() -> KVCacheSpec | None``; ``state_spec() -> StateSpec | None``;
+              ``forward(x[n,hidden], ctx: LayerContext) -> [n,hidden]``.
+feed-forward  ``declare``; ``__init__`` as above; ``forward(x) -> [n,hidden]``.
+norm          ``declare(spec, width)``; ``__init__(spec, width, params, dtype, device)``;
+              ``apply(resid, delta, out_dtype, rows=None) -> normed`` which adds
+              ``delta`` into the 32-bit residual stream and returns the normalised rows.
+block         ``declare(layer_spec, hidden)``; ``__init__(layer_spec, hidden, params, dtype,
+              device, shared)``; ``forward(resid, delta, ctx) -> delta`` where the returned
+              delta is the output not yet added to the residual stream.
+"""
+
+from __future__ import annotations
+
+from ..errors import UnsupportedError
+
+MIXERS: dict = {}
+FEED_FORWARDS: dict = {}
+NORMS: dict = {}
+BLOCKS: dict = {}
+
+
+def register_mixer(kind: str, cls) -> None:
+    MIXERS[kind] = cls
+
+
+def register_feed_forward(kind: str, cls) -> None:
+    FEED_FORWARDS[kind] = cls
+
+
+def register_norm(kind: str, cls) -> None:
+    NORMS[kind] = cls
+
+
+def register_block(kind: str, cls) -> None:
+    BLOCKS[kind] = cls
+
+
+def lookup(registry: dict, kind: str, what: str):
+    if kind not in registry:
+        raise UnsupportedError(f"{what} {kind!r}, the registry knows {', '.join(sorted(registry)) or 'none'}")
+    return registry[kind]
+
+
+def scoped(params: dict, prefix: str) -> dict:
+    """The tensors under ``prefix.``, by their local names."""
+    cut = len(prefix) + 1
+    return {k[cut:]: v for k, v in params.items() if k.startswith(prefix + ".")}
+
+
+def prefixed(decls, prefix: str) -> list:
+    from ..weights.loader import ParamDecl
+
+    return [ParamDecl(f"{prefix}.{d.name}", d.shape, d.role, d.optional) for d in decls]

@@ -1,0 +1,131 @@
+"""The engine against the plain implementation, replayed four ways, in 32-bit
+and in bfloat16: each request alone and whole; most of it in one step and the
+last 32 tokens one by one; in portions of changing size; mixed with other
+requests and so few pages that they are used again."""
+
+from __future__ import annotations
+
+import json
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import replay_util as ru
+from conftest import ROOT, TINY_INIT
+
+pytestmark = pytest.mark.gpu
+
+# max|got - want| / max|want|.  32-bit: the reference's own bound for its tiny
+# fixture (tests/fixtures/tiny/manifest.json: 1e-5).  bfloat16: inputs of every
+# product are rounded to 8 bits of mantissa (2^-9 = 2e-3 a rounding); through two
+# or three layers and a head that is a few times 1e-3 of the largest logit.
+TOLERANCE = {"float32": 1e-5, "bfloat16": 2e-2}
+LENGTHS = {"A": [5, 17, 33, 70, 100, 41], "B": [1, 9, 24, 40, 129, 66], "C": [3, 50, 97, 64, 20, 35]}
+
+
+@pytest.fixture(scope="module")
+def setups(model_dirs):
+    """(model name, dtype) -> (model dir, prompts, plain logits)."""
+    made = {}
+
+    def get(name, dtype):
+        if (name, dtype) not in made:
+            d = model_dirs(name, dtype)
+            prompts = ru.make_prompts(TINY_INIT[name]["config"]["vocab_size"], LENGTHS[name], seed=11)
+            made[(name, dtype)] = (d, prompts, ru.plain_logits(d, prompts))
+        return made[(name, dtype)]
+
+    return get
+
+
+def replay(model_dir, dtype, prompts, steps, max_live, block_size=16):
+    from paged_llm_rs_amd.engine.replay import Replayer
+
+    r = Replayer(model_dir, dtype, max_tokens=ru.pool_tokens(prompts, max_live), block_size=block_size)
+    got = ru.collect(r, steps)
+    assert r.cache.manager.live_sequences == 0
+    assert r.cache.manager.available() == r.cache.manager.total(), "every page came back"
+    return got
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_whole_requests(setups, name, dtype):
+    d, prompts, want = setups(name, dtype)
+    got = replay(d, dtype, prompts, ru.whole(prompts), max_live=1)
+    assert len(got) == sum(len(t) for t in prompts.values())
+    worst, where = ru.worst_error(got, want)
+    assert worst <= TOLERANCE[dtype], f"{worst:.3e} at {where}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,block_size", [("A", 16), ("B", 8), ("C", 4)])
+def test_last_tokens_decoded_one_by_one(setups, name, dtype, block_size):
+    d, prompts, want = setups(name, dtype)
+    got = replay(d, dtype, prompts, ru.tail_decoded(prompts, 32), max_live=1, block_size=block_size)
+    worst, where = ru.worst_error(got, want)
+    assert worst <= TOLERANCE[dtype], f"{worst:.3e} at {where}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,block_size", [("A", 16), ("B", 8), ("C", 4)])
+def test_portions_of_changing_size(setups, name, dtype, block_size):
+    d, prompts, want = setups(name, dtype)
+    got = replay(d, dtype, prompts, ru.portions(prompts), max_live=1, block_size=block_size)
+    worst, where = ru.worst_error(got, want)
+    assert worst <= TOLERANCE[dtype], f"{worst:.3e} at {where}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,block_size,seed", [("A", 16, 1), ("B", 8, 2), ("C", 4, 3), ("B", 16, 4)])
+def test_mixed_requests_with_pages_used_again(setups, name, dtype, block_size, seed):
+    d, prompts, want = setups(name, dtype)
+    steps = ru.mixed(prompts, seed=seed, max_live=4)
+    assert max(len(s["entries"]) for s in steps) >= 3
+    assert any(len(e["tokens"]) > 1 for s in steps for e in s["entries"] if len(s["entries"]) > 1)
+    got = replay(d, dtype, prompts, steps, max_live=4, block_size=block_size)
+    worst, where = ru.worst_error(got, want)
+    assert worst <= TOLERANCE[dtype], f"{worst:.3e} at {where}"
+
+
+def test_schedules_agree_with_each_other_in_32_bit(setups):
+    """The logits at a position do not depend on how the tokens were cut, beyond rounding."""
+    d, prompts, _ = setups("B", "float32")
+    a = replay(d, "float32", prompts, ru.whole(prompts), max_live=1, block_size=8)
+    b = replay(d, "float32", prompts, ru.mixed(prompts, seed=9), max_live=4, block_size=8)
+    scale = max(float(np.abs(v).max()) for v in a.values())
+    worst = max(float(np.abs(a[k] - v).max()) / scale for k, v in b.items())
+    assert worst <= 2e-6, f"{worst:.3e}"
+
+
+def test_trace_run_program(setups, tmp_path):
+    """The program itself: JSON lines in, <step>.f32 out, a ``done`` line after each step."""
+    d, prompts, want = setups("A", "float32")
+    steps = ru.mixed(prompts, seed=5)
+    proc = subprocess.run(
+        [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(d), "--dtype", "float32",
+         "--out", str(tmp_path / "out"), "--max-tokens", str(ru.pool_tokens(prompts, 4))],
+        input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.split("\n")[:len(steps)] == [f"done {s['step']}" for s in steps]
+    vocab = TINY_INIT["A"]["config"]["vocab_size"]
+    fed: dict = {}
+    got = {}
+    for s in steps:
+        wanted = sum(len(e["want"]) for e in s["entries"])
+        path = tmp_path / "out" / f"{s['step']}.f32"
+        assert path.exists() == (wanted > 0)
+        rows = np.fromfile(path, dtype="<f4").reshape(wanted, vocab) if wanted else None
+        row = 0
+        for e in s["entries"]:
+            start = fed.get(e["id"], 0)
+            for w in e["want"]:
+                got[(e["id"], start + w)] = rows[row]
+                row += 1
+            fed[e["id"]] = start + len(e["tokens"])
+    worst, where = ru.worst_error(got, want)
+    assert worst <= TOLERANCE["float32"], f"{worst:.3e} at {where}"
