@@ -1,0 +1,221 @@
+#!/usr/bin/env python3
+"""The headline measurement: Qwen3-0.6B-shape decoding and prefill on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one decode step of the engine's own step function on a batch of
+requests, each with a context of 512 tokens at the start: the cache write, the
+attention over the pages, every projection, the output projection and the greedy
+choice of the next token, which is what the next step is fed.  Weights are random
+(the random-weights mode writes the model folder, the loader reads it back),
+prompts are seeded uniform token ids.  One JSON line is printed.
+
+The sizes are those of BASELINE.json's third configuration.  Peaks are the
+published ones of the MI355X: 8 TB/s of HBM, 2.5 PFLOP/s dense bf16.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import random
+import sys
+import tempfile
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK = 8.0e12            # bytes a second
+MFMA_PEAK = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}
+
+# Qwen3-0.6B shape (BASELINE.json, configs[2]).
+CONFIG = {
+    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "hidden_act": "silu",
+    "attention_bias": False, "sliding_window": None, "hidden_size": 1024, "intermediate_size": 3072,
+    "num_hidden_layers": 28, "num_attention_heads": 16, "num_key_value_heads": 8, "head_dim": 128,
+    "rms_norm_eps": 1e-6, "rope_theta": 1000000.0, "vocab_size": 151936,
+    "max_position_embeddings": 4096, "tie_word_embeddings": True,
+}
+FULL_LAYERS = 28
+CONTEXT = 512
+PREFILL_TOKENS = 2048
+BLOCK_SIZE = 16
+
+
+def say(message: str) -> None:
+    print(f"[bench] {message}", file=sys.stderr, flush=True)
+
+
+def model_bytes_and_flops(cfg: dict, element: int):
+    """(bytes of weights a decode step reads once, matrix flops a token costs)."""
+    H, I, L = cfg["hidden_size"], cfg["intermediate_size"], cfg["num_hidden_layers"]
+    q = cfg["num_attention_heads"] * cfg["head_dim"]
+    kv = cfg["num_key_value_heads"] * cfg["head_dim"]
+    per_layer = H * (q + 2 * kv) + q * H + 2 * H * I + I * H
+    norms = L * (2 * H + 2 * cfg["head_dim"]) + H
+    head = cfg["vocab_size"] * H
+    params = L * per_layer + head
+    return (params + norms) * element, 2 * L * per_layer, 2 * head
+
+
+def kv_bytes_per_token(cfg: dict, element: int) -> int:
+    return 2 * cfg["num_hidden_layers"] * cfg["num_key_value_heads"] * cfg["head_dim"] * element
+
+
+class DecodeBench:
+    """B requests with ``context`` tokens each in the cache, then timed decode steps."""
+
+    def __init__(self, model, cache, batch: int, context: int, seed: int):
+        from paged_llm_rs_amd.engine.batch import StepEntry
+
+        self.model, self.cache, self.batch = model, cache, batch
+        self.StepEntry = StepEntry
+        rng = random.Random(seed)
+        vocab = model.spec.vocab_size
+        self.ids = list(range(1, batch + 1))
+        self.next_tokens = None
+        from paged_llm_rs_amd.engine.step import commit_step, run_step
+        from paged_llm_rs_amd import kernels
+        self.run_step, self.commit_step, self.kernels = run_step, commit_step, kernels
+        firsts = []
+        for i in self.ids:
+            cache.manager.add_sequence(i)
+            prompt = [rng.randrange(vocab) for _ in range(context)]
+            assert cache.manager.reserve(i, context)
+            entry = [StepEntry(i, prompt, 0, [context - 1])]
+            logits = run_step(model, cache, entry)
+            commit_step(cache, entry)
+            firsts.append(int(kernels.argmax(logits).item()))
+        self.tokens = firsts
+
+    def step(self) -> None:
+        manager = self.cache.manager
+        entries = []
+        for i, tok in zip(self.ids, self.tokens):
+            assert manager.reserve(i, 1)
+            entries.append(self.StepEntry(i, [tok], manager.tokens(i), [0]))
+        logits = self.run_step(self.model, self.cache, entries)
+        self.tokens = self.kernels.argmax(logits).cpu().tolist()   # the tokens the next step is fed
+        self.commit_step(self.cache, entries)
+
+    def free(self) -> None:
+        for i in self.ids:
+            self.cache.manager.free_sequence(i)
+
+
+def timed(fn, steps: int, warmup: int) -> float:
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - start) / steps
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=50)
+    parser.add_argument("--warmup", type=int, default=10)
+    parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--layers", type=int, default=FULL_LAYERS,
+                        help="fewer layers than the model has, where memory or time needs it; both numbers are reported")
+    parser.add_argument("--skip-points", action="store_true", help="leave out batch 1 and 64 and the prefill")
+    args = parser.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU; this engine has no multi-GPU path (N must be 1)")
+        return 2
+
+    import torch
+
+    from paged_llm_rs_amd import write_random_model
+    from paged_llm_rs_amd.cache import PagedCache
+    from paged_llm_rs_amd.engine.batch import StepEntry
+    from paged_llm_rs_amd.engine.step import commit_step, require_gpu, run_step
+    from paged_llm_rs_amd.parts.model import load_model
+
+    device = require_gpu("cuda:0")
+    cfg = dict(CONFIG)
+    cfg["num_hidden_layers"] = args.layers
+    tmp = tempfile.TemporaryDirectory()
+    say(f"writing a random {args.layers}-layer model folder")
+    t0 = time.time()
+    folder = write_random_model(Path(tmp.name) / "model", cfg, seed=0, std=0.02, gain_std=0.1, dtype="bfloat16")
+    say(f"written in {time.time() - t0:.0f} s; loading")
+    config, model = load_model(folder, "bfloat16", device)
+    say("loaded")
+
+    element = 2
+    weight_bytes, layer_flops, head_flops = model_bytes_and_flops(cfg, element)
+    kv_token = kv_bytes_per_token(cfg, element)
+    largest = max(64, args.batch)
+    pages = (largest * (CONTEXT + args.steps + args.warmup + 64) + PREFILL_TOKENS + 64) // BLOCK_SIZE + largest
+    cache = PagedCache(model.cache_layout, BLOCK_SIZE, pages, torch.bfloat16, device, max_seqs=largest + 1)
+
+    def decode_point(batch: int, steps: int, warmup: int):
+        bench = DecodeBench(model, cache, batch, CONTEXT, seed=batch)
+        seconds = timed(bench.step, steps, warmup)
+        context_mid = CONTEXT + warmup + steps / 2
+        bench.free()
+        return seconds, batch / seconds, weight_bytes + batch * context_mid * kv_token
+
+    say(f"decode, batch {args.batch}")
+    seconds, value, step_bytes = decode_point(args.batch, args.steps, args.warmup)
+    line = {
+        "metric": "Qwen3-0.6B bf16: decode tok/s @ batch 8, ctx 512",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(seconds * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic: random weights, uniform random token ids",
+        "config": {
+            "model": "Qwen3-0.6B shape", "global_batch": args.batch, "seq_len": CONTEXT, "parallelism": "none",
+            "layers": args.layers, "layers_full": FULL_LAYERS, "hidden": cfg["hidden_size"],
+            "q_heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
+            "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
+            "tied": True, "block_size": BLOCK_SIZE, "max_context": cfg["max_position_embeddings"],
+            "prefill_tokens": PREFILL_TOKENS,
+        },
+        "roofline": {"bound": "hbm", "achieved": round(step_bytes / seconds / 1e9, 1), "peak": HBM_PEAK / 1e9,
+                     "unit": "GB/s", "frac": round(step_bytes / seconds / HBM_PEAK, 4)},
+    }
+
+    if not args.skip_points:
+        points = {}
+        for batch in (1, 64):
+            say(f"decode, batch {batch}")
+            s, v, _ = decode_point(batch, max(args.steps // 2, 5), max(args.warmup // 2, 2))
+            points[f"decode_b{batch}"] = round(v, 1)
+        line["points"] = points
+
+        say(f"prefill, {PREFILL_TOKENS} tokens")
+        rng = random.Random(2048)
+        prompt = [rng.randrange(cfg["vocab_size"]) for _ in range(PREFILL_TOKENS)]
+
+        def prefill():
+            cache.manager.add_sequence(1000)
+            assert cache.manager.reserve(1000, PREFILL_TOKENS)
+            entry = [StepEntry(1000, prompt, 0, [PREFILL_TOKENS - 1])]
+            run_step(model, cache, entry)
+            cache.manager.free_sequence(1000)
+
+        seconds_prefill = timed(prefill, 5, 2)
+        d, nq = cfg["head_dim"], cfg["num_attention_heads"]
+        attention_flops = args.layers * 4 * nq * d * (PREFILL_TOKENS * (PREFILL_TOKENS + 1) // 2)
+        flops = layer_flops * PREFILL_TOKENS + head_flops + attention_flops
+        line["prefill"] = {"value": round(PREFILL_TOKENS / seconds_prefill, 1), "tokens": PREFILL_TOKENS,
+                           "ms": round(seconds_prefill * 1e3, 3),
+                           "frac": round(flops / seconds_prefill / MFMA_PEAK["bf16"], 4)}
+
+    print(json.dumps(line), flush=True)
+    tmp.cleanup()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

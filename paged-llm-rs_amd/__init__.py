@@ -11,5 +11,22 @@
 
 from .errors import (ConfigError, IoError, PagedLLMError, TensorError, UnsupportedError, WeightError)
 
-__all__ = ["ConfigError", "IoError", "PagedLLMError", "TensorError", "UnsupportedError", "WeightError"]
+
+
+def __getattr__(name):
+    # Engine and generate import torch and the native libraries; they load on first use.
+    if name in ("Engine", "generate", "Replayer"):
+        from . import engine
+        return getattr(engine, name)
+    if name in ("load_config", "register_architecture"):
+        from . import config
+        return getattr(config, name)
+    if name == "write_random_model":
+        from .weights import write_random_model
+        return write_random_model
+    raise AttributeError(name)
+
+
+__all__ = ["Engine", "generate", "Replayer", "load_config", "register_architecture", "write_random_model",
+           "ConfigError", "IoError", "PagedLLMError", "TensorError", "UnsupportedError", "WeightError"]
 __version__ = "0.1.0"

@@ -1,0 +1,262 @@
+"""The engine loop and the Python entry point.
+
+One iteration (reference: crates/pagedllm-server/src/engine.rs:180-250): ask the
+scheduler for a plan, run the step function, choose a token for every request a
+token comes back for, commit.  A failed step fails the requests in it and
+commits nothing; lengths only move after a step has succeeded.
+"""
+
+from __future__ import annotations
+
+import itertools
+import time
+from dataclasses import dataclass, field
+from pathlib import Path
+from typing import Optional
+
+import torch
+
+from .. import kernels
+from ..cache import PagedCache
+from ..config import GenerationConfig
+from ..errors import ConfigError, PagedLLMError
+from ..parts.model import DTYPES, load_model
+from ..sampling.sampler import Sampling
+from ..weights.safetensors_io import SafetensorsFile
+from . import scheduler as sched
+from .step import require_gpu, run_step
+
+_seed_counter = itertools.count()
+
+
+def default_seed() -> int:
+    """A seed for a request that names none: the clock mixed with a counter, so two
+    requests in the same second do not draw the same tokens (reference: routes.rs:69-80)."""
+    n = next(_seed_counter)
+    return (int(time.time()) * 0x9E3779B97F4A7C15 + n * 0xBF58476D1CE4E5B9) & (2 ** 64 - 1)
+
+
+def checkpoint_dtype(model_dir) -> str:
+    """``auto``: whatever the checkpoint stores its embedding in (reference: model/mod.rs:175)."""
+    f = SafetensorsFile(Path(model_dir) / "model.safetensors")
+    try:
+        for name in f.names():
+            if name.endswith("embed_tokens.weight"):
+                return "float32" if f.dtype(name) in (torch.float32, torch.float64) else "bfloat16"
+    finally:
+        f.close()
+    return "bfloat16"
+
+
+@dataclass
+class Completion:
+    """What a finished request returns."""
+    tokens: list = field(default_factory=list)
+    finish: str = ""
+    prompt_tokens: int = 0
+    preemptions: int = 0
+
+
+class Engine:
+    """A model, its cache and its scheduler on one GPU.
+
+    The options carry the names and meanings of the reference's command line
+    (crates/pagedllm-server/src/main.rs:20-71): ``dtype`` auto|f32|bf16,
+    ``block_size`` (16), ``cache_mib`` (3584), ``max_batch`` (16), ``prefix_cache``
+    (on), ``chunk`` (128; None or "off" runs a prompt whole), ``max_tokens`` (512,
+    the budget of a request that names none).  ``num_blocks`` sets the pool
+    directly instead of ``cache_mib``.
+    """
+
+    def __init__(self, model, dtype: str = "auto", block_size: int = 16, cache_mib: int = 3584,
+                 num_blocks: Optional[int] = None, max_batch: int = 16, chunk=128, prefix_cache: bool = True,
+                 max_tokens: int = 512, device="cuda:0", sampler: str = "device"):
+        self.device = require_gpu(device)
+        dtype = {"auto": None, "f32": "float32", "bf16": "bfloat16"}.get(dtype, dtype)
+        if dtype is None:
+            dtype = checkpoint_dtype(model)
+        if dtype not in ("float32", "bfloat16"):
+            raise ConfigError(f"dtype {dtype!r}, which is none of auto, f32, bf16")
+        if chunk == "off":
+            chunk = None
+        if chunk is not None and int(chunk) < 1:
+            raise ConfigError("--chunk 0 would carry nothing")
+        if sampler not in ("device", "host"):
+            raise ConfigError(f"sampler {sampler!r}, which is neither device nor host")
+        self.dtype = dtype
+        self.model_dir = Path(model)
+        self.config, self.model = load_model(model, dtype, self.device)
+        self.generation = GenerationConfig.from_dir(model)
+        element = 4 if dtype == "float32" else 2
+        layout = self.model.cache_layout
+        if num_blocks is None:
+            # The page count follows from the byte budget, so changing the page
+            # size compares two layouts at the same memory (reference: main.rs:89-120).
+            num_blocks = layout.blocks_within(int(cache_mib) << 20, block_size, element)
+        self.block_size, self.num_blocks = block_size, num_blocks
+        self.bytes_per_token = layout.bytes_per_token(element)
+        self.cache = PagedCache(layout, block_size, num_blocks, DTYPES[dtype], self.device,
+                                max_seqs=max(max_batch * 2, 8))
+        self.scheduler = sched.Scheduler(self.cache.manager, max_batch=max_batch,
+                                         chunk=None if chunk is None else int(chunk),
+                                         max_positions=self.model.spec.max_positions, prefix_cache=prefix_cache)
+        self.default_max_tokens = max_tokens
+        self.sampler = sampler
+        self._next_id = 1
+        self._results: dict = {}
+        self._open: dict = {}
+        self._greedy: dict = {}
+        self._chunk = None if chunk is None else int(chunk)
+
+    # -- requests -------------------------------------------------------------------------
+
+    def resolve_sampling(self, temperature=None, top_k=None, top_p=None) -> Sampling:
+        """The request's value, else the model's generation config, else temperature 1;
+        an explicit temperature of zero drops top-k and top-p (reference: routes.rs:106-126)."""
+        if temperature is None:
+            temperature = self.generation.temperature if self.generation.temperature is not None else 1.0
+        if temperature <= 0.0:
+            return Sampling(float(temperature), None, None)
+        return Sampling(float(temperature), top_k if top_k is not None else self.generation.top_k,
+                        top_p if top_p is not None else self.generation.top_p)
+
+    def submit(self, prompt, max_tokens: Optional[int] = None, temperature=0.0, top_k=None, top_p=None,
+               seed: Optional[int] = None, stop_tokens=None) -> int:
+        prompt = [int(t) for t in prompt]
+        if not prompt:
+            raise ConfigError("cannot generate from an empty prompt")
+        vocab = self.model.spec.vocab_size
+        if min(prompt) < 0 or max(prompt) >= vocab:
+            raise ConfigError(f"a prompt token outside the vocabulary of {vocab}")
+        how = self.resolve_sampling(temperature, top_k, top_p)
+        stops = list(self.generation.eos_token_ids) if stop_tokens is None else [int(t) for t in stop_tokens]
+        seq_id = self._next_id
+        self._next_id += 1
+        self.scheduler.submit(seq_id, prompt, how.temperature, how.top_k, how.top_p,
+                              self.default_max_tokens if max_tokens is None else int(max_tokens), stops,
+                              default_seed() if seed is None else int(seed))
+        self._open[seq_id] = Completion(prompt_tokens=len(prompt))
+        self._greedy[seq_id] = how.is_greedy
+        return seq_id
+
+    def cancel(self, seq_id: int) -> None:
+        self.scheduler.cancel(seq_id)
+        self._open.pop(seq_id, None)
+
+    # -- the loop ---------------------------------------------------------------------------
+
+    def _choose(self, plan, logits: torch.Tensor) -> list:
+        """One token per id of the plan.  Greedy rows are an argmax on the device;
+        the logits of the others go to the host sampler with the request's generator."""
+        if not plan.ids:
+            return []      # a portion in the middle of a prompt: the logits have no rows and are not touched
+        if logits.shape[0] != len(plan.ids):
+            raise PagedLLMError(f"{logits.shape[0]} rows of logits for {len(plan.ids)} requests")
+        greedy = [self._greedy.get(i, True) for i in plan.ids]
+        chosen = [0] * len(plan.ids)
+        if self.sampler == "device" and any(greedy):
+            picked = kernels.argmax(logits).cpu().tolist()
+            for row, g in enumerate(greedy):
+                if g:
+                    chosen[row] = picked[row]
+        rows_on_host = [r for r, g in enumerate(greedy) if not (g and self.sampler == "device")]
+        if rows_on_host:
+            index = torch.tensor(rows_on_host, device=logits.device)
+            host = logits.index_select(0, index).cpu().numpy()
+            for k, row in enumerate(rows_on_host):
+                chosen[row] = self.scheduler.sample_on_host(plan.ids[row], host[k])
+        return chosen
+
+    def step(self):
+        """One iteration.  Returns the outcome, or None when there is nothing to run."""
+        plan = self.scheduler.plan()
+        if plan.kind == sched.IDLE:
+            outcome = self.scheduler.drain_finished()
+            self._record(outcome)
+            return outcome if outcome.finished else None
+        sampled = []
+        if plan.entries:
+            try:
+                logits = run_step(self.model, self.cache, plan.entries)
+                sampled = self._choose(plan, logits)
+            except PagedLLMError:
+                # A failed step fails every request in it; nothing was committed
+                # (reference: engine.rs:340-348).
+                for e in plan.entries:
+                    self.scheduler.cancel(e.seq_id)
+                    done = self._open.pop(e.seq_id, None)
+                    if done is not None:
+                        done.finish = "failed"
+                        self._results[e.seq_id] = done
+                raise
+        outcome = self.scheduler.commit(sampled)
+        self._record(outcome)
+        return outcome
+
+    def _record(self, outcome) -> None:
+        for seq_id, token in outcome.tokens:
+            if seq_id in self._open:
+                self._open[seq_id].tokens.append(token)
+        for f in outcome.finished:
+            done = self._open.pop(f.id, None)
+            if done is None:
+                continue
+            done.finish, done.prompt_tokens, done.preemptions = f.finish, f.prompt_tokens, f.preemptions
+            self._greedy.pop(f.id, None)
+            self._results[f.id] = done
+
+    def run(self) -> None:
+        """Run until every submitted request has finished."""
+        while self._open:
+            if self.step() is None and self._open:
+                raise PagedLLMError("the scheduler idles while requests are open")
+
+    def take_result(self, seq_id: int) -> Completion:
+        return self._results.pop(seq_id)
+
+    def generate(self, prompts, max_tokens: Optional[int] = None, temperature=0.0, top_k=None, top_p=None,
+                 seed: int = 0, stop_tokens=None) -> list:
+        """Generate for a list of prompts (lists of token ids).  Returns, in order,
+        dicts of ``tokens``, ``finish`` ("stop" or "length"), ``prompt_tokens`` and
+        ``preemptions``.  Request i draws from seed + i."""
+        ids = [self.submit(p, max_tokens, temperature, top_k, top_p, seed + i, stop_tokens)
+               for i, p in enumerate(prompts)]
+        self.run()
+        out = []
+        for i in ids:
+            c = self.take_result(i)
+            out.append({"tokens": c.tokens, "finish": c.finish, "prompt_tokens": c.prompt_tokens,
+                        "preemptions": c.preemptions})
+        return out
+
+    def metrics(self) -> dict:
+        m = self.scheduler.metrics()
+        manager = self.cache.manager
+        m.update({k: manager.counter(k) for k in
+                  ("available", "total", "in_use", "cached_blocks", "handed_out", "hits", "misses", "evictions")})
+        m["wasted_tokens"] = self.scheduler.wasted_tokens()
+        return m
+
+    def describe(self) -> str:
+        """The start-up banner (reference: main.rs:133-158)."""
+        chunk = self.scheduler_chunk
+        return (
+            f"paged-llm-rs_amd\n  model    {self.model_dir}\n"
+            f"  backend  MI355X (gfx950), dtype {self.dtype}, chunk {chunk if chunk else 'off'}\n"
+            f"  sampling temperature {self.generation.temperature}, top_p {self.generation.top_p}, "
+            f"top_k {self.generation.top_k}, from the model's generation config\n"
+            f"  stop     {self.generation.eos_token_ids}\n"
+            f"  cache    {self.num_blocks} blocks of {self.block_size} tokens, "
+            f"{self.cache.bytes / 2 ** 30:.2f} GiB, {self.bytes_per_token} bytes a token, "
+            f"{self.num_blocks * self.block_size} tokens held at once")
+
+    @property
+    def scheduler_chunk(self):
+        return self._chunk
+
+
+def generate(model, prompts, max_tokens: int = 16, temperature=0.0, top_k=None, top_p=None, seed: int = 0,
+             stop_tokens=None, **engine_options) -> list:
+    """Load ``model`` (a folder), generate for ``prompts`` and return the completions."""
+    return Engine(model, **engine_options).generate(prompts, max_tokens, temperature, top_k, top_p, seed,
+                                                    stop_tokens)

@@ -234,6 +234,19 @@ def argmax(logits: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tenso
     return out
 
 
+_attention_mode = "kernel"
+
+
+def set_attention(mode: str) -> None:
+    """``kernel``: the matrix-core kernels where they apply; ``tensor``: the plain
+    kernel with 32-bit arithmetic that they are checked against (the reference's
+    flag of the same name chooses between its kernel and its tensor path)."""
+    global _attention_mode
+    if mode not in ("kernel", "tensor"):
+        raise TensorError(f"attention {mode!r}, which is neither tensor nor kernel")
+    _attention_mode = mode
+
+
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nkv: int, d: int,
                     scale: float, window: int = 0) -> torch.Tensor:
     """Attention for every token of a step.  ``qkv`` rows begin with the rotated queries."""

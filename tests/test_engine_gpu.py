@@ -1,0 +1,143 @@
+"""Generation through the entry point: greedy against the plain implementation,
+what happens when pages run out, prefix sharing, sampling with a seed, the
+command line."""
+
+from __future__ import annotations
+
+import json
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+import replay_util as ru
+from conftest import ROOT, TINY_INIT, load_plain
+
+pytestmark = pytest.mark.gpu
+
+
+def plain_greedy_check(model_dir, prompt, produced, noise):
+    """Every produced token is the plain implementation's argmax, or differs from it
+    by less than the engine's rounding noise (the reference's rule for bfloat16:
+    tests/reference_model.rs:260-297)."""
+    cfg, weights = load_plain(model_dir)
+    tokens = list(prompt)
+    for token in produced:
+        logits = plain.forward(weights, cfg, tokens)[-1]
+        best = int(torch.argmax(logits))
+        if token != best:
+            gap = float(logits[best] - logits[token])
+            assert gap <= noise * float(logits.abs().max()), f"token {token} against {best}: gap {gap:.3e}"
+        tokens.append(token)
+
+
+@pytest.mark.parametrize("name,dtype,chunk", [("A", "f32", 128), ("B", "f32", 7), ("B", "bf16", 7),
+                                              ("A", "bf16", None), ("C", "f32", 5)])
+def test_greedy_generation_matches_the_plain_implementation(model_dirs, name, dtype, chunk):
+    from paged_llm_rs_amd import Engine
+
+    long_name = "float32" if dtype == "f32" else "bfloat16"
+    d = model_dirs(name, long_name)
+    vocab = TINY_INIT[name]["config"]["vocab_size"]
+    prompts = list(ru.make_prompts(vocab, [5, 17, 33, 1], seed=3).values())
+    engine = Engine(d, dtype=dtype, block_size=8, num_blocks=64, max_batch=4, chunk=chunk)
+    out = engine.generate(prompts, max_tokens=16, temperature=0.0, stop_tokens=[])
+    for prompt, result in zip(prompts, out):
+        assert result["finish"] == "length" and len(result["tokens"]) == 16
+        assert result["prompt_tokens"] == len(prompt)
+        plain_greedy_check(d, prompt, result["tokens"], 1e-5 if dtype == "f32" else 2e-2)
+    m = engine.metrics()
+    assert m["available"] == m["total"] and m["tokens"] == 64
+
+
+def test_running_out_of_pages_changes_no_token(model_dirs):
+    """Eviction recomputes a request from its history; the tokens it had already
+    returned stay returned and the rest come out the same."""
+    from paged_llm_rs_amd import Engine
+
+    d = model_dirs("A", "float32")
+    prompts = list(ru.make_prompts(256, [9, 12, 7, 10], seed=8).values())
+    roomy = Engine(d, dtype="f32", block_size=4, num_blocks=64, max_batch=4, chunk=16, prefix_cache=False)
+    want = roomy.generate(prompts, max_tokens=24, stop_tokens=[])
+    tight = Engine(d, dtype="f32", block_size=4, num_blocks=18, max_batch=4, chunk=16, prefix_cache=False)
+    got = tight.generate(prompts, max_tokens=24, stop_tokens=[])
+    assert tight.metrics()["preemptions"] > 0, "the pool was meant to run dry"
+    assert [g["tokens"] for g in got] == [w["tokens"] for w in want]
+    assert sum(g["preemptions"] for g in got) == tight.metrics()["preemptions"]
+    assert tight.metrics()["available"] == 18
+
+
+def test_a_prompt_the_pool_cannot_hold_is_refused(model_dirs):
+    from paged_llm_rs_amd import Engine
+
+    engine = Engine(model_dirs("A", "float32"), dtype="f32", block_size=4, num_blocks=4, max_batch=2, chunk=8)
+    out = engine.generate([[1] * 40, [2, 3]], max_tokens=3, stop_tokens=[])
+    assert out[0]["finish"] == "length" and out[0]["tokens"] == []
+    assert len(out[1]["tokens"]) == 3
+
+
+def test_prefix_sharing_changes_no_token(model_dirs):
+    """Two prompts with a common head of 16 tokens (two pages of 8): shared and
+    unshared runs give the same tokens (reference: tests/prefix.rs:87-139)."""
+    from paged_llm_rs_amd import Engine
+
+    d = model_dirs("B", "float32")
+    head = list(ru.make_prompts(384, [16], seed=5).values())[0]
+    tails = list(ru.make_prompts(384, [9, 24, 3], seed=6).values())
+    prompts = [head + t for t in tails] + [head + tails[0]]
+    on = Engine(d, dtype="f32", block_size=8, num_blocks=64, max_batch=1, chunk=7, prefix_cache=True)
+    off = Engine(d, dtype="f32", block_size=8, num_blocks=64, max_batch=1, chunk=7, prefix_cache=False)
+    got = on.generate(prompts, max_tokens=8, stop_tokens=[])
+    want = off.generate(prompts, max_tokens=8, stop_tokens=[])
+    assert [g["tokens"] for g in got] == [w["tokens"] for w in want]
+    assert on.metrics()["cached_tokens"] >= 3 * 16 and off.metrics()["cached_tokens"] == 0
+    assert got[0]["tokens"] == got[3]["tokens"], "the same prompt gives the same tokens"
+
+
+@pytest.mark.parametrize("sampler", ["device", "host"])
+def test_sampling_with_a_seed_repeats_and_stop_tokens_end_a_request(model_dirs, sampler):
+    from paged_llm_rs_amd import Engine
+
+    d = model_dirs("B", "float32")
+    prompts = list(ru.make_prompts(384, [1, 9, 24, 40], seed=1).values())
+    engine = Engine(d, dtype="f32", block_size=8, num_blocks=64, max_batch=4, chunk=7, sampler=sampler)
+    a = engine.generate(prompts, max_tokens=12, temperature=0.8, seed=1234, stop_tokens=[])
+    b = engine.generate(prompts, max_tokens=12, temperature=0.8, seed=1234, stop_tokens=[])
+    c = engine.generate(prompts, max_tokens=12, temperature=0.8, seed=99, stop_tokens=[])
+    assert [x["tokens"] for x in a] == [x["tokens"] for x in b]
+    assert [x["tokens"] for x in a] != [x["tokens"] for x in c]
+    # the plain sampler on the plain logits, with the request's own generator, picks the same tokens
+    cfg, weights = load_plain(d)
+    rng = plain.SplitMix64(1234 + 1)
+    tokens = list(prompts[1])
+    for produced in a[1]["tokens"]:
+        logits = plain.forward(weights, cfg, tokens)[-1].float().numpy()
+        assert plain.sample(logits, 0.8, None, None, rng) == produced
+        tokens.append(produced)
+    # a stop token ends the request and is not part of the output
+    stop = a[0]["tokens"][3]
+    cut = engine.generate(prompts[:1], max_tokens=12, temperature=0.8, seed=1234, stop_tokens=[stop])
+    assert cut[0]["finish"] == "stop" and cut[0]["tokens"] == a[0]["tokens"][:a[0]["tokens"].index(stop)]
+    # top_k 1 is greedy whatever the temperature
+    g = engine.generate(prompts[:2], max_tokens=6, temperature=0.0, stop_tokens=[])
+    k = engine.generate(prompts[:2], max_tokens=6, temperature=3.0, top_k=1, seed=5, stop_tokens=[])
+    assert [x["tokens"] for x in g] == [x["tokens"] for x in k]
+
+
+def test_the_command_line(model_dirs, tmp_path):
+    d = model_dirs("A", "float32")
+    proc = subprocess.run(
+        [sys.executable, str(ROOT / "bin" / "pagedllm"), "--model", str(d), "--dtype", "f32", "--max-tokens", "5",
+         "--block-size", "16", "--cache-mib", "1", "--max-batch", "2", "--chunk", "off", "--prefix-cache", "off",
+         "--prompt-ids", "3,17,42,8", "--prompt-ids", "1 2 3", "--temperature", "0", "--stop-ids", ""],
+        capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = [json.loads(l) for l in proc.stdout.strip().splitlines()]
+    assert len(lines) == 2 and all(len(l["tokens"]) == 5 and l["finish"] == "length" for l in lines)
+    assert "blocks of 16 tokens" in proc.stderr
+    plain_greedy_check(d, [3, 17, 42, 8], lines[0]["tokens"], 1e-5)
+    bad = subprocess.run([sys.executable, str(ROOT / "bin" / "pagedllm"), "--model", str(d), "--chunk", "0"],
+                         capture_output=True, text=True, timeout=600)
+    assert bad.returncode == 1 and "--chunk 0" in bad.stderr

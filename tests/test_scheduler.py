@@ -1,0 +1,474 @@
+"""The scheduler's decisions without a model: every step is answered with a constant
+token.  The scenarios are the reference's own (scheduler.rs:832-1369)."""
+
+from __future__ import annotations
+
+import random
+
+import pytest
+
+from paged_llm_rs_amd.cache import CacheManager, GroupGeometry
+from paged_llm_rs_amd.engine import scheduler as sched
+from paged_llm_rs_amd.errors import ConfigError
+
+
+def scheduler(blocks, block_size, max_batch, chunk=128, window=0, state_slots=0, max_positions=0):
+    manager = CacheManager([GroupGeometry(block_size, blocks, window)], state_slots)
+    return sched.Scheduler(manager, max_batch=max_batch, chunk=chunk, max_positions=max_positions)
+
+
+def submit(s, seq_id, prompt_len, max_tokens, prompt=None):
+    s.submit(seq_id, prompt if prompt is not None else [1] * prompt_len, 0.0, None, None, max_tokens, [99], seq_id)
+
+
+def step(s, token=7):
+    plan = s.plan()
+    outcome = s.commit([token] * len(plan.ids))
+    return plan, outcome
+
+
+def test_a_prompt_is_admitted_before_anything_decodes():
+    """scheduler.rs:832-845"""
+    s = scheduler(64, 4, 4, chunk=None)
+    submit(s, 1, 3, 10)
+    submit(s, 2, 5, 10)
+    assert step(s)[0].kind == sched.PREFILL
+    assert step(s)[0].kind == sched.PREFILL
+    assert step(s)[0].kind == sched.DECODE
+    assert s.running == 2
+
+
+def test_a_sequence_takes_only_the_blocks_its_tokens_need():
+    """scheduler.rs:847-856"""
+    s = scheduler(64, 16, 4)
+    submit(s, 1, 20, 100)
+    step(s)
+    assert s.manager.in_use() == 2 and s.manager.available() == 62
+
+
+def test_a_block_is_taken_only_when_the_last_one_fills():
+    """scheduler.rs:858-871"""
+    s = scheduler(64, 4, 4)
+    submit(s, 1, 3, 20)
+    step(s)
+    assert s.manager.in_use() == 1
+    step(s)
+    assert s.manager.in_use() == 1
+    step(s)
+    assert s.manager.in_use() == 2
+
+
+def test_late_arrivals_join_the_running_batch():
+    """scheduler.rs:873-893"""
+    s = scheduler(64, 8, 4, chunk=None)
+    submit(s, 1, 3, 20)
+    for _ in range(4):
+        step(s)
+    submit(s, 2, 3, 20)
+    assert step(s)[0].kind == sched.PREFILL
+    plan, _ = step(s)
+    assert plan.kind == sched.DECODE and plan.ids == [1, 2]
+    assert len(plan.entries) == 2
+    assert plan.entries[0].start != plan.entries[1].start
+
+
+def test_a_stop_token_ends_a_sequence_and_gives_its_blocks_back():
+    """scheduler.rs:895-906"""
+    s = scheduler(64, 4, 4)
+    submit(s, 1, 6, 10)
+    step(s)
+    assert s.manager.in_use() == 2
+    _, outcome = step(s, 99)
+    assert outcome.tokens == [], "the stop token is not output"
+    assert [(f.id, f.finish) for f in outcome.finished] == [(1, "stop")]
+    assert s.manager.available() == 64
+
+
+def test_the_pool_running_dry_evicts_the_newest_and_recomputes_it():
+    """scheduler.rs:908-932"""
+    s = scheduler(4, 4, 50, chunk=None)
+    submit(s, 1, 4, 50)
+    submit(s, 2, 4, 50)
+    step(s)
+    step(s)
+    assert s.manager.available() == 2
+    for _ in range(10):
+        step(s)
+    m = s.metrics()
+    assert m["preemptions"] > 0 and m["recomputed_tokens"] > 0
+    assert s.waiting + s.running == 2, "what was evicted went back to the queue"
+
+
+def test_the_sequence_that_arrived_first_is_never_the_one_evicted():
+    """scheduler.rs:934-954"""
+    s = scheduler(4, 4, 50)
+    submit(s, 1, 4, 50)
+    submit(s, 2, 4, 50)
+    step(s)
+    step(s)
+    for _ in range(12):
+        step(s)
+        assert 1 in s.running_ids() or s.waiting > 0
+    assert s.metrics()["preemptions"] > 0
+
+
+def test_a_prompt_longer_than_the_whole_pool_is_refused():
+    """scheduler.rs:956-966"""
+    s = scheduler(2, 4, 4)
+    submit(s, 1, 20, 10)
+    plan = s.plan()
+    assert plan.kind == sched.REFUSED and plan.refused == 1
+    outcome = s.commit([])
+    assert [(f.id, f.finish) for f in outcome.finished] == [(1, "length")]
+    assert s.waiting == 0 and s.manager.available() == 2
+
+
+def test_cancelling_gives_the_blocks_back_at_once():
+    """scheduler.rs:968-977"""
+    s = scheduler(8, 4, 4)
+    submit(s, 1, 8, 100)
+    step(s)
+    assert s.manager.in_use() == 2
+    s.cancel(1)
+    assert s.manager.available() == 8 and s.running == 0
+    submit(s, 2, 8, 100)
+    s.cancel(2)
+    assert s.waiting == 0
+
+
+def test_an_idle_scheduler_plans_nothing():
+    """scheduler.rs:979-983"""
+    assert scheduler(8, 4, 4).plan().kind == sched.IDLE
+
+
+def test_a_second_request_with_the_same_prompt_reuses_the_blocks_of_the_first():
+    """scheduler.rs:985-1005"""
+    s = scheduler(64, 4, 4)
+    submit(s, 1, 12, 4)
+    for _ in range(5):
+        step(s)
+    assert s.running == 0
+    first = s.metrics()
+    assert first["cached_tokens"] == 0 and first["prefilled_tokens"] >= 12
+    submit(s, 2, 12, 4)
+    step(s)
+    second = s.metrics()
+    assert second["cached_tokens"] == 8
+    assert second["prefilled_tokens"] - first["prefilled_tokens"] == 4
+
+
+def test_sharing_stops_where_the_prompts_stop_agreeing():
+    """scheduler.rs:1007-1032"""
+    s = scheduler(64, 4, 4)
+    common = list(range(12))
+    submit(s, 1, 0, 2, prompt=common + [100, 101, 102, 103])
+    for _ in range(4):
+        step(s)
+    before = s.metrics()["cached_tokens"]
+    submit(s, 2, 0, 2, prompt=common + [200, 201, 202, 203])
+    step(s)
+    assert s.metrics()["cached_tokens"] - before == 12
+
+
+def test_a_prefix_can_be_shared_while_its_first_owner_is_still_generating():
+    """scheduler.rs:1034-1052"""
+    s = scheduler(64, 4, 100)
+    submit(s, 1, 12, 50)
+    for _ in range(3):
+        step(s)
+    assert s.running == 1
+    submit(s, 2, 12, 50)
+    step(s)
+    assert s.metrics()["cached_tokens"] == 8
+    assert s.running == 2
+
+
+def test_nothing_is_shared_when_the_cache_is_off():
+    """scheduler.rs:1054-1068"""
+    s = scheduler(64, 4, 4)
+    s.set_prefix_cache(False)
+    for seq_id in (1, 2):
+        submit(s, seq_id, 12, 4)
+        for _ in range(5):
+            step(s)
+    assert s.metrics()["cached_tokens"] == 0 and s.metrics()["prefix_hit_rate"] == 0.0
+
+
+def test_cached_blocks_give_way_before_a_sequence_is_refused():
+    """scheduler.rs:1070-1096"""
+    s = scheduler(5, 4, 4)
+    for seq_id in (1, 2, 3):
+        submit(s, seq_id, 0, 2, prompt=[t + seq_id * 1000 for t in range(12)])
+        for _ in range(4):
+            step(s)
+    assert s.waiting == 0 and s.running == 0
+    assert s.manager.counter("evictions") > 0
+
+
+def test_what_paging_wastes_is_bounded_by_one_block_a_sequence():
+    """scheduler.rs:1098-1113"""
+    s = scheduler(64, 16, 8)
+    for seq_id in range(1, 5):
+        submit(s, seq_id, 20, 50)
+    for _ in range(4):
+        step(s)
+    assert s.running == 4
+    assert s.wasted_tokens() < 4 * 16
+
+
+def test_the_average_batch_counts_only_decode_passes():
+    """scheduler.rs:1115-1130"""
+    s = scheduler(64, 8, 4, chunk=None)
+    submit(s, 1, 2, 10)
+    submit(s, 2, 2, 10)
+    for _ in range(5):
+        step(s)
+    m = s.metrics()
+    assert m["prefills"] == 2 and m["steps"] == 5
+    assert abs(m["mean_batch"] - 2.0) < 1e-9
+
+
+def test_a_long_prompt_is_fed_a_slice_at_a_time_within_the_budget():
+    """scheduler.rs:1132-1163"""
+    s = scheduler(64, 8, 8, chunk=16)
+    submit(s, 1, 100, 4)
+    slices = fed = 0
+    while True:
+        plan, outcome = step(s)
+        if plan.kind == sched.DECODE:
+            break
+        assert plan.kind == sched.MIXED
+        assert plan.num_tokens <= 16
+        slices += 1
+        fed += plan.num_tokens
+        assert slices < 20
+        if not outcome.tokens:
+            assert fed < 100, "the prompt ran out without producing a token"
+    assert slices >= 6 and fed == 100
+
+
+def test_a_prompt_arriving_mid_flight_does_not_stop_the_sequences_already_decoding():
+    """scheduler.rs:1165-1194"""
+    s = scheduler(64, 8, 8, chunk=16)
+    submit(s, 1, 4, 40)
+    submit(s, 2, 4, 40)
+    for _ in range(6):
+        step(s)
+    assert s.running == 2
+    submit(s, 3, 90, 40)
+    for _ in range(5):
+        plan, outcome = step(s)
+        assert plan.kind == sched.MIXED
+        produced = [i for i, _ in outcome.tokens]
+        assert 1 in produced and 2 in produced and 3 not in produced
+
+
+def test_a_prompts_last_slice_is_the_one_that_produces_its_first_token():
+    """scheduler.rs:1196-1210"""
+    s = scheduler(64, 8, 8, chunk=16)
+    submit(s, 1, 40, 4)
+    answered = [bool(step(s)[1].tokens) for _ in range(4)]
+    assert answered == [False, False, True, True]
+
+
+def test_the_budget_covers_the_decodes_and_the_slice_together():
+    """scheduler.rs:1212-1237"""
+    s = scheduler(64, 8, 8, chunk=8)
+    for seq_id in (1, 2, 3):
+        submit(s, seq_id, 2, 40)
+    for _ in range(6):
+        step(s)
+    assert s.running == 3
+    submit(s, 9, 60, 40)
+    plan, _ = step(s)
+    assert plan.kind == sched.MIXED and plan.num_tokens == 8
+    assert dict(plan.advanced)[9] == 5
+    # decodes come first, then the slice
+    assert [len(e.tokens) for e in plan.entries] == [1, 1, 1, 5]
+
+
+def test_chunking_off_gives_a_prompt_its_own_pass_and_on_does_not():
+    """scheduler.rs:1239-1256"""
+    for chunk, alone in ((None, True), (16, False)):
+        s = scheduler(64, 8, 8, chunk=chunk)
+        submit(s, 1, 4, 40)
+        for _ in range(3):
+            step(s)
+        submit(s, 2, 20, 40)
+        _, outcome = step(s)
+        assert any(i == 1 for i, _ in outcome.tokens) == (not alone)
+
+
+def test_a_dry_pool_evicts_under_chunking_too():
+    """scheduler.rs:1258-1280"""
+    s = scheduler(6, 4, 50, chunk=8)
+    for seq_id in (1, 2, 3):
+        submit(s, seq_id, 4, 50)
+    for _ in range(20):
+        step(s)
+    m = s.metrics()
+    assert m["preemptions"] > 0 and m["tokens"] > 20
+    assert s.running + s.waiting == 3
+
+
+def test_a_slices_tokens_carry_the_positions_they_hold_in_the_prompt():
+    """scheduler.rs:1282-1330"""
+    s = scheduler(64, 8, 8, chunk=16)
+    submit(s, 1, 4, 40)
+    for _ in range(3):
+        step(s)
+    assert s.running == 1
+    submit(s, 2, 0, 4, prompt=list(range(100, 140)))
+    expected = 0
+    for _ in range(3):
+        plan = s.plan()
+        assert plan.kind == sched.MIXED
+        entry = [e for e in plan.entries if e.seq_id == 2][0]
+        assert plan.entries[-1] is entry, "the resident's rows come first"
+        assert entry.start == expected
+        assert entry.tokens == list(range(100 + expected, 100 + expected + len(entry.tokens)))
+        assert dict(plan.advanced)[2] == len(entry.tokens)
+        expected += len(entry.tokens)
+        assert entry.want == ([len(entry.tokens) - 1] if expected == 40 else [])
+        s.commit([7] * len(plan.ids))
+    assert expected == 40
+
+
+def test_a_prompt_that_is_admitted_gets_a_slice_in_the_pass_that_admitted_it():
+    """scheduler.rs:1332-1369"""
+    s = scheduler(9, 4, 8, chunk=64)
+    for seq_id in range(1, 5):
+        submit(s, seq_id, 4, 30)
+    before = s.metrics()["prefills"]
+    for _ in range(60):
+        plan = s.plan()
+        after = s.metrics()["prefills"]
+        if after > before:
+            assert plan.kind in (sched.MIXED, sched.PREFILL)
+            assert plan.advanced, "a sequence was admitted and the pass ran nothing for it"
+        before = after
+        s.commit([7] * len(plan.ids))
+    assert s.metrics()["prefills"] >= 4
+
+
+# --- beyond the reference's scenarios ---------------------------------------------------------------
+
+def test_bad_requests_are_refused_at_submission():
+    """session/sampler refusals: scheduler.rs:68-70, sampler.rs:72-95"""
+    s = scheduler(8, 4, 4)
+    with pytest.raises(ConfigError):
+        s.submit(1, [], 0.0, None, None, 4, [], 0)
+    with pytest.raises(ConfigError):
+        s.submit(1, [1], -0.5, None, None, 4, [], 0)
+    with pytest.raises(ConfigError):
+        s.submit(1, [1], 1.0, 0, None, 4, [], 0)
+    with pytest.raises(ConfigError):
+        s.submit(1, [1], 1.0, None, 1.5, 4, [], 0)
+    with pytest.raises(ConfigError):
+        sched.Scheduler(CacheManager([GroupGeometry(4, 4)]), chunk=0)
+
+
+def test_a_request_stops_at_the_models_longest_position():
+    s = scheduler(64, 4, 4, max_positions=10)
+    submit(s, 1, 8, 100)
+    produced = 0
+    for _ in range(10):
+        _, outcome = step(s)
+        produced += len(outcome.tokens)
+        if outcome.finished:
+            assert outcome.finished[0].finish == "length"
+            break
+    # positions 0..9 exist: 8 prompt tokens, then tokens fed at 8 and 9, and the last one sampled is never fed
+    assert produced == 3 and s.running == 0
+    submit(s, 2, 11, 5)
+    assert s.plan().kind == sched.REFUSED
+
+
+def test_a_request_alone_that_outgrows_the_pool_ends_instead_of_idling_forever():
+    s = scheduler(2, 4, 4)
+    submit(s, 1, 6, 100)
+    finished = None
+    for _ in range(8):
+        plan = s.plan()
+        if plan.kind == sched.IDLE:
+            finished = s.drain_finished().finished
+            break
+        s.commit([7] * len(plan.ids))
+    assert finished and finished[0].finish == "length" and finished[0].generated == 3
+    assert s.manager.available() == 2
+
+
+def test_state_slots_limit_admission_and_are_marked_fresh_once():
+    s = scheduler(64, 4, 8, chunk=16, state_slots=2)
+    for seq_id in (1, 2, 3):
+        submit(s, seq_id, 20, 3)
+    plan = s.plan()
+    assert plan.entries[0].state_slot == 0 and plan.entries[0].fresh_state
+    s.commit([7] * len(plan.ids))
+    plan = s.plan()
+    assert not plan.entries[0].fresh_state, "a slot is cleared once, before its first use"
+    s.commit([7] * len(plan.ids))
+    seen = set()
+    for _ in range(40):
+        plan = s.plan()
+        if plan.kind == sched.IDLE:
+            break
+        assert s.running <= 2
+        for e in plan.entries:
+            seen.add(e.seq_id)
+            assert e.state_slot in (0, 1)
+        s.commit([7] * len(plan.ids))
+    assert seen == {1, 2, 3}
+    assert s.manager.free_state_slots == 2
+
+
+def test_a_windowed_group_serves_a_prompt_longer_than_its_pool():
+    s = scheduler(8, 4, 4, chunk=8, window=8)
+    submit(s, 1, 100, 5)
+    produced = 0
+    for _ in range(40):
+        plan = s.plan()
+        if plan.kind == sched.IDLE:
+            break
+        assert plan.kind != sched.REFUSED
+        produced += len(s.commit([7] * len(plan.ids)).tokens)
+        assert s.manager.in_use() <= 5
+    assert produced == 5
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_every_request_finishes_and_every_page_returns_under_random_load(seed):
+    rng = random.Random(seed)
+    bs = rng.choice([2, 4, 16])
+    blocks = rng.randrange(8, 30)
+    chunk = rng.choice([None, 8, 32])
+    s = scheduler(blocks, bs, rng.randrange(1, 6), chunk=chunk)
+    submitted = {}
+    finished = {}
+    next_id = 1
+    for it in range(3000):
+        if next_id <= 25 and rng.random() < 0.15:
+            n = rng.randrange(1, bs * blocks // 2)
+            submit(s, next_id, 0, rng.randrange(1, 12), prompt=[rng.randrange(5) for _ in range(n)])
+            submitted[next_id] = n
+            next_id += 1
+        plan = s.plan()
+        if plan.kind == sched.IDLE:
+            for f in s.drain_finished().finished:
+                finished[f.id] = f
+            if next_id > 25 and not s.running and not s.waiting:
+                break
+            continue
+        if chunk:
+            assert plan.num_tokens <= chunk
+        starts = {e.seq_id: e.start for e in plan.entries}
+        for e in plan.entries:
+            assert e.start == s.manager.tokens(e.seq_id), "a portion starts where the cache has got to"
+            assert e.start + len(e.tokens) <= s.manager.capacity(e.seq_id)
+        token = 99 if rng.random() < 0.05 else 7
+        for f in s.commit([token] * len(plan.ids)).finished:
+            finished[f.id] = f
+        assert s.manager.in_use() + s.manager.available() == blocks
+    assert set(finished) == set(submitted), "a request was lost"
+    assert s.manager.available() == blocks and s.manager.live_sequences == 0
+    assert all(f.finish in ("stop", "length") for f in finished.values())
