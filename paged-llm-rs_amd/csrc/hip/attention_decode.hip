@@ -1,0 +1,329 @@
+// Paged attention for single tokens in bfloat16: a decoded token, or a token of
+// a short prompt portion, reading the keys 0..position of its request through
+// the block table.  The work is a stream of the request's keys and values
+// through the chip, so the kernel is built around 16-byte loads that are all in
+// flight together:
+//
+//   grid (kv head x query-head tile, token, split).  A workgroup of four waves
+//   owns one stretch of the context (split-KV) of one kv head and serves up to
+//   GT of the query heads that share it, so keys and values are read once per
+//   kv head, not once per query head.
+//   A group of LPK lanes owns one key: each lane holds 8 of its values.  A wave
+//   handles 64/LPK keys with one load instruction and four such instructions are
+//   issued back to back for keys and for values.
+//   Softmax is online (running maximum and sum in 32-bit, base-2 exponentials
+//   with log2(e) folded into the query scale).  The lane groups and waves keep
+//   separate running states that are merged through LDS at the end; with more
+//   than one split the partial results go to a workspace and a second kernel
+//   merges them.
+#include "common.hpp"
+
+#define AD_WAVES 4
+#define AD_UNROLL 4
+
+struct __attribute__((aligned(16))) u32x4 {
+    uint32_t v[4];
+};
+
+__device__ __forceinline__ void unpack8(const u32x4& p, float* f) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[2 * i] = __uint_as_float(p.v[i] << 16);
+        f[2 * i + 1] = __uint_as_float(p.v[i] & 0xffff0000u);
+    }
+}
+
+template <int LPK>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+    for (int off = LPK / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, PL_WAVE);
+    return v;
+}
+
+// LPK: lanes a key (a power of two, LPK*8 >= d).  GT: query heads a workgroup serves.
+template <int LPK, int GT>
+__global__ void __launch_bounds__(256)
+paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
+                              float* __restrict__ part_acc, float* __restrict__ part_ml,
+                              const int* __restrict__ positions, const int* __restrict__ seq_of,
+                              const int* __restrict__ q_len, int short_limit,
+                              const int* __restrict__ block_table, int max_blocks, int block_size,
+                              const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool, int nq,
+                              int nkv, int d, float scale_log2e, int window, int splits, int tiles) {
+    constexpr int KPW = PL_WAVE / LPK;  // keys a wave handles with one load
+    constexpr int GROUPS = AD_WAVES * KPW;
+    extern __shared__ float lds[];  // [GROUPS][GT][2] running max and sum, then [GROUPS][GT][d] accumulators
+
+    const int t = blockIdx.y;
+    const int pos = positions[t];
+    if (pos < 0) return;
+    const int seq = seq_of[t];
+    if (q_len && q_len[seq] >= short_limit) return;  // a long portion: the tiled kernel's
+
+    const int g = nq / nkv;
+    const int kvh = blockIdx.x / tiles;
+    const int tile = blockIdx.x % tiles;
+    const int h0 = kvh * g + tile * GT;               // first query head of this workgroup
+    const int heads = min(GT, g - tile * GT);         // how many of the GT are real
+    const int split = blockIdx.z;
+
+    const int lane = threadIdx.x % PL_WAVE;
+    const int wave = threadIdx.x / PL_WAVE;
+    const int sub = lane / LPK;   // which of the wave's keys
+    const int dl = lane % LPK;    // which 8 values of the head
+    const bool d_ok = dl * 8 < d;
+
+    // the stretch of keys of this split, in whole rounds of the workgroup
+    const int first = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+    const int total = pos + 1 - first;
+    constexpr int ROUND = AD_WAVES * KPW * AD_UNROLL;
+    const int per_split = pl_ceil_div(pl_ceil_div(total, splits), ROUND) * ROUND;
+    const int s_begin = first + split * per_split;
+    const int s_end = min(pos + 1, s_begin + per_split);
+
+    float qf[GT][8];
+#pragma unroll
+    for (int hq = 0; hq < GT; ++hq) {
+        if (hq < heads && d_ok) {
+            const u32x4 raw = *reinterpret_cast<const u32x4*>(q + static_cast<size_t>(t) * q_stride +
+                                                              static_cast<size_t>(h0 + hq) * d + dl * 8);
+            unpack8(raw, qf[hq]);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) qf[hq][i] *= scale_log2e;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) qf[hq][i] = 0.f;
+        }
+    }
+
+    float m[GT], l[GT], acc[GT][8];
+#pragma unroll
+    for (int hq = 0; hq < GT; ++hq) {
+        m[hq] = -INFINITY;
+        l[hq] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[hq][i] = 0.f;
+    }
+
+    const int* table = block_table + static_cast<size_t>(seq) * max_blocks;
+    const size_t row_stride = static_cast<size_t>(nkv) * d;
+    const size_t head_off = static_cast<size_t>(kvh) * d + dl * 8;
+    const bool pow2 = (block_size & (block_size - 1)) == 0;
+    const int shift = 31 - __clz(block_size);
+
+    for (int base = s_begin + wave * KPW * AD_UNROLL; base < s_end; base += ROUND) {
+        u32x4 kraw[AD_UNROLL], vraw[AD_UNROLL];
+        bool ok[AD_UNROLL];
+#pragma unroll
+        for (int u = 0; u < AD_UNROLL; ++u) {
+            const int j = base + u * KPW + sub;
+            ok[u] = j < s_end;
+            int blk = -1;
+            int within = 0;
+            if (ok[u]) {
+                const int bi = pow2 ? (j >> shift) : (j / block_size);
+                within = pow2 ? (j & (block_size - 1)) : (j - bi * block_size);
+                blk = table[bi];
+            }
+            ok[u] = ok[u] && blk >= 0;
+            if (ok[u] && d_ok) {
+                const size_t off = (static_cast<size_t>(blk) * block_size + within) * row_stride + head_off;
+                kraw[u] = *reinterpret_cast<const u32x4*>(k_pool + off);
+                vraw[u] = *reinterpret_cast<const u32x4*>(v_pool + off);
+            } else {
+                kraw[u] = u32x4{{0u, 0u, 0u, 0u}};
+                vraw[u] = u32x4{{0u, 0u, 0u, 0u}};
+            }
+        }
+        float s[AD_UNROLL][GT];
+#pragma unroll
+        for (int u = 0; u < AD_UNROLL; ++u) {
+            float kf[8];
+            unpack8(kraw[u], kf);
+#pragma unroll
+            for (int hq = 0; hq < GT; ++hq) {
+                float dot = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) dot = fmaf(qf[hq][i], kf[i], dot);
+                dot = group_sum<LPK>(dot);
+                s[u][hq] = ok[u] ? dot : -INFINITY;
+            }
+        }
+#pragma unroll
+        for (int hq = 0; hq < GT; ++hq) {
+            float m_new = m[hq];
+#pragma unroll
+            for (int u = 0; u < AD_UNROLL; ++u) m_new = fmaxf(m_new, s[u][hq]);
+            if (m_new == -INFINITY) continue;  // nothing seen yet by this lane group
+            const float corr = exp2f(m[hq] - m_new);
+            float p[AD_UNROLL];
+            float psum = 0.f;
+#pragma unroll
+            for (int u = 0; u < AD_UNROLL; ++u) {
+                p[u] = exp2f(s[u][hq] - m_new);
+                psum += p[u];
+            }
+            l[hq] = l[hq] * corr + psum;
+            m[hq] = m_new;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[hq][i] *= corr;
+#pragma unroll
+            for (int u = 0; u < AD_UNROLL; ++u) {
+                float vf[8];
+                unpack8(vraw[u], vf);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[hq][i] = fmaf(p[u], vf[i], acc[hq][i]);
+            }
+        }
+    }
+
+    // merge the lane groups of the four waves
+    float* ml = lds;                              // [GROUPS][GT][2]
+    float* accs = lds + GROUPS * GT * 2;          // [GROUPS][GT][d]
+    const int group = wave * KPW + sub;
+#pragma unroll
+    for (int hq = 0; hq < GT; ++hq) {
+        if (dl == 0) {
+            ml[(group * GT + hq) * 2] = m[hq];
+            ml[(group * GT + hq) * 2 + 1] = l[hq];
+        }
+        if (d_ok) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) accs[(static_cast<size_t>(group) * GT + hq) * d + dl * 8 + i] = acc[hq][i];
+        }
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < heads * d; idx += blockDim.x) {
+        const int hq = idx / d, dd = idx % d;
+        float big = -INFINITY;
+        for (int gr = 0; gr < GROUPS; ++gr) big = fmaxf(big, ml[(gr * GT + hq) * 2]);
+        float sum = 0.f, a = 0.f;
+        if (big != -INFINITY) {
+            for (int gr = 0; gr < GROUPS; ++gr) {
+                const float mg = ml[(gr * GT + hq) * 2];
+                if (mg == -INFINITY) continue;
+                const float w = exp2f(mg - big);
+                sum += ml[(gr * GT + hq) * 2 + 1] * w;
+                a += accs[(static_cast<size_t>(gr) * GT + hq) * d + dd] * w;
+            }
+        }
+        const int h = h0 + hq;
+        if (splits == 1) {
+            out[(static_cast<size_t>(t) * nq + h) * d + dd] = from_float<bf16_t>(sum > 0.f ? a / sum : 0.f);
+        } else {
+            const size_t pi = (static_cast<size_t>(t) * nq + h) * splits + split;
+            part_acc[pi * d + dd] = a;
+            if (dd == 0) {
+                part_ml[pi * 2] = big;
+                part_ml[pi * 2 + 1] = sum;
+            }
+        }
+    }
+}
+
+// Merges the splits of one (token, query head): out = sum_s a_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).
+__global__ void paged_attention_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+                                             bf16_t* __restrict__ out, const int* __restrict__ positions,
+                                             const int* __restrict__ seq_of, const int* __restrict__ q_len,
+                                             int short_limit, int nq, int d, int splits) {
+    const int t = blockIdx.x, h = blockIdx.y;
+    if (positions[t] < 0) return;
+    if (q_len && q_len[seq_of[t]] >= short_limit) return;
+    const size_t base = (static_cast<size_t>(t) * nq + h) * splits;
+    float big = -INFINITY;
+    for (int s = 0; s < splits; ++s) big = fmaxf(big, part_ml[(base + s) * 2]);
+    for (int dd = threadIdx.x; dd < d; dd += blockDim.x) {
+        float sum = 0.f, a = 0.f;
+        if (big != -INFINITY) {
+            for (int s = 0; s < splits; ++s) {
+                const float ms = part_ml[(base + s) * 2];
+                if (ms == -INFINITY) continue;
+                const float w = exp2f(ms - big);
+                sum += part_ml[(base + s) * 2 + 1] * w;
+                a += part_acc[(base + s) * d + dd] * w;
+            }
+        }
+        out[(static_cast<size_t>(t) * nq + h) * d + dd] = from_float<bf16_t>(sum > 0.f ? a / sum : 0.f);
+    }
+}
+
+template <int LPK, int GT>
+static int launch_decode(const void* q, int q_stride, void* out, float* part_acc, float* part_ml,
+                         const int* positions, const int* seq_of, const int* q_len, int short_limit,
+                         const int* block_table, int max_blocks, int block_size, const void* k_pool,
+                         const void* v_pool, int n, int nq, int nkv, int d, float scale, int window, int splits,
+                         hipStream_t stream) {
+    constexpr int KPW = PL_WAVE / LPK;
+    constexpr int GROUPS = AD_WAVES * KPW;
+    const int g = nq / nkv;
+    const int tiles = pl_ceil_div(g, GT);
+    const size_t lds_bytes = (static_cast<size_t>(GROUPS) * GT * 2 + static_cast<size_t>(GROUPS) * GT * d) * sizeof(float);
+    PL_REQUIRE(lds_bytes <= 160 * 1024, "decode attention: %zu bytes of LDS for head size %d", lds_bytes, d);
+    if (lds_bytes > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_decode_kernel<LPK, GT>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+        PL_REQUIRE(e == hipSuccess, "decode attention: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
+    }
+    dim3 grid(nkv * tiles, n, splits);
+    PL_REQUIRE(n <= 65535 && splits <= 65535, "decode attention: %d tokens or %d splits are more than one launch covers", n, splits);
+    paged_attention_decode_kernel<LPK, GT><<<grid, 256, lds_bytes, stream>>>(
+        static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), part_acc, part_ml, positions, seq_of,
+        q_len, short_limit, block_table, max_blocks, block_size, static_cast<const bf16_t*>(k_pool),
+        static_cast<const bf16_t*>(v_pool), nq, nkv, d, scale * 1.4426950408889634f, window, splits, tiles);
+    PL_CHECK_LAUNCH("paged_attention_decode");
+    if (splits > 1) {
+        dim3 mgrid(n, nq);
+        paged_attention_merge_kernel<<<mgrid, 64, 0, stream>>>(part_acc, part_ml, static_cast<bf16_t*>(out), positions,
+                                                               seq_of, q_len, short_limit, nq, d, splits);
+        PL_CHECK_LAUNCH("paged_attention_merge");
+    }
+    return 0;
+}
+
+template <int LPK>
+static int dispatch_gt(int gt, const void* q, int q_stride, void* out, float* part_acc, float* part_ml,
+                       const int* positions, const int* seq_of, const int* q_len, int short_limit,
+                       const int* block_table, int max_blocks, int block_size, const void* k_pool,
+                       const void* v_pool, int n, int nq, int nkv, int d, float scale, int window, int splits,
+                       hipStream_t stream) {
+#define AD_CALL(G)                                                                                              \
+    return launch_decode<LPK, G>(q, q_stride, out, part_acc, part_ml, positions, seq_of, q_len, short_limit,   \
+                                 block_table, max_blocks, block_size, k_pool, v_pool, n, nq, nkv, d, scale,    \
+                                 window, splits, stream)
+    switch (gt) {
+        case 1: AD_CALL(1);
+        case 2: AD_CALL(2);
+        case 4: AD_CALL(4);
+        default: AD_CALL(8);
+    }
+#undef AD_CALL
+}
+
+// bfloat16 only.  With splits > 1 the workspace needs n*nq*splits*d floats (part_acc) and n*nq*splits*2 (part_ml).
+// q_len (may be null) and short_limit leave the tokens of requests with q_len >= short_limit to the tiled kernel.
+extern "C" int pl_paged_attention_decode(const void* q, int q_stride, void* out, float* part_acc, float* part_ml,
+                                         const int* positions, const int* seq_of, const int* q_len, int short_limit,
+                                         const int* block_table, int max_blocks, int block_size, const void* k_pool,
+                                         const void* v_pool, int n, int nq, int nkv, int d, float scale, int window,
+                                         int splits, hipStream_t stream) {
+    PL_REQUIRE(d > 0 && d <= 256 && d % 16 == 0, "decode attention: head size %d, which has to be a multiple of 16 up to 256", d);
+    PL_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "decode attention: %d query heads over %d key heads", nq, nkv);
+    PL_REQUIRE(block_size > 0 && max_blocks > 0 && q_stride >= nq * d && q_stride % 8 == 0 && window >= 0 && splits >= 1,
+               "decode attention: block size %d, %d blocks a row, query stride %d, window %d, %d splits", block_size,
+               max_blocks, q_stride, window, splits);
+    PL_REQUIRE(splits == 1 || (part_acc && part_ml), "decode attention: %d splits without a workspace", splits);
+    if (n <= 0) return 0;
+    const int g = nq / nkv;
+    const int gt = g >= 8 ? 8 : (g > 2 ? 4 : g);   // 1, 2, 4 or 8 query heads a workgroup; the rest are more tiles
+    const int chunks = d / 8;
+#define AD_LPK(L)                                                                                                  \
+    return dispatch_gt<L>(gt, q, q_stride, out, part_acc, part_ml, positions, seq_of, q_len, short_limit,        \
+                          block_table, max_blocks, block_size, k_pool, v_pool, n, nq, nkv, d, scale, window,      \
+                          splits, stream)
+    if (chunks <= 2) AD_LPK(2);
+    if (chunks <= 4) AD_LPK(4);
+    if (chunks <= 8) AD_LPK(8);
+    if (chunks <= 16) AD_LPK(16);
+    AD_LPK(32);
+#undef AD_LPK
+}

@@ -98,4 +98,4 @@ void pl_set_error(const char* fmt, ...);
         }                                                                       \
     } while (0)
 
-static inline int pl_ceil_div(int a, int b) { return (a + b - 1) / b; }
+__host__ __device__ static inline int pl_ceil_div(int a, int b) { return (a + b - 1) / b; }

@@ -35,6 +35,8 @@ def _signatures(lib) -> None:
         "pl_gemm_plain": [p, p, p, i, i, i, i, i, i, i, p],
         "pl_paged_attention_plain": [p, i, p, p, p, p, i, i, p, p, i, i, i, i, f, i, i, p],
         "pl_argmax": [p, p, i, i, p],
+        "pl_gemm_skinny": [p, p, p, i, i, i, i, i, p],
+        "pl_paged_attention_decode": [p, i, p, p, p, p, p, p, i, p, i, i, p, p, i, i, i, i, f, i, i, p],
     }
     for name, argtypes in table.items():
         fn = getattr(lib, name)
@@ -236,9 +238,15 @@ def argmax(logits: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tenso
 
 _attention_mode = "kernel"
 
+# A request that brings fewer tokens than this to a step has each of them served
+# like a decoded token (one row of queries against its keys); longer portions go
+# to the tiled kernel.
+SHORT_PORTION = 16
+SKINNY_ROWS = 64
+
 
 def set_attention(mode: str) -> None:
-    """``kernel``: the matrix-core kernels where they apply; ``tensor``: the plain
+    """``kernel``: the fast bfloat16 kernels where they apply; ``tensor``: the plain
     kernel with 32-bit arithmetic that they are checked against (the reference's
     flag of the same name chooses between its kernel and its tensor path)."""
     global _attention_mode
@@ -247,17 +255,92 @@ def set_attention(mode: str) -> None:
     _attention_mode = mode
 
 
+def decode_splits(tokens: int, nq: int, nkv: int, max_ctx: int) -> int:
+    """How many stretches the context is cut into, so that a launch fills the chip:
+    about a thousand workgroups, each with at least 128 keys."""
+    g = nq // nkv
+    gt = 8 if g >= 8 else (4 if g > 2 else g)
+    base = max(tokens * nkv * ((g + gt - 1) // gt), 1)
+    return max(1, min((1024 + base - 1) // base, (max_ctx + 127) // 128, 64))
+
+
+def paged_attention_decode(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, positions: torch.Tensor,
+                           seq_of: torch.Tensor, block_table: torch.Tensor, block_size: int,
+                           k_pool: torch.Tensor, v_pool: torch.Tensor, nq: int, nkv: int, d: int, scale: float,
+                           window: int = 0, splits: int = 1, q_len: torch.Tensor | None = None,
+                           short_limit: int = 0) -> torch.Tensor:
+    """bfloat16 attention of single tokens over their requests' pages, split along the context."""
+    n = positions.numel()
+    _need(q, "query buffer", None, torch.bfloat16)
+    if q.dim() != 2 or q.shape[0] != n or q.shape[1] != q_row_stride or q_row_stride < nq * d:
+        raise TensorError(f"query buffer has shape {tuple(q.shape)} for {n} tokens and row stride {q_row_stride}")
+    _need(out, "attention output", (n, nq * d), torch.bfloat16)
+    _need(positions, "positions", (n,), torch.int32)
+    _need(seq_of, "request index of each token", (n,), torch.int32)
+    _need(block_table, "block table", None, torch.int32)
+    if q_len is not None:
+        _need(q_len, "tokens of each request", (block_table.shape[0],), torch.int32)
+    for pool, what in ((k_pool, "key pool"), (v_pool, "value pool")):
+        _need(pool, what, None, torch.bfloat16)
+        if pool.dim() != 2 or pool.shape[1] != nkv * d or pool.shape[0] % block_size != 0:
+            raise TensorError(f"{what} has shape {tuple(pool.shape)}, expected [pages*{block_size}, {nkv * d}]")
+    part_acc = part_ml = None
+    if splits > 1:
+        part_acc = torch.empty((n * nq * splits * d,), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((n * nq * splits * 2,), dtype=torch.float32, device=q.device)
+    _check(library().pl_paged_attention_decode(
+        q.data_ptr(), q_row_stride, out.data_ptr(), _ptr(part_acc), _ptr(part_ml), positions.data_ptr(),
+        seq_of.data_ptr(), _ptr(q_len), int(short_limit), block_table.data_ptr(), block_table.shape[1], block_size,
+        k_pool.data_ptr(), v_pool.data_ptr(), n, nq, nkv, d, float(scale), int(window or 0), int(splits), _stream()))
+    return out
+
+
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nkv: int, d: int,
                     scale: float, window: int = 0) -> torch.Tensor:
     """Attention for every token of a step.  ``qkv`` rows begin with the rotated queries."""
+    if qkv.dtype == torch.bfloat16 and _attention_mode == "kernel" and batch.max_q_len < SHORT_PORTION:
+        splits = decode_splits(batch.num_tokens, nq, nkv, batch.max_ctx_len)
+        return paged_attention_decode(qkv, qkv.shape[1], out, batch.positions, batch.seq_of, kv.block_table,
+                                      kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window, splits)
     return paged_attention_plain(qkv, qkv.shape[1], out, batch.positions, batch.seq_of, kv.block_table,
                                  kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window)
 
 
-def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
-    """y = x . w^T for bfloat16 operands with 32-bit accumulation."""
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
+                swiglu: bool = False) -> torch.Tensor:
+    """y = x . w^T for up to 64 rows of bfloat16 on the matrix cores, the weights streamed once.
+    With ``swiglu`` the rows of ``w`` are [gate | up] and y = silu(x . gate^T) * (x . up^T)."""
+    n, K = x.shape
     _need(x, "matrix product input", None, torch.bfloat16)
     _need(w, "weight", None, torch.bfloat16)
+    if w.dim() != 2 or w.shape[1] != K:
+        raise TensorError(f"weight has shape {tuple(w.shape)} for an input of width {K}")
+    N_out = w.shape[0] // 2 if swiglu else w.shape[0]
+    if swiglu and w.shape[0] % 2:
+        raise TensorError(f"fused gate/up weight has an odd number of rows, {w.shape[0]}")
+    if out_dtype not in (torch.bfloat16, torch.float32):
+        raise TensorError(f"matrix product output {out_dtype}")
+    out = torch.empty((n, N_out), dtype=out_dtype, device=x.device)
+    _check(library().pl_gemm_skinny(x.data_ptr(), w.data_ptr(), out.data_ptr(), n, N_out, K, 1 if swiglu else 0,
+                                    1 if out_dtype == torch.float32 else 0, _stream()))
+    return out
+
+
+def skinny_applies(x: torch.Tensor) -> bool:
+    return x.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_ROWS and x.shape[1] % 8 == 0
+
+
+def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """y = x . w^T for bfloat16 operands with 32-bit accumulation: few rows stream the
+    weights through the hand-written kernel, many rows go to the library's product."""
+    _need(x, "matrix product input", None, torch.bfloat16)
+    _need(w, "weight", None, torch.bfloat16)
+    if skinny_applies(x):
+        return gemm_skinny(x, w, out_dtype)
     if out_dtype == torch.float32:
+        if x.shape[1] % 8 == 0:
+            # more wanted rows than one skinny launch takes: 64 at a time
+            return torch.cat([gemm_skinny(x[i:i + SKINNY_ROWS].contiguous(), w, torch.float32)
+                              for i in range(0, x.shape[0], SKINNY_ROWS)], dim=0)
         return gemm_plain(x, w, out_dtype=torch.float32)
     return torch.mm(x, w.t())

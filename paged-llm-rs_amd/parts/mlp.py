@@ -27,7 +27,12 @@ class GatedMlp:
         self.down_proj = Linear(params["down_proj.weight"])
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return self.down_proj.forward(kernels.swiglu(self.gate_up_proj.forward(x)))
+        if kernels.skinny_applies(x):
+            # few rows: the activation is the epilogue of the weight stream
+            act = kernels.gemm_skinny(x, self.gate_up_proj.weight, swiglu=True)
+        else:
+            act = kernels.swiglu(self.gate_up_proj.forward(x))
+        return self.down_proj.forward(act)
 
 
 register_feed_forward("gated_mlp", GatedMlp)

@@ -1,0 +1,368 @@
+"""Each kernel alone against a plain 32-bit (or 64-bit) torch reference of the same
+operation, at other sizes than the engine's tiny models use."""
+
+from __future__ import annotations
+
+import math
+import random
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def rel(got, want):
+    got, want = got.double().cpu(), want.double().cpu()
+    assert got.shape == want.shape
+    return float((got - want).abs().max() / want.abs().max().clamp_min(1e-30))
+
+
+def tol(dtype):
+    return 2e-6 if dtype == torch.float32 else 1e-2
+
+
+@pytest.fixture(autouse=True)
+def _seed():
+    torch.manual_seed(1234)
+
+
+# --- embedding -------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("V,H", [(331, 100), (1000, 1024), (50, 24)])
+def test_embed(dtype, V, H):
+    from paged_llm_rs_amd import kernels
+
+    table = torch.randn(V, H, device=DEV).to(dtype)
+    ids = torch.tensor([0, V - 1, 7, 7, -1, V // 2], dtype=torch.int32, device=DEV)
+    out = kernels.embed(ids, table)
+    assert out.dtype == torch.float32
+    want = table.float()[ids.clamp_min(0).long()]
+    want[4] = 0
+    assert torch.equal(out, want)
+
+
+# --- residual add + norm -----------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,H", [(1, 24), (7, 100), (33, 1024), (5, 5120)])
+def test_add_rmsnorm(dtype, n, H):
+    from paged_llm_rs_amd import kernels
+
+    resid = torch.randn(n, H, device=DEV) * 3
+    delta = torch.randn(n, H, device=DEV).to(dtype)
+    gain = (torch.rand(H, device=DEV) + 0.5).to(dtype)
+    eps = 1e-5
+    x = resid.double() + delta.double()
+    want = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * gain.double()
+    out = torch.empty(n, H, dtype=dtype, device=DEV)
+    r = resid.clone()
+    kernels.add_rmsnorm(r, delta, gain, eps, out)
+    assert rel(out, want) < tol(dtype)
+    assert rel(r, x) < 1e-6, "the sum is written back in 32-bit"
+    # no delta; gathered rows leave the stream untouched; a 32-bit gain beside 16-bit activations
+    r2 = resid.clone()
+    rows = torch.tensor([n - 1, 0], dtype=torch.int32, device=DEV)
+    out2 = torch.empty(2, H, dtype=dtype, device=DEV)
+    kernels.add_rmsnorm(r2, delta, gain.float(), eps, out2, rows=rows)
+    assert torch.equal(r2, resid)
+    assert rel(out2, want[[n - 1, 0]]) < tol(dtype)
+    out3 = torch.empty(n, H, dtype=dtype, device=DEV)
+    kernels.add_rmsnorm(resid.clone(), None, gain, eps, out3)
+    x0 = resid.double()
+    assert rel(out3, x0 / torch.sqrt((x0 * x0).mean(-1, keepdim=True) + eps) * gain.double()) < tol(dtype)
+
+
+# --- q/k norm, rotation, cache write --------------------------------------------------------------------
+
+def rope_ref(x, pos, theta, rot):
+    """x [n, heads, d] float64; rotate the first ``rot`` values of each head, halves paired."""
+    half = rot // 2
+    inv = torch.tensor([1.0 / theta ** (2.0 * i / rot) for i in range(half)], dtype=torch.float64, device=x.device)
+    ang = pos.double()[:, None] * inv[None]
+    c, s = ang.cos()[:, None, :], ang.sin()[:, None, :]
+    out = x.clone()
+    x1, x2 = x[..., :half], x[..., half:rot]
+    out[..., :half] = x1 * c - x2 * s
+    out[..., half:rot] = x2 * c + x1 * s
+    return out
+
+
+def tables(max_pos, rot, theta):
+    half = rot // 2
+    inv = torch.tensor([1.0 / theta ** (2.0 * i / rot) for i in range(half)], dtype=torch.float64)
+    ang = torch.arange(max_pos, dtype=torch.float64)[:, None] * inv[None]
+    return ang.cos().float().to(DEV), ang.sin().float().to(DEV)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nq,nkv,d,bs,norm", [(4, 2, 16, 4, True), (6, 1, 48, 16, True), (3, 3, 128, 8, False),
+                                              (8, 2, 256, 2, True), (5, 5, 80, 16, True)])
+def test_qk_norm_rope_kv_write(dtype, nq, nkv, d, bs, norm):
+    from paged_llm_rs_amd import kernels
+
+    n, S, pages = 11, 3, 64      # positions up to 31: 16 pages a request at a page size of 2
+    theta, eps = 1e4, 1e-5
+    qkv = torch.randn(n, (nq + 2 * nkv) * d, device=DEV).to(dtype)
+    seq_of = torch.tensor([0, 0, 0, 0, 1, 2, 2, 2, 2, 2, 1], dtype=torch.int32, device=DEV)
+    positions = torch.tensor([5, 6, 7, 8, 30, 0, 1, 2, 3, -1, 31], dtype=torch.int32, device=DEV)
+    perm = torch.randperm(pages)[: S * 16].reshape(S, 16).to(torch.int32).to(DEV)
+    k_pool = torch.zeros(pages * bs, nkv * d, dtype=dtype, device=DEV)
+    v_pool = torch.zeros_like(k_pool)
+    q_gain = (torch.rand(d, device=DEV) + 0.5).to(dtype) if norm else None
+    k_gain = (torch.rand(d, device=DEV) + 0.5).to(dtype) if norm else None
+    cos, sin = tables(64, d, theta)
+    before = qkv.clone()
+    kernels.qk_norm_rope_kv_write(qkv, q_gain, k_gain, eps, cos, sin, d, positions, seq_of, perm, bs, k_pool, v_pool,
+                                  nq, nkv, d)
+    x = before.double().reshape(n, nq + 2 * nkv, d)
+    q, k, v = x[:, :nq], x[:, nq:nq + nkv], x[:, nq + nkv:]
+    if norm:
+        q = q / torch.sqrt((q * q).mean(-1, keepdim=True) + eps) * q_gain.double()
+        k = k / torch.sqrt((k * k).mean(-1, keepdim=True) + eps) * k_gain.double()
+    pos = positions.clamp_min(0)
+    q, k = rope_ref(q, pos, theta, d), rope_ref(k, pos, theta, d)
+    live = positions >= 0
+    got_q = qkv.reshape(n, nq + 2 * nkv, d)[:, :nq]
+    assert rel(got_q[live], q[live]) < tol(dtype)
+    assert torch.equal(got_q[~live], before.reshape(n, -1, d)[:, :nq][~live]), "a padding row is left alone"
+    for t in range(n):
+        if positions[t] < 0:
+            continue
+        p = int(positions[t])
+        slot = int(perm[int(seq_of[t]), p // bs]) * bs + p % bs
+        assert rel(k_pool[slot].reshape(nkv, d), k[t]) < tol(dtype)
+        assert torch.equal(v_pool[slot].reshape(nkv, d), before.reshape(n, -1, d)[t, nq + nkv:]), "v is copied as it is"
+    written = {int(perm[int(seq_of[t]), int(positions[t]) // bs]) * bs + int(positions[t]) % bs
+               for t in range(n) if positions[t] >= 0}
+    untouched = torch.ones(pages * bs, dtype=torch.bool)
+    untouched[list(written)] = False
+    assert not k_pool[untouched.to(DEV)].any() and not v_pool[untouched.to(DEV)].any(), "nothing else was written"
+    # without the cache write only q changes
+    k2, v2 = torch.zeros_like(k_pool), torch.zeros_like(v_pool)
+    again = before.clone()
+    kernels.qk_norm_rope_kv_write(again, q_gain, k_gain, eps, cos, sin, d, positions, seq_of, perm, bs, k2, v2,
+                                  nq, nkv, d, write_kv=False)
+    assert not k2.any() and not v2.any()
+    assert torch.equal(again.reshape(n, -1, d)[:, :nq], got_q)
+
+
+def test_rotation_of_part_of_a_head_and_refused_sizes():
+    from paged_llm_rs_amd import kernels
+    from paged_llm_rs_amd.errors import TensorError
+
+    n, nq, nkv, d, rot, bs = 3, 2, 1, 32, 16, 4
+    qkv = torch.randn(n, (nq + 2 * nkv) * d, device=DEV)
+    positions = torch.tensor([3, 4, 9], dtype=torch.int32, device=DEV)
+    seq_of = torch.zeros(n, dtype=torch.int32, device=DEV)
+    bt = torch.arange(4, dtype=torch.int32, device=DEV).reshape(1, 4)
+    kp = torch.zeros(16, d, device=DEV)
+    vp = torch.zeros(16, d, device=DEV)
+    cos, sin = tables(16, rot, 1e4)
+    before = qkv.clone()
+    kernels.qk_norm_rope_kv_write(qkv, None, None, 0.0, cos, sin, rot, positions, seq_of, bt, bs, kp, vp, nq, nkv, d)
+    want = rope_ref(before.double().reshape(n, 4, d)[:, :nq], positions, 1e4, rot)
+    assert rel(qkv.reshape(n, 4, d)[:, :nq], want) < 2e-6
+    assert torch.equal(qkv.reshape(n, 4, d)[:, :nq, rot:], before.reshape(n, 4, d)[:, :nq, rot:])
+    with pytest.raises(TensorError, match="multiple of 16"):
+        kernels.qk_norm_rope_kv_write(torch.zeros(1, 4 * 24, device=DEV), None, None, 0.0, None, None, 0,
+                                      positions[:1], seq_of[:1], bt, bs, torch.zeros(16, 24, device=DEV),
+                                      torch.zeros(16, 24, device=DEV), 2, 1, 24)
+
+
+# --- feed-forward ------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu(dtype):
+    from paged_llm_rs_amd import kernels
+
+    gu = torch.randn(9, 2 * 212, device=DEV).to(dtype)
+    want = torch.nn.functional.silu(gu.double()[:, :212]) * gu.double()[:, 212:]
+    assert rel(kernels.swiglu(gu), want) < tol(dtype)
+    assert float(kernels.swiglu(torch.zeros(1, 8, device=DEV)).abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,N,K", [(1, 5, 3), (7, 331, 100), (70, 130, 257), (64, 64, 64), (3, 1000, 1024)])
+def test_gemm_plain(dtype, n, N, K):
+    from paged_llm_rs_amd import kernels
+
+    x = torch.randn(n, K, device=DEV).to(dtype)
+    w = torch.randn(N, K, device=DEV).to(dtype)
+    want = x.double() @ w.double().T
+    assert rel(kernels.gemm_plain(x, w), want) < (2e-6 if dtype == torch.float32 else 6e-3)
+    assert rel(kernels.gemm_plain(x, w, out_dtype=torch.float32), want) < 2e-6
+    # a row's result does not depend on what else is in the batch: bitwise
+    alone = kernels.gemm_plain(x[:1].contiguous(), w, out_dtype=torch.float32)
+    assert torch.equal(alone, kernels.gemm_plain(x, w, out_dtype=torch.float32)[:1])
+
+
+@pytest.mark.parametrize("n", [1, 2, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(16, 32), (331, 104), (4096, 1024), (1024, 3072), (50, 8), (1000, 2056)])
+def test_gemm_skinny(n, N, K):
+    from paged_llm_rs_amd import kernels
+
+    x = torch.randn(n, K, device=DEV).to(torch.bfloat16)
+    w = torch.randn(N, K, device=DEV).to(torch.bfloat16)
+    want = x.double() @ w.double().T
+    assert rel(kernels.gemm_skinny(x, w, torch.float32), want) < 1e-5, "products of bfloat16 summed in 32-bit"
+    assert rel(kernels.gemm_skinny(x, w, torch.bfloat16), want) < 6e-3
+    if N % 2 == 0:
+        g, u = want[:, :N // 2], want[:, N // 2:]
+        act = torch.nn.functional.silu(g) * u
+        assert rel(kernels.gemm_skinny(x, w, torch.float32, swiglu=True), act) < 2e-5
+    # one-hot rows pick single weights: a wrong operand layout cannot pass this
+    eye = torch.zeros(min(n, K), K, device=DEV, dtype=torch.bfloat16)
+    idx = torch.randperm(K)[:eye.shape[0]]
+    eye[torch.arange(eye.shape[0]), idx] = 1
+    assert torch.equal(kernels.gemm_skinny(eye, w, torch.bfloat16), w[:, idx].T.contiguous())
+
+
+def test_gemm_skinny_refusals():
+    from paged_llm_rs_amd import kernels
+    from paged_llm_rs_amd.errors import TensorError
+
+    with pytest.raises(TensorError, match="multiple of 8"):
+        kernels.gemm_skinny(torch.zeros(2, 100, device=DEV, dtype=torch.bfloat16),
+                            torch.zeros(5, 100, device=DEV, dtype=torch.bfloat16))
+    with pytest.raises(TensorError, match="up to 64"):
+        kernels.gemm_skinny(torch.zeros(65, 64, device=DEV, dtype=torch.bfloat16),
+                            torch.zeros(5, 64, device=DEV, dtype=torch.bfloat16))
+
+
+# --- attention ------------------------------------------------------------------------------------------------
+
+def build_paged(nkv, d, bs, ctx_lens, dtype, seed=0, pages_extra=7):
+    """Random keys and values for requests of the given lengths, scattered over shuffled pages."""
+    g = torch.Generator().manual_seed(seed)
+    S = len(ctx_lens)
+    need = [(c + bs - 1) // bs for c in ctx_lens]
+    pages = sum(need) + pages_extra
+    order = torch.randperm(pages, generator=g).tolist()
+    max_blocks = max(need) + 2
+    bt = torch.full((S, max_blocks), -1, dtype=torch.int32)
+    k_pool = torch.randn(pages * bs, nkv * d, generator=g).to(dtype)
+    v_pool = torch.randn(pages * bs, nkv * d, generator=g).to(dtype)
+    keys, values = [], []
+    at = 0
+    for s, c in enumerate(ctx_lens):
+        for b in range(need[s]):
+            bt[s, b] = order[at]
+            at += 1
+        slots = [int(bt[s, p // bs]) * bs + p % bs for p in range(c)]
+        keys.append(k_pool[slots].reshape(c, nkv, d).double())
+        values.append(v_pool[slots].reshape(c, nkv, d).double())
+    return bt.to(DEV), k_pool.to(DEV), v_pool.to(DEV), keys, values
+
+
+def attention_ref(q, keys, values, pos, g, scale, window):
+    """q [nq, d] float64 at position pos against keys/values [ctx, nkv, d]."""
+    out = []
+    first = max(0, pos + 1 - window) if window else 0
+    for h in range(q.shape[0]):
+        k = keys[first:pos + 1, h // g]
+        v = values[first:pos + 1, h // g]
+        p = torch.softmax(k @ q[h] * scale, dim=0)
+        out.append(p @ v)
+    return torch.stack(out)
+
+
+ATTENTION_CASES = [
+    # nq, nkv, d, block size, context lengths, window
+    (4, 2, 16, 4, [1, 5, 33], 0),
+    (6, 1, 32, 8, [70, 9], 0),
+    (6, 2, 48, 16, [100, 17, 64], 0),
+    (16, 8, 128, 16, [513, 40], 0),
+    (8, 1, 64, 16, [200, 129], 0),
+    (3, 3, 80, 2, [37, 12], 0),
+    (12, 2, 112, 16, [90], 0),
+    (32, 2, 128, 16, [300], 0),
+    (4, 2, 256, 16, [77, 150], 0),
+    (4, 2, 64, 16, [300, 31], 48),
+    (2, 2, 16, 4, [50], 7),
+]
+
+
+@pytest.mark.parametrize("kernel", ["plain-f32", "plain-bf16", "decode-1", "decode-3", "decode-8"])
+@pytest.mark.parametrize("nq,nkv,d,bs,ctx_lens,window", ATTENTION_CASES)
+def test_paged_attention_of_single_tokens(kernel, nq, nkv, d, bs, ctx_lens, window):
+    from paged_llm_rs_amd import kernels
+
+    dtype = torch.float32 if kernel == "plain-f32" else torch.bfloat16
+    bt, k_pool, v_pool, keys, values = build_paged(nkv, d, bs, ctx_lens, dtype, seed=d + bs)
+    # several tokens a request, at its end and in its middle, plus a padding row
+    toks = []
+    for s, c in enumerate(ctx_lens):
+        for p in sorted({c - 1, c // 2, 0, min(c - 1, bs), max(0, c - 2)}):
+            toks.append((s, p))
+    n = len(toks) + 1
+    stride = (nq + 2 * nkv) * d
+    q = torch.randn(n, stride, device=DEV).to(dtype)
+    positions = torch.tensor([p for _, p in toks] + [-1], dtype=torch.int32, device=DEV)
+    seq_of = torch.tensor([s for s, _ in toks] + [0], dtype=torch.int32, device=DEV)
+    scale = 1 / math.sqrt(d)
+    out = torch.full((n, nq * d), 7.0, dtype=dtype, device=DEV)
+    if kernel.startswith("plain"):
+        kernels.paged_attention_plain(q, stride, out, positions, seq_of, bt, bs, k_pool, v_pool, nq, nkv, d, scale, window)
+    else:
+        kernels.paged_attention_decode(q, stride, out, positions, seq_of, bt, bs, k_pool, v_pool, nq, nkv, d, scale,
+                                       window, splits=int(kernel.split("-")[1]))
+    g = nq // nkv
+    for i, (s, p) in enumerate(toks):
+        want = attention_ref(q[i, :nq * d].double().cpu().reshape(nq, d), keys[s], values[s], p, g, scale, window)
+        err = rel(out[i].reshape(nq, d), want)
+        assert err < (2e-6 if dtype == torch.float32 else 1e-2), f"token {i} (request {s}, position {p}): {err:.3e}"
+    assert bool((out[-1] == 7.0).all()), "a padding row is not written"
+
+
+@pytest.mark.parametrize("kernel", ["plain", "decode"])
+def test_a_far_key_among_hundreds_is_found(kernel):
+    """Random scores hide a lost key; here one key far back (just across a page edge,
+    then just inside a window's edge) carries nearly all the weight, and its value is the answer."""
+    from paged_llm_rs_amd import kernels
+
+    nq, nkv, d, bs = 4, 2, 64, 16
+    dtype = torch.bfloat16
+    for ctx, target, window in [(700, 16, 0), (700, 15, 0), (700, 699, 0), (700, 0, 0), (700, 700 - 100, 100),
+                                (700, 700 - 101, 100)]:
+        bt, k_pool, v_pool, keys, values = build_paged(nkv, d, bs, [ctx], dtype, seed=ctx + target)
+        stride = (nq + 2 * nkv) * d
+        q = torch.randn(1, stride, device=DEV).to(dtype)
+        slot = int(bt[0, target // bs]) * bs + target % bs
+        for kvh in range(nkv):
+            k_pool[slot, kvh * d:(kvh + 1) * d] = (q[0, kvh * 2 * d: kvh * 2 * d + d].float() * 4).to(dtype)
+            keys[0][target, kvh] = k_pool[slot, kvh * d:(kvh + 1) * d].double().cpu()
+        positions = torch.tensor([ctx - 1], dtype=torch.int32, device=DEV)
+        seq_of = torch.zeros(1, dtype=torch.int32, device=DEV)
+        out = torch.zeros(1, nq * d, dtype=dtype, device=DEV)
+        scale = 1 / math.sqrt(d)
+        if kernel == "plain":
+            kernels.paged_attention_plain(q, stride, out, positions, seq_of, bt, bs, k_pool, v_pool, nq, nkv, d, scale, window)
+        else:
+            kernels.paged_attention_decode(q, stride, out, positions, seq_of, bt, bs, k_pool, v_pool, nq, nkv, d,
+                                           scale, window, splits=4)
+        want = attention_ref(q[0, :nq * d].double().cpu().reshape(nq, d), keys[0], values[0], ctx - 1, 2, scale, window)
+        assert rel(out[0].reshape(nq, d), want) < 1e-2, (ctx, target, window)
+        inside = window == 0 or target > ctx - 1 - window
+        hit = rel(out[0].reshape(nq, d)[0], values[0][target, 0]) < 0.2
+        assert hit == inside, f"key {target} of {ctx} with window {window}: found {hit}, visible {inside}"
+
+
+# --- sampling ------------------------------------------------------------------------------------------------------
+
+def test_argmax_first_maximum_wins():
+    from paged_llm_rs_amd import kernels
+
+    logits = torch.randn(5, 151936, device=DEV)
+    logits[0, 77] = logits[0, 99999] = 50.0
+    logits[1, 151935] = 60.0
+    logits[2, 0] = 70.0
+    logits[3] = -5.0
+    got = kernels.argmax(logits).cpu().tolist()
+    assert got[:4] == [77, 151935, 0, 0]
+    assert got[4] == int(torch.argmax(logits[4]))
+    small = torch.tensor([[1.0, 3.0, 3.0, 2.0]], device=DEV)
+    assert kernels.argmax(small).item() == 1
