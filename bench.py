@@ -68,7 +68,7 @@ def kv_bytes_per_token(cfg: dict, element: int) -> int:
 class DecodeBench:
     """B requests with ``context`` tokens each in the cache, then timed decode steps."""
 
-    def __init__(self, model, cache, batch: int, context: int, seed: int):
+    def __init__(self, model, cache, runner, batch: int, context: int, seed: int):
         from paged_llm_rs_amd.engine.batch import StepEntry
 
         self.model, self.cache, self.batch = model, cache, batch
@@ -80,6 +80,7 @@ class DecodeBench:
         from paged_llm_rs_amd.engine.step import commit_step, run_step
         from paged_llm_rs_amd import kernels
         self.run_step, self.commit_step, self.kernels = run_step, commit_step, kernels
+        self.runner = runner
         firsts = []
         for i in self.ids:
             cache.manager.add_sequence(i)
@@ -97,8 +98,8 @@ class DecodeBench:
         for i, tok in zip(self.ids, self.tokens):
             assert manager.reserve(i, 1)
             entries.append(self.StepEntry(i, [tok], manager.tokens(i), [0]))
-        logits = self.run_step(self.model, self.cache, entries)
-        self.tokens = self.kernels.argmax(logits).cpu().tolist()   # the tokens the next step is fed
+        out = self.runner.run(entries)
+        self.tokens = out.greedy_tokens().cpu().tolist()   # the tokens the next step is fed
         self.commit_step(self.cache, entries)
 
     def free(self) -> None:
@@ -127,6 +128,7 @@ def main() -> int:
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--layers", type=int, default=FULL_LAYERS,
                         help="fewer layers than the model has, where memory or time needs it; both numbers are reported")
+    parser.add_argument("--no-graphs", action="store_true", help="run decode steps eagerly instead of as HIP graphs")
     parser.add_argument("--skip-points", action="store_true", help="leave out batch 1 and 64 and the prefill")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -138,7 +140,7 @@ def main() -> int:
     from paged_llm_rs_amd import write_random_model
     from paged_llm_rs_amd.cache import PagedCache
     from paged_llm_rs_amd.engine.batch import StepEntry
-    from paged_llm_rs_amd.engine.step import commit_step, require_gpu, run_step
+    from paged_llm_rs_amd.engine.step import StepRunner, commit_step, require_gpu, run_step
     from paged_llm_rs_amd.parts.model import load_model
 
     device = require_gpu("cuda:0")
@@ -159,8 +161,10 @@ def main() -> int:
     pages = (largest * (CONTEXT + args.steps + args.warmup + 64) + PREFILL_TOKENS + 64) // BLOCK_SIZE + largest
     cache = PagedCache(model.cache_layout, BLOCK_SIZE, pages, torch.bfloat16, device, max_seqs=largest + 1)
 
+    runner = StepRunner(model, cache, graphs=not args.no_graphs)
+
     def decode_point(batch: int, steps: int, warmup: int):
-        bench = DecodeBench(model, cache, batch, CONTEXT, seed=batch)
+        bench = DecodeBench(model, cache, runner, batch, CONTEXT, seed=batch)
         seconds = timed(bench.step, steps, warmup)
         context_mid = CONTEXT + warmup + steps / 2
         bench.free()

@@ -16,7 +16,6 @@ from typing import Optional
 
 import torch
 
-from .. import kernels
 from ..cache import PagedCache
 from ..config import GenerationConfig
 from ..errors import ConfigError, PagedLLMError
@@ -24,7 +23,7 @@ from ..parts.model import DTYPES, load_model
 from ..sampling.sampler import Sampling
 from ..weights.safetensors_io import SafetensorsFile
 from . import scheduler as sched
-from .step import require_gpu, run_step
+from .step import StepRunner, require_gpu
 
 _seed_counter = itertools.count()
 
@@ -70,7 +69,7 @@ class Engine:
 
     def __init__(self, model, dtype: str = "auto", block_size: int = 16, cache_mib: int = 3584,
                  num_blocks: Optional[int] = None, max_batch: int = 16, chunk=128, prefix_cache: bool = True,
-                 max_tokens: int = 512, device="cuda:0", sampler: str = "device"):
+                 max_tokens: int = 512, device="cuda:0", sampler: str = "device", graphs: bool = True):
         self.device = require_gpu(device)
         dtype = {"auto": None, "f32": "float32", "bf16": "bfloat16"}.get(dtype, dtype)
         if dtype is None:
@@ -100,6 +99,7 @@ class Engine:
         self.scheduler = sched.Scheduler(self.cache.manager, max_batch=max_batch,
                                          chunk=None if chunk is None else int(chunk),
                                          max_positions=self.model.spec.max_positions, prefix_cache=prefix_cache)
+        self.runner = StepRunner(self.model, self.cache, graphs=graphs)
         self.default_max_tokens = max_tokens
         self.sampler = sampler
         self._next_id = 1
@@ -145,17 +145,18 @@ class Engine:
 
     # -- the loop ---------------------------------------------------------------------------
 
-    def _choose(self, plan, logits: torch.Tensor) -> list:
+    def _choose(self, plan, output) -> list:
         """One token per id of the plan.  Greedy rows are an argmax on the device;
         the logits of the others go to the host sampler with the request's generator."""
         if not plan.ids:
             return []      # a portion in the middle of a prompt: the logits have no rows and are not touched
+        logits = output.logits
         if logits.shape[0] != len(plan.ids):
             raise PagedLLMError(f"{logits.shape[0]} rows of logits for {len(plan.ids)} requests")
         greedy = [self._greedy.get(i, True) for i in plan.ids]
         chosen = [0] * len(plan.ids)
         if self.sampler == "device" and any(greedy):
-            picked = kernels.argmax(logits).cpu().tolist()
+            picked = output.greedy_tokens().cpu().tolist()
             for row, g in enumerate(greedy):
                 if g:
                     chosen[row] = picked[row]
@@ -177,8 +178,7 @@ class Engine:
         sampled = []
         if plan.entries:
             try:
-                logits = run_step(self.model, self.cache, plan.entries)
-                sampled = self._choose(plan, logits)
+                sampled = self._choose(plan, self.runner.run(plan.entries))
             except PagedLLMError:
                 # A failed step fails every request in it; nothing was committed
                 # (reference: engine.rs:340-348).

@@ -12,12 +12,12 @@ from ..cache import PagedCache
 from ..errors import ConfigError
 from ..parts.model import DTYPES, load_model
 from .batch import StepEntry
-from .step import commit_step, require_gpu, run_step
+from .step import StepRunner, commit_step, require_gpu
 
 
 class Replayer:
     def __init__(self, model_dir, dtype: str, max_tokens: int, block_size: int = 16, device="cuda:0",
-                 max_live: int = 64):
+                 max_live: int = 64, graphs: bool = True):
         device = require_gpu(device)
         self.config, self.model = load_model(model_dir, dtype, device)
         if max_tokens < 1:
@@ -27,6 +27,7 @@ class Replayer:
         tokens = (max_tokens + 63) // 64 * 64
         self.cache = PagedCache(self.model.cache_layout, block_size, max(tokens // block_size, 1),
                                 DTYPES[dtype], device, max_seqs=max_live)
+        self.runner = StepRunner(self.model, self.cache, graphs=graphs)
         self.ids: dict = {}
         self.next_id = 1
 
@@ -54,7 +55,7 @@ class Replayer:
                                           state_slot=slot, fresh_state=fresh and slot >= 0))
         logits = None
         if step_entries:
-            out = run_step(self.model, self.cache, step_entries)
+            out = self.runner.run(step_entries).logits
             commit_step(self.cache, step_entries)
             if out.shape[0] > 0:
                 logits = out.to(torch.float32).cpu().numpy().astype("<f4", copy=False)

@@ -1,14 +1,29 @@
 """The step function: run the tokens a step brings, as one batch, from the
 cache, and return the logits at the wanted places (reference:
 model/mod.rs:305-352).  Pages are written; the lengths in the cache manager do
-not move: whoever asked for the step records it once it has succeeded."""
+not move: whoever asked for the step records it once it has succeeded.
+
+A step in which every request brings exactly one token (plain decoding) is
+launch-bound: some two hundred small kernels.  Such steps are captured once as a
+HIP graph over static buffers, per (requests, pages a request) bucket, and
+replayed; the descriptor of the step is written into a pinned host buffer by the
+native cache manager and copied in with one transfer.  Every other step runs
+eagerly.  Both ways run the same model code and the same kernels.
+"""
 
 from __future__ import annotations
 
+from dataclasses import dataclass
+from typing import Optional
+
+import numpy as np
 import torch
 
-from ..errors import TensorError
+from .. import kernels
+from ..errors import ConfigError, PagedLLMError, TensorError
 from .batch import StepBatch, build_batch
+
+GRAPH_MAX_REQUESTS = 64
 
 
 def require_gpu(device) -> torch.device:
@@ -32,3 +47,158 @@ def commit_step(cache, entries) -> None:
     """Record that the step ran: every request has its tokens written."""
     for e in entries:
         cache.manager.advance(e.seq_id, len(e.tokens))
+
+
+@dataclass
+class StepOutput:
+    logits: torch.Tensor                      # [wanted, vocabulary], 32-bit, on the device
+    greedy: Optional[torch.Tensor] = None     # [wanted] int32 on the device, when already computed
+
+    def greedy_tokens(self) -> torch.Tensor:
+        if self.greedy is None:
+            self.greedy = kernels.argmax(self.logits)
+        return self.greedy
+
+
+def _bucket(n: int, least: int = 1) -> int:
+    b = least
+    while b < n:
+        b *= 2
+    return b
+
+
+class DecodeGraph:
+    """One decode step for up to ``cap`` requests with up to ``widths[g]`` pages each, captured."""
+
+    def __init__(self, model, cache, cap: int, widths: list):
+        self.model, self.cache, self.cap, self.widths = model, cache, cap, list(widths)
+        pieces = [("token_ids", cap), ("positions", cap), ("seq_of", cap), ("q_start", cap), ("q_len", cap),
+                  ("ctx_len", cap), ("state_slots", cap), ("logit_rows", cap)]
+        pieces += [(f"block_table_{g}", cap * w) for g, w in enumerate(widths)]
+        self.layout, offset = {}, 0
+        for name, count in pieces:
+            self.layout[name] = (offset, count)
+            offset += (count + 3) // 4 * 4
+        self.host = torch.zeros(offset, dtype=torch.int32).pin_memory()
+        self.host_np = self.host.numpy()
+        self.ids = np.zeros(cap, dtype=np.uint64)
+        self.device_buf = torch.zeros(offset, dtype=torch.int32, device=model.device)
+        block_size = cache.block_size
+        self.batch = StepBatch(self.device_buf, self.layout, cap, cap, list(widths), cap, 1,
+                               max(widths or [1]) * block_size, [])
+        h = self.host_np
+        for name in ("seq_of", "q_start", "logit_rows"):
+            b, c = self.layout[name]
+            h[b:b + c] = np.arange(cap, dtype=np.int32)
+        b, c = self.layout["q_len"]
+        h[b:b + c] = 1
+        self._idle_rows(0)
+        self.graph = None
+        self.logits = None
+        self.tokens = None
+
+    def _view(self, name):
+        b, c = self.layout[name]
+        return self.host_np[b:b + c]
+
+    def _idle_rows(self, live: int) -> None:
+        """Rows past the live requests are padding: position -1, no pages."""
+        self._view("token_ids")[live:] = 0
+        self._view("positions")[live:] = -1
+        self._view("ctx_len")[live:] = 0
+        self._view("state_slots")[live:] = -1
+        for g, w in enumerate(self.widths):
+            self._view(f"block_table_{g}").reshape(self.cap, w)[live:] = -1
+
+    def _forward(self):
+        logits = self.model.forward(self.batch, self.cache)
+        return logits, kernels.argmax(logits)
+
+    def capture(self) -> None:
+        self.device_buf.copy_(self.host)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self._forward()        # everything that initialises lazily does so outside the capture
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.logits, self.tokens = self._forward()
+
+    def fill(self, entries) -> None:
+        """Write the step's descriptor into the pinned buffer.  Raises when a table is wider than the bucket."""
+        live = len(entries)
+        manager = self.cache.manager
+        self.ids[:live] = [e.seq_id for e in entries]
+        positions = self._view("positions")
+        manager.fill_step(self.ids.ctypes.data, live, positions.ctypes.data, 0, 0, 0)
+        for g, w in enumerate(self.widths):
+            manager.fill_step(self.ids.ctypes.data, live, 0, g, self._view(f"block_table_{g}").ctypes.data, w)
+        tokens = self._view("token_ids")
+        tokens[:live] = [e.tokens[0] for e in entries]
+        vocab, limit = self.model.spec.vocab_size, self.model.spec.max_positions
+        if tokens[:live].min() < 0 or tokens[:live].max() >= vocab:
+            raise ConfigError(f"a token id outside the vocabulary of {vocab}")
+        if limit and positions[:live].max() >= limit:
+            raise ConfigError(f"position {int(positions[:live].max())} is past the model's {limit}")
+        self._view("ctx_len")[:live] = positions[:live] + 1
+        self._view("state_slots")[:live] = [e.state_slot for e in entries]
+        self._idle_rows(live)
+
+    def run(self, entries) -> StepOutput:
+        live = len(entries)
+        self.fill(entries)
+        if self.graph is None:
+            self.capture()
+        self.device_buf.copy_(self.host, non_blocking=True)
+        self.graph.replay()
+        return StepOutput(self.logits[:live], self.tokens[:live])
+
+
+class StepRunner:
+    """Runs steps for one model and cache, keeping the captured decode graphs."""
+
+    def __init__(self, model, cache, graphs: bool = True):
+        self.model, self.cache, self.use_graphs = model, cache, graphs
+        self._graphs: dict = {}
+        self.graph_steps = 0
+        self.eager_steps = 0
+
+    def _is_plain_decode(self, entries) -> bool:
+        return (self.use_graphs and 0 < len(entries) <= GRAPH_MAX_REQUESTS
+                and all(len(e.tokens) == 1 and e.want == [0] for e in entries))
+
+    def _widths_needed(self, entries) -> list:
+        manager = self.cache.manager
+        return [max(len(manager.table(e.seq_id, g)) for e in entries) for g in range(len(self.cache.layout.groups))]
+
+    def run(self, entries) -> StepOutput:
+        entries = list(entries)
+        if not entries:
+            raise ConfigError("an empty batch")
+        if not self._is_plain_decode(entries):
+            self.eager_steps += 1
+            return StepOutput(run_step(self.model, self.cache, entries))
+        if len({e.seq_id for e in entries}) != len(entries):
+            raise ConfigError("a request appears twice in one step")
+        for e in entries:
+            if e.fresh_state and e.state_slot >= 0:
+                self.cache.clear_state_slot(e.state_slot)
+        cap = _bucket(len(entries))
+        graph = self._graphs.get(cap)
+        if graph is not None:
+            try:
+                out = graph.run(entries)
+                self.graph_steps += 1
+                return out
+            except ConfigError as error:
+                if "for room of" not in str(error):
+                    raise
+        # no graph for this many requests yet, or a request has outgrown the bucket's table
+        widths = [_bucket(w + 1, 32) for w in self._widths_needed(entries)]
+        graph = DecodeGraph(self.model, self.cache, cap, widths)
+        self._graphs[cap] = graph
+        out = graph.run(entries)
+        self.graph_steps += 1
+        return out

@@ -34,7 +34,7 @@ def _signatures(lib) -> None:
         "pl_swiglu": [p, p, i, i, i, p],
         "pl_gemm_plain": [p, p, p, i, i, i, i, i, i, i, p],
         "pl_paged_attention_plain": [p, i, p, p, p, p, i, i, p, p, i, i, i, i, f, i, i, p],
-        "pl_argmax": [p, p, i, i, p],
+        "pl_argmax": [p, p, p, p, i, i, p],
         "pl_gemm_skinny": [p, p, p, i, i, i, i, i, p],
         "pl_paged_attention_decode": [p, i, p, p, p, p, p, p, i, p, i, i, p, p, i, i, i, i, f, i, i, p],
     }
@@ -232,7 +232,10 @@ def argmax(logits: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tenso
     if out is None:
         out = torch.empty((m,), dtype=torch.int32, device=logits.device)
     _need(out, "chosen tokens", (m,), torch.int32)
-    _check(library().pl_argmax(logits.data_ptr(), out.data_ptr(), m, V, _stream()))
+    scratch_v = torch.empty((m * 64,), dtype=torch.float32, device=logits.device)
+    scratch_i = torch.empty((m * 64,), dtype=torch.int32, device=logits.device)
+    _check(library().pl_argmax(logits.data_ptr(), out.data_ptr(), scratch_v.data_ptr(), scratch_i.data_ptr(),
+                               m, V, _stream()))
     return out
 
 

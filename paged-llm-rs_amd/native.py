@@ -32,6 +32,7 @@ def _signatures(lib) -> None:
         "plh_cache_publish_full": ([vp, u64, P(u32), sz], lg),
         "plh_cache_set_prefix_cache": ([vp, i32], None), "plh_cache_sharing_possible": ([vp], i32),
         "plh_cache_table": ([vp, u64, sz, vp, sz], lg), "plh_cache_table_len": ([vp, u64, sz], lg),
+        "plh_cache_fill_step": ([vp, sz, vp, vp, sz, vp, sz], lg),
         "plh_cache_state_slot": ([vp, u64], lg), "plh_cache_wasted_tokens": ([vp, u64], lg),
         "plh_cache_counter": ([vp, sz, i32], u64), "plh_cache_live_sequences": ([vp], lg),
         "plh_cache_free_state_slots": ([vp], i32), "plh_cache_holders": ([vp, sz, i32], lg),

@@ -141,3 +141,52 @@ def test_the_command_line(model_dirs, tmp_path):
     bad = subprocess.run([sys.executable, str(ROOT / "bin" / "pagedllm"), "--model", str(d), "--chunk", "0"],
                          capture_output=True, text=True, timeout=600)
     assert bad.returncode == 1 and "--chunk 0" in bad.stderr
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_captured_decode_step_replays_like_the_eager_one(model_dirs, dtype):
+    """Every replay of the decode graph is checked against the eager step, with eager
+    work and synchronisations in between, over requests that come and go, cross page
+    edges and outgrow the graph's table."""
+    from paged_llm_rs_amd.engine.replay import Replayer
+
+    d = model_dirs("B", dtype)
+    prompts = ru.make_prompts(384, [30, 3, 17, 9, 40], seed=21)
+    steps = []
+    live = {}
+    order = list(prompts.items())
+    rng = __import__("random").Random(4)
+    fed = {}
+    # a first step with whole prompt heads (eager), then single tokens (graph), requests ending at different times
+    heads = {n: max(1, len(t) - rng.choice([3, 8, 14])) for n, t in order}
+    steps.append({"step": 0, "entries": [{"id": n, "tokens": t[:heads[n]], "want": [heads[n] - 1]} for n, t in order[:4]],
+                  "end": []})
+    fed = {n: heads[n] for n, _ in order[:4]}
+    k = 1
+    while fed:
+        entries, end = [], []
+        for n in list(fed):
+            t = prompts[n]
+            entries.append({"id": n, "tokens": [t[fed[n]]], "want": [0]})
+            fed[n] += 1
+            if fed[n] == len(t):
+                end.append(n)
+                del fed[n]
+        steps.append({"step": k, "entries": entries, "end": end})
+        k += 1
+        if k == 4:      # a late arrival: one eager step in the middle, then it joins the graph steps
+            n, t = order[4]
+            steps.append({"step": k, "entries": [{"id": n, "tokens": t[:heads[n]], "want": [heads[n] - 1]}], "end": []})
+            fed[n] = heads[n]
+            k += 1
+    eager = Replayer(d, dtype, max_tokens=64 * 5, block_size=8, graphs=False)
+    graph = Replayer(d, dtype, max_tokens=64 * 5, block_size=8, graphs=True)
+    a = ru.collect(eager, steps)
+    b = ru.collect(graph, steps)
+    assert graph.runner.graph_steps > 10 and eager.runner.graph_steps == 0
+    assert a.keys() == b.keys()
+    for key in a:
+        assert np.array_equal(a[key], b[key]), f"{key}: a replay differs from the eager step"
+
+
+import numpy as np  # noqa: E402
