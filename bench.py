@@ -130,6 +130,8 @@ def main() -> int:
                         help="fewer layers than the model has, where memory or time needs it; both numbers are reported")
     parser.add_argument("--no-graphs", action="store_true", help="run decode steps eagerly instead of as HIP graphs")
     parser.add_argument("--skip-points", action="store_true", help="leave out batch 1 and 64 and the prefill")
+    parser.add_argument("--only", choices=["decode", "prefill"], default=None,
+                        help="run one part alone (for a profiler): the decode steps at --batch, or the prefill")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU; this engine has no multi-GPU path (N must be 1)")
@@ -170,33 +172,7 @@ def main() -> int:
         bench.free()
         return seconds, batch / seconds, weight_bytes + batch * context_mid * kv_token
 
-    say(f"decode, batch {args.batch}")
-    seconds, value, step_bytes = decode_point(args.batch, args.steps, args.warmup)
-    line = {
-        "metric": "Qwen3-0.6B bf16: decode tok/s @ batch 8, ctx 512",
-        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(seconds * 1e3, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16", "data": "synthetic: random weights, uniform random token ids",
-        "config": {
-            "model": "Qwen3-0.6B shape", "global_batch": args.batch, "seq_len": CONTEXT, "parallelism": "none",
-            "layers": args.layers, "layers_full": FULL_LAYERS, "hidden": cfg["hidden_size"],
-            "q_heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
-            "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
-            "tied": True, "block_size": BLOCK_SIZE, "max_context": cfg["max_position_embeddings"],
-            "prefill_tokens": PREFILL_TOKENS,
-        },
-        "roofline": {"bound": "hbm", "achieved": round(step_bytes / seconds / 1e9, 1), "peak": HBM_PEAK / 1e9,
-                     "unit": "GB/s", "frac": round(step_bytes / seconds / HBM_PEAK, 4)},
-    }
-
-    if not args.skip_points:
-        points = {}
-        for batch in (1, 64):
-            say(f"decode, batch {batch}")
-            s, v, _ = decode_point(batch, max(args.steps // 2, 5), max(args.warmup // 2, 2))
-            points[f"decode_b{batch}"] = round(v, 1)
-        line["points"] = points
-
+    def prefill_point():
         say(f"prefill, {PREFILL_TOKENS} tokens")
         rng = random.Random(2048)
         prompt = [rng.randrange(cfg["vocab_size"]) for _ in range(PREFILL_TOKENS)]
@@ -212,9 +188,42 @@ def main() -> int:
         d, nq = cfg["head_dim"], cfg["num_attention_heads"]
         attention_flops = args.layers * 4 * nq * d * (PREFILL_TOKENS * (PREFILL_TOKENS + 1) // 2)
         flops = layer_flops * PREFILL_TOKENS + head_flops + attention_flops
-        line["prefill"] = {"value": round(PREFILL_TOKENS / seconds_prefill, 1), "tokens": PREFILL_TOKENS,
-                           "ms": round(seconds_prefill * 1e3, 3),
-                           "frac": round(flops / seconds_prefill / MFMA_PEAK["bf16"], 4)}
+        return {"value": round(PREFILL_TOKENS / seconds_prefill, 1), "tokens": PREFILL_TOKENS,
+                "ms": round(seconds_prefill * 1e3, 3),
+                "frac": round(flops / seconds_prefill / MFMA_PEAK["bf16"], 4)}
+
+    if args.only == "prefill":
+        print(json.dumps({"prefill": prefill_point()}), flush=True)
+        tmp.cleanup()
+        return 0
+
+    say(f"decode, batch {args.batch}")
+    seconds, value, step_bytes = decode_point(args.batch, args.steps, args.warmup)
+    line = {
+        "metric": f"Qwen3-0.6B bf16: decode tok/s @ batch {args.batch}, ctx 512",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(seconds * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic: random weights, uniform random token ids",
+        "config": {
+            "model": "Qwen3-0.6B shape", "global_batch": args.batch, "seq_len": CONTEXT, "parallelism": "none",
+            "layers": args.layers, "layers_full": FULL_LAYERS, "hidden": cfg["hidden_size"],
+            "q_heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
+            "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
+            "tied": True, "block_size": BLOCK_SIZE, "max_context": cfg["max_position_embeddings"],
+            "prefill_tokens": PREFILL_TOKENS,
+        },
+        "roofline": {"bound": "hbm", "achieved": round(step_bytes / seconds / 1e9, 1), "peak": HBM_PEAK / 1e9,
+                     "unit": "GB/s", "frac": round(step_bytes / seconds / HBM_PEAK, 4)},
+    }
+
+    if not args.skip_points and args.only is None:
+        points = {}
+        for batch in (1, 64):
+            say(f"decode, batch {batch}")
+            s, v, _ = decode_point(batch, max(args.steps // 2, 5), max(args.warmup // 2, 2))
+            points[f"decode_b{batch}"] = round(v, 1)
+        line["points"] = points
+        line["prefill"] = prefill_point()
 
     print(json.dumps(line), flush=True)
     tmp.cleanup()
