@@ -1,0 +1,338 @@
+// Paged attention for portions of prompts in bfloat16 on the matrix cores.
+//
+// A request brings q_len consecutive tokens to the step; the first stands at
+// position start = ctx_len - q_len.  Token i reads the keys 0..start+i (or the
+// last `window` of them) of its request through the block table; the keys of
+// its own step are already in the cache.  Requests that bring fewer than
+// `short_limit` tokens are left to the kernel for single tokens.
+//
+// One workgroup of NW waves owns 32*NW consecutive tokens of one request and
+// one query head; each wave owns 32 of them.  Keys are walked in tiles of 64:
+//
+//   S^T = K . Q^T     v_mfma_f32_32x32x16_bf16, A = a tile of keys from LDS,
+//                     B = the wave's queries, held in registers for the whole
+//                     kernel.  A lane then holds, for ONE query (lane % 32), 16
+//                     scores of each 32-key tile, so the softmax statistics are
+//                     a reduction inside the lane and one exchange with lane^32.
+//   O^T += V^T . P^T  the lane's probabilities, rounded to bfloat16, are the B
+//                     operand as they stand: the contraction index of a matrix
+//                     product may be permuted freely, so V^T is read from LDS in
+//                     the order in which the scores lie in the registers.
+//
+// V is transposed on its way into LDS (two keys packed into a 32-bit word) so
+// that the keys of one head element are contiguous.  Maximum, sum and the
+// output are 32-bit; exponentials are base 2 with log2(e) folded into the scale.
+#include "common.hpp"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+#define AP_BN 64   // keys a tile
+#define AP_KPAD 8  // padding of a row of keys in LDS, in elements
+#define AP_VPAD 4  // padding of a row of transposed values in LDS, in elements
+
+struct __attribute__((aligned(16))) ap_u32x4 {
+    uint32_t v[4];
+};
+struct __attribute__((aligned(8))) ap_u32x2 {
+    uint32_t v[2];
+};
+
+union ap_frag {
+    bf16x8 vec;
+    ap_u32x4 raw;
+    ap_u32x2 half[2];
+    uint32_t w[4];
+};
+
+__device__ __forceinline__ uint32_t ap_pack2(float lo, float hi) {
+    return static_cast<uint32_t>(bf16_bits_from_float(lo)) | (static_cast<uint32_t>(bf16_bits_from_float(hi)) << 16);
+}
+
+// DT: the head is padded to 32*DT elements.  NW: waves a workgroup.
+template <int DT, int NW>
+__global__ void __launch_bounds__(64 * NW)
+paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
+                               const int* __restrict__ q_start, const int* __restrict__ q_len,
+                               const int* __restrict__ ctx_len, int short_limit, int tiles_a_request,
+                               int num_seqs, const int* __restrict__ block_table, int max_blocks,
+                               int block_size, const bf16_t* __restrict__ k_pool,
+                               const bf16_t* __restrict__ v_pool, int nq, int nkv, int d, float scale_log2e,
+                               int window, int total_work) {
+    constexpr int DP = 32 * DT;
+    constexpr int BM = 32 * NW;
+    constexpr int NT = 64 * NW;
+    constexpr int KROW = DP + AP_KPAD;     // elements a row of Ks
+    constexpr int VROW = AP_BN + AP_VPAD;  // elements a row of Vt
+    extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+    uint16_t* Ks = lds;                    // [AP_BN][KROW]
+    uint16_t* Vt = lds + AP_BN * KROW;     // [DP][VROW]
+
+    // Workgroups are dealt round-robin to the eight XCDs; consecutive pieces of
+    // work (the token tiles of one head) go to one XCD, whose L2 then holds the
+    // keys and values they share.
+    int work = blockIdx.x;
+    if ((total_work & 7) == 0) work = (blockIdx.x & 7) * (total_work >> 3) + (blockIdx.x >> 3);
+    // work = (request * nq + head) * tiles + (tiles - 1 - tile): late tiles, which read the most keys, first
+    const int tile = tiles_a_request - 1 - work % tiles_a_request;
+    const int head = (work / tiles_a_request) % nq;
+    const int seq = work / (tiles_a_request * nq);
+    if (seq >= num_seqs) return;
+
+    const int count = q_len[seq];
+    if (count < short_limit) return;
+    const int q0 = tile * BM;
+    if (q0 >= count) return;
+    const int start = ctx_len[seq] - count;  // position of the request's first token in this step
+    const int row0 = q_start[seq];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int r32 = lane & 31;
+    const int h = lane >> 5;
+    const int kvh = head / (nq / nkv);
+
+    // columns d..DP of the key tile are never loaded: they meet zero queries and must be finite
+    if (d < DP) {
+        for (int idx = tid; idx < AP_BN * (DP - d); idx += NT) {
+            const int key = idx / (DP - d), c = idx % (DP - d);
+            Ks[key * KROW + d + c] = 0;
+        }
+    }
+
+    // the wave's queries: lane holds query wq = q0 + wave*32 + r32, elements 16*kk + 8*h .. +8
+    const int wq = q0 + wave * 32 + r32;
+    const bool q_ok = wq < count;
+    ap_frag qf[2 * DT];
+#pragma unroll
+    for (int kk = 0; kk < 2 * DT; ++kk) {
+        const int e0 = 16 * kk + 8 * h;
+        if (q_ok && e0 < d)
+            qf[kk].raw = *reinterpret_cast<const ap_u32x4*>(q + static_cast<size_t>(row0 + wq) * q_stride +
+                                                            static_cast<size_t>(head) * d + e0);
+        else
+            qf[kk].raw = ap_u32x4{{0u, 0u, 0u, 0u}};
+    }
+    const int q_pos = start + wq;                               // position of this lane's query
+    const int wave_first = start + q0 + wave * 32;              // position of the wave's first query
+    const int wave_last = start + min(q0 + wave * 32 + 31, count - 1);
+    const bool wave_active = q0 + wave * 32 < count;
+
+    f32x16 o[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[dt][r] = 0.f;
+    float m = -INFINITY, lsum = 0.f;
+
+    const int last_pos = start + min(q0 + BM, count) - 1;       // the last key any query of the tile sees
+    const int first_pos = (window > 0 && start + q0 + 1 > window) ? start + q0 + 1 - window : 0;
+    const int* table = block_table + static_cast<size_t>(seq) * max_blocks;
+    const size_t row_stride = static_cast<size_t>(nkv) * d;
+    const size_t head_off = static_cast<size_t>(kvh) * d;
+    const int cpr = d / 8;                                      // 16-byte pieces a row
+    const bool pow2 = (block_size & (block_size - 1)) == 0;
+    const int shift = 31 - __clz(block_size);
+
+    for (int k0 = (first_pos / AP_BN) * AP_BN; k0 <= last_pos; k0 += AP_BN) {
+        __syncthreads();  // the previous tile has been read by every wave
+        // keys: 16 consecutive lanes (d = 128) read one row
+        for (int idx = tid; idx < AP_BN * cpr; idx += NT) {
+            const int key = idx / cpr, c = idx - key * cpr;
+            const int j = k0 + key;
+            ap_u32x4 val = ap_u32x4{{0u, 0u, 0u, 0u}};
+            if (j <= last_pos) {
+                const int bi = pow2 ? (j >> shift) : (j / block_size);
+                const int within = pow2 ? (j & (block_size - 1)) : (j - bi * block_size);
+                const int blk = table[bi];
+                if (blk >= 0)
+                    val = *reinterpret_cast<const ap_u32x4*>(
+                        k_pool + (static_cast<size_t>(blk) * block_size + within) * row_stride + head_off + c * 8);
+            }
+            *reinterpret_cast<ap_u32x4*>(Ks + key * KROW + c * 8) = val;
+        }
+        // values: a thread takes two neighbouring keys and stores them transposed, one pair a word
+        for (int idx = tid; idx < (AP_BN / 2) * cpr; idx += NT) {
+            const int pair = idx / cpr, c = idx - pair * cpr;
+            ap_u32x4 v0 = ap_u32x4{{0u, 0u, 0u, 0u}}, v1 = v0;
+            const int j = k0 + 2 * pair;
+            if (j <= last_pos) {
+                const int bi = pow2 ? (j >> shift) : (j / block_size);
+                const int within = pow2 ? (j & (block_size - 1)) : (j - bi * block_size);
+                const int blk = table[bi];
+                if (blk >= 0)
+                    v0 = *reinterpret_cast<const ap_u32x4*>(
+                        v_pool + (static_cast<size_t>(blk) * block_size + within) * row_stride + head_off + c * 8);
+            }
+            if (j + 1 <= last_pos) {
+                const int bi = pow2 ? ((j + 1) >> shift) : ((j + 1) / block_size);
+                const int within = pow2 ? ((j + 1) & (block_size - 1)) : (j + 1 - bi * block_size);
+                const int blk = table[bi];
+                if (blk >= 0)
+                    v1 = *reinterpret_cast<const ap_u32x4*>(
+                        v_pool + (static_cast<size_t>(blk) * block_size + within) * row_stride + head_off + c * 8);
+            }
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const uint32_t even = (v0.v[w] & 0xffffu) | (v1.v[w] << 16);
+                const uint32_t odd = (v0.v[w] >> 16) | (v1.v[w] & 0xffff0000u);
+                *reinterpret_cast<uint32_t*>(Vt + (c * 8 + 2 * w) * VROW + 2 * pair) = even;
+                *reinterpret_cast<uint32_t*>(Vt + (c * 8 + 2 * w + 1) * VROW + 2 * pair) = odd;
+            }
+        }
+        __syncthreads();
+
+        // a wave whose queries all stand before this tile, or that has no queries, has nothing to add
+        if (!wave_active || k0 > wave_last) continue;
+        if (window > 0 && k0 + AP_BN - 1 <= wave_first - window) continue;
+
+        // scores, transposed: s[kt][4*j + i] is key k0 + 32*kt + 8*j + 4*h + i against query r32
+        f32x16 s[2];
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[kt][r] = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < 2 * DT; ++kk) {
+                ap_frag a;
+                a.raw = *reinterpret_cast<const ap_u32x4*>(Ks + (32 * kt + r32) * KROW + 16 * kk + 8 * h);
+                s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.vec, qf[kk].vec, s[kt], 0, 0, 0);
+            }
+        }
+        const bool edge = k0 + AP_BN - 1 > wave_first || window > 0;  // some key of the tile is hidden from some query
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float v = s[kt][r] * scale_log2e;
+                if (edge) {
+                    const int key = k0 + 32 * kt + 8 * (r >> 2) + 4 * h + (r & 3);
+                    const bool seen = key <= q_pos && (window <= 0 || key > q_pos - window);
+                    v = seen ? v : -INFINITY;
+                }
+                s[kt][r] = v;
+                mx = fmaxf(mx, v);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, PL_WAVE));
+        const float m_new = fmaxf(m, mx);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        const float corr = exp2f(m - m_use);
+        float psum = 0.f;
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float p = exp2f(s[kt][r] - m_use);
+                s[kt][r] = p;
+                psum += p;
+            }
+        lsum = lsum * corr + psum;
+        m = m_new;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[dt][r] *= corr;
+
+        // O^T += V^T . P^T, sixteen keys a product: registers 8*half .. 8*half+7 of tile kt are the
+        // keys 32*kt + 16*half + {4h..4h+3} and + 8 + {4h..4h+3}
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                ap_frag b;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) b.w[w] = ap_pack2(s[kt][8 * half + 2 * w], s[kt][8 * half + 2 * w + 1]);
+                const int key_off = 32 * kt + 16 * half + 4 * h;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    ap_frag a;
+                    const uint16_t* row = Vt + (32 * dt + r32) * VROW + key_off;
+                    a.half[0] = *reinterpret_cast<const ap_u32x2*>(row);
+                    a.half[1] = *reinterpret_cast<const ap_u32x2*>(row + 8);
+                    o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.vec, b.vec, o[dt], 0, 0, 0);
+                }
+            }
+    }
+
+    if (!q_ok) return;
+    const float total = lsum + __shfl_xor(lsum, 32, PL_WAVE);
+    const float inv = total > 0.f ? 1.f / total : 0.f;
+    // o[dt][4*j + i] is element 32*dt + 8*j + 4*h + i of query r32
+    bf16_t* orow = out + (static_cast<size_t>(row0 + wq) * nq + head) * d;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int e0 = 32 * dt + 8 * j + 4 * h;
+            if (e0 < d) {
+                ap_u32x2 w;
+                w.v[0] = ap_pack2(o[dt][4 * j] * inv, o[dt][4 * j + 1] * inv);
+                w.v[1] = ap_pack2(o[dt][4 * j + 2] * inv, o[dt][4 * j + 3] * inv);
+                *reinterpret_cast<ap_u32x2*>(orow + e0) = w;
+            }
+        }
+}
+
+template <int DT, int NW>
+static int launch_prefill(const void* q, int q_stride, void* out, const int* q_start, const int* q_len,
+                          const int* ctx_len, int short_limit, int num_seqs, int max_q_len, const int* block_table,
+                          int max_blocks, int block_size, const void* k_pool, const void* v_pool, int nq, int nkv,
+                          int d, float scale, int window, hipStream_t stream) {
+    constexpr int DP = 32 * DT;
+    constexpr int BM = 32 * NW;
+    const size_t lds_bytes = (static_cast<size_t>(AP_BN) * (DP + AP_KPAD) + static_cast<size_t>(DP) * (AP_BN + AP_VPAD)) * 2;
+    if (lds_bytes > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_prefill_kernel<DT, NW>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+        PL_REQUIRE(e == hipSuccess, "prefill attention: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
+    }
+    const int tiles = pl_ceil_div(max_q_len, BM);
+    const long long total = static_cast<long long>(tiles) * nq * num_seqs;
+    PL_REQUIRE(total > 0 && total < (1ll << 30), "prefill attention: %lld workgroups", total);
+    paged_attention_prefill_kernel<DT, NW><<<static_cast<int>(total), 64 * NW, lds_bytes, stream>>>(
+        static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), q_start, q_len, ctx_len, short_limit, tiles,
+        num_seqs, block_table, max_blocks, block_size, static_cast<const bf16_t*>(k_pool),
+        static_cast<const bf16_t*>(v_pool), nq, nkv, d, scale * 1.4426950408889634f, window, static_cast<int>(total));
+    PL_CHECK_LAUNCH("paged_attention_prefill");
+    return 0;
+}
+
+// bfloat16 only.  q rows begin with the nq*d rotated query values; request s brings the rows
+// q_start[s] .. q_start[s] + q_len[s] - 1, which stand at the positions ctx_len[s] - q_len[s] .. ctx_len[s] - 1.
+// Requests with q_len < short_limit are skipped.  max_q_len bounds q_len over the requests.
+extern "C" int pl_paged_attention_prefill(const void* q, int q_stride, void* out, const int* q_start,
+                                          const int* q_len, const int* ctx_len, int short_limit, int num_seqs,
+                                          int max_q_len, const int* block_table, int max_blocks, int block_size,
+                                          const void* k_pool, const void* v_pool, int nq, int nkv, int d,
+                                          float scale, int window, hipStream_t stream) {
+    PL_REQUIRE(d > 0 && d <= 256 && d % 16 == 0, "prefill attention: head size %d, which has to be a multiple of 16 up to 256", d);
+    PL_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "prefill attention: %d query heads over %d key heads", nq, nkv);
+    PL_REQUIRE(block_size > 0 && max_blocks > 0 && q_stride >= nq * d && q_stride % 8 == 0 && window >= 0,
+               "prefill attention: block size %d, %d blocks a row, query stride %d, window %d", block_size, max_blocks,
+               q_stride, window);
+    PL_REQUIRE((nkv * d) % 8 == 0, "prefill attention: a cache row of %d elements is not read 16 bytes at a time", nkv * d);
+    if (num_seqs <= 0 || max_q_len <= 0) return 0;
+    const int dt = pl_ceil_div(d, 32);
+    // few tokens a request: 64-token tiles give twice the workgroups
+    const bool small = max_q_len <= 64;
+#define AP_CALL(D)                                                                                                 \
+    return small ? launch_prefill<D, 2>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len, \
+                                        block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale,   \
+                                        window, stream)                                                            \
+                 : launch_prefill<D, 4>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len, \
+                                        block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale,   \
+                                        window, stream)
+    switch (dt) {
+        case 1: AP_CALL(1);
+        case 2: AP_CALL(2);
+        case 3: AP_CALL(3);
+        case 4: AP_CALL(4);
+        case 5: AP_CALL(5);
+        case 6: AP_CALL(6);
+        case 7: AP_CALL(7);
+        default: AP_CALL(8);
+    }
+#undef AP_CALL
+}

@@ -34,7 +34,8 @@ class StepBatch:
     """Device tensors of one step (all int32)."""
 
     def __init__(self, packed: torch.Tensor, layout: dict, num_tokens: int, num_seqs: int, max_blocks: list,
-                 num_logit_rows: int, max_q_len: int, max_ctx_len: int, seq_ids: list):
+                 num_logit_rows: int, max_q_len: int, max_ctx_len: int, seq_ids: list,
+                 short_tokens: int | None = None):
         self.packed = packed
         self.num_tokens = num_tokens
         self.num_seqs = num_seqs
@@ -42,6 +43,8 @@ class StepBatch:
         self.max_q_len = max_q_len
         self.max_ctx_len = max_ctx_len
         self.seq_ids = seq_ids
+        # tokens of requests that bring fewer than SHORT_PORTION tokens: the single-token kernel's share
+        self.short_tokens = num_tokens if short_tokens is None else short_tokens
 
         def view(name, *shape):
             begin, count = layout[name]
@@ -131,5 +134,6 @@ def build_batch(entries, manager, num_groups: int, vocab_size: int, max_position
         begin, count = layout[name]
         host[begin:begin + count] = arr
     packed = torch.from_numpy(host).to(device)
+    from ..kernels import SHORT_PORTION
     return StepBatch(packed, layout, n, S, max_blocks, len(logit_rows), int(q_len.max()), int(ctx_len.max()),
-                     [e.seq_id for e in entries])
+                     [e.seq_id for e in entries], short_tokens=int(q_len[q_len < SHORT_PORTION].sum()))

@@ -37,6 +37,7 @@ def _signatures(lib) -> None:
         "pl_argmax": [p, p, p, p, i, i, p],
         "pl_gemm_skinny": [p, p, p, i, i, i, i, i, p],
         "pl_paged_attention_decode": [p, i, p, p, p, p, p, p, i, p, i, i, p, p, i, i, i, i, f, i, i, p],
+        "pl_paged_attention_prefill": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, p],
     }
     for name, argtypes in table.items():
         fn = getattr(lib, name)
@@ -298,15 +299,56 @@ def paged_attention_decode(q: torch.Tensor, q_row_stride: int, out: torch.Tensor
     return out
 
 
+def paged_attention_prefill(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, q_start: torch.Tensor,
+                            q_len: torch.Tensor, ctx_len: torch.Tensor, max_q_len: int, block_table: torch.Tensor,
+                            block_size: int, k_pool: torch.Tensor, v_pool: torch.Tensor, nq: int, nkv: int, d: int,
+                            scale: float, window: int = 0, short_limit: int = 0) -> torch.Tensor:
+    """bfloat16 attention of prompt portions on the matrix cores.  Request s brings the rows
+    q_start[s] .. q_start[s]+q_len[s]-1 at the positions ctx_len[s]-q_len[s] .. ctx_len[s]-1;
+    requests with fewer than ``short_limit`` tokens are skipped."""
+    n = q.shape[0]
+    S = block_table.shape[0]
+    _need(q, "query buffer", None, torch.bfloat16)
+    if q.dim() != 2 or q.shape[1] != q_row_stride or q_row_stride < nq * d:
+        raise TensorError(f"query buffer has shape {tuple(q.shape)} for row stride {q_row_stride}")
+    _need(out, "attention output", (n, nq * d), torch.bfloat16)
+    _need(block_table, "block table", None, torch.int32)
+    for t, what in ((q_start, "first row of each request"), (q_len, "tokens of each request"),
+                    (ctx_len, "context length of each request")):
+        _need(t, what, (S,), torch.int32)
+    for pool, what in ((k_pool, "key pool"), (v_pool, "value pool")):
+        _need(pool, what, None, torch.bfloat16)
+        if pool.dim() != 2 or pool.shape[1] != nkv * d or pool.shape[0] % block_size != 0:
+            raise TensorError(f"{what} has shape {tuple(pool.shape)}, expected [pages*{block_size}, {nkv * d}]")
+    if not 0 < max_q_len <= n:
+        raise TensorError(f"the longest portion is said to have {max_q_len} of the step's {n} tokens")
+    _check(library().pl_paged_attention_prefill(
+        q.data_ptr(), q_row_stride, out.data_ptr(), q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(),
+        int(short_limit), S, int(max_q_len), block_table.data_ptr(), block_table.shape[1], block_size,
+        k_pool.data_ptr(), v_pool.data_ptr(), nq, nkv, d, float(scale), int(window or 0), _stream()))
+    return out
+
+
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nkv: int, d: int,
                     scale: float, window: int = 0) -> torch.Tensor:
-    """Attention for every token of a step.  ``qkv`` rows begin with the rotated queries."""
-    if qkv.dtype == torch.bfloat16 and _attention_mode == "kernel" and batch.max_q_len < SHORT_PORTION:
-        splits = decode_splits(batch.num_tokens, nq, nkv, batch.max_ctx_len)
-        return paged_attention_decode(qkv, qkv.shape[1], out, batch.positions, batch.seq_of, kv.block_table,
-                                      kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window, splits)
-    return paged_attention_plain(qkv, qkv.shape[1], out, batch.positions, batch.seq_of, kv.block_table,
-                                 kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window)
+    """Attention for every token of a step.  ``qkv`` rows begin with the rotated queries.
+    In bfloat16 the long portions go to the tiled kernel and the tokens of short ones
+    (decoded tokens among them) to the kernel for single tokens; both read the same pages."""
+    if qkv.dtype != torch.bfloat16 or _attention_mode != "kernel":
+        return paged_attention_plain(qkv, qkv.shape[1], out, batch.positions, batch.seq_of, kv.block_table,
+                                     kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window)
+    stride = qkv.shape[1]
+    if batch.max_q_len >= SHORT_PORTION:
+        paged_attention_prefill(qkv, stride, out, batch.q_start, batch.q_len, batch.ctx_len, batch.max_q_len,
+                                kv.block_table, kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window,
+                                short_limit=SHORT_PORTION)
+        if batch.short_tokens == 0:
+            return out
+    mixed = batch.max_q_len >= SHORT_PORTION
+    splits = decode_splits(batch.short_tokens, nq, nkv, batch.max_ctx_len)
+    return paged_attention_decode(qkv, stride, out, batch.positions, batch.seq_of, kv.block_table,
+                                  kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window, splits,
+                                  q_len=batch.q_len if mixed else None, short_limit=SHORT_PORTION if mixed else 0)
 
 
 def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,

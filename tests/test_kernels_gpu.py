@@ -351,6 +351,94 @@ def test_a_far_key_among_hundreds_is_found(kernel):
         assert hit == inside, f"key {target} of {ctx} with window {window}: found {hit}, visible {inside}"
 
 
+PORTION_CASES = [
+    # nq, nkv, d, block size, [(context length after the step, tokens of the step)], window
+    (4, 2, 16, 4, [(40, 40), (70, 17), (5, 1)], 0),
+    (6, 1, 32, 8, [(200, 130), (9, 9)], 0),
+    (6, 2, 48, 16, [(150, 64), (33, 33), (64, 16)], 0),
+    (16, 8, 128, 16, [(513, 300), (40, 2), (129, 129)], 0),
+    (3, 3, 80, 2, [(97, 65)], 0),
+    (4, 2, 112, 16, [(260, 129)], 0),
+    (2, 1, 256, 16, [(150, 77)], 0),
+    (4, 2, 64, 16, [(300, 140), (31, 31)], 48),
+    (2, 2, 16, 4, [(90, 70)], 7),
+    (2, 2, 32, 16, [(500, 200)], 64),
+]
+
+
+@pytest.mark.parametrize("nq,nkv,d,bs,requests,window", PORTION_CASES)
+def test_paged_attention_of_portions(nq, nkv, d, bs, requests, window):
+    """The tiled kernel takes the requests that bring 16 tokens or more, the single-token kernel
+    the others; together they fill every row of the step."""
+    from paged_llm_rs_amd import kernels
+
+    dtype = torch.bfloat16
+    ctx_lens = [c for c, _ in requests]
+    bt, k_pool, v_pool, keys, values = build_paged(nkv, d, bs, ctx_lens, dtype, seed=d + bs + len(requests))
+    n = sum(c for _, c in requests)
+    stride = (nq + 2 * nkv) * d
+    q = torch.randn(n, stride, device=DEV).to(dtype)
+    q_start, q_len, positions, seq_of = [], [], [], []
+    for s, (ctx, count) in enumerate(requests):
+        q_start.append(len(positions))
+        q_len.append(count)
+        positions += list(range(ctx - count, ctx))
+        seq_of += [s] * count
+    as_i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    q_start_t, q_len_t, ctx_t = as_i32(q_start), as_i32(q_len), as_i32(ctx_lens)
+    scale = 1 / math.sqrt(d)
+    out = torch.full((n, nq * d), 7.0, dtype=dtype, device=DEV)
+    limit = kernels.SHORT_PORTION
+    kernels.paged_attention_prefill(q, stride, out, q_start_t, q_len_t, ctx_t, max(q_len), bt, bs, k_pool, v_pool,
+                                    nq, nkv, d, scale, window, short_limit=limit)
+    for s, (ctx, count) in enumerate(requests):
+        if count < limit:
+            rows = out[q_start[s]:q_start[s] + count]
+            assert bool((rows == 7.0).all()), "a short request is left to the other kernel"
+    kernels.paged_attention_decode(q, stride, out, as_i32(positions), as_i32(seq_of), bt, bs, k_pool, v_pool, nq, nkv, d,
+                                   scale, window, splits=2, q_len=q_len_t, short_limit=limit)
+    g = nq // nkv
+    worst = 0.0
+    for i in range(n):
+        s, p = seq_of[i], positions[i]
+        want = attention_ref(q[i, :nq * d].double().cpu().reshape(nq, d), keys[s], values[s], p, g, scale, window)
+        err = rel(out[i].reshape(nq, d), want)
+        worst = max(worst, err)
+        assert err < 1e-2, f"token {i} (request {s}, position {p}): {err:.3e}"
+
+
+def test_a_far_key_is_found_from_inside_a_portion():
+    """One key carries nearly all the weight of one query in the middle of a long portion: a key of an
+    earlier step across a page edge, a key of the same step, the query's own key, and keys at a window's edge."""
+    from paged_llm_rs_amd import kernels
+
+    nq, nkv, d, bs = 4, 2, 64, 16
+    dtype = torch.bfloat16
+    ctx, count = 700, 333
+    start = ctx - count
+    for query, target, window in [(500, 16, 0), (500, 15, 0), (500, 500, 0), (500, 0, 0), (699, 698, 0),
+                                  (start, start - 1, 0), (start + 127, start + 64, 0), (start + 128, start + 127, 0),
+                                  (500, 401, 100), (500, 400, 100), (start + 1, start + 1 - 99, 100)]:
+        bt, k_pool, v_pool, keys, values = build_paged(nkv, d, bs, [ctx], dtype, seed=query + target)
+        stride = (nq + 2 * nkv) * d
+        q = torch.randn(count, stride, device=DEV).to(dtype)
+        row = query - start
+        slot = int(bt[0, target // bs]) * bs + target % bs
+        for kvh in range(nkv):
+            k_pool[slot, kvh * d:(kvh + 1) * d] = (q[row, kvh * 2 * d: kvh * 2 * d + d].float() * 4).to(dtype)
+            keys[0][target, kvh] = k_pool[slot, kvh * d:(kvh + 1) * d].double().cpu()
+        as_i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+        out = torch.zeros(count, nq * d, dtype=dtype, device=DEV)
+        scale = 1 / math.sqrt(d)
+        kernels.paged_attention_prefill(q, stride, out, as_i32([0]), as_i32([count]), as_i32([ctx]), count, bt, bs,
+                                        k_pool, v_pool, nq, nkv, d, scale, window, short_limit=16)
+        want = attention_ref(q[row, :nq * d].double().cpu().reshape(nq, d), keys[0], values[0], query, 2, scale, window)
+        assert rel(out[row].reshape(nq, d), want) < 1e-2, (query, target, window)
+        inside = target <= query and (window == 0 or target > query - window)
+        hit = rel(out[row].reshape(nq, d)[0], values[0][target, 0]) < 0.2
+        assert hit == inside, f"key {target} for the query at {query} with window {window}: found {hit}, visible {inside}"
+
+
 # --- sampling ------------------------------------------------------------------------------------------------------
 
 def test_argmax_first_maximum_wins():
