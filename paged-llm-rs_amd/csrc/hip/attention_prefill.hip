@@ -27,6 +27,9 @@
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
+#ifndef AP_OCC
+#define AP_OCC 2  // waves a SIMD the registers are kept within
+#endif
 #define AP_BN 64   // keys a tile
 #define AP_KPAD 8  // padding of a row of keys in LDS, in elements
 #define AP_VPAD 4  // padding of a row of transposed values in LDS, in elements
@@ -45,13 +48,18 @@ union ap_frag {
     uint32_t w[4];
 };
 
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+// Two floats rounded to nearest-even bfloat16 in one word (the hardware's packed conversion).
 __device__ __forceinline__ uint32_t ap_pack2(float lo, float hi) {
-    return static_cast<uint32_t>(bf16_bits_from_float(lo)) | (static_cast<uint32_t>(bf16_bits_from_float(hi)) << 16);
+    const f32x2 pair = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
 }
 
 // DT: the head is padded to 32*DT elements.  NW: waves a workgroup.
 template <int DT, int NW>
-__global__ void __launch_bounds__(64 * NW)
+__global__ void __launch_bounds__(64 * NW, AP_OCC * 4 / NW)
 paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
                                const int* __restrict__ q_start, const int* __restrict__ q_len,
                                const int* __restrict__ ctx_len, int short_limit, int tiles_a_request,
@@ -88,18 +96,10 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // the same for the whole wave: kept scalar
     const int r32 = lane & 31;
     const int h = lane >> 5;
     const int kvh = head / (nq / nkv);
-
-    // columns d..DP of the key tile are never loaded: they meet zero queries and must be finite
-    if (d < DP) {
-        for (int idx = tid; idx < AP_BN * (DP - d); idx += NT) {
-            const int key = idx / (DP - d), c = idx % (DP - d);
-            Ks[key * KROW + d + c] = 0;
-        }
-    }
 
     // the wave's queries: lane holds query wq = q0 + wave*32 + r32, elements 16*kk + 8*h .. +8
     const int wq = q0 + wave * 32 + r32;
@@ -131,57 +131,104 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     const int* table = block_table + static_cast<size_t>(seq) * max_blocks;
     const size_t row_stride = static_cast<size_t>(nkv) * d;
     const size_t head_off = static_cast<size_t>(kvh) * d;
-    const int cpr = d / 8;                                      // 16-byte pieces a row
-    const bool pow2 = (block_size & (block_size - 1)) == 0;
-    const int shift = 31 - __clz(block_size);
+    const int cpr = d / 8;                                      // 16-byte pieces of a row of the head
+    // floor(2^32 / block_size): the high half of j * bs_magic is j / block_size or one less
+    const uint32_t bs_magic = block_size == 1 ? 0xffffffffu : static_cast<uint32_t>(0x100000000ull / static_cast<uint32_t>(block_size));
 
-    for (int k0 = (first_pos / AP_BN) * AP_BN; k0 <= last_pos; k0 += AP_BN) {
-        __syncthreads();  // the previous tile has been read by every wave
-        // keys: 16 consecutive lanes (d = 128) read one row
-        for (int idx = tid; idx < AP_BN * cpr; idx += NT) {
-            const int key = idx / cpr, c = idx - key * cpr;
-            const int j = k0 + key;
-            ap_u32x4 val = ap_u32x4{{0u, 0u, 0u, 0u}};
-            if (j <= last_pos) {
-                const int bi = pow2 ? (j >> shift) : (j / block_size);
-                const int within = pow2 ? (j & (block_size - 1)) : (j - bi * block_size);
-                const int blk = table[bi];
-                if (blk >= 0)
-                    val = *reinterpret_cast<const ap_u32x4*>(
-                        k_pool + (static_cast<size_t>(blk) * block_size + within) * row_stride + head_off + c * 8);
-            }
-            *reinterpret_cast<ap_u32x4*>(Ks + key * KROW + c * 8) = val;
+    // A tile travels global memory -> registers -> LDS.  The loads of the next tile are issued before
+    // the products of this one, so that their latency passes behind the matrix cores.
+    constexpr int CP = DP / 8;                                  // 16-byte pieces of a padded row
+    constexpr int KI = (AP_BN * CP + NT - 1) / NT;              // pieces of the key tile a thread carries
+    constexpr int VI = (AP_BN / 2 * CP + NT - 1) / NT;          // pairs of pieces of the value tile
+    ap_u32x4 kreg[KI], vreg0[VI], vreg1[VI];
+
+    // Loads are unconditional, from an address that is valid in any case, and what they bring is
+    // masked afterwards where the key does not exist: a load inside a branch would be waited for
+    // at the branch's end, one load after the other.  The page numbers of a tile are looked up one
+    // tile before its keys and values are loaded, so that no load waits for another.
+    int kblk[KI], kwithin[KI], vblk[VI][2], vwithin[VI][2];
+    auto locate = [&](int j, int& blk, int& within) {           // page and place in the page of key j
+        const bool in = j <= last_pos;
+        const int jj = in ? j : last_pos;
+        int bi = static_cast<int>(__umulhi(static_cast<uint32_t>(jj), bs_magic));
+        within = jj - bi * block_size;
+        const int low = within >= block_size ? 1 : 0;            // the estimate is the quotient or one less
+        bi += low;
+        within -= low * block_size;
+        const int got = table[bi];
+        blk = in ? got : -1;
+    };
+    auto lookup = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < KI; ++i) locate(k0 + ((tid + i * NT) / CP) % AP_BN, kblk[i], kwithin[i]);
+#pragma unroll
+        for (int i = 0; i < VI; ++i) {
+            const int pair = ((tid + i * NT) / CP) % (AP_BN / 2);
+            locate(k0 + 2 * pair, vblk[i][0], vwithin[i][0]);
+            locate(k0 + 2 * pair + 1, vblk[i][1], vwithin[i][1]);
         }
-        // values: a thread takes two neighbouring keys and stores them transposed, one pair a word
-        for (int idx = tid; idx < (AP_BN / 2) * cpr; idx += NT) {
-            const int pair = idx / cpr, c = idx - pair * cpr;
-            ap_u32x4 v0 = ap_u32x4{{0u, 0u, 0u, 0u}}, v1 = v0;
-            const int j = k0 + 2 * pair;
-            if (j <= last_pos) {
-                const int bi = pow2 ? (j >> shift) : (j / block_size);
-                const int within = pow2 ? (j & (block_size - 1)) : (j - bi * block_size);
-                const int blk = table[bi];
-                if (blk >= 0)
-                    v0 = *reinterpret_cast<const ap_u32x4*>(
-                        v_pool + (static_cast<size_t>(blk) * block_size + within) * row_stride + head_off + c * 8);
-            }
-            if (j + 1 <= last_pos) {
-                const int bi = pow2 ? ((j + 1) >> shift) : ((j + 1) / block_size);
-                const int within = pow2 ? ((j + 1) & (block_size - 1)) : (j + 1 - bi * block_size);
-                const int blk = table[bi];
-                if (blk >= 0)
-                    v1 = *reinterpret_cast<const ap_u32x4*>(
-                        v_pool + (static_cast<size_t>(blk) * block_size + within) * row_stride + head_off + c * 8);
-            }
+    };
+    auto row_of = [&](int blk, int within) -> size_t {
+        return (static_cast<size_t>(max(blk, 0)) * block_size + within) * row_stride;
+    };
+    auto fetch = [&]() {
+#pragma unroll
+        for (int i = 0; i < KI; ++i) {
+            const int c = (tid + i * NT) % CP;
+            const ap_u32x4 got = *reinterpret_cast<const ap_u32x4*>(k_pool + row_of(kblk[i], kwithin[i]) + head_off + min(c, cpr - 1) * 8);
+            const uint32_t keep = (kblk[i] >= 0 && c < cpr) ? 0xffffffffu : 0u;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) kreg[i].v[w] = got.v[w] & keep;
+        }
+#pragma unroll
+        for (int i = 0; i < VI; ++i) {
+            const int c = (tid + i * NT) % CP;
+            const size_t col = head_off + min(c, cpr - 1) * 8;
+            const ap_u32x4 got0 = *reinterpret_cast<const ap_u32x4*>(v_pool + row_of(vblk[i][0], vwithin[i][0]) + col);
+            const ap_u32x4 got1 = *reinterpret_cast<const ap_u32x4*>(v_pool + row_of(vblk[i][1], vwithin[i][1]) + col);
+            const uint32_t keep0 = (vblk[i][0] >= 0 && c < cpr) ? 0xffffffffu : 0u;
+            const uint32_t keep1 = (vblk[i][1] >= 0 && c < cpr) ? 0xffffffffu : 0u;
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
-                const uint32_t even = (v0.v[w] & 0xffffu) | (v1.v[w] << 16);
-                const uint32_t odd = (v0.v[w] >> 16) | (v1.v[w] & 0xffff0000u);
-                *reinterpret_cast<uint32_t*>(Vt + (c * 8 + 2 * w) * VROW + 2 * pair) = even;
-                *reinterpret_cast<uint32_t*>(Vt + (c * 8 + 2 * w + 1) * VROW + 2 * pair) = odd;
+                vreg0[i].v[w] = got0.v[w] & keep0;
+                vreg1[i].v[w] = got1.v[w] & keep1;
             }
         }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int i = 0; i < KI; ++i) {
+            const int idx = tid + i * NT;
+            const int key = idx / CP, c = idx % CP;
+            if (idx < AP_BN * CP) *reinterpret_cast<ap_u32x4*>(Ks + key * KROW + c * 8) = kreg[i];
+        }
+        // values are stored transposed, two neighbouring keys a word
+#pragma unroll
+        for (int i = 0; i < VI; ++i) {
+            const int idx = tid + i * NT;
+            const int pair = idx / CP, c = idx % CP;
+            if (idx < AP_BN / 2 * CP) {
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const uint32_t even = (vreg0[i].v[w] & 0xffffu) | (vreg1[i].v[w] << 16);
+                    const uint32_t odd = (vreg0[i].v[w] >> 16) | (vreg1[i].v[w] & 0xffff0000u);
+                    *reinterpret_cast<uint32_t*>(Vt + (c * 8 + 2 * w) * VROW + 2 * pair) = even;
+                    *reinterpret_cast<uint32_t*>(Vt + (c * 8 + 2 * w + 1) * VROW + 2 * pair) = odd;
+                }
+            }
+        }
+    };
+
+    const int k_first = (first_pos / AP_BN) * AP_BN;
+    lookup(k_first);
+    fetch();
+    lookup(k_first + AP_BN);
+    for (int k0 = k_first; k0 <= last_pos; k0 += AP_BN) {
+        __syncthreads();  // the previous tile has been read by every wave
+        stash();
         __syncthreads();
+        fetch();                     // tile k0 + AP_BN, all zeros past the last key
+        lookup(k0 + 2 * AP_BN);
 
         // a wave whose queries all stand before this tile, or that has no queries, has nothing to add
         if (!wave_active || k0 > wave_last) continue;
@@ -193,38 +240,50 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) s[kt][r] = 0.f;
+            ap_frag a[2 * DT];
 #pragma unroll
-            for (int kk = 0; kk < 2 * DT; ++kk) {
-                ap_frag a;
-                a.raw = *reinterpret_cast<const ap_u32x4*>(Ks + (32 * kt + r32) * KROW + 16 * kk + 8 * h);
-                s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.vec, qf[kk].vec, s[kt], 0, 0, 0);
-            }
+            for (int kk = 0; kk < 2 * DT; ++kk)
+                a[kk].raw = *reinterpret_cast<const ap_u32x4*>(Ks + (32 * kt + r32) * KROW + 16 * kk + 8 * h);
+#pragma unroll
+            for (int kk = 0; kk < 2 * DT; ++kk)
+                s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kk].vec, qf[kk].vec, s[kt], 0, 0, 0);
         }
-        const bool edge = k0 + AP_BN - 1 > wave_first || window > 0;  // some key of the tile is hidden from some query
+        // Key k0 + c + 4*h, c a constant of the register, is seen by this lane's query iff c <= reach
+        // (and c > reach - window).  Tiles that lie before every query of the wave need no test.
+        const bool edge = k0 + AP_BN - 1 > wave_first || window > 0;
+        const int reach = q_pos - k0 - 4 * h;
+        const int behind = window > 0 ? reach - window : -(1 << 30);
         float mx = -INFINITY;
+        if (edge) {
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
+            for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                float v = s[kt][r] * scale_log2e;
-                if (edge) {
-                    const int key = k0 + 32 * kt + 8 * (r >> 2) + 4 * h + (r & 3);
-                    const bool seen = key <= q_pos && (window <= 0 || key > q_pos - window);
-                    v = seen ? v : -INFINITY;
+                for (int r = 0; r < 16; ++r) {
+                    const int c = 32 * kt + 8 * (r >> 2) + (r & 3);
+                    const float v = (c <= reach && c > behind) ? s[kt][r] * scale_log2e : -INFINITY;
+                    s[kt][r] = v;
+                    mx = fmaxf(mx, v);
                 }
-                s[kt][r] = v;
-                mx = fmaxf(mx, v);
-            }
+        } else {
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float v = s[kt][r] * scale_log2e;
+                    s[kt][r] = v;
+                    mx = fmaxf(mx, v);
+                }
+        }
         mx = fmaxf(mx, __shfl_xor(mx, 32, PL_WAVE));
         const float m_new = fmaxf(m, mx);
         const float m_use = m_new == -INFINITY ? 0.f : m_new;
-        const float corr = exp2f(m - m_use);
+        const float corr = __builtin_amdgcn_exp2f(m - m_use);
         float psum = 0.f;
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const float p = exp2f(s[kt][r] - m_use);
+                const float p = __builtin_amdgcn_exp2f(s[kt][r] - m_use);  // v_exp_f32: arguments are <= 0, tiny results may flush
                 s[kt][r] = p;
                 psum += p;
             }
@@ -245,14 +304,16 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
 #pragma unroll
                 for (int w = 0; w < 4; ++w) b.w[w] = ap_pack2(s[kt][8 * half + 2 * w], s[kt][8 * half + 2 * w + 1]);
                 const int key_off = 32 * kt + 16 * half + 4 * h;
+                ap_frag a[DT];
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
-                    ap_frag a;
                     const uint16_t* row = Vt + (32 * dt + r32) * VROW + key_off;
-                    a.half[0] = *reinterpret_cast<const ap_u32x2*>(row);
-                    a.half[1] = *reinterpret_cast<const ap_u32x2*>(row + 8);
-                    o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.vec, b.vec, o[dt], 0, 0, 0);
+                    a[dt].half[0] = *reinterpret_cast<const ap_u32x2*>(row);
+                    a[dt].half[1] = *reinterpret_cast<const ap_u32x2*>(row + 8);
                 }
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+                    o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[dt].vec, b.vec, o[dt], 0, 0, 0);
             }
     }
 
@@ -316,7 +377,12 @@ extern "C" int pl_paged_attention_prefill(const void* q, int q_stride, void* out
     if (num_seqs <= 0 || max_q_len <= 0) return 0;
     const int dt = pl_ceil_div(d, 32);
     // few tokens a request: 64-token tiles give twice the workgroups
-    const bool small = max_q_len <= 64;
+#ifdef AP_FORCE_SMALL
+    const bool small = AP_FORCE_SMALL;
+#else
+    // two waves have twice the pieces of a tile to carry each: only small heads leave them the registers
+    const bool small = max_q_len <= 64 && dt <= 2;
+#endif
 #define AP_CALL(D)                                                                                                 \
     return small ? launch_prefill<D, 2>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len, \
                                         block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale,   \
