@@ -10,8 +10,7 @@
 
 #define PL_WAVE 64
 
-// bfloat16 as its sixteen bits; conversions written out so that rounding is
-// round-to-nearest-even everywhere and does not depend on a header's choice.
+// bfloat16 as its sixteen bits.
 struct bf16_t {
     uint16_t bits;
 };
@@ -21,13 +20,9 @@ __device__ __forceinline__ float to_float(bf16_t x) {
     return __uint_as_float(static_cast<uint32_t>(x.bits) << 16);
 }
 
+// Round-to-nearest-even through the hardware's conversion (v_cvt_pk_bf16_f32); a NaN stays a NaN.
 __device__ __forceinline__ uint16_t bf16_bits_from_float(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) {
-        return static_cast<uint16_t>((u >> 16) | 0x0040u);  // quiet NaN
-    }
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return static_cast<uint16_t>(u >> 16);
+    return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
 }
 
 template <typename T>
