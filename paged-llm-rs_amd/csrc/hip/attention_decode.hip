@@ -68,7 +68,7 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
     const int split = blockIdx.z;
 
     const int lane = threadIdx.x % PL_WAVE;
-    const int wave = threadIdx.x / PL_WAVE;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PL_WAVE);  // the same for the whole wave: kept scalar
     const int sub = lane / LPK;   // which of the wave's keys
     const int dl = lane % LPK;    // which 8 values of the head
     const bool d_ok = dl * 8 < d;
@@ -107,34 +107,50 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
 
     const int* table = block_table + static_cast<size_t>(seq) * max_blocks;
     const size_t row_stride = static_cast<size_t>(nkv) * d;
-    const size_t head_off = static_cast<size_t>(kvh) * d + dl * 8;
-    const bool pow2 = (block_size & (block_size - 1)) == 0;
-    const int shift = 31 - __clz(block_size);
+    const size_t head_off = static_cast<size_t>(kvh) * d + min(dl * 8, d - 8);
+    // floor(2^32 / block_size): the high half of j * bs_magic is j / block_size or one less
+    const uint32_t bs_magic = block_size == 1 ? 0xffffffffu : static_cast<uint32_t>(0x100000000ull / static_cast<uint32_t>(block_size));
 
-    for (int base = s_begin + wave * KPW * AD_UNROLL; base < s_end; base += ROUND) {
+    // Loads are unconditional, from an address that is valid in any case, and masked afterwards:
+    // a load inside a branch is waited for at the branch's end, one after the other.  The pages
+    // of a round are looked up during the round before, so that no load waits for another.
+    int blk[AD_UNROLL], within[AD_UNROLL];
+    auto lookup = [&](int base) {
+#pragma unroll
+        for (int u = 0; u < AD_UNROLL; ++u) {
+            const int j = base + u * KPW + sub;
+            const bool in = j < s_end;
+            const int jj = in ? j : pos;                          // the token's own place always has a page
+            int bi = static_cast<int>(__umulhi(static_cast<uint32_t>(jj), bs_magic));
+            int w = jj - bi * block_size;
+            const int low = w >= block_size ? 1 : 0;              // the estimate is the quotient or one less
+            bi += low;
+            w -= low * block_size;
+            const int got = table[bi];
+            blk[u] = in ? got : -1;
+            within[u] = w;
+        }
+    };
+    const int first_base = s_begin + wave * KPW * AD_UNROLL;
+    lookup(first_base);
+
+    for (int base = first_base; base < s_end; base += ROUND) {
         u32x4 kraw[AD_UNROLL], vraw[AD_UNROLL];
         bool ok[AD_UNROLL];
 #pragma unroll
         for (int u = 0; u < AD_UNROLL; ++u) {
-            const int j = base + u * KPW + sub;
-            ok[u] = j < s_end;
-            int blk = -1;
-            int within = 0;
-            if (ok[u]) {
-                const int bi = pow2 ? (j >> shift) : (j / block_size);
-                within = pow2 ? (j & (block_size - 1)) : (j - bi * block_size);
-                blk = table[bi];
-            }
-            ok[u] = ok[u] && blk >= 0;
-            if (ok[u] && d_ok) {
-                const size_t off = (static_cast<size_t>(blk) * block_size + within) * row_stride + head_off;
-                kraw[u] = *reinterpret_cast<const u32x4*>(k_pool + off);
-                vraw[u] = *reinterpret_cast<const u32x4*>(v_pool + off);
-            } else {
-                kraw[u] = u32x4{{0u, 0u, 0u, 0u}};
-                vraw[u] = u32x4{{0u, 0u, 0u, 0u}};
+            ok[u] = blk[u] >= 0;
+            const size_t off = (static_cast<size_t>(max(blk[u], 0)) * block_size + within[u]) * row_stride + head_off;
+            const u32x4 kgot = *reinterpret_cast<const u32x4*>(k_pool + off);
+            const u32x4 vgot = *reinterpret_cast<const u32x4*>(v_pool + off);
+            const uint32_t keep = (ok[u] && d_ok) ? 0xffffffffu : 0u;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                kraw[u].v[w] = kgot.v[w] & keep;
+                vraw[u].v[w] = vgot.v[w] & keep;
             }
         }
+        lookup(base + ROUND);
         float s[AD_UNROLL][GT];
 #pragma unroll
         for (int u = 0; u < AD_UNROLL; ++u) {
