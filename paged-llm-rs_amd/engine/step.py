@@ -160,7 +160,8 @@ class StepRunner:
     """Runs steps for one model and cache, keeping the captured decode graphs."""
 
     def __init__(self, model, cache, graphs: bool = True):
-        self.model, self.cache, self.use_graphs = model, cache, graphs
+        self.model, self.cache = model, cache
+        self.use_graphs = graphs and getattr(model, "graph_safe", True)
         self._graphs: dict = {}
         self.graph_steps = 0
         self.eager_steps = 0

@@ -38,6 +38,12 @@ class PreNormBlock:
         self.feed_forward = lookup(FEED_FORWARDS, layer.feed_forward.kind, "feed-forward")(
             layer.feed_forward, hidden, scoped(params, n["feed_forward"]), dtype, device, shared)
 
+    @property
+    def graph_safe(self) -> bool:
+        """Whether a step through this block may be captured as a HIP graph: a part that
+        reads device values on the host, or allocates by data, sets ``graph_safe = False``."""
+        return getattr(self.mixer, "graph_safe", True) and getattr(self.feed_forward, "graph_safe", True)
+
     def forward(self, resid, delta, ctx):
         normed = self.norm1.apply(resid, delta, self.dtype)
         mixed = self.mixer.forward(normed, ctx)

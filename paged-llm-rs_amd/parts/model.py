@@ -87,6 +87,7 @@ class DecoderModel:
             if entry.cache_from is not None and not 0 <= entry.cache_from < len(self.blocks):
                 raise ConfigError(f"the schedule reads the cache of layer {entry.cache_from} of {len(self.blocks)}")
         self.cache_layout = CacheLayout.from_blocks(self.blocks, spec.schedule)
+        self.graph_safe = all(getattr(b, "graph_safe", True) for b in self.blocks)
 
     # -- the forward pass of one step -------------------------------------------------
 

@@ -10,10 +10,15 @@ mixer         ``declare(spec, hidden) -> [ParamDecl]`` (local names);
               ``__init__(spec, hidden, params, dtype, device, shared)``;
               ``cache_spec() -> KVCacheSpec | None``; ``state_spec() -> StateSpec | None``;
               ``forward(x[n,hidden], ctx: LayerContext) -> [n,hidden]``.
+              Optional ``graph_safe = False`` when its forward cannot be captured as a HIP graph.
 feed-forward  ``declare``; ``__init__`` as above; ``forward(x) -> [n,hidden]``.
 norm          ``declare(spec, width)``; ``__init__(spec, width, params, dtype, device)``;
               ``apply(resid, delta, out_dtype, rows=None) -> normed`` which adds
               ``delta`` into the 32-bit residual stream and returns the normalised rows.
+position      ``__init__(spec, device)`` giving ``dim`` (how many elements of a head are rotated),
+              ``cos`` and ``sin`` ([max_positions, dim/2], 32-bit, on the device) and
+              ``max_positions``: the rotation by pairs (i, i + dim/2) that the attention kernels
+              apply is fixed, the angles are the encoding's own.
 block         ``declare(layer_spec, hidden)``; ``__init__(layer_spec, hidden, params, dtype,
               device, shared)``; ``forward(resid, delta, ctx) -> delta`` where the returned
               delta is the output not yet added to the residual stream.
@@ -27,6 +32,7 @@ MIXERS: dict = {}
 FEED_FORWARDS: dict = {}
 NORMS: dict = {}
 BLOCKS: dict = {}
+POSITIONS: dict = {}
 
 
 def register_mixer(kind: str, cls) -> None:
@@ -43,6 +49,10 @@ def register_norm(kind: str, cls) -> None:
 
 def register_block(kind: str, cls) -> None:
     BLOCKS[kind] = cls
+
+
+def register_position(kind: str, cls) -> None:
+    POSITIONS[kind] = cls
 
 
 def lookup(registry: dict, kind: str, what: str):

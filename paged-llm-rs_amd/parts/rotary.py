@@ -10,6 +10,7 @@ from __future__ import annotations
 import torch
 
 from ..errors import UnsupportedError
+from .registry import POSITIONS, lookup, register_position
 
 
 class RotaryTables:
@@ -27,9 +28,13 @@ class RotaryTables:
         self.max_positions = spec.max_positions
 
 
-def rotary_tables(spec, device, shared: dict) -> RotaryTables:
-    """Layers with the same position spec share one pair of tables."""
-    key = ("rotary", spec, str(device))
+register_position("rotary_half", RotaryTables)
+
+
+def rotary_tables(spec, device, shared: dict):
+    """The tables of a position spec, built by the class its ``kind`` names; layers
+    with the same spec share one pair."""
+    key = ("position", spec, str(device))
     if key not in shared:
-        shared[key] = RotaryTables(spec, device)
+        shared[key] = lookup(POSITIONS, spec.kind, "position encoding")(spec, device)
     return shared[key]

@@ -1,0 +1,349 @@
+"""Each part alone against the plain implementation's function for it, a toy
+mixer with state of its own registered from outside the package, long decoding,
+the first tokens of a sequence, and long portions over earlier context."""
+
+from __future__ import annotations
+
+import math
+import types
+from dataclasses import dataclass
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen3 as plain
+import replay_util as ru
+from conftest import TINY_INIT, load_plain, rel_err
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+TOL = {torch.float32: 2e-5, torch.bfloat16: 2e-2}
+
+
+def randn(*shape, std=1.0, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g) * std
+
+
+# --- norm -----------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width,eps", [(100, 1e-5), (1024, 1e-6)])
+def test_norm_part(dtype, width, eps):
+    from paged_llm_rs_amd.config import NormSpec
+    from paged_llm_rs_amd.parts import NORMS
+
+    gain = (1 + randn(width, std=0.2, seed=1)).to(dtype)
+    part = NORMS["rms_norm"](NormSpec("rms_norm", eps), width, {"weight": gain.to(DEV)}, dtype, DEV)
+    resid = randn(7, width, seed=2)
+    delta = randn(7, width, seed=3).to(dtype)
+    stream = resid.to(DEV).clone()
+    out = part.apply(stream, delta.to(DEV), dtype)
+    summed = resid.double() + delta.double()
+    assert rel_err(stream, summed) < 1e-6, "the residual sum is 32-bit and written back"
+    assert rel_err(out, plain.rms_norm(summed, gain.double(), eps)) < TOL[dtype]
+    rows = torch.tensor([5, 0, 5], dtype=torch.int32, device=DEV)
+    picked = part.apply(stream, None, dtype, rows=rows)
+    assert rel_err(picked, plain.rms_norm(summed[[5, 0, 5]], gain.double(), eps)) < TOL[dtype]
+
+
+# --- position encoding -------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dim,theta", [(16, 10000.0), (48, 1e6)])
+def test_position_part(dim, theta):
+    from paged_llm_rs_amd.config import PositionSpec
+    from paged_llm_rs_amd.parts import POSITIONS
+
+    tables = POSITIONS["rotary_half"](PositionSpec("rotary_half", dim, theta, 300), DEV)
+    positions = torch.tensor([0, 1, 7, 299])
+    cos, sin = plain.rope_tables(dim, positions, theta)       # [n, dim], the half table twice
+    assert rel_err(tables.cos[positions], cos[:, :dim // 2]) < 1e-6
+    assert rel_err(tables.sin[positions], sin[:, :dim // 2]) < 1e-6
+
+
+# --- feed-forward --------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows", [3, 70])
+def test_feed_forward_part(dtype, rows):
+    from paged_llm_rs_amd.config import GatedMlpSpec
+    from paged_llm_rs_amd.parts import FEED_FORWARDS
+
+    hidden, inter = 96, 200
+    w = {"m.gate_proj.weight": randn(inter, hidden, std=0.1, seed=1).to(dtype),
+         "m.up_proj.weight": randn(inter, hidden, std=0.1, seed=2).to(dtype),
+         "m.down_proj.weight": randn(hidden, inter, std=0.1, seed=3).to(dtype)}
+    part = FEED_FORWARDS["gated_mlp"](GatedMlpSpec("gated_mlp", inter, "silu"), hidden,
+                                      {k[2:]: v.to(DEV) for k, v in w.items()}, dtype, DEV, {})
+    x = randn(rows, hidden, seed=4).to(dtype)
+    want = plain.swiglu_mlp(x.double(), {k: v.double() for k, v in w.items()}, "m")
+    assert rel_err(part.forward(x.to(DEV)), want) < TOL[dtype]
+
+
+# --- mixer ---------------------------------------------------------------------------------------------------
+
+def one_layer_cache(mixer, block_size, pages, dtype):
+    from paged_llm_rs_amd.cache import CacheLayout, PagedCache
+    from paged_llm_rs_amd.config import ScheduleEntry
+
+    layout = CacheLayout.from_blocks([types.SimpleNamespace(mixer=mixer)], [ScheduleEntry(0)])
+    return PagedCache(layout, block_size, pages, dtype, DEV, max_seqs=4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nq,nkv,d,block_size", [(4, 2, 16, 4), (6, 1, 32, 16), (6, 3, 48, 8)])
+def test_attention_part_in_portions(dtype, nq, nkv, d, block_size):
+    """The mixer alone over its own pages: a sequence fed in portions (a long one, a short one, single
+    tokens) gives what the plain attention gives for the whole sequence."""
+    from paged_llm_rs_amd.config import AttentionSpec, NormSpec, PositionSpec
+    from paged_llm_rs_amd.engine.batch import StepEntry, build_batch
+    from paged_llm_rs_amd.parts import MIXERS, LayerContext
+
+    hidden, eps, theta, n = 40, 1e-5, 5e5, 61
+    cfg = {"num_attention_heads": nq, "num_key_value_heads": nkv, "head_dim": d, "rms_norm_eps": eps,
+           "rope_theta": theta}
+    w = {"a.q_proj.weight": randn(nq * d, hidden, std=0.2, seed=1), "a.k_proj.weight": randn(nkv * d, hidden, std=0.2, seed=2),
+         "a.v_proj.weight": randn(nkv * d, hidden, std=0.2, seed=3), "a.o_proj.weight": randn(hidden, nq * d, std=0.2, seed=4),
+         "a.q_norm.weight": 1 + randn(d, std=0.2, seed=5), "a.k_norm.weight": 1 + randn(d, std=0.2, seed=6)}
+    w = {k: v.to(dtype) for k, v in w.items()}
+    spec = AttentionSpec("paged_attention", nq, nkv, d, NormSpec("rms_norm", eps),
+                         PositionSpec("rotary_half", d, theta, 128), None, None)
+    mixer = MIXERS["paged_attention"](spec, hidden, {k[2:]: v.to(DEV) for k, v in w.items()}, dtype, DEV, {})
+    cache = one_layer_cache(mixer, block_size, 24, dtype)
+    x = randn(n, hidden, seed=7).to(dtype)
+    want = plain.attention(x.double(), {k: v.double() for k, v in w.items()}, "a", cfg, torch.arange(n))
+    cache.manager.add_sequence(1)
+    got, at = [], 0
+    for count in (20, 1, 17, 1, 1, 19, 2):
+        assert cache.manager.reserve(1, count)
+        entries = [StepEntry(1, [0] * count, at, [])]
+        batch = build_batch(entries, cache.manager, 1, 10, 128, DEV)
+        got.append(mixer.forward(x[at:at + count].to(DEV).contiguous(), LayerContext(batch, cache, 0, 0, True)))
+        cache.manager.advance(1, count)
+        at += count
+    assert at == n
+    assert rel_err(torch.cat(got), want) < TOL[dtype]
+
+
+# --- block ---------------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_block_part(model_dirs, dtype):
+    """One layer of a tiny model through the block class, fed the plain implementation's own input."""
+    from paged_llm_rs_amd.cache import PagedCache
+    from paged_llm_rs_amd.engine.batch import StepEntry, build_batch
+    from paged_llm_rs_amd.parts import LayerContext, load_model
+
+    name = "float32" if dtype == torch.float32 else "bfloat16"
+    d = model_dirs("C", name)
+    cfg, weights = load_plain(d)
+    _, model = load_model(d, name, DEV)
+    n = 23
+    x = randn(n, cfg["hidden_size"], seed=9)
+    want = plain.decoder_block(x.double(), {k: v.double() for k, v in weights.items()}, "model.layers.1", cfg, torch.arange(n))
+    cache = PagedCache(model.cache_layout, 8, 8, dtype, DEV, max_seqs=2)
+    cache.manager.add_sequence(1)
+    assert cache.manager.reserve(1, n)
+    batch = build_batch([StepEntry(1, [0] * n, 0, [])], cache.manager, 1, cfg["vocab_size"], 0, DEV)
+    resid = x.to(DEV).clone()
+    delta = model.blocks[1].forward(resid, None, LayerContext(batch, cache, 1, 1, True))
+    assert rel_err(resid.double() + delta.double(), want) < TOL[dtype]
+
+
+# --- a toy mixer with state of its own, defined here ---------------------------------------------------------------------
+
+@dataclass(frozen=True)
+class RunningMeanSpec:
+    kind: str = "running_mean"
+
+
+class RunningMeanMixer:
+    """out[t] = W . mean(x[0..t]): the sum so far and the count are the request's state."""
+    graph_safe = False      # it reads the step's layout on the host
+
+    @staticmethod
+    def declare(spec, hidden):
+        from paged_llm_rs_amd.weights.loader import ParamDecl
+        return [ParamDecl("proj.weight", (hidden, hidden))]
+
+    def __init__(self, spec, hidden, params, dtype, device, shared):
+        self.w, self.hidden = params["proj.weight"], hidden
+
+    def cache_spec(self):
+        return None
+
+    def state_spec(self):
+        from paged_llm_rs_amd.cache import StateSpec
+        return StateSpec((self.hidden + 1,), torch.float32)
+
+    def forward(self, x, ctx):
+        batch, state, H = ctx.batch, ctx.state(), self.hidden
+        out = torch.empty_like(x)
+        starts, counts, slots = (t.cpu().tolist() for t in (batch.q_start, batch.q_len, batch.state_slots))
+        for a, n, slot in zip(starts, counts, slots):
+            assert slot >= 0, "a request of a model with state has a slot"
+            sums = state[slot, :H] + x[a:a + n].float().cumsum(0)
+            seen = state[slot, H] + torch.arange(1, n + 1, device=x.device)
+            out[a:a + n] = ((sums / seen[:, None]) @ self.w.float().t()).to(x.dtype)
+            state[slot, :H] = sums[-1]
+            state[slot, H] = seen[-1]
+        return out
+
+
+class ToyConfig:
+    """Layer 0 mixes by running mean, layer 1 by attention; both read ``hidden_size`` and so on from config.json."""
+
+    def __init__(self, d):
+        self.d = d
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls(dict(d))
+
+    def to_dict(self):
+        return dict(self.d)
+
+    def model_spec(self):
+        from paged_llm_rs_amd.config import (AttentionSpec, GatedMlpSpec, LayerSpec, ModelSpec, NormSpec, PositionSpec,
+                                             ScheduleEntry)
+        d = self.d
+        norm = NormSpec("rms_norm", d["rms_norm_eps"])
+        ffn = GatedMlpSpec("gated_mlp", d["intermediate_size"], "silu")
+        attention = AttentionSpec("paged_attention", d["num_attention_heads"], d["num_key_value_heads"], d["head_dim"],
+                                  norm, PositionSpec("rotary_half", d["head_dim"], d["rope_theta"],
+                                                     d["max_position_embeddings"]), None, None)
+        layers = (LayerSpec("pre_norm", RunningMeanSpec(), ffn, norm, "model.layers.0"),
+                  LayerSpec("pre_norm", attention, ffn, norm, "model.layers.1"))
+        return ModelSpec(d["hidden_size"], d["vocab_size"], layers, (ScheduleEntry(0), ScheduleEntry(1)), norm,
+                         d["tie_word_embeddings"], d["max_position_embeddings"])
+
+
+TOY = {"architectures": ["ToyForCausalLM"], "model_type": "toy", "hidden_size": 48, "intermediate_size": 80,
+       "num_attention_heads": 2, "num_key_value_heads": 1, "head_dim": 16, "rms_norm_eps": 1e-5, "rope_theta": 1e4,
+       "vocab_size": 97, "max_position_embeddings": 256, "tie_word_embeddings": True}
+
+
+def toy_plain(weights, tokens):
+    w = {k: v.double() for k, v in weights.items()}
+    n = len(tokens)
+    x = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+    eps = TOY["rms_norm_eps"]
+    normed = plain.rms_norm(x, w["model.layers.0.input_layernorm.weight"], eps)
+    mean = normed.cumsum(0) / torch.arange(1, n + 1, dtype=torch.float64)[:, None]
+    x = x + mean @ w["model.layers.0.self_attn.proj.weight"].T
+    x = x + plain.swiglu_mlp(plain.rms_norm(x, w["model.layers.0.post_attention_layernorm.weight"], eps), w, "model.layers.0.mlp")
+    x = plain.decoder_block(x, w, "model.layers.1", TOY, torch.arange(n))
+    return plain.rms_norm(x, w["model.norm.weight"], eps) @ w["model.embed_tokens.weight"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path, dtype):
+    """A mixer that keeps a running mean in a state slot, an architecture that uses it in one layer
+    beside attention in another: registered here, written by the random-weights mode, replayed in
+    portions mixed with other requests, and generated from through the engine."""
+    from safetensors.torch import load_file
+
+    from paged_llm_rs_amd import Engine, register_architecture, write_random_model
+    from paged_llm_rs_amd.engine.replay import Replayer
+    from paged_llm_rs_amd.parts import register_mixer
+
+    register_mixer("running_mean", RunningMeanMixer)
+    register_architecture("ToyForCausalLM", ToyConfig, model_type="toy")
+    folder = write_random_model(tmp_path / "toy", TOY, seed=5, std=0.1, gain_std=0.2, dtype=dtype)
+    weights = load_file(str(folder / "model.safetensors"))
+    assert "model.layers.0.self_attn.proj.weight" in weights and "model.layers.1.self_attn.q_proj.weight" in weights
+    prompts = ru.make_prompts(TOY["vocab_size"], [30, 9, 41, 17, 25], seed=3)
+    want = {name: toy_plain(weights, toks) for name, toks in prompts.items()}
+    tolerance = 1e-5 if dtype == "float32" else 2e-2
+    for steps, live in ((ru.whole(prompts), 1), (ru.mixed(prompts, seed=7, max_live=3), 3)):
+        r = Replayer(folder, dtype, max_tokens=ru.pool_tokens(prompts, live), block_size=8, max_live=4)
+        assert not r.runner.use_graphs and r.cache.layout.states, "the toy's state slots exist and its steps run eagerly"
+        got = ru.collect(r, steps)
+        worst, where = ru.worst_error(got, want)
+        assert worst <= tolerance, f"{worst:.3e} at {where}"
+        assert r.cache.manager.free_state_slots == 4, "every state slot came back"
+    engine = Engine(folder, dtype="f32" if dtype == "float32" else "bf16", block_size=8, num_blocks=16, max_batch=3, chunk=8)
+    out = engine.generate(list(prompts.values())[:3], max_tokens=5, temperature=0.0, stop_tokens=[])
+    for prompt, result in zip(prompts.values(), out):
+        tokens = list(prompt)
+        for produced in result["tokens"]:
+            logits = toy_plain(weights, tokens)[-1]
+            best = int(torch.argmax(logits))
+            if produced != best:
+                assert float(logits[best] - logits[produced]) <= tolerance * float(logits.abs().max())
+            tokens.append(produced)
+
+
+# --- long decoding, first tokens, long portions -----------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,block_size", [("A", 16), ("C", 4)])
+def test_long_decoding(model_dirs, name, dtype, block_size):
+    """Three hundred tokens decoded one by one, two requests side by side, over many page edges."""
+    from paged_llm_rs_amd.engine.replay import Replayer
+
+    d = model_dirs(name, dtype)
+    prompts = ru.make_prompts(TINY_INIT[name]["config"]["vocab_size"], [330, 301], seed=21)
+    want = ru.plain_logits(d, prompts)
+    steps = [{"step": 0, "entries": [{"id": n, "tokens": t[:20 + 11 * i], "want": [19 + 11 * i]}
+                                     for i, (n, t) in enumerate(prompts.items())], "end": []}]
+    at = {n: 20 + 11 * i for i, n in enumerate(prompts)}
+    while at:
+        entries = [{"id": n, "tokens": [prompts[n][p]], "want": [0]} for n, p in at.items()]
+        at = {n: p + 1 for n, p in at.items()}
+        end = [n for n, p in at.items() if p == len(prompts[n])]
+        for n in end:
+            del at[n]
+        steps.append({"step": len(steps), "entries": entries, "end": end})
+    r = Replayer(d, dtype, max_tokens=ru.pool_tokens(prompts, 2), block_size=block_size)
+    got = ru.collect(r, steps)
+    assert r.runner.graph_steps > 250, "decoding runs as captured graphs"
+    worst, where = ru.worst_error(got, want)
+    assert worst <= (1e-5 if dtype == "float32" else 2e-2), f"{worst:.3e} at {where}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_the_first_tokens_of_a_sequence(model_dirs, name, dtype):
+    """Positions 0, 1, 2, ...: fed one by one from an empty cache, as a portion of two, and whole."""
+    from paged_llm_rs_amd.engine.replay import Replayer
+
+    d = model_dirs(name, dtype)
+    prompts = ru.make_prompts(TINY_INIT[name]["config"]["vocab_size"], [6, 1, 2, 3], seed=8)
+    want = ru.plain_logits(d, prompts)
+    one_by_one = []
+    for n, t in prompts.items():
+        for p, token in enumerate(t):
+            one_by_one.append({"step": len(one_by_one), "entries": [{"id": n, "tokens": [token], "want": [0]}],
+                               "end": [n] if p == len(t) - 1 else []})
+    for steps in (one_by_one, ru.portions(prompts, sizes=(2, 1, 3)), ru.whole(prompts)):
+        r = Replayer(d, dtype, max_tokens=64, block_size=4)
+        worst, where = ru.worst_error(ru.collect(r, steps), want)
+        assert worst <= (1e-5 if dtype == "float32" else 2e-2), f"{worst:.3e} at {where}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,block_size", [("A", 16), ("B", 8)])
+def test_long_portions_over_earlier_context(model_dirs, name, dtype, block_size):
+    """Portions of more than a hundred tokens that read hundreds of earlier keys through the pages (the tiled
+    attention kernel's case in bfloat16), beside a request that decodes."""
+    from paged_llm_rs_amd.engine.replay import Replayer
+
+    d = model_dirs(name, dtype)
+    prompts = ru.make_prompts(TINY_INIT[name]["config"]["vocab_size"], [450, 40], seed=31)
+    want = ru.plain_logits(d, prompts)
+    long, short = prompts["r0"], prompts["r1"]
+    cuts = [0, 130, 131, 300, 429, 450]
+    steps = [{"step": 0, "entries": [{"id": "r1", "tokens": short[:30], "want": [29]}], "end": []}]
+    for i in range(len(cuts) - 1):
+        a, b = cuts[i], cuts[i + 1]
+        entries = [{"id": "r0", "tokens": long[a:b], "want": sorted({0, (b - a) // 2, b - a - 1})}]
+        if 30 + i < len(short):
+            entries.append({"id": "r1", "tokens": [short[30 + i]], "want": [0]})
+        steps.append({"step": len(steps), "entries": entries, "end": ["r0"] if b == len(long) else []})
+    steps.append({"step": len(steps), "entries": [{"id": "r1", "tokens": short[35:], "want": [0, 4]}], "end": ["r1"]})
+    r = Replayer(d, dtype, max_tokens=ru.pool_tokens(prompts, 2), block_size=block_size)
+    worst, where = ru.worst_error(ru.collect(r, steps), want)
+    assert worst <= (1e-5 if dtype == "float32" else 2e-2), f"{worst:.3e} at {where}"
