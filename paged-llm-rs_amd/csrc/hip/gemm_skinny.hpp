@@ -1,0 +1,345 @@
+// y[n, N] = x[n, K] . w[N, K]^T for few rows (n <= 64), bfloat16 weights, 32-bit accumulate,
+// on the matrix cores, with what comes before and after the product fused into it.
+//
+// With few rows the product is a stream of the weight matrix through the chip:
+// every weight is read once and the time is the time of that read, which is the
+// time of one trip to memory if the whole matrix is asked for at once.  One
+// workgroup of four waves owns 16 output columns (16 rows of w); the waves split
+// K between them and each asks for its whole share before it multiplies, and
+// their partial tiles are added in a fixed order through LDS.  Each wave feeds
+// v_mfma_f32_16x16x32_bf16 straight from global memory: both operands are
+// contiguous along K, so a lane's 16 bytes are one load.
+//
+// Before the product (PRO):
+//   PRO_BF16  x is bfloat16 [n, K].
+//   PRO_NORM  x is the 32-bit residual stream; row r of the product reads row rows[r] of it (or r).
+//             The product runs over bf16(x * gain) and the result is scaled by
+//             1 / sqrt(mean(x^2) + eps) of its row afterwards: the statistic is summed from the
+//             very values the product loads, so the norm costs no pass of its own.
+// After the product (EPI):
+//   EPI_STORE   y = result (bfloat16 or 32-bit).
+//   EPI_SWIGLU  the workgroup owns 16 gate columns and the 16 up columns that belong to
+//               them (rows c and N + c of w) and stores silu(gate) * up.
+//   EPI_ADD     the 32-bit residual stream takes the result: resid[r, c] += result.  Every
+//               element has one owner, so the sum does not depend on timing.
+#pragma once
+#include "common.hpp"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
+
+#define SK_TILE_N 16
+#define SK_KSTEP 32
+
+#define PRO_BF16 0
+#define PRO_NORM 1
+#define EPI_STORE 0
+#define EPI_SWIGLU 1
+#define EPI_ADD 2
+
+struct __attribute__((aligned(16))) sk_f32x4 {
+    float v[4];
+};
+struct __attribute__((aligned(16))) sk_u32x4 {
+    uint32_t v[4];
+};
+
+__device__ __forceinline__ bf16x8 sk_load8(const bf16_t* p) {
+    return *reinterpret_cast<const bf16x8*>(p);
+}
+
+__device__ __forceinline__ bf16x8 sk_zero8() {
+    bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+    return z;
+}
+
+// Eight consecutive gains as 32-bit floats, whichever way they are stored.
+template <typename GT>
+__device__ __forceinline__ void sk_load_gain(const void* gain, int k, float* out);
+template <>
+__device__ __forceinline__ void sk_load_gain<float>(const void* gain, int k, float* out) {
+    const sk_f32x4 a = *reinterpret_cast<const sk_f32x4*>(static_cast<const float*>(gain) + k);
+    const sk_f32x4 b = *reinterpret_cast<const sk_f32x4*>(static_cast<const float*>(gain) + k + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        out[e] = a.v[e];
+        out[4 + e] = b.v[e];
+    }
+}
+template <>
+__device__ __forceinline__ void sk_load_gain<bf16_t>(const void* gain, int k, float* out) {
+    const sk_u32x4 raw = *reinterpret_cast<const sk_u32x4*>(static_cast<const bf16_t*>(gain) + k);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        out[2 * e] = __uint_as_float(raw.v[e] << 16);
+        out[2 * e + 1] = __uint_as_float(raw.v[e] & 0xffff0000u);
+    }
+}
+
+// MT: 16-row tiles of x (n <= 16*MT).  UNR: K steps a wave asks for at once.  WV: the most waves a
+// workgroup may have (it is launched with as many as give every wave one round of loads, or WV).
+// GT: the gain's type.
+// A workgroup walks the column tiles blockIdx.x, blockIdx.x + gridDim.x, ...; when a wave's share of
+// K fits one round of loads, its rows of x are loaded (and normalised) once and stay in registers.
+template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT, typename GT>
+__global__ void __launch_bounds__(64 * WV)
+gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OUT* __restrict__ y,
+                   const void* __restrict__ gain, float eps, const int* __restrict__ rows, int n, int N_out,
+                   int K) {
+    constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
+    __shared__ float red[WV][BT][MT][256];
+    __shared__ float ssq_lds[WV][MT * 16];
+    const int nwaves = blockDim.x / PL_WAVE;
+
+    const int lane = threadIdx.x % PL_WAVE;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PL_WAVE);
+    const int c = lane % 16;  // column of the tile (a row of w), and the row of x inside its tile
+    const int g = lane / 16;  // which 8 of the 32 values of a K step
+    const int num_tiles = pl_ceil_div(N_out, SK_TILE_N);
+
+    // K is cut into one stretch of whole steps a wave.
+    const int steps = (K + SK_KSTEP - 1) / SK_KSTEP;
+    const int per_wave = (steps + nwaves - 1) / nwaves;
+    const int kbeg = wave * per_wave * SK_KSTEP;
+    const int kend = min(K, (wave + 1) * per_wave * SK_KSTEP);
+    const bool one_round = per_wave <= UNR;
+
+    const bf16_t* xb = static_cast<const bf16_t*>(x_);
+    const float* xf = static_cast<const float*>(x_);
+    size_t xrow[MT];
+    bool row_ok[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int row = m * 16 + c;
+        row_ok[m] = row < n;
+        int src = row_ok[m] ? row : 0;
+        if (PRO == PRO_NORM && rows) src = rows[src];
+        xrow[m] = static_cast<size_t>(src) * K;
+    }
+
+    bf16x8 ax[MT][UNR];
+    float ssq[MT];
+    sk_f32x4 raw[PRO == PRO_NORM ? MT : 1][UNR][2];
+    float gn[PRO == PRO_NORM ? UNR : 1][8];
+
+    // The rows of x for the K steps k0, k0 + 32, ...: asked for from a place that exists in any case
+    // (a load inside a branch is waited for at the branch's end) ...
+    auto ask_x = [&](int k0) {
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+            const int at = k0 + u * SK_KSTEP + g * 8;
+            const int kk = at < kend ? at : 0;  // K is a multiple of 8, so a chunk is whole or absent
+            if (PRO == PRO_NORM) sk_load_gain<GT>(gain, kk, gn[u]);
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                if (PRO == PRO_BF16) {
+                    ax[m][u] = sk_load8(xb + xrow[m] + kk);
+                } else {
+                    raw[m][u][0] = *reinterpret_cast<const sk_f32x4*>(xf + xrow[m] + kk);
+                    raw[m][u][1] = *reinterpret_cast<const sk_f32x4*>(xf + xrow[m] + kk + 4);
+                }
+            }
+        }
+    };
+    // ... and, once they are there, masked, summed into the row's statistic and rounded.
+    auto take_x = [&](int k0) {
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+            const bool k_ok = k0 + u * SK_KSTEP + g * 8 < kend;
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const bool ok = k_ok && row_ok[m];
+                if (PRO == PRO_BF16) {
+                    ax[m][u] = ok ? ax[m][u] : sk_zero8();
+                } else {
+                    f32x8 v;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float xv = ok ? raw[m][u][e / 4].v[e % 4] : 0.f;
+                        ssq[m] = fmaf(xv, xv, ssq[m]);
+                        v[e] = xv * gn[u][e];
+                    }
+                    ax[m][u] = __builtin_convertvector(v, bf16x8);
+                }
+            }
+        }
+    };
+
+#pragma unroll
+    for (int m = 0; m < MT; ++m) ssq[m] = 0.f;
+    bool x_asked = one_round && kbeg < kend;
+    if (x_asked) ask_x(kbeg);
+
+    for (int tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
+        const int n0 = tile * SK_TILE_N;
+        const bool col_ok = n0 + c < N_out;
+        const bf16_t* wrow[BT];
+        wrow[0] = w + static_cast<size_t>(col_ok ? n0 + c : 0) * K;
+        if (BT == 2) wrow[BT - 1] = w + static_cast<size_t>(N_out + (col_ok ? n0 + c : 0)) * K;
+
+        f32x4 acc[BT][MT];
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int b = 0; b < BT; ++b) acc[b][m] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (!one_round) {
+#pragma unroll
+            for (int m = 0; m < MT; ++m) ssq[m] = 0.f;
+        }
+
+        for (int k0 = kbeg; k0 < kend; k0 += SK_KSTEP * UNR) {
+            bf16x8 bw[BT][UNR];
+#pragma unroll
+            for (int u = 0; u < UNR; ++u) {
+                const int at = k0 + u * SK_KSTEP + g * 8;
+                const bool k_ok = at < kend;
+                const int kk = k_ok ? at : 0;
+#pragma unroll
+                for (int b = 0; b < BT; ++b) {
+                    const bf16x8 got = sk_load8(wrow[b] + kk);
+                    bw[b][u] = (k_ok && col_ok) ? got : sk_zero8();
+                }
+            }
+            // the weights are asked for first: they come from furthest away
+            if (!one_round) {
+                ask_x(k0);
+                take_x(k0);
+            } else if (x_asked) {
+                take_x(kbeg);
+                x_asked = false;
+            }
+#pragma unroll
+            for (int u = 0; u < UNR; ++u)
+#pragma unroll
+                for (int m = 0; m < MT; ++m)
+#pragma unroll
+                    for (int b = 0; b < BT; ++b)
+                        acc[b][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[m][u], bw[b][u], acc[b][m], 0, 0, 0);
+        }
+
+        // A lane holds rows (lane/16)*4 + i, i = 0..3, of column lane%16 of its 16x16 tile.
+#pragma unroll
+        for (int b = 0; b < BT; ++b)
+#pragma unroll
+            for (int m = 0; m < MT; ++m)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) red[wave][b][m][lane * 4 + i] = acc[b][m][i];
+        if (PRO == PRO_NORM) {
+            // the four lanes that hold a row's four chunks of a K step, then the four waves
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                float s = ssq[m];
+                s += __shfl_xor(s, 16, PL_WAVE);
+                s += __shfl_xor(s, 32, PL_WAVE);
+                if (g == 0) ssq_lds[wave][m * 16 + c] = s;
+            }
+        }
+        __syncthreads();
+
+        const int t = threadIdx.x % 256;   // with more than four waves the first four finish the tile
+        const int src_lane = t / 4, i = t % 4;
+        const int row_in_tile = (src_lane / 16) * 4 + i;
+        const int col = n0 + src_lane % 16;
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const int row = m * 16 + row_in_tile;
+            float v[BT];
+#pragma unroll
+            for (int b = 0; b < BT; ++b) {
+                float s = 0.f;
+#pragma unroll
+                for (int wv = 0; wv < nwaves; ++wv) s += red[wv][b][m][t];
+                v[b] = s;
+            }
+            if (PRO == PRO_NORM) {
+                float total = 0.f;
+#pragma unroll
+                for (int wv = 0; wv < nwaves; ++wv) total += ssq_lds[wv][m * 16 + row_in_tile];
+                const float rinv = 1.f / sqrtf(total / static_cast<float>(K) + eps);
+#pragma unroll
+                for (int b = 0; b < BT; ++b) v[b] *= rinv;
+            }
+            if (threadIdx.x < 256 && row < n && col < N_out) {
+                float r = v[0];
+                if (EPI == EPI_SWIGLU) r = v[0] / (1.f + __expf(-v[0])) * v[BT - 1];
+                const size_t at = static_cast<size_t>(row) * N_out + col;
+                if (EPI == EPI_ADD)
+                    y[at] = from_float<OUT>(to_float(y[at]) + r);
+                else
+                    y[at] = from_float<OUT>(r);
+            }
+        }
+        __syncthreads();  // the next tile writes the same LDS
+    }
+}
+
+// More column tiles than this many workgroups are walked in a loop, which keeps a wave's rows of x
+// in its registers from tile to tile: eight workgroups a compute unit are as many as stay resident.
+#define SK_MAX_GRID 2048
+
+template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT>
+static int launch_one(int waves, const void* x, const void* w, void* y, const void* gain, int gain_dtype, float eps,
+                      const int* rows, int n, int N_out, int K, hipStream_t stream) {
+    const int grid = min(pl_ceil_div(N_out, SK_TILE_N), SK_MAX_GRID);
+    if (PRO == PRO_NORM && gain_dtype == PL_DTYPE_F32)
+        gemm_skinny_kernel<MT, UNR, WV, PRO, EPI, OUT, float><<<grid, 64 * waves, 0, stream>>>(
+            x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps, rows, n, N_out, K);
+    else
+        gemm_skinny_kernel<MT, UNR, WV, PRO, EPI, OUT, bf16_t><<<grid, 64 * waves, 0, stream>>>(
+            x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps, rows, n, N_out, K);
+    PL_CHECK_LAUNCH("gemm_skinny");
+    return 0;
+}
+
+// As many waves as give each one round of loads, between four and sixteen: the whole matrix is then
+// asked for at once and the kernel's time is one trip to memory.
+template <int MT, int PRO, int EPI, typename OUT>
+static int launch_unr(const void* x, const void* w, void* y, const void* gain, int gain_dtype, float eps,
+                      const int* rows, int n, int N_out, int K, hipStream_t stream) {
+    constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
+    constexpr int COST = BT + MT * (PRO == PRO_NORM ? 2 : 1);  // 16-byte registers a K step holds in flight
+    constexpr int UNR = COST <= 4 ? 8 : (COST <= 6 ? 4 : 2);
+    // the partial tiles of all waves lie in LDS side by side, a kilobyte a tile: at most 48 of them
+    // (a product that starts with a norm holds its rows twice, raw and rounded: four waves leave it the registers)
+    constexpr int MAXWV = PRO == PRO_NORM ? 4 : (BT * MT <= 3 ? 16 : (BT * MT <= 6 ? 8 : 4));
+    const int steps = pl_ceil_div(K, SK_KSTEP);
+    const int waves = max(4, min(MAXWV, pl_ceil_div(steps, UNR)));
+    if (waves <= 4) return launch_one<MT, UNR, 4, PRO, EPI, OUT>(4, x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream);
+    if constexpr (MAXWV >= 8) {
+        if (waves <= 8) return launch_one<MT, UNR, 8, PRO, EPI, OUT>(waves, x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream);
+    }
+    if constexpr (MAXWV >= 16) {
+        return launch_one<MT, UNR, 16, PRO, EPI, OUT>(waves, x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream);
+    }
+    return -1;  // not reached: waves <= MAXWV
+}
+
+template <int PRO, int EPI, typename OUT>
+static int launch_mt(const void* x, const void* w, void* y, const void* gain, int gain_dtype, float eps,
+                     const int* rows, int n, int N_out, int K, hipStream_t stream) {
+    switch (pl_ceil_div(n, 16)) {
+        case 1: return launch_unr<1, PRO, EPI, OUT>(x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream);
+        case 2: return launch_unr<2, PRO, EPI, OUT>(x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream);
+        case 3: return launch_unr<3, PRO, EPI, OUT>(x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream);
+        default: return launch_unr<4, PRO, EPI, OUT>(x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream);
+    }
+}
+
+template <int PRO>
+static int sk_launch(int epilogue, int out_f32, const void* x, const void* w, void* y, const void* gain,
+                      int gain_dtype, float eps, const int* rows, int n, int N_out, int K, hipStream_t stream) {
+    if (epilogue == EPI_STORE)
+        return out_f32 ? launch_mt<PRO, EPI_STORE, float>(x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream)
+                       : launch_mt<PRO, EPI_STORE, bf16_t>(x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream);
+    if (epilogue == EPI_SWIGLU)
+        return out_f32 ? launch_mt<PRO, EPI_SWIGLU, float>(x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream)
+                       : launch_mt<PRO, EPI_SWIGLU, bf16_t>(x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream);
+    if constexpr (PRO == PRO_NORM) {
+        pl_set_error("skinny product: a product that reads the residual stream cannot add into it");
+        return -1;
+    } else {
+        return launch_mt<PRO, EPI_ADD, float>(x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream);
+    }
+}
+

@@ -35,7 +35,7 @@ def _signatures(lib) -> None:
         "pl_gemm_plain": [p, p, p, i, i, i, i, i, i, i, p],
         "pl_paged_attention_plain": [p, i, p, p, p, p, i, i, p, p, i, i, i, i, f, i, i, p],
         "pl_argmax": [p, p, p, p, i, i, p],
-        "pl_gemm_skinny": [p, p, p, i, i, i, i, i, p],
+        "pl_gemm_skinny": [p, p, p, p, i, f, p, i, i, i, i, i, p],
         "pl_paged_attention_decode": [p, i, p, p, p, p, p, p, i, p, i, i, p, p, i, i, i, i, f, i, i, p],
         "pl_paged_attention_prefill": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, p],
     }
@@ -351,28 +351,58 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nk
                                   q_len=batch.q_len if mixed else None, short_limit=SHORT_PORTION if mixed else 0)
 
 
-def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
-                swiglu: bool = False) -> torch.Tensor:
-    """y = x . w^T for up to 64 rows of bfloat16 on the matrix cores, the weights streamed once.
-    With ``swiglu`` the rows of ``w`` are [gate | up] and y = silu(x . gate^T) * (x . up^T)."""
-    n, K = x.shape
-    _need(x, "matrix product input", None, torch.bfloat16)
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, swiglu: bool = False,
+                norm_gain: torch.Tensor | None = None, eps: float = 0.0, rows: torch.Tensor | None = None,
+                add_into: torch.Tensor | None = None) -> torch.Tensor:
+    """y = x . w^T for up to 64 rows on the matrix cores, the bfloat16 weights streamed once.
+
+    ``x`` is bfloat16 [n, K]; or, with ``norm_gain``, the 32-bit residual stream, whose rows
+    (``rows[i]`` for output row i when a row list is given) are RMS-normalised on the way in.
+    With ``swiglu`` the rows of ``w`` are [gate | up] and y = silu(x . gate^T) * (x . up^T).
+    With ``add_into`` (the 32-bit residual stream, [n, N]) the result is added there and that
+    tensor is returned."""
+    K = x.shape[1]
+    if norm_gain is None:
+        _need(x, "matrix product input", None, torch.bfloat16)
+        n = x.shape[0]
+        if rows is not None:
+            raise TensorError("a row list goes with a norm")
+    else:
+        _need(x, "residual stream", None, torch.float32)
+        _need(norm_gain, "norm gain", (K,))
+        n = x.shape[0] if rows is None else rows.numel()
+        if rows is not None:
+            _need(rows, "row list", (n,), torch.int32)
     _need(w, "weight", None, torch.bfloat16)
-    if w.dim() != 2 or w.shape[1] != K:
-        raise TensorError(f"weight has shape {tuple(w.shape)} for an input of width {K}")
+    if x.dim() != 2 or w.dim() != 2 or w.shape[1] != K:
+        raise TensorError(f"weight has shape {tuple(w.shape)} for an input of shape {tuple(x.shape)}")
     N_out = w.shape[0] // 2 if swiglu else w.shape[0]
     if swiglu and w.shape[0] % 2:
         raise TensorError(f"fused gate/up weight has an odd number of rows, {w.shape[0]}")
-    if out_dtype not in (torch.bfloat16, torch.float32):
-        raise TensorError(f"matrix product output {out_dtype}")
-    out = torch.empty((n, N_out), dtype=out_dtype, device=x.device)
-    _check(library().pl_gemm_skinny(x.data_ptr(), w.data_ptr(), out.data_ptr(), n, N_out, K, 1 if swiglu else 0,
-                                    1 if out_dtype == torch.float32 else 0, _stream()))
+    if add_into is not None:
+        if swiglu or norm_gain is not None:
+            raise TensorError("a product that adds into the residual stream has a plain input and no activation")
+        _need(add_into, "residual stream", (n, N_out), torch.float32)
+        out, epilogue, out_f32 = add_into, 2, 1
+    else:
+        if out_dtype not in (torch.bfloat16, torch.float32):
+            raise TensorError(f"matrix product output {out_dtype}")
+        out = torch.empty((n, N_out), dtype=out_dtype, device=x.device)
+        epilogue, out_f32 = (1 if swiglu else 0), (1 if out_dtype == torch.float32 else 0)
+    _check(library().pl_gemm_skinny(
+        x.data_ptr(), w.data_ptr(), out.data_ptr(), _ptr(norm_gain),
+        _code(norm_gain, "norm gain") if norm_gain is not None else F32, float(eps), _ptr(rows), n, N_out, K,
+        epilogue, out_f32, _stream()))
     return out
 
 
 def skinny_applies(x: torch.Tensor) -> bool:
     return x.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_ROWS and x.shape[1] % 8 == 0
+
+
+def fused_norm_applies(rows_out: int, width: int, weight: torch.Tensor) -> bool:
+    """Whether norm and product run as one kernel: few rows of a bfloat16 model."""
+    return weight.dtype == torch.bfloat16 and 0 < rows_out <= SKINNY_ROWS and width % 8 == 0
 
 
 def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:

@@ -63,7 +63,12 @@ class PagedAttention:
     def state_spec(self):
         return None
 
-    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+    # forward takes a norm still to run in place of rows, and may add its result into ctx.residual
+    fuses = True
+
+    def forward(self, x, ctx):
+        """``x``: normalised rows, or a PendingNorm.  Where ``ctx.residual`` is given and the output
+        projection can add into it, None comes back."""
         batch = ctx.batch
         kv = ctx.kv()
         qkv = self.qkv_proj.forward(x)
@@ -74,9 +79,9 @@ class PagedAttention:
             qkv, self.q_gain, self.k_gain, self.eps, cos, sin, rot, batch.positions, batch.seq_of,
             kv.block_table, kv.block_size, kv.k_pool, kv.v_pool, self.nq, self.nkv, self.d,
             write_kv=ctx.writes_cache)
-        out = torch.empty((x.shape[0], self.nq * self.d), dtype=x.dtype, device=x.device)
+        out = torch.empty((qkv.shape[0], self.nq * self.d), dtype=qkv.dtype, device=qkv.device)
         kernels.paged_attention(qkv, out, batch, kv, self.nq, self.nkv, self.d, self.scale, self.window)
-        return self.o_proj.forward(out)
+        return self.o_proj.forward(out, add_into=ctx.residual)
 
 
 register_mixer("paged_attention", PagedAttention)

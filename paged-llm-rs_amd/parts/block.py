@@ -4,11 +4,14 @@ feed-forward, residual (reference: model/mod.rs:84-136).
 The residual stream is 32-bit.  A block receives the stream and the previous
 block's output that has not been added yet, adds it inside its first norm, and
 returns its own feed-forward output unadded, so that every residual sum is
-fused with the norm that follows it.
+fused with the norm that follows it.  With few rows the fusion goes the other
+way: a part that can adds its output into the stream as the last stage of its
+product kernel and the norm becomes the first stage of the next product.
 """
 
 from __future__ import annotations
 
+from .norm import PendingNorm
 from .registry import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, lookup, prefixed, register_block, scoped)
 
 
@@ -45,10 +48,24 @@ class PreNormBlock:
         return getattr(self.mixer, "graph_safe", True) and getattr(self.feed_forward, "graph_safe", True)
 
     def forward(self, resid, delta, ctx):
-        normed = self.norm1.apply(resid, delta, self.dtype)
-        mixed = self.mixer.forward(normed, ctx)
-        normed = self.norm2.apply(resid, mixed, self.dtype)
-        return self.feed_forward.forward(normed)
+        """``delta``: what the block before has not added to the stream yet, or None.  Returns this
+        block's own unadded output, or None when the feed-forward added it itself."""
+        mixer_fuses = getattr(self.mixer, "fuses", False)
+        ffn_fuses = getattr(self.feed_forward, "fuses", False)
+        if delta is None and mixer_fuses:
+            x = PendingNorm(self.norm1, resid, self.dtype)       # every sum is in the stream already
+        else:
+            x = self.norm1.apply(resid, delta, self.dtype)
+        ctx.residual = resid if mixer_fuses else None
+        mixed = self.mixer.forward(x, ctx)
+        ctx.residual = None
+        if mixed is None and ffn_fuses:
+            x = PendingNorm(self.norm2, resid, self.dtype)
+        else:
+            x = self.norm2.apply(resid, mixed, self.dtype)
+        if ffn_fuses:
+            return self.feed_forward.forward(x, residual=resid)
+        return self.feed_forward.forward(x)
 
 
 register_block("pre_norm", PreNormBlock)

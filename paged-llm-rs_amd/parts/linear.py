@@ -8,6 +8,7 @@ import torch
 
 from .. import kernels
 from ..errors import TensorError
+from .norm import PendingNorm
 
 
 class Linear:
@@ -24,7 +25,21 @@ class Linear:
         concatenation."""
         return cls(torch.cat(list(weights), dim=0))
 
-    def forward(self, x: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    def forward(self, x, out_dtype: torch.dtype | None = None, add_into: torch.Tensor | None = None,
+                swiglu: bool = False):
+        """The product of ``x`` (rows, or a norm still to run) with the weight.
+
+        ``swiglu``: the weight is [gate | up] stacked and silu(gate) * up comes back.
+        ``add_into``: the 32-bit residual stream; where the product kernel can add its result
+        there itself it does and None comes back, otherwise the result comes back unadded."""
+        if isinstance(x, PendingNorm):
+            if x.width != self.in_features:
+                raise TensorError(f"a linear of {self.in_features} inputs given a stream of width {x.width}")
+            if (getattr(x.norm, "fuses_into_product", False) and add_into is None
+                    and kernels.fused_norm_applies(x.num_rows, self.in_features, self.weight)):
+                return kernels.gemm_skinny(x.resid, self.weight, out_dtype or x.out_dtype, swiglu=swiglu,
+                                           norm_gain=x.norm.gain, eps=x.norm.eps, rows=x.rows)
+            x = x.materialize()
         if x.dim() != 2 or x.shape[1] != self.in_features:
             raise TensorError(f"a linear of {self.in_features} inputs given {tuple(x.shape)}")
         if x.dtype != self.weight.dtype:
@@ -32,5 +47,13 @@ class Linear:
         out_dtype = out_dtype or x.dtype
         if x.dtype == torch.float32:
             # the true 32-bit path: vector-unit multiply-add only
-            return kernels.gemm_plain(x, self.weight, out_dtype=torch.float32)
+            y = kernels.gemm_plain(x, self.weight, out_dtype=torch.float32)
+            return kernels.swiglu(y) if swiglu else y
+        if kernels.skinny_applies(x):
+            if add_into is not None and not swiglu:
+                kernels.gemm_skinny(x, self.weight, add_into=add_into)
+                return None
+            return kernels.gemm_skinny(x, self.weight, out_dtype, swiglu=swiglu)
+        if swiglu:
+            return kernels.swiglu(kernels.linear_bf16(x, self.weight, x.dtype))
         return kernels.linear_bf16(x, self.weight, out_dtype)

@@ -26,13 +26,14 @@ class GatedMlp:
         self.gate_up_proj = Linear.fused([params["gate_proj.weight"], params["up_proj.weight"]])
         self.down_proj = Linear(params["down_proj.weight"])
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
-        if kernels.skinny_applies(x):
-            # few rows: the activation is the epilogue of the weight stream
-            act = kernels.gemm_skinny(x, self.gate_up_proj.weight, swiglu=True)
-        else:
-            act = kernels.swiglu(self.gate_up_proj.forward(x))
-        return self.down_proj.forward(act)
+    # forward takes a norm still to run in place of rows, and may add its result into the stream
+    fuses = True
+
+    def forward(self, x, residual: torch.Tensor | None = None):
+        """``x``: normalised rows, or a PendingNorm.  With ``residual`` (the 32-bit stream) the
+        result is added there where the product kernel can do it, and None comes back."""
+        act = self.gate_up_proj.forward(x, swiglu=True)      # few rows: the activation is the product's epilogue
+        return self.down_proj.forward(act, add_into=residual)
 
 
 register_feed_forward("gated_mlp", GatedMlp)

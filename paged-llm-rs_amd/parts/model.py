@@ -18,6 +18,7 @@ from ..errors import ConfigError, UnsupportedError, WeightError
 from ..weights.loader import ParamDecl, load_weights
 from . import attention, block, mlp, norm  # noqa: F401  (register the built-in parts)
 from .linear import Linear
+from .norm import PendingNorm
 from .registry import BLOCKS, NORMS, lookup, prefixed, scoped
 
 DTYPES = {"float32": torch.float32, "f32": torch.float32, "bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
@@ -42,7 +43,7 @@ class LayerContext:
     """What one run of one layer sees of the step: the batch, its own pages (or
     the pages of the layer it reads from) and its state slots."""
 
-    __slots__ = ("batch", "cache", "layer", "cache_layer", "writes_cache")
+    __slots__ = ("batch", "cache", "layer", "cache_layer", "writes_cache", "residual")
 
     def __init__(self, batch, cache, layer: int, cache_layer: int, writes_cache: bool):
         self.batch = batch
@@ -50,6 +51,8 @@ class LayerContext:
         self.layer = layer
         self.cache_layer = cache_layer
         self.writes_cache = writes_cache
+        # the 32-bit stream, while a mixer that adds its own output runs; None otherwise
+        self.residual = None
 
     def kv(self):
         return self.cache.layer_view(self.cache_layer, self.batch)
@@ -105,7 +108,10 @@ class DecoderModel:
             # A portion in the middle of a prompt runs only to fill the cache.
             # Nothing further is launched for it.
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
-        normed = self.norm.apply(resid, delta, self.dtype, rows=batch.logit_rows)
+        if delta is None:
+            normed = PendingNorm(self.norm, resid, self.dtype, rows=batch.logit_rows)
+        else:
+            normed = self.norm.apply(resid, delta, self.dtype, rows=batch.logit_rows)
         return self.lm_head.forward(normed, out_dtype=torch.float32)
 
 

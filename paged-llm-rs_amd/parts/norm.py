@@ -9,8 +9,35 @@ from ..weights.loader import ParamDecl
 from .registry import register_norm
 
 
+class PendingNorm:
+    """A norm that has not run yet: the 32-bit stream it will read (every sum already in
+    it), the norm, the type its output would have, and the rows wanted (all, or a list).
+
+    A part that is handed one may pass it on to ``Linear.forward``, which runs norm and
+    product as one kernel where that pays, or call ``materialize()`` for the normalised rows."""
+
+    __slots__ = ("norm", "resid", "out_dtype", "rows")
+
+    def __init__(self, norm, resid: torch.Tensor, out_dtype: torch.dtype, rows=None):
+        self.norm, self.resid, self.out_dtype, self.rows = norm, resid, out_dtype, rows
+
+    @property
+    def num_rows(self) -> int:
+        return self.resid.shape[0] if self.rows is None else self.rows.numel()
+
+    @property
+    def width(self) -> int:
+        return self.resid.shape[1]
+
+    def materialize(self) -> torch.Tensor:
+        return self.norm.apply(self.resid, None, self.out_dtype, rows=self.rows)
+
+
 class RmsNorm:
     """x / sqrt(mean(x^2) + eps) * gain, statistic and product in 32-bit."""
+
+    # a product kernel can take this norm as its first stage: it needs ``gain`` and ``eps`` only
+    fuses_into_product = True
 
     @staticmethod
     def declare(spec, width: int) -> list:

@@ -221,6 +221,43 @@ def test_gemm_skinny(n, N, K):
     assert torch.equal(kernels.gemm_skinny(eye, w, torch.bfloat16), w[:, idx].T.contiguous())
 
 
+@pytest.mark.parametrize("n", [1, 8, 17, 64])
+@pytest.mark.parametrize("N,K,gain_dtype", [(48, 104, torch.float32), (4096, 1024, torch.bfloat16), (250, 2056, torch.float32)])
+def test_gemm_skinny_with_the_norm_before_and_the_residual_after(n, N, K, gain_dtype):
+    """The norm as the product's first stage (statistic from the values the product loads, rows picked
+    by a list), SwiGLU or the residual sum as its last."""
+    from paged_llm_rs_amd import kernels
+
+    eps = 1e-5
+    stream = torch.randn(n + 3, K, device=DEV) * 3.0
+    stream[0] *= 50.0                                         # rows of very different size: the statistic is a row's own
+    gain = (1 + 0.3 * torch.randn(K, device=DEV)).to(gain_dtype)
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
+
+    def normed(rows):
+        x = stream[rows].double()
+        return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * gain.double()
+
+    all_rows = list(range(n))
+    want = normed(all_rows) @ w.double().T
+    got = kernels.gemm_skinny(stream[:n].contiguous(), w, torch.float32, norm_gain=gain, eps=eps)
+    assert rel(got, want) < 6e-3, "bfloat16 inputs, 32-bit sums"
+    picked = [(7 * i + 2) % (n + 3) for i in range(n)]
+    rows = torch.tensor(picked, dtype=torch.int32, device=DEV)
+    got = kernels.gemm_skinny(stream, w, torch.bfloat16, norm_gain=gain, eps=eps, rows=rows)
+    assert rel(got, normed(picked) @ w.double().T) < 1e-2
+    if N % 2 == 0:
+        g, u = want[:, :N // 2], want[:, N // 2:]
+        got = kernels.gemm_skinny(stream[:n].contiguous(), w, torch.float32, swiglu=True, norm_gain=gain, eps=eps)
+        assert rel(got, torch.nn.functional.silu(g) * u) < 1e-2
+    # the residual sum: every element of the stream takes its own column's product, once
+    x = torch.randn(n, K, device=DEV).to(torch.bfloat16)
+    resid = torch.randn(n, N, device=DEV)
+    want = resid.double() + x.double() @ w.double().T
+    assert kernels.gemm_skinny(x, w, add_into=resid) is resid
+    assert rel(resid, want) < 1e-5
+
+
 def test_gemm_skinny_refusals():
     from paged_llm_rs_amd import kernels
     from paged_llm_rs_amd.errors import TensorError
