@@ -9,8 +9,8 @@
 //   GT of the query heads that share it, so keys and values are read once per
 //   kv head, not once per query head.
 //   A group of LPK lanes owns one key: each lane holds 8 of its values.  A wave
-//   handles 64/LPK keys with one load instruction and four such instructions are
-//   issued back to back for keys and for values.
+//   handles 64/LPK keys with one load instruction and four or eight such
+//   instructions are issued back to back for keys and for values.
 //   Softmax is online (running maximum and sum in 32-bit, base-2 exponentials
 //   with log2(e) folded into the query scale).  The lane groups and waves keep
 //   separate running states that are merged through LDS at the end; with more
@@ -19,7 +19,6 @@
 #include "common.hpp"
 
 #define AD_WAVES 4
-#define AD_UNROLL 4
 
 struct __attribute__((aligned(16))) u32x4 {
     uint32_t v[4];
@@ -41,7 +40,8 @@ __device__ __forceinline__ float group_sum(float v) {
 }
 
 // LPK: lanes a key (a power of two, LPK*8 >= d).  GT: query heads a workgroup serves.
-template <int LPK, int GT>
+// U: keys a lane group asks for at once.
+template <int LPK, int GT, int U>
 __global__ void __launch_bounds__(256)
 paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
                               float* __restrict__ part_acc, float* __restrict__ part_ml,
@@ -76,7 +76,7 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
     // the stretch of keys of this split, in whole rounds of the workgroup
     const int first = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
     const int total = pos + 1 - first;
-    constexpr int ROUND = AD_WAVES * KPW * AD_UNROLL;
+    constexpr int ROUND = AD_WAVES * KPW * U;
     const int per_split = pl_ceil_div(pl_ceil_div(total, splits), ROUND) * ROUND;
     const int s_begin = first + split * per_split;
     const int s_end = min(pos + 1, s_begin + per_split);
@@ -114,10 +114,10 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
     // Loads are unconditional, from an address that is valid in any case, and masked afterwards:
     // a load inside a branch is waited for at the branch's end, one after the other.  The pages
     // of a round are looked up during the round before, so that no load waits for another.
-    int blk[AD_UNROLL], within[AD_UNROLL];
+    int blk[U], within[U];
     auto lookup = [&](int base) {
 #pragma unroll
-        for (int u = 0; u < AD_UNROLL; ++u) {
+        for (int u = 0; u < U; ++u) {
             const int j = base + u * KPW + sub;
             const bool in = j < s_end;
             const int jj = in ? j : pos;                          // the token's own place always has a page
@@ -131,14 +131,14 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
             within[u] = w;
         }
     };
-    const int first_base = s_begin + wave * KPW * AD_UNROLL;
+    const int first_base = s_begin + wave * KPW * U;
     lookup(first_base);
 
     for (int base = first_base; base < s_end; base += ROUND) {
-        u32x4 kraw[AD_UNROLL], vraw[AD_UNROLL];
-        bool ok[AD_UNROLL];
+        u32x4 kraw[U], vraw[U];
+        bool ok[U];
 #pragma unroll
-        for (int u = 0; u < AD_UNROLL; ++u) {
+        for (int u = 0; u < U; ++u) {
             ok[u] = blk[u] >= 0;
             const size_t off = (static_cast<size_t>(max(blk[u], 0)) * block_size + within[u]) * row_stride + head_off;
             const u32x4 kgot = *reinterpret_cast<const u32x4*>(k_pool + off);
@@ -151,9 +151,9 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
             }
         }
         lookup(base + ROUND);
-        float s[AD_UNROLL][GT];
+        float s[U][GT];
 #pragma unroll
-        for (int u = 0; u < AD_UNROLL; ++u) {
+        for (int u = 0; u < U; ++u) {
             float kf[8];
             unpack8(kraw[u], kf);
 #pragma unroll
@@ -169,13 +169,13 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
         for (int hq = 0; hq < GT; ++hq) {
             float m_new = m[hq];
 #pragma unroll
-            for (int u = 0; u < AD_UNROLL; ++u) m_new = fmaxf(m_new, s[u][hq]);
+            for (int u = 0; u < U; ++u) m_new = fmaxf(m_new, s[u][hq]);
             if (m_new == -INFINITY) continue;  // nothing seen yet by this lane group
             const float corr = exp2f(m[hq] - m_new);
-            float p[AD_UNROLL];
+            float p[U];
             float psum = 0.f;
 #pragma unroll
-            for (int u = 0; u < AD_UNROLL; ++u) {
+            for (int u = 0; u < U; ++u) {
                 p[u] = exp2f(s[u][hq] - m_new);
                 psum += p[u];
             }
@@ -184,7 +184,7 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
 #pragma unroll
             for (int i = 0; i < 8; ++i) acc[hq][i] *= corr;
 #pragma unroll
-            for (int u = 0; u < AD_UNROLL; ++u) {
+            for (int u = 0; u < U; ++u) {
                 float vf[8];
                 unpack8(vraw[u], vf);
 #pragma unroll
@@ -238,29 +238,45 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
 }
 
 // Merges the splits of one (token, query head): out = sum_s a_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).
-__global__ void paged_attention_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
-                                             bf16_t* __restrict__ out, const int* __restrict__ positions,
-                                             const int* __restrict__ seq_of, const int* __restrict__ q_len,
-                                             int short_limit, int nq, int d, int splits) {
-    const int t = blockIdx.x, h = blockIdx.y;
-    if (positions[t] < 0) return;
-    if (q_len && q_len[seq_of[t]] >= short_limit) return;
+// (The merge is a kernel of its own because the end of a kernel is the cheapest way on this chip to make
+// one workgroup's results visible to another: a device-wide fence inside a kernel writes back and
+// invalidates a whole L2.)  One thread an output element; every load is asked for before any is used.
+#define AD_MAX_SPLITS 64
+
+template <int SP>
+__global__ void __launch_bounds__(256)
+paged_attention_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+                             bf16_t* __restrict__ out, const int* __restrict__ positions,
+                             const int* __restrict__ seq_of, const int* __restrict__ q_len, int short_limit,
+                             int nq, int d, int splits, int n) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    const int per_token = nq * d;
+    const int t = min(idx / per_token, n - 1);
+    const int rest = idx - t * per_token;
+    const int h = rest / d, dd = rest - h * d;
     const size_t base = (static_cast<size_t>(t) * nq + h) * splits;
-    float big = -INFINITY;
-    for (int s = 0; s < splits; ++s) big = fmaxf(big, part_ml[(base + s) * 2]);
-    for (int dd = threadIdx.x; dd < d; dd += blockDim.x) {
-        float sum = 0.f, a = 0.f;
-        if (big != -INFINITY) {
-            for (int s = 0; s < splits; ++s) {
-                const float ms = part_ml[(base + s) * 2];
-                if (ms == -INFINITY) continue;
-                const float w = exp2f(ms - big);
-                sum += part_ml[(base + s) * 2 + 1] * w;
-                a += part_acc[(base + s) * d + dd] * w;
-            }
-        }
-        out[(static_cast<size_t>(t) * nq + h) * d + dd] = from_float<bf16_t>(sum > 0.f ? a / sum : 0.f);
+    const int pos = positions[t];
+    const int len = q_len ? q_len[seq_of[t]] : 0;
+    float ms[SP], ls[SP], as[SP];
+#pragma unroll
+    for (int s = 0; s < SP; ++s) {
+        const int sc = min(s, splits - 1);
+        ms[s] = part_ml[(base + sc) * 2];
+        ls[s] = part_ml[(base + sc) * 2 + 1];
+        as[s] = part_acc[(base + sc) * d + dd];
     }
+    if (idx >= n * per_token || pos < 0 || (q_len && len >= short_limit)) return;
+    float big = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < SP; ++s) big = fmaxf(big, s < splits ? ms[s] : -INFINITY);
+    float sum = 0.f, a = 0.f;
+#pragma unroll
+    for (int s = 0; s < SP; ++s) {
+        const float w = (s < splits && ms[s] != -INFINITY) ? exp2f(ms[s] - big) : 0.f;
+        sum = fmaf(ls[s], w, sum);
+        a = fmaf(as[s], w, a);
+    }
+    out[(static_cast<size_t>(t) * nq + h) * d + dd] = from_float<bf16_t>(sum > 0.f ? a / sum : 0.f);
 }
 
 template <int LPK, int GT>
@@ -271,26 +287,34 @@ static int launch_decode(const void* q, int q_stride, void* out, float* part_acc
                          hipStream_t stream) {
     constexpr int KPW = PL_WAVE / LPK;
     constexpr int GROUPS = AD_WAVES * KPW;
+    constexpr int U = GT <= 2 ? 8 : 4;   // fewer heads a workgroup leave registers for more keys in flight
     const int g = nq / nkv;
     const int tiles = pl_ceil_div(g, GT);
     const size_t lds_bytes = (static_cast<size_t>(GROUPS) * GT * 2 + static_cast<size_t>(GROUPS) * GT * d) * sizeof(float);
     PL_REQUIRE(lds_bytes <= 160 * 1024, "decode attention: %zu bytes of LDS for head size %d", lds_bytes, d);
     if (lds_bytes > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_decode_kernel<LPK, GT>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_decode_kernel<LPK, GT, U>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
         PL_REQUIRE(e == hipSuccess, "decode attention: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
     }
     dim3 grid(nkv * tiles, n, splits);
     PL_REQUIRE(n <= 65535 && splits <= 65535, "decode attention: %d tokens or %d splits are more than one launch covers", n, splits);
-    paged_attention_decode_kernel<LPK, GT><<<grid, 256, lds_bytes, stream>>>(
+    paged_attention_decode_kernel<LPK, GT, U><<<grid, 256, lds_bytes, stream>>>(
         static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), part_acc, part_ml, positions, seq_of,
         q_len, short_limit, block_table, max_blocks, block_size, static_cast<const bf16_t*>(k_pool),
         static_cast<const bf16_t*>(v_pool), nq, nkv, d, scale * 1.4426950408889634f, window, splits, tiles);
     PL_CHECK_LAUNCH("paged_attention_decode");
     if (splits > 1) {
-        dim3 mgrid(n, nq);
-        paged_attention_merge_kernel<<<mgrid, 64, 0, stream>>>(part_acc, part_ml, static_cast<bf16_t*>(out), positions,
-                                                               seq_of, q_len, short_limit, nq, d, splits);
+        const int mgrid = pl_ceil_div(n * nq * d, 256);
+#define AD_MERGE(SP)                                                                                              \
+    paged_attention_merge_kernel<SP><<<mgrid, 256, 0, stream>>>(part_acc, part_ml, static_cast<bf16_t*>(out),     \
+                                                                positions, seq_of, q_len, short_limit, nq, d,     \
+                                                                splits, n)
+        if (splits <= 4) AD_MERGE(4);
+        else if (splits <= 8) AD_MERGE(8);
+        else if (splits <= 16) AD_MERGE(16);
+        else AD_MERGE(AD_MAX_SPLITS);
+#undef AD_MERGE
         PL_CHECK_LAUNCH("paged_attention_merge");
     }
     return 0;
@@ -324,7 +348,7 @@ extern "C" int pl_paged_attention_decode(const void* q, int q_stride, void* out,
                                          int splits, hipStream_t stream) {
     PL_REQUIRE(d > 0 && d <= 256 && d % 16 == 0, "decode attention: head size %d, which has to be a multiple of 16 up to 256", d);
     PL_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "decode attention: %d query heads over %d key heads", nq, nkv);
-    PL_REQUIRE(block_size > 0 && max_blocks > 0 && q_stride >= nq * d && q_stride % 8 == 0 && window >= 0 && splits >= 1,
+    PL_REQUIRE(block_size > 0 && max_blocks > 0 && q_stride >= nq * d && q_stride % 8 == 0 && window >= 0 && splits >= 1 && splits <= AD_MAX_SPLITS,
                "decode attention: block size %d, %d blocks a row, query stride %d, window %d, %d splits", block_size,
                max_blocks, q_stride, window, splits);
     PL_REQUIRE(splits == 1 || (part_acc && part_ml), "decode attention: %d splits without a workspace", splits);
