@@ -54,43 +54,32 @@ __device__ __forceinline__ bf16x8 sk_zero8() {
     return z;
 }
 
-// Eight consecutive gains as 32-bit floats, whichever way they are stored.
-template <typename GT>
-__device__ __forceinline__ void sk_load_gain(const void* gain, int k, float* out);
-template <>
-__device__ __forceinline__ void sk_load_gain<float>(const void* gain, int k, float* out) {
-    const sk_f32x4 a = *reinterpret_cast<const sk_f32x4*>(static_cast<const float*>(gain) + k);
-    const sk_f32x4 b = *reinterpret_cast<const sk_f32x4*>(static_cast<const float*>(gain) + k + 4);
+// Eight consecutive gains (32-bit floats).
+__device__ __forceinline__ void sk_load_gain(const float* gain, int k, float* out) {
+    const sk_f32x4 a = *reinterpret_cast<const sk_f32x4*>(gain + k);
+    const sk_f32x4 b = *reinterpret_cast<const sk_f32x4*>(gain + k + 4);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         out[e] = a.v[e];
         out[4 + e] = b.v[e];
     }
 }
-template <>
-__device__ __forceinline__ void sk_load_gain<bf16_t>(const void* gain, int k, float* out) {
-    const sk_u32x4 raw = *reinterpret_cast<const sk_u32x4*>(static_cast<const bf16_t*>(gain) + k);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        out[2 * e] = __uint_as_float(raw.v[e] << 16);
-        out[2 * e + 1] = __uint_as_float(raw.v[e] & 0xffff0000u);
-    }
-}
 
 // MT: 16-row tiles of x (n <= 16*MT).  UNR: K steps a wave asks for at once.  WV: the most waves a
 // workgroup may have (it is launched with as many as give every wave one round of loads, or WV).
-// GT: the gain's type.
+// The gain is 32-bit.
 // A workgroup walks the column tiles blockIdx.x, blockIdx.x + gridDim.x, ...; when a wave's share of
 // K fits one round of loads, its rows of x are loaded (and normalised) once and stay in registers.
-template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT, typename GT>
+template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT>
 __global__ void __launch_bounds__(64 * WV)
 gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OUT* __restrict__ y,
-                   const void* __restrict__ gain, float eps, const int* __restrict__ rows, int n, int N_out,
+                   const float* __restrict__ gain, float eps, const int* __restrict__ rows, int n, int N_out,
                    int K) {
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
-    __shared__ float red[WV][BT][MT][256];
-    __shared__ float ssq_lds[WV][MT * 16];
     const int nwaves = blockDim.x / PL_WAVE;
+    extern __shared__ float sk_lds[];
+    float* red = sk_lds;                                   // [nwaves][BT][MT][256] partial tiles
+    float* ssq_lds = sk_lds + nwaves * BT * MT * 256;      // [nwaves][MT * 16] partial sums of squares
 
     const int lane = threadIdx.x % PL_WAVE;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PL_WAVE);
@@ -130,7 +119,7 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
         for (int u = 0; u < UNR; ++u) {
             const int at = k0 + u * SK_KSTEP + g * 8;
             const int kk = at < kend ? at : 0;  // K is a multiple of 8, so a chunk is whole or absent
-            if (PRO == PRO_NORM) sk_load_gain<GT>(gain, kk, gn[u]);
+            if (PRO == PRO_NORM) sk_load_gain(gain, kk, gn[u]);
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
                 if (PRO == PRO_BF16) {
@@ -224,7 +213,7 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
 #pragma unroll
             for (int m = 0; m < MT; ++m)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) red[wave][b][m][lane * 4 + i] = acc[b][m][i];
+                for (int i = 0; i < 4; ++i) red[((wave * BT + b) * MT + m) * 256 + lane * 4 + i] = acc[b][m][i];
         if (PRO == PRO_NORM) {
             // the four lanes that hold a row's four chunks of a K step, then the four waves
 #pragma unroll
@@ -232,7 +221,7 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
                 float s = ssq[m];
                 s += __shfl_xor(s, 16, PL_WAVE);
                 s += __shfl_xor(s, 32, PL_WAVE);
-                if (g == 0) ssq_lds[wave][m * 16 + c] = s;
+                if (g == 0) ssq_lds[wave * MT * 16 + m * 16 + c] = s;
             }
         }
         __syncthreads();
@@ -249,13 +238,13 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
             for (int b = 0; b < BT; ++b) {
                 float s = 0.f;
 #pragma unroll
-                for (int wv = 0; wv < nwaves; ++wv) s += red[wv][b][m][t];
+                for (int wv = 0; wv < nwaves; ++wv) s += red[((wv * BT + b) * MT + m) * 256 + t];
                 v[b] = s;
             }
             if (PRO == PRO_NORM) {
                 float total = 0.f;
 #pragma unroll
-                for (int wv = 0; wv < nwaves; ++wv) total += ssq_lds[wv][m * 16 + row_in_tile];
+                for (int wv = 0; wv < nwaves; ++wv) total += ssq_lds[wv * MT * 16 + m * 16 + row_in_tile];
                 const float rinv = 1.f / sqrtf(total / static_cast<float>(K) + eps);
 #pragma unroll
                 for (int b = 0; b < BT; ++b) v[b] *= rinv;
@@ -279,67 +268,77 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
 #define SK_MAX_GRID 2048
 
 template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT>
-static int launch_one(int waves, const void* x, const void* w, void* y, const void* gain, int gain_dtype, float eps,
+static int launch_one(int waves, const void* x, const void* w, void* y, const float* gain, float eps,
                       const int* rows, int n, int N_out, int K, hipStream_t stream) {
+    constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
     const int grid = min(pl_ceil_div(N_out, SK_TILE_N), SK_MAX_GRID);
-    if (PRO == PRO_NORM && gain_dtype == PL_DTYPE_F32)
-        gemm_skinny_kernel<MT, UNR, WV, PRO, EPI, OUT, float><<<grid, 64 * waves, 0, stream>>>(
-            x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps, rows, n, N_out, K);
-    else
-        gemm_skinny_kernel<MT, UNR, WV, PRO, EPI, OUT, bf16_t><<<grid, 64 * waves, 0, stream>>>(
-            x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps, rows, n, N_out, K);
+    const size_t lds_bytes = static_cast<size_t>(waves) * (BT * MT * 256 + MT * 16) * sizeof(float);
+    if (lds_bytes > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny_kernel<MT, UNR, WV, PRO, EPI, OUT>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+        PL_REQUIRE(e == hipSuccess, "skinny product: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
+    }
+    gemm_skinny_kernel<MT, UNR, WV, PRO, EPI, OUT><<<grid, 64 * waves, lds_bytes, stream>>>(
+        x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps, rows, n, N_out, K);
     PL_CHECK_LAUNCH("gemm_skinny");
     return 0;
 }
 
-// As many waves as give each one round of loads, between four and sixteen: the whole matrix is then
-// asked for at once and the kernel's time is one trip to memory.
+// How many waves, and how many K steps each asks for at once.  What a wave holds in flight has to fit
+// its registers (512 a lane with four waves, 256 with eight, 128 with sixteen); within that, the
+// fewest waves whose one round of loads covers K are taken, so that the whole matrix is asked for at
+// once and the kernel's time is one trip to memory.  The numbers are the largest that compile
+// without spilling (0: that many waves have no room).
+template <int MT, int PRO, int EPI>
+struct SkShape {
+    static constexpr bool TWO = EPI == EPI_SWIGLU;     // two weight tiles a step
+    static constexpr int U4 = PRO == PRO_NORM ? (MT == 1 ? 8 : (MT == 2 ? 4 : 2)) : ((TWO && MT >= 3) ? 4 : 8);
+    static constexpr int U8 = PRO == PRO_NORM ? 0 : (TWO ? (MT == 1 ? 8 : (MT <= 3 ? 4 : 2)) : (MT <= 2 ? 8 : 4));
+    static constexpr int U16 = PRO == PRO_NORM ? 0 : (TWO ? (MT == 1 ? 4 : (MT <= 3 ? 2 : 1)) : (MT == 1 ? 8 : (MT == 2 ? 4 : 2)));
+};
+
 template <int MT, int PRO, int EPI, typename OUT>
-static int launch_unr(const void* x, const void* w, void* y, const void* gain, int gain_dtype, float eps,
+static int launch_unr(const void* x, const void* w, void* y, const float* gain, float eps,
                       const int* rows, int n, int N_out, int K, hipStream_t stream) {
-    constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
-    constexpr int COST = BT + MT * (PRO == PRO_NORM ? 2 : 1);  // 16-byte registers a K step holds in flight
-    constexpr int UNR = COST <= 4 ? 8 : (COST <= 6 ? 4 : 2);
-    // the partial tiles of all waves lie in LDS side by side, a kilobyte a tile: at most 48 of them
-    // (a product that starts with a norm holds its rows twice, raw and rounded: four waves leave it the registers)
-    constexpr int MAXWV = PRO == PRO_NORM ? 4 : (BT * MT <= 3 ? 16 : (BT * MT <= 6 ? 8 : 4));
+    using S = SkShape<MT, PRO, EPI>;
     const int steps = pl_ceil_div(K, SK_KSTEP);
-    const int waves = max(4, min(MAXWV, pl_ceil_div(steps, UNR)));
-    if (waves <= 4) return launch_one<MT, UNR, 4, PRO, EPI, OUT>(4, x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream);
-    if constexpr (MAXWV >= 8) {
-        if (waves <= 8) return launch_one<MT, UNR, 8, PRO, EPI, OUT>(waves, x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream);
+    const int most = max(4 * S::U4, max(8 * S::U8, 16 * S::U16));
+    const int need = min(steps, most);     // beyond that, several rounds
+    if (need <= 4 * S::U4)
+        return launch_one<MT, S::U4, 4, PRO, EPI, OUT>(4, x, w, y, gain, eps, rows, n, N_out, K, stream);
+    if constexpr (S::U8 > 0) {
+        if (need <= 8 * S::U8 || S::U16 == 0)
+            return launch_one<MT, S::U8, 8, PRO, EPI, OUT>(max(5, min(8, pl_ceil_div(steps, S::U8))), x, w, y, gain, eps, rows, n, N_out, K, stream);
     }
-    if constexpr (MAXWV >= 16) {
-        return launch_one<MT, UNR, 16, PRO, EPI, OUT>(waves, x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream);
+    if constexpr (S::U16 > 0) {
+        return launch_one<MT, S::U16, 16, PRO, EPI, OUT>(max(9, min(16, pl_ceil_div(steps, S::U16))), x, w, y, gain, eps, rows, n, N_out, K, stream);
     }
-    return -1;  // not reached: waves <= MAXWV
+    return launch_one<MT, S::U4, 4, PRO, EPI, OUT>(4, x, w, y, gain, eps, rows, n, N_out, K, stream);
 }
 
 template <int PRO, int EPI, typename OUT>
-static int launch_mt(const void* x, const void* w, void* y, const void* gain, int gain_dtype, float eps,
+static int launch_mt(const void* x, const void* w, void* y, const float* gain, float eps,
                      const int* rows, int n, int N_out, int K, hipStream_t stream) {
     switch (pl_ceil_div(n, 16)) {
-        case 1: return launch_unr<1, PRO, EPI, OUT>(x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream);
-        case 2: return launch_unr<2, PRO, EPI, OUT>(x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream);
-        case 3: return launch_unr<3, PRO, EPI, OUT>(x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream);
-        default: return launch_unr<4, PRO, EPI, OUT>(x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream);
+        case 1: return launch_unr<1, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, stream);
+        case 2: return launch_unr<2, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, stream);
+        case 3: return launch_unr<3, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, stream);
+        default: return launch_unr<4, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, stream);
     }
 }
 
 template <int PRO>
-static int sk_launch(int epilogue, int out_f32, const void* x, const void* w, void* y, const void* gain,
-                      int gain_dtype, float eps, const int* rows, int n, int N_out, int K, hipStream_t stream) {
+static int sk_launch(int epilogue, int out_f32, const void* x, const void* w, void* y, const float* gain,
+                      float eps, const int* rows, int n, int N_out, int K, hipStream_t stream) {
     if (epilogue == EPI_STORE)
-        return out_f32 ? launch_mt<PRO, EPI_STORE, float>(x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream)
-                       : launch_mt<PRO, EPI_STORE, bf16_t>(x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream);
-    if (epilogue == EPI_SWIGLU)
-        return out_f32 ? launch_mt<PRO, EPI_SWIGLU, float>(x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream)
-                       : launch_mt<PRO, EPI_SWIGLU, bf16_t>(x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream);
+        return out_f32 ? launch_mt<PRO, EPI_STORE, float>(x, w, y, gain, eps, rows, n, N_out, K, stream)
+                       : launch_mt<PRO, EPI_STORE, bf16_t>(x, w, y, gain, eps, rows, n, N_out, K, stream);
+    if (epilogue == EPI_SWIGLU) return launch_mt<PRO, EPI_SWIGLU, bf16_t>(x, w, y, gain, eps, rows, n, N_out, K, stream);
     if constexpr (PRO == PRO_NORM) {
         pl_set_error("skinny product: a product that reads the residual stream cannot add into it");
         return -1;
     } else {
-        return launch_mt<PRO, EPI_ADD, float>(x, w, y, gain, gain_dtype, eps, rows, n, N_out, K, stream);
+        return launch_mt<PRO, EPI_ADD, float>(x, w, y, gain, eps, rows, n, N_out, K, stream);
     }
 }
 

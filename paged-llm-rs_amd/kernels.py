@@ -35,7 +35,7 @@ def _signatures(lib) -> None:
         "pl_gemm_plain": [p, p, p, i, i, i, i, i, i, i, p],
         "pl_paged_attention_plain": [p, i, p, p, p, p, i, i, p, p, i, i, i, i, f, i, i, p],
         "pl_argmax": [p, p, p, p, i, i, p],
-        "pl_gemm_skinny": [p, p, p, p, i, f, p, i, i, i, i, i, p],
+        "pl_gemm_skinny": [p, p, p, p, f, p, i, i, i, i, i, p],
         "pl_paged_attention_decode": [p, i, p, p, p, p, p, p, i, p, i, i, p, p, i, i, i, i, f, i, i, p],
         "pl_paged_attention_prefill": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, p],
     }
@@ -358,7 +358,7 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
 
     ``x`` is bfloat16 [n, K]; or, with ``norm_gain``, the 32-bit residual stream, whose rows
     (``rows[i]`` for output row i when a row list is given) are RMS-normalised on the way in.
-    With ``swiglu`` the rows of ``w`` are [gate | up] and y = silu(x . gate^T) * (x . up^T).
+    With ``swiglu`` the rows of ``w`` are [gate | up] and y = silu(x . gate^T) * (x . up^T), in bfloat16.
     With ``add_into`` (the 32-bit residual stream, [n, N]) the result is added there and that
     tensor is returned."""
     K = x.shape[1]
@@ -369,7 +369,7 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
             raise TensorError("a row list goes with a norm")
     else:
         _need(x, "residual stream", None, torch.float32)
-        _need(norm_gain, "norm gain", (K,))
+        _need(norm_gain, "norm gain", (K,), torch.float32)
         n = x.shape[0] if rows is None else rows.numel()
         if rows is not None:
             _need(rows, "row list", (n,), torch.int32)
@@ -385,13 +385,12 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
         _need(add_into, "residual stream", (n, N_out), torch.float32)
         out, epilogue, out_f32 = add_into, 2, 1
     else:
-        if out_dtype not in (torch.bfloat16, torch.float32):
-            raise TensorError(f"matrix product output {out_dtype}")
+        if out_dtype not in (torch.bfloat16, torch.float32) or (swiglu and out_dtype != torch.bfloat16):
+            raise TensorError(f"matrix product output {out_dtype}" + (" after the activation" if swiglu else ""))
         out = torch.empty((n, N_out), dtype=out_dtype, device=x.device)
         epilogue, out_f32 = (1 if swiglu else 0), (1 if out_dtype == torch.float32 else 0)
     _check(library().pl_gemm_skinny(
-        x.data_ptr(), w.data_ptr(), out.data_ptr(), _ptr(norm_gain),
-        _code(norm_gain, "norm gain") if norm_gain is not None else F32, float(eps), _ptr(rows), n, N_out, K,
+        x.data_ptr(), w.data_ptr(), out.data_ptr(), _ptr(norm_gain), float(eps), _ptr(rows), n, N_out, K,
         epilogue, out_f32, _stream()))
     return out
 

@@ -38,7 +38,7 @@ class Linear:
             if (getattr(x.norm, "fuses_into_product", False) and add_into is None
                     and kernels.fused_norm_applies(x.num_rows, self.in_features, self.weight)):
                 return kernels.gemm_skinny(x.resid, self.weight, out_dtype or x.out_dtype, swiglu=swiglu,
-                                           norm_gain=x.norm.gain, eps=x.norm.eps, rows=x.rows)
+                                           norm_gain=x.norm.gain32, eps=x.norm.eps, rows=x.rows)
             x = x.materialize()
         if x.dim() != 2 or x.shape[1] != self.in_features:
             raise TensorError(f"a linear of {self.in_features} inputs given {tuple(x.shape)}")

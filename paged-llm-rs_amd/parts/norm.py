@@ -36,7 +36,7 @@ class PendingNorm:
 class RmsNorm:
     """x / sqrt(mean(x^2) + eps) * gain, statistic and product in 32-bit."""
 
-    # a product kernel can take this norm as its first stage: it needs ``gain`` and ``eps`` only
+    # a product kernel can take this norm as its first stage: it needs ``gain32`` and ``eps`` only
     fuses_into_product = True
 
     @staticmethod
@@ -47,6 +47,8 @@ class RmsNorm:
         self.eps = float(spec.eps)
         self.width = width
         self.gain = params["weight"]
+        # the product kernels that take the norm as their first stage read the gain in 32-bit
+        self.gain32 = self.gain if self.gain.dtype == torch.float32 else self.gain.float()
 
     def apply(self, resid: torch.Tensor, delta, out_dtype: torch.dtype, rows=None) -> torch.Tensor:
         n = resid.shape[0] if rows is None else rows.numel()

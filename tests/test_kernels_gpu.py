@@ -213,7 +213,7 @@ def test_gemm_skinny(n, N, K):
     if N % 2 == 0:
         g, u = want[:, :N // 2], want[:, N // 2:]
         act = torch.nn.functional.silu(g) * u
-        assert rel(kernels.gemm_skinny(x, w, torch.float32, swiglu=True), act) < 2e-5
+        assert rel(kernels.gemm_skinny(x, w, swiglu=True), act) < 6e-3
     # one-hot rows pick single weights: a wrong operand layout cannot pass this
     eye = torch.zeros(min(n, K), K, device=DEV, dtype=torch.bfloat16)
     idx = torch.randperm(K)[:eye.shape[0]]
@@ -222,8 +222,8 @@ def test_gemm_skinny(n, N, K):
 
 
 @pytest.mark.parametrize("n", [1, 8, 17, 64])
-@pytest.mark.parametrize("N,K,gain_dtype", [(48, 104, torch.float32), (4096, 1024, torch.bfloat16), (250, 2056, torch.float32)])
-def test_gemm_skinny_with_the_norm_before_and_the_residual_after(n, N, K, gain_dtype):
+@pytest.mark.parametrize("N,K", [(48, 104), (4096, 1024), (250, 2056), (64, 3072)])
+def test_gemm_skinny_with_the_norm_before_and_the_residual_after(n, N, K):
     """The norm as the product's first stage (statistic from the values the product loads, rows picked
     by a list), SwiGLU or the residual sum as its last."""
     from paged_llm_rs_amd import kernels
@@ -231,7 +231,7 @@ def test_gemm_skinny_with_the_norm_before_and_the_residual_after(n, N, K, gain_d
     eps = 1e-5
     stream = torch.randn(n + 3, K, device=DEV) * 3.0
     stream[0] *= 50.0                                         # rows of very different size: the statistic is a row's own
-    gain = (1 + 0.3 * torch.randn(K, device=DEV)).to(gain_dtype)
+    gain = 1 + 0.3 * torch.randn(K, device=DEV)
     w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
 
     def normed(rows):
@@ -248,7 +248,7 @@ def test_gemm_skinny_with_the_norm_before_and_the_residual_after(n, N, K, gain_d
     assert rel(got, normed(picked) @ w.double().T) < 1e-2
     if N % 2 == 0:
         g, u = want[:, :N // 2], want[:, N // 2:]
-        got = kernels.gemm_skinny(stream[:n].contiguous(), w, torch.float32, swiglu=True, norm_gain=gain, eps=eps)
+        got = kernels.gemm_skinny(stream[:n].contiguous(), w, swiglu=True, norm_gain=gain, eps=eps)
         assert rel(got, torch.nn.functional.silu(g) * u) < 1e-2
     # the residual sum: every element of the stream takes its own column's product, once
     x = torch.randn(n, K, device=DEV).to(torch.bfloat16)
