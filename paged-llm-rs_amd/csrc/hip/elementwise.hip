@@ -188,6 +188,124 @@ __global__ void qk_norm_rope_kv_write_kernel(
     }
 }
 
+// The same for the common case that the rotated width is a multiple of 16: a lane holds eight
+// consecutive elements of a head (one 16-byte load in bfloat16), d/8 lanes a head, so a wave works
+// on several heads at once and the partner of an element in the rotation lies whole in another
+// lane, d/16 lanes away.  A workgroup of four waves takes 4 * (64 / (d/8)) heads of one token.
+template <typename T>
+struct qk_vec;
+template <>
+struct qk_vec<bf16_t> {
+    static __device__ __forceinline__ void load(const bf16_t* p, float* out) {
+        struct __attribute__((aligned(16))) raw_t { uint32_t v[4]; };
+        const raw_t raw = *reinterpret_cast<const raw_t*>(p);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            out[2 * e] = __uint_as_float(raw.v[e] << 16);
+            out[2 * e + 1] = __uint_as_float(raw.v[e] & 0xffff0000u);
+        }
+    }
+    static __device__ __forceinline__ void store(bf16_t* p, const float* in) {
+        struct __attribute__((aligned(16))) raw_t { uint32_t v[4]; };
+        raw_t raw;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            raw.v[e] = static_cast<uint32_t>(bf16_bits_from_float(in[2 * e])) |
+                       (static_cast<uint32_t>(bf16_bits_from_float(in[2 * e + 1])) << 16);
+        *reinterpret_cast<raw_t*>(p) = raw;
+    }
+};
+template <>
+struct qk_vec<float> {
+    struct __attribute__((aligned(16))) raw_t { float v[4]; };
+    static __device__ __forceinline__ void load(const float* p, float* out) {
+        const raw_t a = *reinterpret_cast<const raw_t*>(p), b = *reinterpret_cast<const raw_t*>(p + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            out[e] = a.v[e];
+            out[4 + e] = b.v[e];
+        }
+    }
+    static __device__ __forceinline__ void store(float* p, const float* in) {
+        raw_t a, b;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            a.v[e] = in[e];
+            b.v[e] = in[4 + e];
+        }
+        *reinterpret_cast<raw_t*>(p) = a;
+        *reinterpret_cast<raw_t*>(p + 4) = b;
+    }
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+qk_norm_rope_kv_write_wide_kernel(
+    T* __restrict__ qkv, const void* __restrict__ q_gain, const void* __restrict__ k_gain,
+    int gain_dtype, float eps, const float* __restrict__ cos_table,
+    const float* __restrict__ sin_table, int rot, const int* __restrict__ positions,
+    const int* __restrict__ seq_of, const int* __restrict__ block_table, int max_blocks,
+    int block_size, T* __restrict__ k_pool, T* __restrict__ v_pool, int nq, int nkv, int d, int heads) {
+    const int t = blockIdx.x;
+    const int lane = threadIdx.x % PL_WAVE;
+    const int wave = threadIdx.x / PL_WAVE;
+    const int pos = positions[t];
+    if (pos < 0) return;
+
+    const int lph = d / 8;                  // lanes a head
+    const int hpw = PL_WAVE / lph;          // heads a wave
+    const int hw = lane / lph, chunk = lane - hw * lph;
+    const int h = (blockIdx.y * 4 + wave) * hpw + hw;
+    const bool active = hw < hpw && h < heads;
+    const int hh = active ? h : 0;
+    const bool is_q = hh < nq;
+    const bool is_k = !is_q && hh < nq + nkv;
+
+    const int row_width = (nq + 2 * nkv) * d;
+    T* src = qkv + static_cast<size_t>(t) * row_width + static_cast<size_t>(hh) * d + chunk * 8;
+    const int blk = block_table[static_cast<size_t>(seq_of[t]) * max_blocks + pos / block_size];
+    const size_t slot = static_cast<size_t>(blk < 0 ? 0 : blk) * block_size + pos % block_size;
+    T* dst = src;
+    if (!is_q) {
+        const int kvh = is_k ? hh - nq : hh - nq - nkv;
+        dst = (is_k ? k_pool : v_pool) + (slot * nkv + kvh) * d + chunk * 8;
+    }
+    const bool writes = active && (is_q || blk >= 0);   // never write through a hole in the table
+
+    float x[8];
+    qk_vec<T>::load(src, x);
+    const bool plain_copy = !is_q && !is_k;            // v
+    const void* gain = is_q ? q_gain : k_gain;
+
+    // the sum of squares over the lanes of the head (every lane takes part in the exchange)
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss = fmaf(x[e], x[e], ss);
+    float total = 0.f;
+    const int base = hw * lph;
+    for (int j = 0; j < lph; ++j) total += __shfl(ss, min(base + j, PL_WAVE - 1), PL_WAVE);
+    if (gain && !plain_copy) {
+        const float denom = sqrtf(total / static_cast<float>(d) + eps);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = x[e] / denom * load_as_float(gain, gain_dtype, chunk * 8 + e);
+    }
+    // the partner in the rotation: the element rot/2 further on, or back
+    const int half = rot / 2, hc = half / 8;
+    const bool low = chunk < hc;
+    const int partner = min(max(lane + (low ? hc : -hc), 0), PL_WAVE - 1);
+    float px[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) px[e] = __shfl(x[e], partner, PL_WAVE);
+    if (cos_table && !plain_copy && chunk * 8 < rot) {
+        const int at = (low ? chunk : chunk - hc) * 8;
+        const float* c = cos_table + static_cast<size_t>(pos) * half + at;
+        const float* s = sin_table + static_cast<size_t>(pos) * half + at;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = low ? x[e] * c[e] - px[e] * s[e] : x[e] * c[e] + px[e] * s[e];
+    }
+    if (writes) qk_vec<T>::store(dst, x);
+}
+
 extern "C" int pl_qk_norm_rope_kv_write(
     void* qkv, const void* q_gain, const void* k_gain, int gain_dtype, float eps,
     const float* cos_table, const float* sin_table, int rot, const int* positions,
@@ -201,7 +319,24 @@ extern "C" int pl_qk_norm_rope_kv_write(
     PL_REQUIRE((q_gain == nullptr) == (k_gain == nullptr), "qk_norm_rope: one of the two gains is missing");
     if (n <= 0) return 0;
     // Without the cache write (a layer that reads another layer's pages) only the query heads run.
-    dim3 grid(n, write_kv ? nq + 2 * nkv : nq);
+    const int heads = write_kv ? nq + 2 * nkv : nq;
+    if (rot % 16 == 0) {
+        const int per_group = 4 * (PL_WAVE / (d / 8));
+        dim3 wide(n, pl_ceil_div(heads, per_group));
+        if (dtype == PL_DTYPE_F32)
+            qk_norm_rope_kv_write_wide_kernel<float><<<wide, 256, 0, stream>>>(
+                static_cast<float*>(qkv), q_gain, k_gain, gain_dtype, eps, cos_table, sin_table, rot, positions, seq_of,
+                block_table, max_blocks, block_size, static_cast<float*>(k_pool), static_cast<float*>(v_pool), nq, nkv, d, heads);
+        else if (dtype == PL_DTYPE_BF16)
+            qk_norm_rope_kv_write_wide_kernel<bf16_t><<<wide, 256, 0, stream>>>(
+                static_cast<bf16_t*>(qkv), q_gain, k_gain, gain_dtype, eps, cos_table, sin_table, rot, positions, seq_of,
+                block_table, max_blocks, block_size, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), nq, nkv, d, heads);
+        else
+            PL_REQUIRE(false, "qk_norm_rope: dtype code %d", dtype);
+        PL_CHECK_LAUNCH("qk_norm_rope_kv_write");
+        return 0;
+    }
+    dim3 grid(n, heads);
     if (dtype == PL_DTYPE_F32)
         qk_norm_rope_kv_write_kernel<float><<<grid, PL_WAVE, 0, stream>>>(
             static_cast<float*>(qkv), q_gain, k_gain, gain_dtype, eps, cos_table, sin_table, rot, positions, seq_of,
