@@ -260,11 +260,14 @@ def set_attention(mode: str) -> None:
 
 
 def decode_splits(tokens: int, nq: int, nkv: int, max_ctx: int) -> int:
-    """How many stretches the context is cut into, so that a launch fills the chip:
-    about a thousand workgroups, each with at least 128 keys."""
+    """How many stretches the context is cut into, so that a launch fills the chip: none when the
+    tokens and heads alone give two workgroups a compute unit, else up to about a thousand
+    workgroups, each with at least 128 keys (one round of loads)."""
     g = nq // nkv
     gt = 8 if g >= 8 else (4 if g > 2 else g)
     base = max(tokens * nkv * ((g + gt - 1) // gt), 1)
+    if base >= 512:
+        return 1
     return max(1, min((1024 + base - 1) // base, (max_ctx + 127) // 128, 64))
 
 
@@ -397,6 +400,11 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
 
 def skinny_applies(x: torch.Tensor) -> bool:
     return x.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_ROWS and x.shape[1] % 8 == 0
+
+
+# A product with more columns than this walks its column tiles in a loop; the norm as its first stage
+# then costs the registers that keep enough waves resident, and a norm kernel of its own is cheaper.
+FUSED_NORM_MAX_COLUMNS = 32768
 
 
 def fused_norm_applies(rows_out: int, width: int, weight: torch.Tensor) -> bool:

@@ -36,7 +36,8 @@ class Linear:
             if x.width != self.in_features:
                 raise TensorError(f"a linear of {self.in_features} inputs given a stream of width {x.width}")
             if (getattr(x.norm, "fuses_into_product", False) and add_into is None
-                    and kernels.fused_norm_applies(x.num_rows, self.in_features, self.weight)):
+                    and kernels.fused_norm_applies(x.num_rows, self.in_features, self.weight)
+                    and self.out_features <= kernels.FUSED_NORM_MAX_COLUMNS):
                 return kernels.gemm_skinny(x.resid, self.weight, out_dtype or x.out_dtype, swiglu=swiglu,
                                            norm_gain=x.norm.gain32, eps=x.norm.eps, rows=x.rows)
             x = x.materialize()
