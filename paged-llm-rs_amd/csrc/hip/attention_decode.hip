@@ -39,6 +39,71 @@ __device__ __forceinline__ float group_sum(float v) {
     return v;
 }
 
+// What the kernel needs to normalise and rotate queries and the new key itself (a step in which every
+// request brings one token): then no kernel of its own runs for that before attention.
+struct ad_fuse_t {
+    const void* q_gain;       // per-head norm gains, or null
+    const void* k_gain;
+    int gain_dtype;
+    float eps;
+    const float* cos_table;   // [max_pos, rot/2], or null
+    const float* sin_table;
+    int rot;                  // a multiple of 16
+    int mode;                 // 0: q, k and v are ready; 1: q is raw; 2: q is raw, and the token's key and value
+                              //    are taken raw from its row, used, and written into the cache
+};
+
+__device__ __forceinline__ void ad_load_gain8(const void* gain, int dtype, int at, float* out) {
+    if (dtype == PL_DTYPE_F32) {
+        struct __attribute__((aligned(16))) f4 { float v[4]; };
+        const f4 a = *reinterpret_cast<const f4*>(static_cast<const float*>(gain) + at);
+        const f4 b = *reinterpret_cast<const f4*>(static_cast<const float*>(gain) + at + 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            out[i] = a.v[i];
+            out[4 + i] = b.v[i];
+        }
+    } else {
+        unpack8(*reinterpret_cast<const u32x4*>(static_cast<const bf16_t*>(gain) + at), out);
+    }
+}
+
+// One head spread over LPK lanes, eight elements a lane: RMSNorm over the head, rotation by the
+// token's position (the partner of an element lies rot/16 lanes away), rounding to bfloat16 as the
+// stand-alone kernel stores it.  Every lane of the wave takes part in the exchanges.
+template <int LPK>
+__device__ __forceinline__ void ad_norm_rope8(float* x, const void* gain, const ad_fuse_t& f, int d, int dl, int pos) {
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ss = fmaf(x[i], x[i], ss);
+    ss = group_sum<LPK>(ss);
+    const int at = min(dl * 8, d - 8);
+    if (gain) {
+        float gn[8];
+        ad_load_gain8(gain, f.gain_dtype, at, gn);
+        const float denom = sqrtf(ss / static_cast<float>(d) + f.eps);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = x[i] / denom * gn[i];
+    }
+    const int half = f.rot / 2, hc = half / 8;
+    const bool low = dl < hc;
+    const int lane = threadIdx.x % PL_WAVE;
+    const int partner = min(max(lane + (low ? hc : -hc), 0), PL_WAVE - 1);
+    float px[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) px[i] = __shfl(x[i], partner, PL_WAVE);
+    if (f.cos_table && dl * 8 < f.rot) {
+        const int ta = (low ? dl : dl - hc) * 8;
+        float c[8], s[8];
+        ad_load_gain8(f.cos_table + static_cast<size_t>(pos) * half, PL_DTYPE_F32, ta, c);
+        ad_load_gain8(f.sin_table + static_cast<size_t>(pos) * half, PL_DTYPE_F32, ta, s);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = low ? x[i] * c[i] - px[i] * s[i] : x[i] * c[i] + px[i] * s[i];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = to_float(from_float<bf16_t>(x[i]));
+}
+
 // LPK: lanes a key (a power of two, LPK*8 >= d).  GT: query heads a workgroup serves.
 // U: keys a lane group asks for at once.
 template <int LPK, int GT, int U>
@@ -48,8 +113,8 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
                               const int* __restrict__ positions, const int* __restrict__ seq_of,
                               const int* __restrict__ q_len, int short_limit,
                               const int* __restrict__ block_table, int max_blocks, int block_size,
-                              const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool, int nq,
-                              int nkv, int d, float scale_log2e, int window, int splits, int tiles) {
+                              bf16_t* __restrict__ k_pool, bf16_t* __restrict__ v_pool, int nq,
+                              int nkv, int d, float scale_log2e, int window, int splits, int tiles, ad_fuse_t fuse) {
     constexpr int KPW = PL_WAVE / LPK;  // keys a wave handles with one load
     constexpr int GROUPS = AD_WAVES * KPW;
     extern __shared__ float lds[];  // [GROUPS][GT][2] running max and sum, then [GROUPS][GT][d] accumulators
@@ -75,11 +140,12 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
 
     // the stretch of keys of this split, in whole rounds of the workgroup
     const int first = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
-    const int total = pos + 1 - first;
+    const int limit = fuse.mode == 2 ? pos : pos + 1;   // the token's own key is not in the cache yet
+    const int total = max(limit - first, 0);
     constexpr int ROUND = AD_WAVES * KPW * U;
     const int per_split = pl_ceil_div(pl_ceil_div(total, splits), ROUND) * ROUND;
     const int s_begin = first + split * per_split;
-    const int s_end = min(pos + 1, s_begin + per_split);
+    const int s_end = min(limit, s_begin + per_split);
 
     float qf[GT][8];
 #pragma unroll
@@ -88,12 +154,13 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
             const u32x4 raw = *reinterpret_cast<const u32x4*>(q + static_cast<size_t>(t) * q_stride +
                                                               static_cast<size_t>(h0 + hq) * d + dl * 8);
             unpack8(raw, qf[hq]);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) qf[hq][i] *= scale_log2e;
         } else {
 #pragma unroll
             for (int i = 0; i < 8; ++i) qf[hq][i] = 0.f;
         }
+        if (fuse.mode != 0) ad_norm_rope8<LPK>(qf[hq], fuse.q_gain, fuse, d, dl, pos);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) qf[hq][i] *= scale_log2e;
     }
 
     float m[GT], l[GT], acc[GT][8];
@@ -193,6 +260,56 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
         }
     }
 
+    // The token's own key and value, raw in its row: normalised and rotated here, taken into the
+    // running state of one lane group of the last split, and written into the cache by one workgroup.
+    if (fuse.mode == 2 && split == splits - 1 && wave == 0) {
+        const bf16_t* row = q + static_cast<size_t>(t) * q_stride;
+        const int at = min(dl * 8, d - 8);
+        const u32x4 kraw = *reinterpret_cast<const u32x4*>(row + static_cast<size_t>(nq + kvh) * d + at);
+        const u32x4 vraw = *reinterpret_cast<const u32x4*>(row + static_cast<size_t>(nq + nkv + kvh) * d + at);
+        float kf[8], vf[8];
+        unpack8(kraw, kf);
+        unpack8(vraw, vf);
+        if (!d_ok) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) kf[i] = vf[i] = 0.f;
+        }
+        ad_norm_rope8<LPK>(kf, fuse.k_gain, fuse, d, dl, pos);
+        int bi = static_cast<int>(__umulhi(static_cast<uint32_t>(pos), bs_magic));
+        int w = pos - bi * block_size;
+        if (w >= block_size) {
+            bi += 1;
+            w -= block_size;
+        }
+        const int page = table[bi];
+        if (tile == 0 && sub == 0 && d_ok && page >= 0) {
+            const size_t off = (static_cast<size_t>(page) * block_size + w) * row_stride + static_cast<size_t>(kvh) * d + dl * 8;
+            u32x4 packed;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                packed.v[i] = static_cast<uint32_t>(bf16_bits_from_float(kf[2 * i])) |
+                              (static_cast<uint32_t>(bf16_bits_from_float(kf[2 * i + 1])) << 16);
+            *reinterpret_cast<u32x4*>(k_pool + off) = packed;
+            *reinterpret_cast<u32x4*>(v_pool + off) = vraw;
+        }
+#pragma unroll
+        for (int hq = 0; hq < GT; ++hq) {
+            float dot = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) dot = fmaf(qf[hq][i], kf[i], dot);
+            dot = group_sum<LPK>(dot);
+            const float sc = (sub == 0 && page >= 0) ? dot : -INFINITY;
+            const float m_new = fmaxf(m[hq], sc);
+            if (m_new == -INFINITY) continue;
+            const float corr = exp2f(m[hq] - m_new);
+            const float p = exp2f(sc - m_new);
+            l[hq] = l[hq] * corr + p;
+            m[hq] = m_new;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[hq][i] = fmaf(p, vf[i], acc[hq][i] * corr);
+        }
+    }
+
     // merge the lane groups of the four waves
     float* ml = lds;                              // [GROUPS][GT][2]
     float* accs = lds + GROUPS * GT * 2;          // [GROUPS][GT][d]
@@ -282,9 +399,9 @@ paged_attention_merge_kernel(const float* __restrict__ part_acc, const float* __
 template <int LPK, int GT>
 static int launch_decode(const void* q, int q_stride, void* out, float* part_acc, float* part_ml,
                          const int* positions, const int* seq_of, const int* q_len, int short_limit,
-                         const int* block_table, int max_blocks, int block_size, const void* k_pool,
-                         const void* v_pool, int n, int nq, int nkv, int d, float scale, int window, int splits,
-                         hipStream_t stream) {
+                         const int* block_table, int max_blocks, int block_size, void* k_pool,
+                         void* v_pool, int n, int nq, int nkv, int d, float scale, int window, int splits,
+                         const ad_fuse_t& fuse, hipStream_t stream) {
     constexpr int KPW = PL_WAVE / LPK;
     constexpr int GROUPS = AD_WAVES * KPW;
     constexpr int U = GT <= 2 ? 8 : 4;   // fewer heads a workgroup leave registers for more keys in flight
@@ -301,8 +418,8 @@ static int launch_decode(const void* q, int q_stride, void* out, float* part_acc
     PL_REQUIRE(n <= 65535 && splits <= 65535, "decode attention: %d tokens or %d splits are more than one launch covers", n, splits);
     paged_attention_decode_kernel<LPK, GT, U><<<grid, 256, lds_bytes, stream>>>(
         static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), part_acc, part_ml, positions, seq_of,
-        q_len, short_limit, block_table, max_blocks, block_size, static_cast<const bf16_t*>(k_pool),
-        static_cast<const bf16_t*>(v_pool), nq, nkv, d, scale * 1.4426950408889634f, window, splits, tiles);
+        q_len, short_limit, block_table, max_blocks, block_size, static_cast<bf16_t*>(k_pool),
+        static_cast<bf16_t*>(v_pool), nq, nkv, d, scale * 1.4426950408889634f, window, splits, tiles, fuse);
     PL_CHECK_LAUNCH("paged_attention_decode");
     if (splits > 1) {
         const int mgrid = pl_ceil_div(n * nq * d, 256);
@@ -323,13 +440,13 @@ static int launch_decode(const void* q, int q_stride, void* out, float* part_acc
 template <int LPK>
 static int dispatch_gt(int gt, const void* q, int q_stride, void* out, float* part_acc, float* part_ml,
                        const int* positions, const int* seq_of, const int* q_len, int short_limit,
-                       const int* block_table, int max_blocks, int block_size, const void* k_pool,
-                       const void* v_pool, int n, int nq, int nkv, int d, float scale, int window, int splits,
-                       hipStream_t stream) {
+                       const int* block_table, int max_blocks, int block_size, void* k_pool,
+                       void* v_pool, int n, int nq, int nkv, int d, float scale, int window, int splits,
+                       const ad_fuse_t& fuse, hipStream_t stream) {
 #define AD_CALL(G)                                                                                              \
     return launch_decode<LPK, G>(q, q_stride, out, part_acc, part_ml, positions, seq_of, q_len, short_limit,   \
                                  block_table, max_blocks, block_size, k_pool, v_pool, n, nq, nkv, d, scale,    \
-                                 window, splits, stream)
+                                 window, splits, fuse, stream)
     switch (gt) {
         case 1: AD_CALL(1);
         case 2: AD_CALL(2);
@@ -341,17 +458,33 @@ static int dispatch_gt(int gt, const void* q, int q_stride, void* out, float* pa
 
 // bfloat16 only.  With splits > 1 the workspace needs n*nq*splits*d floats (part_acc) and n*nq*splits*2 (part_ml).
 // q_len (may be null) and short_limit leave the tokens of requests with q_len >= short_limit to the tiled kernel.
+// fuse_mode 0: the rows of q are ready and the cache holds every key up to each token's own.  1: the rows of q are
+// the raw projection and are normalised (gains, eps) and rotated (tables, rot a multiple of 16) here.  2: as 1, and
+// each token's key and value are taken raw from its row [q | k | v], used, and written into the cache; every
+// request then has to bring exactly one token.
 extern "C" int pl_paged_attention_decode(const void* q, int q_stride, void* out, float* part_acc, float* part_ml,
                                          const int* positions, const int* seq_of, const int* q_len, int short_limit,
-                                         const int* block_table, int max_blocks, int block_size, const void* k_pool,
-                                         const void* v_pool, int n, int nq, int nkv, int d, float scale, int window,
-                                         int splits, hipStream_t stream) {
+                                         const int* block_table, int max_blocks, int block_size, void* k_pool,
+                                         void* v_pool, int n, int nq, int nkv, int d, float scale, int window,
+                                         int splits, int fuse_mode, const void* q_gain, const void* k_gain,
+                                         int gain_dtype, float eps, const float* cos_table, const float* sin_table,
+                                         int rot, hipStream_t stream) {
     PL_REQUIRE(d > 0 && d <= 256 && d % 16 == 0, "decode attention: head size %d, which has to be a multiple of 16 up to 256", d);
     PL_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "decode attention: %d query heads over %d key heads", nq, nkv);
     PL_REQUIRE(block_size > 0 && max_blocks > 0 && q_stride >= nq * d && q_stride % 8 == 0 && window >= 0 && splits >= 1 && splits <= AD_MAX_SPLITS,
                "decode attention: block size %d, %d blocks a row, query stride %d, window %d, %d splits", block_size,
                max_blocks, q_stride, window, splits);
     PL_REQUIRE(splits == 1 || (part_acc && part_ml), "decode attention: %d splits without a workspace", splits);
+    PL_REQUIRE(fuse_mode >= 0 && fuse_mode <= 2, "decode attention: fuse mode %d", fuse_mode);
+    if (fuse_mode != 0) {
+        PL_REQUIRE(rot >= 0 && rot <= d && rot % 16 == 0, "decode attention: a rotated width of %d of a head of %d is not fused", rot, d);
+        PL_REQUIRE((q_gain == nullptr) == (k_gain == nullptr), "decode attention: one of the two gains is missing");
+        PL_REQUIRE(!q_gain || gain_dtype == PL_DTYPE_F32 || gain_dtype == PL_DTYPE_BF16, "decode attention: gain dtype code %d", gain_dtype);
+        PL_REQUIRE((cos_table == nullptr) == (sin_table == nullptr) && (cos_table || rot == 0), "decode attention: rotation tables");
+        PL_REQUIRE(fuse_mode != 2 || (q_len == nullptr && q_stride >= (nq + 2 * nkv) * d),
+                   "decode attention: the fused cache write is for steps of one token a request over rows [q | k | v]");
+    }
+    const ad_fuse_t fuse{q_gain, k_gain, gain_dtype, eps, cos_table, sin_table, rot, fuse_mode};
     if (n <= 0) return 0;
     const int g = nq / nkv;
     const int gt = g >= 8 ? 8 : (g > 2 ? 4 : g);   // 1, 2, 4 or 8 query heads a workgroup; the rest are more tiles
@@ -359,7 +492,7 @@ extern "C" int pl_paged_attention_decode(const void* q, int q_stride, void* out,
 #define AD_LPK(L)                                                                                                  \
     return dispatch_gt<L>(gt, q, q_stride, out, part_acc, part_ml, positions, seq_of, q_len, short_limit,        \
                           block_table, max_blocks, block_size, k_pool, v_pool, n, nq, nkv, d, scale, window,      \
-                          splits, stream)
+                          splits, fuse, stream)
     if (chunks <= 2) AD_LPK(2);
     if (chunks <= 4) AD_LPK(4);
     if (chunks <= 8) AD_LPK(8);

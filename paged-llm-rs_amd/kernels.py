@@ -36,7 +36,8 @@ def _signatures(lib) -> None:
         "pl_paged_attention_plain": [p, i, p, p, p, p, i, i, p, p, i, i, i, i, f, i, i, p],
         "pl_argmax": [p, p, p, p, i, i, p],
         "pl_gemm_skinny": [p, p, p, p, f, p, i, i, i, i, i, p],
-        "pl_paged_attention_decode": [p, i, p, p, p, p, p, p, i, p, i, i, p, p, i, i, i, i, f, i, i, p],
+        "pl_paged_attention_decode": [p, i, p, p, p, p, p, p, i, p, i, i, p, p, i, i, i, i, f, i, i,
+                                      i, p, p, i, f, p, p, i, p],
         "pl_paged_attention_prefill": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, p],
     }
     for name, argtypes in table.items():
@@ -275,8 +276,10 @@ def paged_attention_decode(q: torch.Tensor, q_row_stride: int, out: torch.Tensor
                            seq_of: torch.Tensor, block_table: torch.Tensor, block_size: int,
                            k_pool: torch.Tensor, v_pool: torch.Tensor, nq: int, nkv: int, d: int, scale: float,
                            window: int = 0, splits: int = 1, q_len: torch.Tensor | None = None,
-                           short_limit: int = 0) -> torch.Tensor:
-    """bfloat16 attention of single tokens over their requests' pages, split along the context."""
+                           short_limit: int = 0, fuse: "QkFusion | None" = None) -> torch.Tensor:
+    """bfloat16 attention of single tokens over their requests' pages, split along the context.
+    With ``fuse`` the rows of ``q`` are the raw projection [q | k | v]: queries (and, when it says so, each
+    token's key) are normalised and rotated inside the kernel, and key and value are written into the pages."""
     n = positions.numel()
     _need(q, "query buffer", None, torch.bfloat16)
     if q.dim() != 2 or q.shape[0] != n or q.shape[1] != q_row_stride or q_row_stride < nq * d:
@@ -295,11 +298,40 @@ def paged_attention_decode(q: torch.Tensor, q_row_stride: int, out: torch.Tensor
     if splits > 1:
         part_acc = torch.empty((n * nq * splits * d,), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((n * nq * splits * 2,), dtype=torch.float32, device=q.device)
+    mode, q_gain, k_gain, gain_code, eps, cos, sin, rot = 0, None, None, F32, 0.0, None, None, 0
+    if fuse is not None:
+        if q_len is not None:
+            raise TensorError("the fused norm, rotation and cache write are for steps of one token a request")
+        mode = 2 if fuse.write_kv else 1
+        q_gain, k_gain, eps, cos, sin, rot = fuse.q_gain, fuse.k_gain, fuse.eps, fuse.cos, fuse.sin, fuse.rot
+        if q_gain is not None:
+            _need(q_gain, "query norm gain", (d,))
+            _need(k_gain, "key norm gain", (d,), q_gain.dtype)
+            gain_code = _code(q_gain, "query norm gain")
+        if cos is not None:
+            _need(cos, "cosine table", None, torch.float32)
+            _need(sin, "sine table", tuple(cos.shape), torch.float32)
+            if cos.dim() != 2 or cos.shape[1] != rot // 2:
+                raise TensorError(f"rotary tables have shape {tuple(cos.shape)}, expected [positions, {rot // 2}]")
+        if mode == 2 and q_row_stride != (nq + 2 * nkv) * d:
+            raise TensorError(f"rows of {q_row_stride} values are not [q | k | v] of {nq}+2*{nkv} heads of {d}")
     _check(library().pl_paged_attention_decode(
         q.data_ptr(), q_row_stride, out.data_ptr(), _ptr(part_acc), _ptr(part_ml), positions.data_ptr(),
         seq_of.data_ptr(), _ptr(q_len), int(short_limit), block_table.data_ptr(), block_table.shape[1], block_size,
-        k_pool.data_ptr(), v_pool.data_ptr(), n, nq, nkv, d, float(scale), int(window or 0), int(splits), _stream()))
+        k_pool.data_ptr(), v_pool.data_ptr(), n, nq, nkv, d, float(scale), int(window or 0), int(splits),
+        mode, _ptr(q_gain), _ptr(k_gain), gain_code, float(eps), _ptr(cos), _ptr(sin), int(rot), _stream()))
     return out
+
+
+class QkFusion:
+    """What turns a raw projection row into queries and keys: the per-head norm's gains and eps, the
+    rotation's tables and width, and whether key and value go into the pages."""
+
+    __slots__ = ("q_gain", "k_gain", "eps", "cos", "sin", "rot", "write_kv")
+
+    def __init__(self, q_gain, k_gain, eps: float, cos, sin, rot: int, write_kv: bool):
+        self.q_gain, self.k_gain, self.eps, self.cos, self.sin = q_gain, k_gain, eps, cos, sin
+        self.rot, self.write_kv = rot, write_kv
 
 
 def paged_attention_prefill(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, q_start: torch.Tensor,
@@ -330,6 +362,24 @@ def paged_attention_prefill(q: torch.Tensor, q_row_stride: int, out: torch.Tenso
         int(short_limit), S, int(max_q_len), block_table.data_ptr(), block_table.shape[1], block_size,
         k_pool.data_ptr(), v_pool.data_ptr(), nq, nkv, d, float(scale), int(window or 0), _stream()))
     return out
+
+
+def attention_step(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nkv: int, d: int, scale: float,
+                   window: int, prepare: QkFusion) -> torch.Tensor:
+    """Everything between the fused q/k/v projection and the output projection for the tokens of a step:
+    per-head norm and rotation of q and k, the write of k and v into the pages, attention.  A step in
+    which every request brings one token (in bfloat16) does all of it in the attention kernel;
+    any other step runs the stand-alone kernel for the first three and then attention."""
+    if (qkv.dtype == torch.bfloat16 and _attention_mode == "kernel" and batch.max_q_len == 1
+            and prepare.rot % 16 == 0):
+        splits = decode_splits(batch.num_tokens, nq, nkv, batch.max_ctx_len)
+        return paged_attention_decode(qkv, qkv.shape[1], out, batch.positions, batch.seq_of, kv.block_table,
+                                      kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window, splits,
+                                      fuse=prepare)
+    qk_norm_rope_kv_write(qkv, prepare.q_gain, prepare.k_gain, prepare.eps, prepare.cos, prepare.sin, prepare.rot,
+                          batch.positions, batch.seq_of, kv.block_table, kv.block_size, kv.k_pool, kv.v_pool,
+                          nq, nkv, d, write_kv=prepare.write_kv)
+    return paged_attention(qkv, out, batch, kv, nq, nkv, d, scale, window)
 
 
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nkv: int, d: int,

@@ -75,12 +75,9 @@ class PagedAttention:
         cos = self.rotary.cos if self.rotary is not None else None
         sin = self.rotary.sin if self.rotary is not None else None
         rot = self.rotary.dim if self.rotary is not None else 0
-        kernels.qk_norm_rope_kv_write(
-            qkv, self.q_gain, self.k_gain, self.eps, cos, sin, rot, batch.positions, batch.seq_of,
-            kv.block_table, kv.block_size, kv.k_pool, kv.v_pool, self.nq, self.nkv, self.d,
-            write_kv=ctx.writes_cache)
+        prepare = kernels.QkFusion(self.q_gain, self.k_gain, self.eps, cos, sin, rot, ctx.writes_cache)
         out = torch.empty((qkv.shape[0], self.nq * self.d), dtype=qkv.dtype, device=qkv.device)
-        kernels.paged_attention(qkv, out, batch, kv, self.nq, self.nkv, self.d, self.scale, self.window)
+        kernels.attention_step(qkv, out, batch, kv, self.nq, self.nkv, self.d, self.scale, self.window, prepare)
         return self.o_proj.forward(out, add_into=ctx.residual)
 
 

@@ -388,6 +388,47 @@ def test_a_far_key_among_hundreds_is_found(kernel):
         assert hit == inside, f"key {target} of {ctx} with window {window}: found {hit}, visible {inside}"
 
 
+@pytest.mark.parametrize("nq,nkv,d,bs,ctx_lens,window,rot,norm", [
+    (16, 8, 128, 16, [513, 40, 1], 0, 128, True), (6, 1, 32, 8, [70, 9], 0, 32, True), (6, 2, 48, 16, [100, 17, 64], 0, 32, False),
+    (4, 2, 64, 16, [300, 31], 48, 64, True), (32, 2, 128, 16, [300], 0, 128, True), (3, 3, 80, 2, [37, 12], 0, 0, True)])
+@pytest.mark.parametrize("splits", [1, 3])
+def test_decode_attention_that_prepares_its_own_queries_and_keys(nq, nkv, d, bs, ctx_lens, window, rot, norm, splits):
+    """One token a request: the norm, the rotation and the cache write inside the attention kernel give what
+    the stand-alone kernel followed by attention gives, in the output and in the pages."""
+    from paged_llm_rs_amd import kernels
+
+    dtype = torch.bfloat16
+    bt, k_pool, v_pool, _, _ = build_paged(nkv, d, bs, ctx_lens, dtype, seed=d + bs + rot)
+    n = len(ctx_lens) + 1
+    stride = (nq + 2 * nkv) * d
+    raw = torch.randn(n, stride, device=DEV).to(dtype)
+    positions = torch.tensor([c - 1 for c in ctx_lens] + [-1], dtype=torch.int32, device=DEV)
+    seq_of = torch.tensor(list(range(len(ctx_lens))) + [0], dtype=torch.int32, device=DEV)
+    q_gain = (1 + 0.2 * torch.randn(d, device=DEV)).to(dtype) if norm else None
+    k_gain = (1 + 0.2 * torch.randn(d, device=DEV)).to(dtype) if norm else None
+    cos = sin = None
+    if rot:
+        angle = torch.arange(600, dtype=torch.float64)[:, None] * (1.0 / 10000 ** (torch.arange(rot // 2, dtype=torch.float64) * 2 / rot))
+        cos, sin = angle.cos().float().to(DEV), angle.sin().float().to(DEV)
+    scale = 1 / math.sqrt(d)
+    apart, k_a, v_a = raw.clone(), k_pool.clone(), v_pool.clone()
+    kernels.qk_norm_rope_kv_write(apart, q_gain, k_gain, 1e-5, cos, sin, rot, positions, seq_of, bt, bs, k_a, v_a, nq, nkv, d)
+    want = torch.full((n, nq * d), 7.0, dtype=dtype, device=DEV)
+    kernels.paged_attention_decode(apart, stride, want, positions, seq_of, bt, bs, k_a, v_a, nq, nkv, d, scale, window, splits)
+    got = torch.full((n, nq * d), 7.0, dtype=dtype, device=DEV)
+    k_b, v_b = k_pool.clone(), v_pool.clone()
+    kernels.paged_attention_decode(raw, stride, got, positions, seq_of, bt, bs, k_b, v_b, nq, nkv, d, scale, window, splits,
+                                   fuse=kernels.QkFusion(q_gain, k_gain, 1e-5, cos, sin, rot, True))
+    assert torch.equal(k_a, k_b) and torch.equal(v_a, v_b), "the same keys and values in the same places"
+    assert rel(got[:-1], want[:-1]) < 4e-3
+    assert bool((got[-1] == 7.0).all()), "a padding row is not written"
+    # queries only: a layer that reads pages another layer wrote
+    again = torch.full((n, nq * d), 7.0, dtype=dtype, device=DEV)
+    kernels.paged_attention_decode(raw, stride, again, positions, seq_of, bt, bs, k_a, v_a, nq, nkv, d, scale, window, splits,
+                                   fuse=kernels.QkFusion(q_gain, k_gain, 1e-5, cos, sin, rot, False))
+    assert rel(again[:-1], want[:-1]) < 4e-3
+
+
 PORTION_CASES = [
     # nq, nkv, d, block size, [(context length after the step, tokens of the step)], window
     (4, 2, 16, 4, [(40, 40), (70, 17), (5, 1)], 0),
