@@ -158,10 +158,19 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
 #pragma unroll
             for (int i = 0; i < 8; ++i) qf[hq][i] = 0.f;
         }
-        if (fuse.mode != 0) ad_norm_rope8<LPK>(qf[hq], fuse.q_gain, fuse, d, dl, pos);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) qf[hq][i] *= scale_log2e;
     }
+    // The queries are normalised, rotated and scaled once the first keys and values have been asked
+    // for, so that this work passes while they are on their way.
+    bool q_ready = false;
+    auto prepare_q = [&]() {
+#pragma unroll
+        for (int hq = 0; hq < GT; ++hq) {
+            if (fuse.mode != 0) ad_norm_rope8<LPK>(qf[hq], fuse.q_gain, fuse, d, dl, pos);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) qf[hq][i] *= scale_log2e;
+        }
+        q_ready = true;
+    };
 
     float m[GT], l[GT], acc[GT][8];
 #pragma unroll
@@ -218,6 +227,7 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
             }
         }
         lookup(base + ROUND);
+        if (!q_ready) prepare_q();
         float s[U][GT];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -262,6 +272,7 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
 
     // The token's own key and value, raw in its row: normalised and rotated here, taken into the
     // running state of one lane group of the last split, and written into the cache by one workgroup.
+    if (!q_ready) prepare_q();
     if (fuse.mode == 2 && split == splits - 1 && wave == 0) {
         const bf16_t* row = q + static_cast<size_t>(t) * q_stride;
         const int at = min(dl * 8, d - 8);
