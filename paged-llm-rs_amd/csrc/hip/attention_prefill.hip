@@ -28,7 +28,13 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 #ifndef AP_OCC
-#define AP_OCC 2  // waves a SIMD the registers are kept within
+#define AP_OCC 2  // waves a SIMD that the registers are kept within (the second launch bound counts waves a SIMD)
+#endif
+#ifndef AP_SMALL_KS
+#define AP_SMALL_KS 2
+#endif
+#ifndef AP_KS
+#define AP_KS 2    // waves a block of 32 tokens in the large tile
 #endif
 #define AP_BN 64   // keys a tile
 #define AP_KPAD 8  // padding of a row of keys in LDS, in elements
@@ -57,9 +63,13 @@ __device__ __forceinline__ uint32_t ap_pack2(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
 }
 
-// DT: the head is padded to 32*DT elements.  NW: waves a workgroup.
-template <int DT, int NW>
-__global__ void __launch_bounds__(64 * NW, AP_OCC * 4 / NW)
+// DT: the head is padded to 32*DT elements.  NW: blocks of 32 tokens a workgroup.  KS: waves a block
+// of tokens (1, or 2: then one wave takes the first 32 keys of every tile and the other the last 32,
+// each with a running state of its own, merged at the end; twice the waves overlap more of the
+// softmax with the products; heads of more than 128 elements have no registers for it).  A workgroup
+// has NW * KS waves.
+template <int DT, int NW, int KS>
+__global__ void __launch_bounds__(64 * NW * KS, DT <= 4 ? AP_OCC : 1)
 paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
                                const int* __restrict__ q_start, const int* __restrict__ q_len,
                                const int* __restrict__ ctx_len, int short_limit, int tiles_a_request,
@@ -69,7 +79,8 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
                                int window, int total_work) {
     constexpr int DP = 32 * DT;
     constexpr int BM = 32 * NW;
-    constexpr int NT = 64 * NW;
+    constexpr int NT = 64 * NW * KS;
+    constexpr int KT = 2 / KS;             // 32-key tiles of a 64-key tile a wave takes
     constexpr int KROW = DP + AP_KPAD;     // elements a row of Ks
     constexpr int VROW = AP_BN + AP_VPAD;  // elements a row of Vt
     extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
@@ -96,7 +107,9 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // the same for the whole wave: kept scalar
+    const int wave_id = __builtin_amdgcn_readfirstlane(tid >> 6);   // the same for the whole wave: kept scalar
+    const int wave = wave_id % NW;                               // which block of 32 tokens
+    const int kt0 = (wave_id / NW) * KT;                         // the wave's first 32-key tile of a 64-key tile
     const int r32 = lane & 31;
     const int h = lane >> 5;
     const int kvh = head / (nq / nkv);
@@ -231,32 +244,32 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         lookup(k0 + 2 * AP_BN);
 
         // a wave whose queries all stand before this tile, or that has no queries, has nothing to add
-        if (!wave_active || k0 > wave_last) continue;
-        if (window > 0 && k0 + AP_BN - 1 <= wave_first - window) continue;
+        if (!wave_active || k0 + 32 * kt0 > wave_last) continue;
+        if (window > 0 && k0 + 32 * (kt0 + KT) - 1 <= wave_first - window) continue;
 
         // scores, transposed: s[kt][4*j + i] is key k0 + 32*kt + 8*j + 4*h + i against query r32
-        f32x16 s[2];
+        f32x16 s[KT];
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
+        for (int kt = 0; kt < KT; ++kt) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) s[kt][r] = 0.f;
             ap_frag a[2 * DT];
 #pragma unroll
             for (int kk = 0; kk < 2 * DT; ++kk)
-                a[kk].raw = *reinterpret_cast<const ap_u32x4*>(Ks + (32 * kt + r32) * KROW + 16 * kk + 8 * h);
+                a[kk].raw = *reinterpret_cast<const ap_u32x4*>(Ks + (32 * (kt0 + kt) + r32) * KROW + 16 * kk + 8 * h);
 #pragma unroll
             for (int kk = 0; kk < 2 * DT; ++kk)
                 s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kk].vec, qf[kk].vec, s[kt], 0, 0, 0);
         }
         // Key k0 + c + 4*h, c a constant of the register, is seen by this lane's query iff c <= reach
         // (and c > reach - window).  Tiles that lie before every query of the wave need no test.
-        const bool edge = k0 + AP_BN - 1 > wave_first || window > 0;
-        const int reach = q_pos - k0 - 4 * h;
+        const bool edge = k0 + 32 * (kt0 + KT) - 1 > wave_first || window > 0;
+        const int reach = q_pos - k0 - 32 * kt0 - 4 * h;
         const int behind = window > 0 ? reach - window : -(1 << 30);
         float mx = -INFINITY;
         if (edge) {
 #pragma unroll
-            for (int kt = 0; kt < 2; ++kt)
+            for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int c = 32 * kt + 8 * (r >> 2) + (r & 3);
@@ -266,7 +279,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
                 }
         } else {
 #pragma unroll
-            for (int kt = 0; kt < 2; ++kt)
+            for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const float v = s[kt][r] * scale_log2e;
@@ -280,7 +293,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         const float corr = __builtin_amdgcn_exp2f(m - m_use);
         float psum = 0.f;
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
+        for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const float p = __builtin_amdgcn_exp2f(s[kt][r] - m_use);  // v_exp_f32: arguments are <= 0, tiny results may flush
@@ -297,13 +310,13 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         // O^T += V^T . P^T, sixteen keys a product: registers 8*half .. 8*half+7 of tile kt are the
         // keys 32*kt + 16*half + {4h..4h+3} and + 8 + {4h..4h+3}
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
+        for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
                 ap_frag b;
 #pragma unroll
                 for (int w = 0; w < 4; ++w) b.w[w] = ap_pack2(s[kt][8 * half + 2 * w], s[kt][8 * half + 2 * w + 1]);
-                const int key_off = 32 * kt + 16 * half + 4 * h;
+                const int key_off = 32 * (kt0 + kt) + 16 * half + 4 * h;
                 ap_frag a[DT];
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
@@ -317,8 +330,34 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
             }
     }
 
+    lsum += __shfl_xor(lsum, 32, PL_WAVE);
+    if (KS == 2) {
+        // The wave of the later keys hands its state to the wave of the earlier ones through LDS
+        // (the tiles are done with): out = (o0 2^(m0-M) + o1 2^(m1-M)) / (l0 2^(m0-M) + l1 2^(m1-M)).
+        float* hand = reinterpret_cast<float*>(lds) + static_cast<size_t>(wave) * (16 * DT + 2) * PL_WAVE;
+        __syncthreads();
+        if (kt0 != 0) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) hand[(dt * 16 + r) * PL_WAVE + lane] = o[dt][r];
+            hand[(16 * DT) * PL_WAVE + lane] = m;
+            hand[(16 * DT + 1) * PL_WAVE + lane] = lsum;
+        }
+        __syncthreads();
+        if (kt0 != 0) return;
+        const float m1 = hand[(16 * DT) * PL_WAVE + lane], l1 = hand[(16 * DT + 1) * PL_WAVE + lane];
+        const float big = fmaxf(m, m1);
+        const float use = big == -INFINITY ? 0.f : big;
+        const float w0 = __builtin_amdgcn_exp2f(m - use), w1 = __builtin_amdgcn_exp2f(m1 - use);
+        lsum = lsum * w0 + l1 * w1;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[dt][r] = o[dt][r] * w0 + hand[(dt * 16 + r) * PL_WAVE + lane] * w1;
+    }
     if (!q_ok) return;
-    const float total = lsum + __shfl_xor(lsum, 32, PL_WAVE);
+    const float total = lsum;
     const float inv = total > 0.f ? 1.f / total : 0.f;
     // o[dt][4*j + i] is element 32*dt + 8*j + 4*h + i of query r32
     bf16_t* orow = out + (static_cast<size_t>(row0 + wq) * nq + head) * d;
@@ -336,23 +375,25 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         }
 }
 
-template <int DT, int NW>
+template <int DT, int NW, int KS>
 static int launch_prefill(const void* q, int q_stride, void* out, const int* q_start, const int* q_len,
                           const int* ctx_len, int short_limit, int num_seqs, int max_q_len, const int* block_table,
                           int max_blocks, int block_size, const void* k_pool, const void* v_pool, int nq, int nkv,
                           int d, float scale, int window, hipStream_t stream) {
     constexpr int DP = 32 * DT;
     constexpr int BM = 32 * NW;
-    const size_t lds_bytes = (static_cast<size_t>(AP_BN) * (DP + AP_KPAD) + static_cast<size_t>(DP) * (AP_BN + AP_VPAD)) * 2;
+    const size_t tile_bytes = (static_cast<size_t>(AP_BN) * (DP + AP_KPAD) + static_cast<size_t>(DP) * (AP_BN + AP_VPAD)) * 2;
+    const size_t hand_bytes = KS == 2 ? static_cast<size_t>(NW) * (16 * DT + 2) * PL_WAVE * sizeof(float) : 0;
+    const size_t lds_bytes = tile_bytes > hand_bytes ? tile_bytes : hand_bytes;
     if (lds_bytes > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_prefill_kernel<DT, NW>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_prefill_kernel<DT, NW, KS>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
         PL_REQUIRE(e == hipSuccess, "prefill attention: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
     }
     const int tiles = pl_ceil_div(max_q_len, BM);
     const long long total = static_cast<long long>(tiles) * nq * num_seqs;
     PL_REQUIRE(total > 0 && total < (1ll << 30), "prefill attention: %lld workgroups", total);
-    paged_attention_prefill_kernel<DT, NW><<<static_cast<int>(total), 64 * NW, lds_bytes, stream>>>(
+    paged_attention_prefill_kernel<DT, NW, KS><<<static_cast<int>(total), 64 * NW * KS, lds_bytes, stream>>>(
         static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), q_start, q_len, ctx_len, short_limit, tiles,
         num_seqs, block_table, max_blocks, block_size, static_cast<const bf16_t*>(k_pool),
         static_cast<const bf16_t*>(v_pool), nq, nkv, d, scale * 1.4426950408889634f, window, static_cast<int>(total));
@@ -380,16 +421,16 @@ extern "C" int pl_paged_attention_prefill(const void* q, int q_stride, void* out
 #ifdef AP_FORCE_SMALL
     const bool small = AP_FORCE_SMALL;
 #else
-    // two waves have twice the pieces of a tile to carry each: only small heads leave them the registers
-    const bool small = max_q_len <= 64 && dt <= 2;
+    // half the threads have twice the pieces of a tile to carry each: large heads leave them no registers for that
+    const bool small = max_q_len <= 64 && dt <= 4;
 #endif
 #define AP_CALL(D)                                                                                                 \
-    return small ? launch_prefill<D, 2>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len, \
-                                        block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale,   \
-                                        window, stream)                                                            \
-                 : launch_prefill<D, 4>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len, \
-                                        block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale,   \
-                                        window, stream)
+    return small ? launch_prefill<D, 2, (D <= 4 ? AP_SMALL_KS : 1)>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len, \
+                                           block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale,   \
+                                           window, stream)                                                            \
+                 : launch_prefill<D, 4, (D <= 4 ? AP_KS : 1)>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len, \
+                                               block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale,   \
+                                               window, stream)
     switch (dt) {
         case 1: AP_CALL(1);
         case 2: AP_CALL(2);
