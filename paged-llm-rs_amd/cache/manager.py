@@ -150,12 +150,13 @@ class CacheManager:
         return native.check(self._lib.plh_cache_table(self._h, seq_id, group, address, capacity))
 
     def fill_step(self, ids_address: int, count: int, positions_address: int, group: int, tables_address: int,
-                  width: int) -> None:
+                  width: int) -> int:
         """For ``count`` requests (64-bit ids at a raw address): where each one's next token goes, and
         the rows of one group's block table (-1 beyond a request's pages), written at raw addresses
-        of 32-bit buffers.  An address of 0 leaves that output out."""
-        native.check(self._lib.plh_cache_fill_step(self._h, count, ids_address, positions_address, group,
-                                                   tables_address, width))
+        of 32-bit buffers.  An address of 0 leaves that output out.  Returns 0, or, when a request has
+        more pages than ``width``, that number of pages (the rows are then not written)."""
+        return native.check(self._lib.plh_cache_fill_step(self._h, count, ids_address, positions_address, group,
+                                                          tables_address, width))
 
     def state_slot(self, seq_id: int) -> int:
         slot = self._lib.plh_cache_state_slot(self._h, seq_id)

@@ -1,6 +1,7 @@
 // The C interface of the host runtime.  Every call returns 0 (or a count) on
 // success and a negative number on failure; the message is read with
 // plh_last_error().  Handles are opaque pointers.
+#include <algorithm>
 #include <cstring>
 #include <string>
 
@@ -125,24 +126,26 @@ long plh_cache_table(void* c, uint64_t id, size_t group, int* out, size_t cap) {
 }
 // For a step of n requests: positions[i] = tokens the cache holds of request i (where its next
 // token goes), and row i of `tables` (n rows of `width`, -1 beyond a request's pages) for one group.
+// Returns 0, or the number of pages of the longest table when that is more than `width`.
 // Either output may be null.
 long plh_cache_fill_step(void* c, size_t n, const uint64_t* ids, int* positions, size_t group, int* tables,
                          size_t width) {
     return guarded([&] {
         auto* cache = static_cast<CacheManager*>(c);
+        size_t widest = 0;
         for (size_t i = 0; i < n; ++i) {
             const SequenceTable& t = cache->table(ids[i]);
             if (t.tokens + 1 > cache->capacity(ids[i]))
                 throw Error("request " + std::to_string(ids[i]) + " has no block for position " + std::to_string(t.tokens));
             if (positions) positions[i] = static_cast<int>(t.tokens);
-            if (tables) {
-                const auto& blocks = t.blocks.at(group);
-                if (blocks.size() > width)
-                    throw Error("a table of " + std::to_string(blocks.size()) + " pages for room of " + std::to_string(width));
-                int* row = tables + i * width;
-                std::memcpy(row, blocks.data(), blocks.size() * sizeof(int));
-                for (size_t b = blocks.size(); b < width; ++b) row[b] = -1;
-            }
+            if (tables) widest = std::max(widest, t.blocks.at(group).size());
+        }
+        if (tables && widest > width) return static_cast<long>(widest);   // nothing is written: the rows need more room
+        for (size_t i = 0; tables && i < n; ++i) {
+            const auto& blocks = cache->table(ids[i]).blocks.at(group);
+            int* row = tables + i * width;
+            std::memcpy(row, blocks.data(), blocks.size() * sizeof(int));
+            for (size_t b = blocks.size(); b < width; ++b) row[b] = -1;
         }
         return 0L;
     });

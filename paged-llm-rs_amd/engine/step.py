@@ -60,6 +60,14 @@ class StepOutput:
         return self.greedy
 
 
+class TableTooWide(Exception):
+    """A request has more pages than the rows of a captured graph's block table have room for."""
+
+    def __init__(self, group: int, pages: int):
+        super().__init__(f"group {group}: a table of {pages} pages")
+        self.group, self.pages = group, pages
+
+
 def _bucket(n: int, least: int = 1) -> int:
     b = least
     while b < n:
@@ -127,14 +135,17 @@ class DecodeGraph:
             self.logits, self.tokens = self._forward()
 
     def fill(self, entries) -> None:
-        """Write the step's descriptor into the pinned buffer.  Raises when a table is wider than the bucket."""
+        """Write the step's descriptor into the pinned buffer.  Raises TableTooWide when a request has
+        outgrown the rows of this graph's block table."""
         live = len(entries)
         manager = self.cache.manager
         self.ids[:live] = [e.seq_id for e in entries]
         positions = self._view("positions")
         manager.fill_step(self.ids.ctypes.data, live, positions.ctypes.data, 0, 0, 0)
         for g, w in enumerate(self.widths):
-            manager.fill_step(self.ids.ctypes.data, live, 0, g, self._view(f"block_table_{g}").ctypes.data, w)
+            pages = manager.fill_step(self.ids.ctypes.data, live, 0, g, self._view(f"block_table_{g}").ctypes.data, w)
+            if pages:
+                raise TableTooWide(g, pages)
         tokens = self._view("token_ids")
         tokens[:live] = [e.tokens[0] for e in entries]
         vocab, limit = self.model.spec.vocab_size, self.model.spec.max_positions
@@ -193,9 +204,8 @@ class StepRunner:
                 out = graph.run(entries)
                 self.graph_steps += 1
                 return out
-            except ConfigError as error:
-                if "for room of" not in str(error):
-                    raise
+            except TableTooWide:
+                pass
         # no graph for this many requests yet, or a request has outgrown the bucket's table
         widths = [_bucket(w + 1, 32) for w in self._widths_needed(entries)]
         graph = DecodeGraph(self.model, self.cache, cap, widths)
