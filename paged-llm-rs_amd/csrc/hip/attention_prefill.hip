@@ -84,8 +84,8 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     constexpr int KROW = DP + AP_KPAD;     // elements a row of Ks
     constexpr int VROW = AP_BN + AP_VPAD;  // elements a row of Vt
     extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
-    uint16_t* Ks = lds;                    // [AP_BN][KROW]
-    uint16_t* Vt = lds + AP_BN * KROW;     // [DP][VROW]
+    // two tiles of keys [AP_BN][KROW] and of transposed values [DP][VROW]: one is read while the next is written
+    constexpr int TILE = AP_BN * KROW + DP * VROW;
 
     // Workgroups are dealt round-robin to the eight XCDs; consecutive pieces of
     // work (the token tiles of one head) go to one XCD, whose L2 then holds the
@@ -208,7 +208,9 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
             }
         }
     };
-    auto stash = [&]() {
+    auto stash = [&](int buf) {
+        uint16_t* Ks = lds + buf * TILE;
+        uint16_t* Vt = Ks + AP_BN * KROW;
 #pragma unroll
         for (int i = 0; i < KI; ++i) {
             const int idx = tid + i * NT;
@@ -236,18 +238,17 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     lookup(k_first);
     fetch();
     lookup(k_first + AP_BN);
-    for (int k0 = k_first; k0 <= last_pos; k0 += AP_BN) {
-        __syncthreads();  // the previous tile has been read by every wave
-        stash();
-        __syncthreads();
-        fetch();                     // tile k0 + AP_BN, all zeros past the last key
-        lookup(k0 + 2 * AP_BN);
-
-        // a wave whose queries all stand before this tile, or that has no queries, has nothing to add
-        if (!wave_active || k0 + 32 * kt0 > wave_last) continue;
-        if (window > 0 && k0 + 32 * (kt0 + KT) - 1 <= wave_first - window) continue;
-
-        // scores, transposed: s[kt][4*j + i] is key k0 + 32*kt + 8*j + 4*h + i against query r32
+    stash(0);
+    fetch();                         // the second tile, all zeros past the last key
+    lookup(k_first + 2 * AP_BN);
+    __syncthreads();
+    // One tile for this wave.  The running maximum is kept on the raw scores; the scale (with log2 e
+    // folded in) enters inside the exponential's argument, one multiply-add an element.  The output is
+    // rescaled only when some query's maximum has grown.
+    auto one_tile = [&](int k0, int cur, bool masked) {
+        const uint16_t* Ks = lds + cur * TILE;
+        const uint16_t* Vt = Ks + AP_BN * KROW;
+        // scores, transposed: s[kt][4*j + i] is key k0 + 32*(kt0+kt) + 8*j + 4*h + i against query r32
         f32x16 s[KT];
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt) {
@@ -261,54 +262,51 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
             for (int kk = 0; kk < 2 * DT; ++kk)
                 s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kk].vec, qf[kk].vec, s[kt], 0, 0, 0);
         }
-        // Key k0 + c + 4*h, c a constant of the register, is seen by this lane's query iff c <= reach
-        // (and c > reach - window).  Tiles that lie before every query of the wave need no test.
-        const bool edge = k0 + 32 * (kt0 + KT) - 1 > wave_first || window > 0;
-        const int reach = q_pos - k0 - 32 * kt0 - 4 * h;
-        const int behind = window > 0 ? reach - window : -(1 << 30);
         float mx = -INFINITY;
-        if (edge) {
+        if (masked) {
+            // Key k0 + c + 4*h, c a constant of the register, is seen by this lane's query iff c <= reach
+            // (and c > reach - window).
+            const int reach = q_pos - k0 - 32 * kt0 - 4 * h;
+            const int behind = window > 0 ? reach - window : -(1 << 30);
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int c = 32 * kt + 8 * (r >> 2) + (r & 3);
-                    const float v = (c <= reach && c > behind) ? s[kt][r] * scale_log2e : -INFINITY;
-                    s[kt][r] = v;
-                    mx = fmaxf(mx, v);
-                }
-        } else {
-#pragma unroll
-            for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float v = s[kt][r] * scale_log2e;
-                    s[kt][r] = v;
-                    mx = fmaxf(mx, v);
+                    s[kt][r] = (c <= reach && c > behind) ? s[kt][r] : -INFINITY;
                 }
         }
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kt][r]);
         mx = fmaxf(mx, __shfl_xor(mx, 32, PL_WAVE));
         const float m_new = fmaxf(m, mx);
         const float m_use = m_new == -INFINITY ? 0.f : m_new;
-        const float corr = __builtin_amdgcn_exp2f(m - m_use);
+        if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {   // the same for the whole wave
+            const float corr = __builtin_amdgcn_exp2f((m - m_use) * scale_log2e);
+            lsum *= corr;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o[dt][r] *= corr;
+            m = m_new;
+        }
+        const float shift = -m_use * scale_log2e;
         float psum = 0.f;
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const float p = __builtin_amdgcn_exp2f(s[kt][r] - m_use);  // v_exp_f32: arguments are <= 0, tiny results may flush
+                // v_exp_f32: arguments are <= 0, tiny results may flush
+                const float p = __builtin_amdgcn_exp2f(fmaf(s[kt][r], scale_log2e, shift));
                 s[kt][r] = p;
                 psum += p;
             }
-        lsum = lsum * corr + psum;
-        m = m_new;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) o[dt][r] *= corr;
+        lsum += psum;
 
         // O^T += V^T . P^T, sixteen keys a product: registers 8*half .. 8*half+7 of tile kt are the
-        // keys 32*kt + 16*half + {4h..4h+3} and + 8 + {4h..4h+3}
+        // keys 32*(kt0+kt) + 16*half + {4h..4h+3} and + 8 + {4h..4h+3}
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
@@ -328,14 +326,39 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
                 for (int dt = 0; dt < DT; ++dt)
                     o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[dt].vec, b.vec, o[dt], 0, 0, 0);
             }
-    }
+    };
 
+    // The registers hold the next tile: it goes into the buffer that nobody reads now (its readers
+    // passed the barrier that ended the round before), and the tile after it is asked for.
+    auto advance = [&](int k0, int cur) {
+        stash(cur ^ 1);
+        fetch();
+        lookup(k0 + 3 * AP_BN);
+    };
+
+    // First the tiles that every query of the workgroup sees whole: no masks, no wave stands idle
+    // (a wave past the request's last token works on zero queries and stores nothing).  Then the
+    // few tiles around the diagonal, where keys are hidden and waves of early tokens are done.
+    int cur = 0, k0 = k_first;
+    const int open_end = window > 0 ? k_first : ((start + q0 + 1) / AP_BN) * AP_BN;   // keys below it are seen by all
+    for (; k0 < open_end; k0 += AP_BN, cur ^= 1) {
+        advance(k0, cur);
+        one_tile(k0, cur, false);
+        __syncthreads();  // this tile has been read, the next one written
+    }
+    for (; k0 <= last_pos; k0 += AP_BN, cur ^= 1) {
+        advance(k0, cur);
+        // a wave whose queries all stand before this tile, or that has no queries, has nothing to add
+        const bool idle = !wave_active || k0 + 32 * kt0 > wave_last ||
+                          (window > 0 && k0 + 32 * (kt0 + KT) - 1 <= wave_first - window);
+        if (!idle) one_tile(k0, cur, true);
+        __syncthreads();
+    }
     lsum += __shfl_xor(lsum, 32, PL_WAVE);
     if (KS == 2) {
         // The wave of the later keys hands its state to the wave of the earlier ones through LDS
         // (the tiles are done with): out = (o0 2^(m0-M) + o1 2^(m1-M)) / (l0 2^(m0-M) + l1 2^(m1-M)).
         float* hand = reinterpret_cast<float*>(lds) + static_cast<size_t>(wave) * (16 * DT + 2) * PL_WAVE;
-        __syncthreads();
         if (kt0 != 0) {
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
@@ -349,7 +372,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         const float m1 = hand[(16 * DT) * PL_WAVE + lane], l1 = hand[(16 * DT + 1) * PL_WAVE + lane];
         const float big = fmaxf(m, m1);
         const float use = big == -INFINITY ? 0.f : big;
-        const float w0 = __builtin_amdgcn_exp2f(m - use), w1 = __builtin_amdgcn_exp2f(m1 - use);
+        const float w0 = __builtin_amdgcn_exp2f((m - use) * scale_log2e), w1 = __builtin_amdgcn_exp2f((m1 - use) * scale_log2e);
         lsum = lsum * w0 + l1 * w1;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
@@ -382,7 +405,7 @@ static int launch_prefill(const void* q, int q_stride, void* out, const int* q_s
                           int d, float scale, int window, hipStream_t stream) {
     constexpr int DP = 32 * DT;
     constexpr int BM = 32 * NW;
-    const size_t tile_bytes = (static_cast<size_t>(AP_BN) * (DP + AP_KPAD) + static_cast<size_t>(DP) * (AP_BN + AP_VPAD)) * 2;
+    const size_t tile_bytes = 2 * (static_cast<size_t>(AP_BN) * (DP + AP_KPAD) + static_cast<size_t>(DP) * (AP_BN + AP_VPAD)) * 2;
     const size_t hand_bytes = KS == 2 ? static_cast<size_t>(NW) * (16 * DT + 2) * PL_WAVE * sizeof(float) : 0;
     const size_t lds_bytes = tile_bytes > hand_bytes ? tile_bytes : hand_bytes;
     if (lds_bytes > 48 * 1024) {
