@@ -55,8 +55,24 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restric
     const T* d = delta ? delta + static_cast<size_t>(r) * H : nullptr;
     T* o = out + static_cast<size_t>(i) * H;
 
+    // A thread keeps up to NORM_KEEP of its elements in registers between the sum and the output, so
+    // that a row is read once (wider rows read the rest again).
+    constexpr int NORM_KEEP = 8;
+    float kept[NORM_KEEP];
     float ss = 0.f;
-    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+#pragma unroll
+    for (int k = 0; k < NORM_KEEP; ++k) {
+        const int c = threadIdx.x + k * blockDim.x;
+        float v = 0.f;
+        if (c < H) {
+            v = x[c];
+            if (d) v += to_float(d[c]);
+            if (write_resid) x[c] = v;
+        }
+        kept[k] = v;
+        ss += v * v;
+    }
+    for (int c = threadIdx.x + NORM_KEEP * blockDim.x; c < H; c += blockDim.x) {
         float v = x[c];
         if (d) v += to_float(d[c]);
         if (write_resid) x[c] = v;
@@ -64,7 +80,12 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restric
     }
     ss = block_sum(ss, scratch);
     const float denom = sqrtf(ss / static_cast<float>(H) + eps);
-    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+#pragma unroll
+    for (int k = 0; k < NORM_KEEP; ++k) {
+        const int c = threadIdx.x + k * blockDim.x;
+        if (c < H) o[c] = from_float<T>(kept[k] / denom * load_as_float(gain, gain_dtype, c));
+    }
+    for (int c = threadIdx.x + NORM_KEEP * blockDim.x; c < H; c += blockDim.x) {
         float v = x[c];
         if (d && !write_resid) v += to_float(d[c]);
         o[c] = from_float<T>(v / denom * load_as_float(gain, gain_dtype, c));
@@ -255,55 +276,72 @@ qk_norm_rope_kv_write_wide_kernel(
     const int lph = d / 8;                  // lanes a head
     const int hpw = PL_WAVE / lph;          // heads a wave
     const int hw = lane / lph, chunk = lane - hw * lph;
-    const int h = (blockIdx.y * 4 + wave) * hpw + hw;
-    const bool active = hw < hpw && h < heads;
-    const int hh = active ? h : 0;
-    const bool is_q = hh < nq;
-    const bool is_k = !is_q && hh < nq + nkv;
-
     const int row_width = (nq + 2 * nkv) * d;
-    T* src = qkv + static_cast<size_t>(t) * row_width + static_cast<size_t>(hh) * d + chunk * 8;
     const int blk = block_table[static_cast<size_t>(seq_of[t]) * max_blocks + pos / block_size];
     const size_t slot = static_cast<size_t>(blk < 0 ? 0 : blk) * block_size + pos % block_size;
-    T* dst = src;
-    if (!is_q) {
-        const int kvh = is_k ? hh - nq : hh - nq - nkv;
-        dst = (is_k ? k_pool : v_pool) + (slot * nkv + kvh) * d + chunk * 8;
-    }
-    const bool writes = active && (is_q || blk >= 0);   // never write through a hole in the table
 
-    float x[8];
-    qk_vec<T>::load(src, x);
-    const bool plain_copy = !is_q && !is_k;            // v
-    const void* gain = is_q ? q_gain : k_gain;
-
-    // the sum of squares over the lanes of the head (every lane takes part in the exchange)
-    float ss = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) ss = fmaf(x[e], x[e], ss);
-    float total = 0.f;
-    const int base = hw * lph;
-    for (int j = 0; j < lph; ++j) total += __shfl(ss, min(base + j, PL_WAVE - 1), PL_WAVE);
-    if (gain && !plain_copy) {
-        const float denom = sqrtf(total / static_cast<float>(d) + eps);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) x[e] = x[e] / denom * load_as_float(gain, gain_dtype, chunk * 8 + e);
-    }
-    // the partner in the rotation: the element rot/2 further on, or back
+    // What does not depend on the head is fetched once: the lane's eight gains of either norm and its
+    // eight angles (the partner in the rotation is the element rot/2 further on, or back).
     const int half = rot / 2, hc = half / 8;
     const bool low = chunk < hc;
     const int partner = min(max(lane + (low ? hc : -hc), 0), PL_WAVE - 1);
-    float px[8];
+    const bool rotates = cos_table && chunk * 8 < rot;
+    float qg[8], kg[8], c[8], sn[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) px[e] = __shfl(x[e], partner, PL_WAVE);
-    if (cos_table && !plain_copy && chunk * 8 < rot) {
-        const int at = (low ? chunk : chunk - hc) * 8;
-        const float* c = cos_table + static_cast<size_t>(pos) * half + at;
-        const float* s = sin_table + static_cast<size_t>(pos) * half + at;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) x[e] = low ? x[e] * c[e] - px[e] * s[e] : x[e] * c[e] + px[e] * s[e];
+    for (int e = 0; e < 8; ++e) {
+        qg[e] = q_gain ? load_as_float(q_gain, gain_dtype, chunk * 8 + e) : 1.f;
+        kg[e] = k_gain ? load_as_float(k_gain, gain_dtype, chunk * 8 + e) : 1.f;
+        c[e] = 1.f;
+        sn[e] = 0.f;
     }
-    if (writes) qk_vec<T>::store(dst, x);
+    if (rotates) {
+        const size_t at = static_cast<size_t>(pos) * half + (low ? chunk : chunk - hc) * 8;
+        qk_vec<float>::load(cos_table + at, c);
+        qk_vec<float>::load(sin_table + at, sn);
+    }
+
+    // the workgroups of a token share its heads: 4 * hpw at a time, gridDim.y groups apart
+    const int per_group = 4 * hpw;
+    for (int first = blockIdx.y * per_group; first < heads; first += gridDim.y * per_group) {
+        const int h = first + wave * hpw + hw;
+        const bool active = hw < hpw && h < heads;
+        const int hh = active ? h : 0;
+        const bool is_q = hh < nq;
+        const bool is_k = !is_q && hh < nq + nkv;
+        T* src = qkv + static_cast<size_t>(t) * row_width + static_cast<size_t>(hh) * d + chunk * 8;
+        T* dst = src;
+        if (!is_q) {
+            const int kvh = is_k ? hh - nq : hh - nq - nkv;
+            dst = (is_k ? k_pool : v_pool) + (slot * nkv + kvh) * d + chunk * 8;
+        }
+        const bool writes = active && (is_q || blk >= 0);   // never write through a hole in the table
+
+        float x[8];
+        qk_vec<T>::load(src, x);
+        const bool plain_copy = !is_q && !is_k;            // v
+        const bool normed = !plain_copy && (is_q ? q_gain != nullptr : k_gain != nullptr);
+
+        // the sum of squares over the lanes of the head (every lane takes part in the exchange)
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss = fmaf(x[e], x[e], ss);
+        float total = 0.f;
+        const int base = hw * lph;
+        for (int j = 0; j < lph; ++j) total += __shfl(ss, min(base + j, PL_WAVE - 1), PL_WAVE);
+        if (normed) {
+            const float denom = sqrtf(total / static_cast<float>(d) + eps);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = x[e] / denom * (is_q ? qg[e] : kg[e]);
+        }
+        float px[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) px[e] = __shfl(x[e], partner, PL_WAVE);
+        if (rotates && !plain_copy) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = low ? x[e] * c[e] - px[e] * sn[e] : x[e] * c[e] + px[e] * sn[e];
+        }
+        if (writes) qk_vec<T>::store(dst, x);
+    }
 }
 
 extern "C" int pl_qk_norm_rope_kv_write(
@@ -321,8 +359,10 @@ extern "C" int pl_qk_norm_rope_kv_write(
     // Without the cache write (a layer that reads another layer's pages) only the query heads run.
     const int heads = write_kv ? nq + 2 * nkv : nq;
     if (rot % 16 == 0) {
+        // many tokens: one workgroup a token walks all its heads and fetches gains and angles once;
+        // few tokens: a workgroup for every 4 * (64 / (d/8)) heads, so that the chip has work
         const int per_group = 4 * (PL_WAVE / (d / 8));
-        dim3 wide(n, pl_ceil_div(heads, per_group));
+        dim3 wide(n, n >= 512 ? 1 : pl_ceil_div(heads, per_group));
         if (dtype == PL_DTYPE_F32)
             qk_norm_rope_kv_write_wide_kernel<float><<<wide, 256, 0, stream>>>(
                 static_cast<float*>(qkv), q_gain, k_gain, gain_dtype, eps, cos_table, sin_table, rot, positions, seq_of,
@@ -365,10 +405,38 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int
     out[idx] = from_float<T>(g / (1.f + expf(-g)) * u);
 }
 
+// The same, eight consecutive elements a thread (one 16-byte load of each half in bfloat16), for
+// widths that are a multiple of eight.
+template <typename T>
+__global__ void __launch_bounds__(256)
+swiglu_wide_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t chunks) {
+    const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= chunks) return;
+    const int per_row = I / 8;
+    const size_t row = idx / per_row;
+    const int c = static_cast<int>(idx - row * per_row) * 8;
+    float g[8], u[8], r[8];
+    qk_vec<T>::load(gu + row * 2 * I + c, g);
+    qk_vec<T>::load(gu + row * 2 * I + I + c, u);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = g[e] / (1.f + expf(-g[e])) * u[e];
+    qk_vec<T>::store(out + row * I + c, r);
+}
+
 extern "C" int pl_swiglu(const void* gu, void* out, int n, int I, int dtype, hipStream_t stream) {
     PL_REQUIRE(n >= 0 && I > 0, "swiglu: rows %d, width %d", n, I);
     const size_t count = static_cast<size_t>(n) * I;
     if (count == 0) return 0;
+    if (I % 8 == 0 && (dtype == PL_DTYPE_F32 || dtype == PL_DTYPE_BF16)) {
+        const size_t chunks = count / 8;
+        const int wide_blocks = static_cast<int>((chunks + 255) / 256);
+        if (dtype == PL_DTYPE_F32)
+            swiglu_wide_kernel<float><<<wide_blocks, 256, 0, stream>>>(static_cast<const float*>(gu), static_cast<float*>(out), I, chunks);
+        else
+            swiglu_wide_kernel<bf16_t><<<wide_blocks, 256, 0, stream>>>(static_cast<const bf16_t*>(gu), static_cast<bf16_t*>(out), I, chunks);
+        PL_CHECK_LAUNCH("swiglu");
+        return 0;
+    }
     const int blocks = static_cast<int>((count + 255) / 256);
     if (dtype == PL_DTYPE_F32)
         swiglu_kernel<float><<<blocks, 256, 0, stream>>>(static_cast<const float*>(gu), static_cast<float*>(out), I, count);
