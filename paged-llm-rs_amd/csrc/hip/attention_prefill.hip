@@ -19,9 +19,10 @@
 //                     product may be permuted freely, so V^T is read from LDS in
 //                     the order in which the scores lie in the registers.
 //
-// V is transposed on its way into LDS (two keys packed into a 32-bit word) so
-// that the keys of one head element are contiguous.  Maximum, sum and the
-// output are 32-bit; exponentials are base 2 with log2(e) folded into the scale.
+// V lies in LDS as it lies in the cache, a row a key; the transposing read of
+// gfx950 (ds_read_b64_tr_b16) hands a lane four keys of one head element.
+// Maximum, sum and the output are 32-bit; exponentials are base 2 with log2(e)
+// folded into the scale.
 #include "common.hpp"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -38,7 +39,6 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 #endif
 #define AP_BN 64   // keys a tile
 #define AP_KPAD 8  // padding of a row of keys in LDS, in elements
-#define AP_VPAD 4  // padding of a row of transposed values in LDS, in elements
 
 struct __attribute__((aligned(16))) ap_u32x4 {
     uint32_t v[4];
@@ -54,6 +54,18 @@ union ap_frag {
     uint32_t w[4];
 };
 
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 ap_bf16x4;
+typedef __attribute__((address_space(3))) ap_bf16x4 ap_lds_bf16x4;
+
+// The transposing read.  Among 16 neighbouring lanes, lane 4e + q gives the address of four
+// elements; lane i receives, as its element e, element i % 4 of what lane 4e + i / 4 pointed at.
+// With lane 4e + q pointing at row e, columns 4q .. 4q+3 of a row-major block, lane i gets
+// column i of the rows 0 .. 3.
+__device__ __forceinline__ ap_u32x2 ap_read_transposed(const uint16_t* at) {
+    const ap_bf16x4 got = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((ap_lds_bf16x4*)(at));
+    return __builtin_bit_cast(ap_u32x2, got);
+}
+
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
@@ -68,6 +80,10 @@ __device__ __forceinline__ uint32_t ap_pack2(float lo, float hi) {
 // each with a running state of its own, merged at the end; twice the waves overlap more of the
 // softmax with the products; heads of more than 128 elements have no registers for it).  A workgroup
 // has NW * KS waves.
+// Padding of a row of values in LDS, in elements: a row is then 16 banks (of 32) further than the one
+// before, and the four rows of 64 bytes that 32 lanes read transposed fall on every bank twice.
+__host__ __device__ constexpr int ap_vpad(int dt) { return dt % 2 == 0 ? 32 : 0; }
+
 template <int DT, int NW, int KS>
 __global__ void __launch_bounds__(64 * NW * KS, DT <= 4 ? AP_OCC : 1)
 paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
@@ -82,10 +98,10 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     constexpr int NT = 64 * NW * KS;
     constexpr int KT = 2 / KS;             // 32-key tiles of a 64-key tile a wave takes
     constexpr int KROW = DP + AP_KPAD;     // elements a row of Ks
-    constexpr int VROW = AP_BN + AP_VPAD;  // elements a row of Vt
+    constexpr int VROW = DP + ap_vpad(DT); // elements a row of Vs
     extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
-    // two tiles of keys [AP_BN][KROW] and of transposed values [DP][VROW]: one is read while the next is written
-    constexpr int TILE = AP_BN * KROW + DP * VROW;
+    // two tiles of keys [AP_BN][KROW] and of values [AP_BN][VROW]: one is read while the next is written
+    constexpr int TILE = AP_BN * KROW + AP_BN * VROW;
 
     // Workgroups are dealt round-robin to the eight XCDs; consecutive pieces of
     // work (the token tiles of one head) go to one XCD, whose L2 then holds the
@@ -152,84 +168,62 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     // the products of this one, so that their latency passes behind the matrix cores.
     constexpr int CP = DP / 8;                                  // 16-byte pieces of a padded row
     constexpr int KI = (AP_BN * CP + NT - 1) / NT;              // pieces of the key tile a thread carries
-    constexpr int VI = (AP_BN / 2 * CP + NT - 1) / NT;          // pairs of pieces of the value tile
-    ap_u32x4 kreg[KI], vreg0[VI], vreg1[VI];
+    ap_u32x4 kreg[KI], vreg[KI];                                // and the same pieces of the value tile
 
     // Loads are unconditional, from an address that is valid in any case, and what they bring is
     // masked afterwards where the key does not exist: a load inside a branch would be waited for
     // at the branch's end, one load after the other.  The page numbers of a tile are looked up one
     // tile before its keys and values are loaded, so that no load waits for another.
-    int kblk[KI], kwithin[KI], vblk[VI][2], vwithin[VI][2];
-    auto locate = [&](int j, int& blk, int& within) {           // page and place in the page of key j
-        const bool in = j <= last_pos;
+    // A lookup leaves the table's answer raw: what depends on it is computed by the fetch, one tile
+    // later, so that the wait for the answer stands there and not in the middle of this tile.
+    int kblk[KI], kwithin[KI];
+    bool kin[KI];
+    auto locate = [&](int j, int& blk, int& within, bool& in) {  // page and place in the page of key j
+        in = j <= last_pos;
         const int jj = in ? j : last_pos;
         int bi = static_cast<int>(__umulhi(static_cast<uint32_t>(jj), bs_magic));
         within = jj - bi * block_size;
         const int low = within >= block_size ? 1 : 0;            // the estimate is the quotient or one less
         bi += low;
         within -= low * block_size;
-        const int got = table[bi];
-        blk = in ? got : -1;
+        blk = table[bi];
     };
     auto lookup = [&](int k0) {
 #pragma unroll
-        for (int i = 0; i < KI; ++i) locate(k0 + ((tid + i * NT) / CP) % AP_BN, kblk[i], kwithin[i]);
-#pragma unroll
-        for (int i = 0; i < VI; ++i) {
-            const int pair = ((tid + i * NT) / CP) % (AP_BN / 2);
-            locate(k0 + 2 * pair, vblk[i][0], vwithin[i][0]);
-            locate(k0 + 2 * pair + 1, vblk[i][1], vwithin[i][1]);
-        }
+        for (int i = 0; i < KI; ++i) locate(k0 + ((tid + i * NT) / CP) % AP_BN, kblk[i], kwithin[i], kin[i]);
     };
     auto row_of = [&](int blk, int within) -> size_t {
         return (static_cast<size_t>(max(blk, 0)) * block_size + within) * row_stride;
     };
+    // What a load brings is masked only when it goes into LDS, one tile later: a mask applied here
+    // would make the wave wait for the load in the middle of the tile that should hide it.
+    uint32_t keep[KI];
     auto fetch = [&]() {
 #pragma unroll
         for (int i = 0; i < KI; ++i) {
             const int c = (tid + i * NT) % CP;
-            const ap_u32x4 got = *reinterpret_cast<const ap_u32x4*>(k_pool + row_of(kblk[i], kwithin[i]) + head_off + min(c, cpr - 1) * 8);
-            const uint32_t keep = (kblk[i] >= 0 && c < cpr) ? 0xffffffffu : 0u;
-#pragma unroll
-            for (int w = 0; w < 4; ++w) kreg[i].v[w] = got.v[w] & keep;
-        }
-#pragma unroll
-        for (int i = 0; i < VI; ++i) {
-            const int c = (tid + i * NT) % CP;
-            const size_t col = head_off + min(c, cpr - 1) * 8;
-            const ap_u32x4 got0 = *reinterpret_cast<const ap_u32x4*>(v_pool + row_of(vblk[i][0], vwithin[i][0]) + col);
-            const ap_u32x4 got1 = *reinterpret_cast<const ap_u32x4*>(v_pool + row_of(vblk[i][1], vwithin[i][1]) + col);
-            const uint32_t keep0 = (vblk[i][0] >= 0 && c < cpr) ? 0xffffffffu : 0u;
-            const uint32_t keep1 = (vblk[i][1] >= 0 && c < cpr) ? 0xffffffffu : 0u;
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                vreg0[i].v[w] = got0.v[w] & keep0;
-                vreg1[i].v[w] = got1.v[w] & keep1;
-            }
+            const size_t at = row_of(kblk[i], kwithin[i]) + head_off + min(c, cpr - 1) * 8;
+            kreg[i] = *reinterpret_cast<const ap_u32x4*>(k_pool + at);
+            vreg[i] = *reinterpret_cast<const ap_u32x4*>(v_pool + at);
+            keep[i] = (kin[i] && kblk[i] >= 0 && c < cpr) ? 0xffffffffu : 0u;
         }
     };
     auto stash = [&](int buf) {
         uint16_t* Ks = lds + buf * TILE;
-        uint16_t* Vt = Ks + AP_BN * KROW;
+        uint16_t* Vs = Ks + AP_BN * KROW;
 #pragma unroll
         for (int i = 0; i < KI; ++i) {
             const int idx = tid + i * NT;
             const int key = idx / CP, c = idx % CP;
-            if (idx < AP_BN * CP) *reinterpret_cast<ap_u32x4*>(Ks + key * KROW + c * 8) = kreg[i];
-        }
-        // values are stored transposed, two neighbouring keys a word
+            ap_u32x4 kk, vv;
 #pragma unroll
-        for (int i = 0; i < VI; ++i) {
-            const int idx = tid + i * NT;
-            const int pair = idx / CP, c = idx % CP;
-            if (idx < AP_BN / 2 * CP) {
-#pragma unroll
-                for (int w = 0; w < 4; ++w) {
-                    const uint32_t even = (vreg0[i].v[w] & 0xffffu) | (vreg1[i].v[w] << 16);
-                    const uint32_t odd = (vreg0[i].v[w] >> 16) | (vreg1[i].v[w] & 0xffff0000u);
-                    *reinterpret_cast<uint32_t*>(Vt + (c * 8 + 2 * w) * VROW + 2 * pair) = even;
-                    *reinterpret_cast<uint32_t*>(Vt + (c * 8 + 2 * w + 1) * VROW + 2 * pair) = odd;
-                }
+            for (int w = 0; w < 4; ++w) {
+                kk.v[w] = kreg[i].v[w] & keep[i];
+                vv.v[w] = vreg[i].v[w] & keep[i];
+            }
+            if (idx < AP_BN * CP) {
+                *reinterpret_cast<ap_u32x4*>(Ks + key * KROW + c * 8) = kk;
+                *reinterpret_cast<ap_u32x4*>(Vs + key * VROW + c * 8) = vv;
             }
         }
     };
@@ -247,7 +241,8 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     // rescaled only when some query's maximum has grown.
     auto one_tile = [&](int k0, int cur, bool masked) {
         const uint16_t* Ks = lds + cur * TILE;
-        const uint16_t* Vt = Ks + AP_BN * KROW;
+        // this lane's corner of a block of 4 keys x 16 head elements that 16 lanes read transposed
+        const uint16_t* Vs = Ks + AP_BN * KROW + (32 * kt0 + 4 * h + ((lane & 15) >> 2)) * VROW + (lane & 16) + 4 * (lane & 3);
         // scores, transposed: s[kt][4*j + i] is key k0 + 32*(kt0+kt) + 8*j + 4*h + i against query r32
         f32x16 s[KT];
 #pragma unroll
@@ -314,13 +309,12 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
                 ap_frag b;
 #pragma unroll
                 for (int w = 0; w < 4; ++w) b.w[w] = ap_pack2(s[kt][8 * half + 2 * w], s[kt][8 * half + 2 * w + 1]);
-                const int key_off = 32 * (kt0 + kt) + 16 * half + 4 * h;
                 ap_frag a[DT];
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
-                    const uint16_t* row = Vt + (32 * dt + r32) * VROW + key_off;
-                    a[dt].half[0] = *reinterpret_cast<const ap_u32x2*>(row);
-                    a[dt].half[1] = *reinterpret_cast<const ap_u32x2*>(row + 8);
+                    const uint16_t* block = Vs + (32 * kt + 16 * half) * VROW + 32 * dt;
+                    a[dt].half[0] = ap_read_transposed(block);
+                    a[dt].half[1] = ap_read_transposed(block + 8 * VROW);
                 }
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt)
@@ -405,7 +399,7 @@ static int launch_prefill(const void* q, int q_stride, void* out, const int* q_s
                           int d, float scale, int window, hipStream_t stream) {
     constexpr int DP = 32 * DT;
     constexpr int BM = 32 * NW;
-    const size_t tile_bytes = 2 * (static_cast<size_t>(AP_BN) * (DP + AP_KPAD) + static_cast<size_t>(DP) * (AP_BN + AP_VPAD)) * 2;
+    const size_t tile_bytes = 2 * (static_cast<size_t>(AP_BN) * (DP + AP_KPAD) + static_cast<size_t>(AP_BN) * (DP + ap_vpad(DT))) * 2;
     const size_t hand_bytes = KS == 2 ? static_cast<size_t>(NW) * (16 * DT + 2) * PL_WAVE * sizeof(float) : 0;
     const size_t lds_bytes = tile_bytes > hand_bytes ? tile_bytes : hand_bytes;
     if (lds_bytes > 48 * 1024) {

@@ -300,47 +300,56 @@ qk_norm_rope_kv_write_wide_kernel(
         qk_vec<float>::load(sin_table + at, sn);
     }
 
-    // the workgroups of a token share its heads: 4 * hpw at a time, gridDim.y groups apart
+    // The workgroups of a token share its heads: 4 * hpw heads make a group, a workgroup takes two
+    // groups at a time (both asked for before either is worked on), gridDim.y pairs apart.
     const int per_group = 4 * hpw;
-    for (int first = blockIdx.y * per_group; first < heads; first += gridDim.y * per_group) {
-        const int h = first + wave * hpw + hw;
-        const bool active = hw < hpw && h < heads;
-        const int hh = active ? h : 0;
-        const bool is_q = hh < nq;
-        const bool is_k = !is_q && hh < nq + nkv;
-        T* src = qkv + static_cast<size_t>(t) * row_width + static_cast<size_t>(hh) * d + chunk * 8;
-        T* dst = src;
-        if (!is_q) {
-            const int kvh = is_k ? hh - nq : hh - nq - nkv;
-            dst = (is_k ? k_pool : v_pool) + (slot * nkv + kvh) * d + chunk * 8;
+    for (int first = blockIdx.y * 2 * per_group; first < heads; first += gridDim.y * 2 * per_group) {
+        T* src[2];
+        T* dst[2];
+        bool writes[2], plain_copy[2], normed[2], is_q[2];
+        float x[2][8];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int hd = first + u * per_group + wave * hpw + hw;
+            const bool active = hw < hpw && hd < heads;
+            const int hh = active ? hd : 0;
+            is_q[u] = hh < nq;
+            const bool is_k = !is_q[u] && hh < nq + nkv;
+            src[u] = qkv + static_cast<size_t>(t) * row_width + static_cast<size_t>(hh) * d + chunk * 8;
+            dst[u] = src[u];
+            if (!is_q[u]) {
+                const int kvh = is_k ? hh - nq : hh - nq - nkv;
+                dst[u] = (is_k ? k_pool : v_pool) + (slot * nkv + kvh) * d + chunk * 8;
+            }
+            writes[u] = active && (is_q[u] || blk >= 0);   // never write through a hole in the table
+            plain_copy[u] = !is_q[u] && !is_k;             // v
+            normed[u] = !plain_copy[u] && (is_q[u] ? q_gain != nullptr : k_gain != nullptr);
+            qk_vec<T>::load(src[u], x[u]);
         }
-        const bool writes = active && (is_q || blk >= 0);   // never write through a hole in the table
-
-        float x[8];
-        qk_vec<T>::load(src, x);
-        const bool plain_copy = !is_q && !is_k;            // v
-        const bool normed = !plain_copy && (is_q ? q_gain != nullptr : k_gain != nullptr);
-
-        // the sum of squares over the lanes of the head (every lane takes part in the exchange)
-        float ss = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) ss = fmaf(x[e], x[e], ss);
-        float total = 0.f;
-        const int base = hw * lph;
-        for (int j = 0; j < lph; ++j) total += __shfl(ss, min(base + j, PL_WAVE - 1), PL_WAVE);
-        if (normed) {
-            const float denom = sqrtf(total / static_cast<float>(d) + eps);
+        for (int u = 0; u < 2; ++u) {
+            // the sum of squares over the lanes of the head (every lane takes part in the exchange)
+            float ss = 0.f;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) x[e] = x[e] / denom * (is_q ? qg[e] : kg[e]);
+            for (int e = 0; e < 8; ++e) ss = fmaf(x[u][e], x[u][e], ss);
+            float total = 0.f;
+            const int base = hw * lph;
+            for (int j = 0; j < lph; ++j) total += __shfl(ss, min(base + j, PL_WAVE - 1), PL_WAVE);
+            if (normed[u]) {
+                const float denom = sqrtf(total / static_cast<float>(d) + eps);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[u][e] = x[u][e] / denom * (is_q[u] ? qg[e] : kg[e]);
+            }
+            float px[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) px[e] = __shfl(x[u][e], partner, PL_WAVE);
+            if (rotates && !plain_copy[u]) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    x[u][e] = low ? x[u][e] * c[e] - px[e] * sn[e] : x[u][e] * c[e] + px[e] * sn[e];
+            }
+            if (writes[u]) qk_vec<T>::store(dst[u], x[u]);
         }
-        float px[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) px[e] = __shfl(x[e], partner, PL_WAVE);
-        if (rotates && !plain_copy) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) x[e] = low ? x[e] * c[e] - px[e] * sn[e] : x[e] * c[e] + px[e] * sn[e];
-        }
-        if (writes) qk_vec<T>::store(dst, x);
     }
 }
 
@@ -359,10 +368,9 @@ extern "C" int pl_qk_norm_rope_kv_write(
     // Without the cache write (a layer that reads another layer's pages) only the query heads run.
     const int heads = write_kv ? nq + 2 * nkv : nq;
     if (rot % 16 == 0) {
-        // many tokens: one workgroup a token walks all its heads and fetches gains and angles once;
-        // few tokens: a workgroup for every 4 * (64 / (d/8)) heads, so that the chip has work
+        // a workgroup takes two groups of 4 * (64 / (d/8)) heads of a token at a time
         const int per_group = 4 * (PL_WAVE / (d / 8));
-        dim3 wide(n, n >= 512 ? 1 : pl_ceil_div(heads, per_group));
+        dim3 wide(n, pl_ceil_div(heads, 2 * per_group));
         if (dtype == PL_DTYPE_F32)
             qk_norm_rope_kv_write_wide_kernel<float><<<wide, 256, 0, stream>>>(
                 static_cast<float*>(qkv), q_gain, k_gain, gain_dtype, eps, cos_table, sin_table, rot, positions, seq_of,
