@@ -66,6 +66,7 @@ __device__ __forceinline__ ap_u32x2 ap_read_transposed(const uint16_t* at) {
     return __builtin_bit_cast(ap_u32x2, got);
 }
 
+typedef uint32_t ap_vec4 __attribute__((ext_vector_type(4)));   // 16 bytes on their way through registers
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
@@ -83,8 +84,15 @@ __device__ __forceinline__ uint32_t ap_pack2(float lo, float hi) {
 // Padding of a row of values in LDS, in elements: a row is then 16 banks (of 32) further than the one
 // before, and the four rows of 64 bytes that 32 lanes read transposed fall on every bank twice.
 __host__ __device__ constexpr int ap_vpad(int dt) { return dt % 2 == 0 ? 32 : 0; }
+__host__ __device__ constexpr int ap_value_buffers(int ks) { return ks == 2 ? 3 : 2; }
 
-template <int DT, int NW, int KS>
+// UP (uniform pages): the 64 / (4*DT) keys whose pieces one wave loads with one instruction lie in one
+// page (the page size is a power of two and at least as many keys).  Page numbers then come through
+// the scalar unit and an address is a scalar base plus a lane's constant: no vector arithmetic a tile.
+// What is loaded is not masked on this path: scores of keys that do not exist are masked anyway, and
+// their values are multiplied by zero, so the pages have to hold finite numbers everywhere (the
+// pools are allocated zeroed).
+template <int DT, int NW, int KS, bool UP>
 __global__ void __launch_bounds__(64 * NW * KS, DT <= 4 ? AP_OCC : 1)
 paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
                                const int* __restrict__ q_start, const int* __restrict__ q_len,
@@ -100,8 +108,13 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     constexpr int KROW = DP + AP_KPAD;     // elements a row of Ks
     constexpr int VROW = DP + ap_vpad(DT); // elements a row of Vs
     extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
-    // two tiles of keys [AP_BN][KROW] and of values [AP_BN][VROW]: one is read while the next is written
-    constexpr int TILE = AP_BN * KROW + AP_BN * VROW;
+    // Two tiles of keys [AP_BN][KROW], then NVB tiles of values [AP_BN][VROW].  The values of a tile
+    // are read one round after its keys, and with two groups of waves half a round apart they live
+    // for three rounds.
+    constexpr int NVB = ap_value_buffers(KS);
+    constexpr int KTILE = AP_BN * KROW, VTILE = AP_BN * VROW;
+    uint16_t* const Kbase = lds;
+    uint16_t* const Vbase = lds + 2 * KTILE;
 
     // Workgroups are dealt round-robin to the eight XCDs; consecutive pieces of
     // work (the token tiles of one head) go to one XCD, whose L2 then holds the
@@ -124,6 +137,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave_id = __builtin_amdgcn_readfirstlane(tid >> 6);   // the same for the whole wave: kept scalar
+    // waves w and w + 4 share a SIMD: with NW == 4 a SIMD holds one wave of either group of keys
     const int wave = wave_id % NW;                               // which block of 32 tokens
     const int kt0 = (wave_id / NW) * KT;                         // the wave's first 32-key tile of a 64-key tile
     const int r32 = lane & 31;
@@ -168,7 +182,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     // the products of this one, so that their latency passes behind the matrix cores.
     constexpr int CP = DP / 8;                                  // 16-byte pieces of a padded row
     constexpr int KI = (AP_BN * CP + NT - 1) / NT;              // pieces of the key tile a thread carries
-    ap_u32x4 kreg[KI], vreg[KI];                                // and the same pieces of the value tile
+    ap_vec4 kreg[KI], vreg[KI];                                 // and the same pieces of the value tile
 
     // Loads are unconditional, from an address that is valid in any case, and what they bring is
     // masked afterwards where the key does not exist: a load inside a branch would be waited for
@@ -176,8 +190,13 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     // tile before its keys and values are loaded, so that no load waits for another.
     // A lookup leaves the table's answer raw: what depends on it is computed by the fetch, one tile
     // later, so that the wait for the answer stands there and not in the middle of this tile.
-    int kblk[KI], kwithin[KI];
+    int kblk[KI], kwithin[KI];       // UP: the page of the wave's keys of piece i and their first row in it
     bool kin[KI];
+    uint32_t keep[KI];
+    const int log2_bs = 31 - __builtin_clz(static_cast<unsigned>(block_size));
+    const uint32_t row_bytes = static_cast<uint32_t>(nkv) * d * 2;
+    // UP: this lane's place beside the wave's base: its row among the wave's rows, its piece of the row
+    const uint32_t lane_place = (lane / CP) * row_bytes + static_cast<uint32_t>(head_off + min(lane % CP, cpr - 1) * 8) * 2;
     auto locate = [&](int j, int& blk, int& within, bool& in) {  // page and place in the page of key j
         in = j <= last_pos;
         const int jj = in ? j : last_pos;
@@ -190,40 +209,68 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     };
     auto lookup = [&](int k0) {
 #pragma unroll
-        for (int i = 0; i < KI; ++i) locate(k0 + ((tid + i * NT) / CP) % AP_BN, kblk[i], kwithin[i], kin[i]);
+        for (int i = 0; i < KI; ++i) {
+            if constexpr (UP) {
+                // the first key of the wave's rows; past the last key the page of the last key serves
+                // (its rows exist, and what they hold is never seen)
+                const int j0 = k0 + (64 * wave_id + i * NT) / CP;
+                kwithin[i] = j0 & (block_size - 1);
+                kblk[i] = table[__builtin_amdgcn_readfirstlane(min(j0, last_pos) >> log2_bs)];
+            } else {
+                locate(k0 + ((tid + i * NT) / CP) % AP_BN, kblk[i], kwithin[i], kin[i]);
+            }
+        }
+    };
+    // UP: the scalar unit answers slowly, so the pages of the tile after the next are asked for at the
+    // start of the half round whose end needs them
+    int ahead_blk[KI], ahead_within[KI];
+    auto look_ahead = [&](int k0) {
+        if constexpr (UP) {
+#pragma unroll
+            for (int i = 0; i < KI; ++i) {
+                const int j0 = k0 + (64 * wave_id + i * NT) / CP;
+                ahead_within[i] = j0 & (block_size - 1);
+                ahead_blk[i] = table[__builtin_amdgcn_readfirstlane(min(j0, last_pos) >> log2_bs)];
+            }
+        }
     };
     auto row_of = [&](int blk, int within) -> size_t {
         return (static_cast<size_t>(max(blk, 0)) * block_size + within) * row_stride;
     };
     // What a load brings is masked only when it goes into LDS, one tile later: a mask applied here
     // would make the wave wait for the load in the middle of the tile that should hide it.
-    uint32_t keep[KI];
     auto fetch = [&]() {
 #pragma unroll
         for (int i = 0; i < KI; ++i) {
-            const int c = (tid + i * NT) % CP;
-            const size_t at = row_of(kblk[i], kwithin[i]) + head_off + min(c, cpr - 1) * 8;
-            kreg[i] = *reinterpret_cast<const ap_u32x4*>(k_pool + at);
-            vreg[i] = *reinterpret_cast<const ap_u32x4*>(v_pool + at);
-            keep[i] = (kin[i] && kblk[i] >= 0 && c < cpr) ? 0xffffffffu : 0u;
+            if constexpr (UP) {
+                const int page = __builtin_amdgcn_readfirstlane(max(kblk[i], 0));
+                const size_t base = (static_cast<size_t>(page) * block_size + kwithin[i]) * row_bytes;
+                kreg[i] = *reinterpret_cast<const ap_vec4*>(reinterpret_cast<const char*>(k_pool) + base + lane_place);
+                vreg[i] = *reinterpret_cast<const ap_vec4*>(reinterpret_cast<const char*>(v_pool) + base + lane_place);
+            } else {
+                const int c = (tid + i * NT) % CP;
+                const size_t at = row_of(kblk[i], kwithin[i]) + head_off + min(c, cpr - 1) * 8;
+                kreg[i] = *reinterpret_cast<const ap_vec4*>(k_pool + at);
+                vreg[i] = *reinterpret_cast<const ap_vec4*>(v_pool + at);
+                keep[i] = (kin[i] && kblk[i] >= 0 && c < cpr) ? 0xffffffffu : 0u;
+            }
         }
     };
-    auto stash = [&](int buf) {
-        uint16_t* Ks = lds + buf * TILE;
-        uint16_t* Vs = Ks + AP_BN * KROW;
+    auto stash = [&](int kbuf, int vbuf) {
+        uint16_t* Ks = Kbase + kbuf * KTILE;
+        uint16_t* Vs = Vbase + vbuf * VTILE;
 #pragma unroll
         for (int i = 0; i < KI; ++i) {
             const int idx = tid + i * NT;
             const int key = idx / CP, c = idx % CP;
-            ap_u32x4 kk, vv;
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                kk.v[w] = kreg[i].v[w] & keep[i];
-                vv.v[w] = vreg[i].v[w] & keep[i];
+            ap_vec4 kk = kreg[i], vv = vreg[i];
+            if constexpr (!UP) {
+                kk &= keep[i];
+                vv &= keep[i];
             }
             if (idx < AP_BN * CP) {
-                *reinterpret_cast<ap_u32x4*>(Ks + key * KROW + c * 8) = kk;
-                *reinterpret_cast<ap_u32x4*>(Vs + key * VROW + c * 8) = vv;
+                *reinterpret_cast<ap_vec4*>(Ks + key * KROW + c * 8) = kk;
+                *reinterpret_cast<ap_vec4*>(Vs + key * VROW + c * 8) = vv;
             }
         }
     };
@@ -232,31 +279,115 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     lookup(k_first);
     fetch();
     lookup(k_first + AP_BN);
-    stash(0);
+    stash(0, 0);
     fetch();                         // the second tile, all zeros past the last key
     lookup(k_first + 2 * AP_BN);
+
+    int staged = 1, staged_v = 1;    // the tile that the registers hold, and the buffer its values go to
     __syncthreads();
-    // One tile for this wave.  The running maximum is kept on the raw scores; the scale (with log2 e
-    // folded in) enters inside the exponential's argument, one multiply-add an element.  The output is
-    // rescaled only when some query's maximum has grown.
-    auto one_tile = [&](int k0, int cur, bool masked) {
-        const uint16_t* Ks = lds + cur * TILE;
-        // this lane's corner of a block of 4 keys x 16 head elements that 16 lanes read transposed
-        const uint16_t* Vs = Ks + AP_BN * KROW + (32 * kt0 + 4 * h + ((lane & 15) >> 2)) * VROW + (lane & 16) + 4 * (lane & 3);
-        // scores, transposed: s[kt][4*j + i] is key k0 + 32*(kt0+kt) + 8*j + 4*h + i against query r32
-        f32x16 s[KT];
+    // The registers hold tile `staged`: it goes into buffers that nobody reads now, the tile after it
+    // is asked for and the one after that looked up.
+    auto advance = [&]() {
+        stash(staged & 1, staged_v);
+        fetch();
+        if constexpr (UP) {
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) s[kt][r] = 0.f;
-            ap_frag a[2 * DT];
-#pragma unroll
-            for (int kk = 0; kk < 2 * DT; ++kk)
-                a[kk].raw = *reinterpret_cast<const ap_u32x4*>(Ks + (32 * (kt0 + kt) + r32) * KROW + 16 * kk + 8 * h);
-#pragma unroll
-            for (int kk = 0; kk < 2 * DT; ++kk)
-                s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kk].vec, qf[kk].vec, s[kt], 0, 0, 0);
+            for (int i = 0; i < KI; ++i) {
+                kblk[i] = ahead_blk[i];
+                kwithin[i] = ahead_within[i];
+            }
+        } else {
+            lookup(k_first + (staged + 2) * AP_BN);
         }
+        ++staged;
+        staged_v = staged_v + 1 == NVB ? 0 : staged_v + 1;
+    };
+
+    // A round has two halves with a barrier after each.  In the first a wave multiplies: the scores of
+    // tile t, and the values of tile t-1 into the output.  In the second it turns the scores of tile t
+    // into probabilities and moves the next tile into LDS.  With KS == 2 the waves of the later keys
+    // run half a round behind the others, so that on every SIMD one wave multiplies while the other
+    // exponentiates.
+    //
+    // The running maximum is kept on the raw scores; the scale (with log2 e folded in) enters inside
+    // the exponential's argument, one multiply-add an element.  The output is rescaled only when some
+    // query's maximum has grown.
+    f32x16 s[KT];
+    ap_frag pb[KT][2];               // probabilities of the tile before, rounded: [kt][half] is 16 keys
+    const int v_corner = (32 * kt0 + 4 * h + ((lane & 15) >> 2)) * VROW + (lane & 16) + 4 * (lane & 3);
+    // The multiplying half of a round: O^T += V^T . P^T for the tile before (sixteen keys a product:
+    // pb[kt][half] holds the keys 32*(kt0+kt) + 16*half + {4h..4h+3} and + 8 + {4h..4h+3}; 16 lanes read a
+    // block of 4 keys x 16 head elements transposed), and the scores of this tile, transposed:
+    // s[kt][4*j + i] is key k0 + 32*(kt0+kt) + 8*j + 4*h + i against query r32.  For heads up to 128 all
+    // operands are asked for before the first product, values first, so that LDS is waited for once.
+    auto multiply = [&](int kbuf, int vbuf, bool with_scores) {
+        const uint16_t* Ks = Kbase + kbuf * KTILE;
+        const uint16_t* Vs = Vbase + vbuf * VTILE + v_corner;
+        if constexpr (DT <= 4 && KT == 1) {
+            ap_frag va[2][DT], ka[2 * DT];
+            auto ask_values = [&](int half, int dt) {
+                const uint16_t* block = Vs + 16 * half * VROW + 32 * dt;
+                va[half][dt].half[0] = ap_read_transposed(block);
+                va[half][dt].half[1] = ap_read_transposed(block + 8 * VROW);
+            };
+            // The scores first (they are done when the softmax asks for them, while the last products
+            // of the values still run), and the values asked for between their products: the reads
+            // of LDS go on while the matrix cores work.
+            if (with_scores) {
+#pragma unroll
+                for (int kk = 0; kk < 2 * DT; ++kk)
+                    ka[kk].raw = *reinterpret_cast<const ap_u32x4*>(Ks + (32 * kt0 + r32) * KROW + 16 * kk + 8 * h);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s[0][r] = 0.f;
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int kk = 0; kk < 2 * DT; ++kk) {
+                    s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk].vec, qf[kk].vec, s[0], 0, 0, 0);
+                    ask_values(kk / DT, kk % DT);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+#pragma unroll
+                for (int kk = 0; kk < 2 * DT; ++kk) ask_values(kk / DT, kk % DT);
+            }
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+                    o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[half][dt].vec, pb[0][half].vec, o[dt], 0, 0, 0);
+        } else {
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    ap_frag a[DT];
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) {
+                        const uint16_t* block = Vs + (32 * kt + 16 * half) * VROW + 32 * dt;
+                        a[dt].half[0] = ap_read_transposed(block);
+                        a[dt].half[1] = ap_read_transposed(block + 8 * VROW);
+                    }
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt)
+                        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[dt].vec, pb[kt][half].vec, o[dt], 0, 0, 0);
+                }
+            if (with_scores) {
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) s[kt][r] = 0.f;
+                    ap_frag a[2 * DT];
+#pragma unroll
+                    for (int kk = 0; kk < 2 * DT; ++kk)
+                        a[kk].raw = *reinterpret_cast<const ap_u32x4*>(Ks + (32 * (kt0 + kt) + r32) * KROW + 16 * kk + 8 * h);
+#pragma unroll
+                    for (int kk = 0; kk < 2 * DT; ++kk)
+                        s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kk].vec, qf[kk].vec, s[kt], 0, 0, 0);
+                }
+            }
+        }
+    };
+    auto soften = [&](int k0, bool masked) {
         float mx = -INFINITY;
         if (masked) {
             // Key k0 + c + 4*h, c a constant of the register, is seen by this lane's query iff c <= reach
@@ -290,7 +421,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         const float shift = -m_use * scale_log2e;
         float psum = 0.f;
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt)
+        for (int kt = 0; kt < KT; ++kt) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 // v_exp_f32: arguments are <= 0, tiny results may flush
@@ -298,61 +429,77 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
                 s[kt][r] = p;
                 psum += p;
             }
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int w = 0; w < 4; ++w)
+                    pb[kt][half].w[w] = ap_pack2(s[kt][8 * half + 2 * w], s[kt][8 * half + 2 * w + 1]);
+        }
         lsum += psum;
-
-        // O^T += V^T . P^T, sixteen keys a product: registers 8*half .. 8*half+7 of tile kt are the
-        // keys 32*(kt0+kt) + 16*half + {4h..4h+3} and + 8 + {4h..4h+3}
-#pragma unroll
-        for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                ap_frag b;
-#pragma unroll
-                for (int w = 0; w < 4; ++w) b.w[w] = ap_pack2(s[kt][8 * half + 2 * w], s[kt][8 * half + 2 * w + 1]);
-                ap_frag a[DT];
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
-                    const uint16_t* block = Vs + (32 * kt + 16 * half) * VROW + 32 * dt;
-                    a[dt].half[0] = ap_read_transposed(block);
-                    a[dt].half[1] = ap_read_transposed(block + 8 * VROW);
-                }
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-                    o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[dt].vec, b.vec, o[dt], 0, 0, 0);
-            }
     };
 
-    // The registers hold the next tile: it goes into the buffer that nobody reads now (its readers
-    // passed the barrier that ended the round before), and the tile after it is asked for.
-    auto advance = [&](int k0, int cur) {
-        stash(cur ^ 1);
-        fetch();
-        lookup(k0 + 3 * AP_BN);
+    // The end of half a round: the products stay on their side of the barrier (the compiler would let
+    // them drift behind it, into the half that should run beside another wave's products).
+    auto half_done = [&]() {
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
     };
-
+    const bool behind_group = KS == 2 && kt0 != 0;
+    if (behind_group) {              // half a round in which the later group only moves a tile
+        look_ahead(k_first + (staged + 2) * AP_BN);
+        advance();
+        half_done();
+    }
     // First the tiles that every query of the workgroup sees whole: no masks, no wave stands idle
     // (a wave past the request's last token works on zero queries and stores nothing).  Then the
     // few tiles around the diagonal, where keys are hidden and waves of early tokens are done.
-    int cur = 0, k0 = k_first;
+    // A tile that left no probabilities (the one before the first, one a wave sat out) left zeros:
+    // the values are multiplied in every round.
+    int k0 = k_first, kbuf = 0, vbuf_before = 0;   // vbuf_before: where the values of the tile before lie
+    auto no_weights = [&]() {
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int w = 0; w < 4; ++w) pb[kt][half].w[w] = 0u;
+    };
+    no_weights();
     const int open_end = window > 0 ? k_first : ((start + q0 + 1) / AP_BN) * AP_BN;   // keys below it are seen by all
-    for (; k0 < open_end; k0 += AP_BN, cur ^= 1) {
-        advance(k0, cur);
-        one_tile(k0, cur, false);
-        __syncthreads();  // this tile has been read, the next one written
+    auto next_tile = [&]() {
+        if (k0 != k_first) vbuf_before = vbuf_before + 1 == NVB ? 0 : vbuf_before + 1;
+        k0 += AP_BN;
+        kbuf ^= 1;
+    };
+    for (; k0 < open_end; next_tile()) {
+        multiply(kbuf, vbuf_before, true);
+        half_done();
+        look_ahead(k_first + (staged + 2) * AP_BN);
+        soften(k0, false);
+        advance();
+        half_done();
     }
-    for (; k0 <= last_pos; k0 += AP_BN, cur ^= 1) {
-        advance(k0, cur);
+    for (; k0 <= last_pos; next_tile()) {
         // a wave whose queries all stand before this tile, or that has no queries, has nothing to add
         const bool idle = !wave_active || k0 + 32 * kt0 > wave_last ||
                           (window > 0 && k0 + 32 * (kt0 + KT) - 1 <= wave_first - window);
-        if (!idle) one_tile(k0, cur, true);
-        __syncthreads();
+        multiply(kbuf, vbuf_before, !idle);
+        half_done();
+        look_ahead(k_first + (staged + 2) * AP_BN);
+        if (!idle) soften(k0, true);
+        else no_weights();
+        advance();
+        half_done();
     }
+    multiply(kbuf, vbuf_before, false);
+    if (KS == 2 && !behind_group) half_done();   // the later group is half a round behind
     lsum += __shfl_xor(lsum, 32, PL_WAVE);
     if (KS == 2) {
         // The wave of the later keys hands its state to the wave of the earlier ones through LDS
         // (the tiles are done with): out = (o0 2^(m0-M) + o1 2^(m1-M)) / (l0 2^(m0-M) + l1 2^(m1-M)).
         float* hand = reinterpret_cast<float*>(lds) + static_cast<size_t>(wave) * (16 * DT + 2) * PL_WAVE;
+        __syncthreads();             // the tiles are done with in every wave
         if (kt0 != 0) {
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
@@ -392,30 +539,60 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         }
 }
 
-template <int DT, int NW, int KS>
+template <int DT, int NW, int KS, bool UP>
 static int launch_prefill(const void* q, int q_stride, void* out, const int* q_start, const int* q_len,
                           const int* ctx_len, int short_limit, int num_seqs, int max_q_len, const int* block_table,
                           int max_blocks, int block_size, const void* k_pool, const void* v_pool, int nq, int nkv,
                           int d, float scale, int window, hipStream_t stream) {
     constexpr int DP = 32 * DT;
     constexpr int BM = 32 * NW;
-    const size_t tile_bytes = 2 * (static_cast<size_t>(AP_BN) * (DP + AP_KPAD) + static_cast<size_t>(AP_BN) * (DP + ap_vpad(DT))) * 2;
+    const size_t tile_bytes = (2 * static_cast<size_t>(AP_BN) * (DP + AP_KPAD) +
+                               ap_value_buffers(KS) * static_cast<size_t>(AP_BN) * (DP + ap_vpad(DT))) * 2;
     const size_t hand_bytes = KS == 2 ? static_cast<size_t>(NW) * (16 * DT + 2) * PL_WAVE * sizeof(float) : 0;
     const size_t lds_bytes = tile_bytes > hand_bytes ? tile_bytes : hand_bytes;
     if (lds_bytes > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_prefill_kernel<DT, NW, KS>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_prefill_kernel<DT, NW, KS, UP>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
         PL_REQUIRE(e == hipSuccess, "prefill attention: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
     }
     const int tiles = pl_ceil_div(max_q_len, BM);
     const long long total = static_cast<long long>(tiles) * nq * num_seqs;
     PL_REQUIRE(total > 0 && total < (1ll << 30), "prefill attention: %lld workgroups", total);
-    paged_attention_prefill_kernel<DT, NW, KS><<<static_cast<int>(total), 64 * NW * KS, lds_bytes, stream>>>(
+    paged_attention_prefill_kernel<DT, NW, KS, UP><<<static_cast<int>(total), 64 * NW * KS, lds_bytes, stream>>>(
         static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), q_start, q_len, ctx_len, short_limit, tiles,
         num_seqs, block_table, max_blocks, block_size, static_cast<const bf16_t*>(k_pool),
         static_cast<const bf16_t*>(v_pool), nq, nkv, d, scale * 1.4426950408889634f, window, static_cast<int>(total));
     PL_CHECK_LAUNCH("paged_attention_prefill");
     return 0;
+}
+
+template <int D>
+static int ap_dispatch(bool small, bool uniform_pages, const void* q, int q_stride, void* out, const int* q_start,
+                       const int* q_len, const int* ctx_len, int short_limit, int num_seqs, int max_q_len,
+                       const int* block_table, int max_blocks, int block_size, const void* k_pool, const void* v_pool,
+                       int nq, int nkv, int d, float scale, int window, hipStream_t stream) {
+#define AP_LAUNCH(NW, KS, UP)                                                                                      \
+    launch_prefill<D, NW, KS, UP>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len,    \
+                                  block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale, window, stream)
+    constexpr bool can_fit = 64 % (4 * D) == 0;
+    if constexpr (D <= 4) {
+        if (small) {
+            if constexpr (can_fit) {
+                if (uniform_pages) return AP_LAUNCH(2, AP_SMALL_KS, true);
+            }
+            return AP_LAUNCH(2, AP_SMALL_KS, false);
+        }
+        if constexpr (can_fit) {
+            if (uniform_pages) return AP_LAUNCH(4, AP_KS, true);
+        }
+        return AP_LAUNCH(4, AP_KS, false);
+    } else {
+        if constexpr (can_fit) {
+            if (uniform_pages) return AP_LAUNCH(4, 1, true);
+        }
+        return AP_LAUNCH(4, 1, false);
+    }
+#undef AP_LAUNCH
 }
 
 // bfloat16 only.  q rows begin with the nq*d rotated query values; request s brings the rows
@@ -441,13 +618,11 @@ extern "C" int pl_paged_attention_prefill(const void* q, int q_stride, void* out
     // half the threads have twice the pieces of a tile to carry each: large heads leave them no registers for that
     const bool small = max_q_len <= 64 && dt <= 4;
 #endif
+    // one instruction of a wave loads 64 / (4*D) keys: they share a page when pages are a power of two that large
+    const bool pages_fit = (block_size & (block_size - 1)) == 0 && block_size * 4 * dt >= 64 && 64 % (4 * dt) == 0;
 #define AP_CALL(D)                                                                                                 \
-    return small ? launch_prefill<D, 2, (D <= 4 ? AP_SMALL_KS : 1)>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len, \
-                                           block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale,   \
-                                           window, stream)                                                            \
-                 : launch_prefill<D, 4, (D <= 4 ? AP_KS : 1)>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len, \
-                                               block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale,   \
-                                               window, stream)
+    return ap_dispatch<D>(small, pages_fit, q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len, \
+                          block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale, window, stream)
     switch (dt) {
         case 1: AP_CALL(1);
         case 2: AP_CALL(2);
