@@ -353,6 +353,91 @@ qk_norm_rope_kv_write_wide_kernel(
     }
 }
 
+// Heads of 128 elements that are rotated whole: a head is a row of 16 lanes, so the sum of squares
+// and the exchange with the rotation's partner (8 lanes further on or back) go through the lanes'
+// own data paths (DPP) instead of LDS.  One wave works on four heads of a token, a workgroup on 16.
+__device__ __forceinline__ float qk_dpp_quad_xor1(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true));   // quad_perm [1,0,3,2]
+}
+__device__ __forceinline__ float qk_dpp_quad_xor2(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true));   // quad_perm [2,3,0,1]
+}
+__device__ __forceinline__ float qk_dpp_half_mirror(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, true));  // lane i of 8 takes 7-i
+}
+__device__ __forceinline__ float qk_dpp_mirror(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, true));  // lane i of 16 takes 15-i
+}
+__device__ __forceinline__ float qk_dpp_ror8(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, true));  // lane i of 16 takes i^8
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+qk_norm_rope_kv_write_128_kernel(
+    T* __restrict__ qkv, const void* __restrict__ q_gain, const void* __restrict__ k_gain,
+    int gain_dtype, float eps, const float* __restrict__ cos_table,
+    const float* __restrict__ sin_table, const int* __restrict__ positions,
+    const int* __restrict__ seq_of, const int* __restrict__ block_table, int max_blocks,
+    int block_size, T* __restrict__ k_pool, T* __restrict__ v_pool, int nq, int nkv, int heads) {
+    constexpr int D = 128;
+    const int t = blockIdx.x;
+    const int pos = positions[t];
+    if (pos < 0) return;
+    const int hd = blockIdx.y * 16 + threadIdx.x / 16;     // this lane's head
+    const int chunk = threadIdx.x % 16;                    // its eight elements of the head
+    const bool active = hd < heads;
+    const int hh = active ? hd : 0;
+    const bool is_q = hh < nq, is_k = !is_q && hh < nq + nkv;
+    T* src = qkv + static_cast<size_t>(t) * (nq + 2 * nkv) * D + static_cast<size_t>(hh) * D + chunk * 8;
+    float x[8];
+    qk_vec<T>::load(src, x);
+    const int blk = block_table[static_cast<size_t>(seq_of[t]) * max_blocks + pos / block_size];
+
+    const bool low = chunk < 8;
+    const void* gain = is_q ? q_gain : k_gain;
+    float g[8], c[8], sn[8];
+    if (gain && !(!is_q && !is_k)) {
+        if (gain_dtype == PL_DTYPE_F32) qk_vec<float>::load(static_cast<const float*>(gain) + chunk * 8, g);
+        else qk_vec<bf16_t>::load(static_cast<const bf16_t*>(gain) + chunk * 8, g);
+    }
+    if (cos_table) {
+        const size_t at = static_cast<size_t>(pos) * (D / 2) + (chunk & 7) * 8;
+        qk_vec<float>::load(cos_table + at, c);
+        qk_vec<float>::load(sin_table + at, sn);
+    }
+
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss = fmaf(x[e], x[e], ss);
+    ss += qk_dpp_quad_xor1(ss);
+    ss += qk_dpp_quad_xor2(ss);
+    ss += qk_dpp_half_mirror(ss);
+    ss += qk_dpp_mirror(ss);
+    const bool is_v = !is_q && !is_k;
+    if (gain && !is_v) {
+        const float denom = sqrtf(ss / static_cast<float>(D) + eps);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = x[e] / denom * g[e];
+    }
+    if (cos_table) {
+        float px[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) px[e] = qk_dpp_ror8(x[e]);
+        if (!is_v) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = low ? x[e] * c[e] - px[e] * sn[e] : x[e] * c[e] + px[e] * sn[e];
+        }
+    }
+    T* dst = src;
+    if (!is_q) {
+        const size_t slot = static_cast<size_t>(blk < 0 ? 0 : blk) * block_size + pos % block_size;
+        const int kvh = is_k ? hh - nq : hh - nq - nkv;
+        dst = (is_k ? k_pool : v_pool) + (slot * nkv + kvh) * D + chunk * 8;
+    }
+    if (active && (is_q || blk >= 0)) qk_vec<T>::store(dst, x);   // never write through a hole in the table
+}
+
 extern "C" int pl_qk_norm_rope_kv_write(
     void* qkv, const void* q_gain, const void* k_gain, int gain_dtype, float eps,
     const float* cos_table, const float* sin_table, int rot, const int* positions,
@@ -367,6 +452,21 @@ extern "C" int pl_qk_norm_rope_kv_write(
     if (n <= 0) return 0;
     // Without the cache write (a layer that reads another layer's pages) only the query heads run.
     const int heads = write_kv ? nq + 2 * nkv : nq;
+    if (d == 128 && (rot == 128 || !cos_table)) {
+        dim3 rows(n, pl_ceil_div(heads, 16));
+        if (dtype == PL_DTYPE_F32)
+            qk_norm_rope_kv_write_128_kernel<float><<<rows, 256, 0, stream>>>(
+                static_cast<float*>(qkv), q_gain, k_gain, gain_dtype, eps, cos_table, sin_table, positions, seq_of,
+                block_table, max_blocks, block_size, static_cast<float*>(k_pool), static_cast<float*>(v_pool), nq, nkv, heads);
+        else if (dtype == PL_DTYPE_BF16)
+            qk_norm_rope_kv_write_128_kernel<bf16_t><<<rows, 256, 0, stream>>>(
+                static_cast<bf16_t*>(qkv), q_gain, k_gain, gain_dtype, eps, cos_table, sin_table, positions, seq_of,
+                block_table, max_blocks, block_size, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), nq, nkv, heads);
+        else
+            PL_REQUIRE(false, "qk_norm_rope: dtype code %d", dtype);
+        PL_CHECK_LAUNCH("qk_norm_rope_kv_write");
+        return 0;
+    }
     if (rot % 16 == 0) {
         // a workgroup takes two groups of 4 * (64 / (d/8)) heads of a token at a time
         const int per_group = 4 * (PL_WAVE / (d / 8));

@@ -100,7 +100,8 @@ def tables(max_pos, rot, theta):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("nq,nkv,d,bs,norm", [(4, 2, 16, 4, True), (6, 1, 48, 16, True), (3, 3, 128, 8, False),
-                                              (8, 2, 256, 2, True), (5, 5, 80, 16, True)])
+                                              (8, 2, 256, 2, True), (5, 5, 80, 16, True), (16, 8, 128, 16, True),
+                                              (7, 1, 128, 4, True)])
 def test_qk_norm_rope_kv_write(dtype, nq, nkv, d, bs, norm):
     from paged_llm_rs_amd import kernels
 
