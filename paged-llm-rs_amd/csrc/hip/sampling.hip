@@ -77,3 +77,296 @@ extern "C" int pl_argmax(const float* logits, int* out, float* scratch_v, int* s
     PL_CHECK_LAUNCH("argmax");
     return 0;
 }
+
+// ---------------------------------------------------------------------------
+// Temperature, top-k, top-p and the draw, one workgroup a row (reference:
+// crates/pagedllm/src/sampler.rs: scale, sort downwards, keep k, softmax, keep
+// the shortest head of mass top_p, walk it with one uniform number).
+//
+// Nothing is sorted here.  Every step of that recipe asks for a place in the
+// downward order at which a running sum crosses a mark: the k-th candidate (a
+// sum of ones), the candidate at which the mass reaches top_p of the total,
+// the candidate at which it reaches the drawn point.  Such a place is found by
+// two histogram passes over a 24-bit key that falls as the logit rises:
+//     key = min(2^26 - 1, (max - y) * 2^20) >> 2,   y = logit / temperature,
+// 12 bits a pass.  Logits closer than 4e-6 share a key and count as equal: they
+// are ordered by index, as equal logits are in the recipe.  Logits more than 64
+// below the maximum share the last key; their mass is zero.
+//
+// Masses are exp(y - max) in fixed point (2^40), added as integers: a sum does
+// not depend on the order of its terms, so a row and a uniform number give the
+// same token on every run.
+// ---------------------------------------------------------------------------
+#define SM_THREADS 1024
+#define SM_BINS 4096
+#define SM_NO_LIMIT 0x7fffffff
+
+struct sm_shared {
+    unsigned long long sum[SM_BINS];   // mass, or count, a bin
+    unsigned int count[SM_BINS];       // candidates a bin (second pass)
+    int first[SM_BINS];                // lowest index a bin (second pass)
+    unsigned long long wave_sum[SM_THREADS / PL_WAVE];
+    float red_v[SM_THREADS / PL_WAVE];
+    int red_i[SM_THREADS / PL_WAVE];
+    unsigned long long found_before;   // sum over the bins before the one found
+    unsigned long long found_in;       // sum of the bin found
+    int found_bin;
+    int nth_index;
+};
+
+__device__ __forceinline__ uint32_t sm_key(float y, float top) {
+    if (!(y == y)) return (1u << 24) - 1;                      // a NaN is the last candidate
+    const float t = (top - y) * 1048576.f;                      // >= 0, +inf for -inf
+    const uint32_t q = t >= 67108863.f ? 67108863u : static_cast<uint32_t>(t);
+    return q >> 2;
+}
+
+__device__ __forceinline__ unsigned long long sm_mass(float y, float top) {
+    // 2^40 * exp(y - top): zero from about 28 below the maximum on
+    const float p = __builtin_amdgcn_exp2f((y - top) * 1.4426950408889634f + 40.f);
+    return (y == y) ? static_cast<unsigned long long>(p) : 0ull;
+}
+
+// The first bin, going up, at which the running sum of sm.sum reaches `mark` (mark >= 1; the last bin
+// that holds anything if the sum never gets there).  Leaves found_bin, found_before, found_in.
+__device__ void sm_find(sm_shared& sm, unsigned long long before, unsigned long long mark) {
+    constexpr int PER = SM_BINS / SM_THREADS;                  // bins a thread
+    const int tid = threadIdx.x, lane = tid % PL_WAVE, wave = tid / PL_WAVE;
+    unsigned long long mine = 0;
+#pragma unroll
+    for (int b = 0; b < PER; ++b) mine += sm.sum[tid * PER + b];
+    // running sum over the threads of the wave, then over the waves
+    unsigned long long run = mine;
+#pragma unroll
+    for (int off = 1; off < PL_WAVE; off <<= 1) {
+        const unsigned long long other = __shfl_up(run, off, PL_WAVE);
+        if (lane >= off) run += other;
+    }
+    if (lane == PL_WAVE - 1) sm.wave_sum[wave] = run;
+    if (tid == 0) sm.found_bin = -1;
+    __syncthreads();
+    unsigned long long ahead = before;
+    for (int w = 0; w < wave; ++w) ahead += sm.wave_sum[w];
+    const unsigned long long through = ahead + run, upto = through - mine;   // sums through / before this thread's bins
+    if (upto < mark && mark <= through) {
+        unsigned long long at = upto;
+        for (int b = 0; b < PER; ++b) {
+            const unsigned long long v = sm.sum[tid * PER + b];
+            if (at + v >= mark) {
+                sm.found_bin = tid * PER + b;
+                sm.found_before = at;
+                sm.found_in = v;
+                break;
+            }
+            at += v;
+        }
+    }
+    __syncthreads();
+    if (sm.found_bin < 0) {                                     // the mark lies past the total: the last bin in use
+        if (tid == SM_THREADS - 1) {
+            unsigned long long total = through;
+            int b = SM_BINS - 1;
+            while (b > 0 && sm.sum[b] == 0) --b;
+            sm.found_bin = b;
+            sm.found_in = sm.sum[b];
+            unsigned long long tail = 0;
+            for (int c = b; c < SM_BINS; ++c) tail += sm.sum[c];
+            sm.found_before = total - tail;
+        }
+        __syncthreads();
+    }
+}
+
+// Which candidates are still in: keys below `key`, and of that key the indices below `limit`.
+struct sm_kept {
+    uint32_t key;
+    int limit;
+    __device__ __forceinline__ bool has(uint32_t k, int i) const { return k < key || (k == key && i < limit); }
+};
+
+// The place, in the order of key then index, at which the running sum of `weight` over the kept
+// candidates reaches `mark`.  Returns the key found; `limit` becomes the index after the candidate at
+// which the mark is reached, `before` the sum over the kept candidates of lower keys, `through` the sum
+// up to and with that candidate, and `token` that candidate.  WEIGHTED: masses, else ones.
+template <bool WEIGHTED>
+__device__ uint32_t sm_select(sm_shared& sm, const float* __restrict__ x, int V, float inverse, float top, sm_kept kept,
+                              unsigned long long mark, int& limit, unsigned long long& through, int& token) {
+    const int tid = threadIdx.x;
+    // first pass: the upper 12 bits
+    for (int b = tid; b < SM_BINS; b += SM_THREADS) sm.sum[b] = 0;
+    __syncthreads();
+    for (int i = tid; i < V; i += SM_THREADS) {
+        const float y = x[i] * inverse;
+        const uint32_t k = sm_key(y, top);
+        if (!kept.has(k, i)) continue;
+        const unsigned long long w = WEIGHTED ? sm_mass(y, top) : 1ull;
+        if (w) atomicAdd(&sm.sum[k >> 12], w);
+    }
+    __syncthreads();
+    sm_find(sm, 0, mark);
+    const uint32_t upper = sm.found_bin;
+    const unsigned long long before_upper = sm.found_before;
+    __syncthreads();
+    // second pass: the lower 12 bits of the candidates of that bin
+    for (int b = tid; b < SM_BINS; b += SM_THREADS) {
+        sm.sum[b] = 0;
+        sm.count[b] = 0;
+        sm.first[b] = SM_NO_LIMIT;
+    }
+    __syncthreads();
+    for (int i = tid; i < V; i += SM_THREADS) {
+        const float y = x[i] * inverse;
+        const uint32_t k = sm_key(y, top);
+        if ((k >> 12) != upper || !kept.has(k, i)) continue;
+        const unsigned long long w = WEIGHTED ? sm_mass(y, top) : 1ull;
+        if (!WEIGHTED || w) {
+            atomicAdd(&sm.sum[k & 0xfff], w);
+            atomicAdd(&sm.count[k & 0xfff], 1u);
+            atomicMin(&sm.first[k & 0xfff], i);
+        }
+    }
+    __syncthreads();
+    sm_find(sm, before_upper, mark);
+    const uint32_t key = (upper << 12) | static_cast<uint32_t>(sm.found_bin);
+    const unsigned long long before = sm.found_before, in_bin = sm.found_in;
+    const unsigned int many = sm.count[sm.found_bin];
+    const int lowest = sm.first[sm.found_bin];
+    __syncthreads();
+    if (many <= 1) {                                            // the usual case: one candidate has this key
+        limit = many == 1 ? lowest + 1 : SM_NO_LIMIT;
+        through = before + in_bin;
+        token = many == 1 ? lowest : 0;
+        return key;
+    }
+    // Several candidates share the key: they are walked in the order of their indices, a stretch of
+    // SM_THREADS indices at a time, until the running sum reaches the mark.
+    unsigned long long run = before;
+    if (tid == 0) sm.nth_index = -1;
+    __syncthreads();
+    const int lane = tid % PL_WAVE, wave = tid / PL_WAVE;
+    for (int base = 0; base < V; base += SM_THREADS) {
+        const int i = base + tid;
+        unsigned long long w = 0;
+        if (i < V) {
+            const float y = x[i] * inverse;
+            const uint32_t k = sm_key(y, top);
+            if (k == key && kept.has(k, i)) w = WEIGHTED ? sm_mass(y, top) : 1ull;
+        }
+        unsigned long long scan = w;
+#pragma unroll
+        for (int off = 1; off < PL_WAVE; off <<= 1) {
+            const unsigned long long other = __shfl_up(scan, off, PL_WAVE);
+            if (lane >= off) scan += other;
+        }
+        if (lane == PL_WAVE - 1) sm.wave_sum[wave] = scan;
+        __syncthreads();
+        unsigned long long ahead = run, all = 0;
+        for (int v = 0; v < SM_THREADS / PL_WAVE; ++v) {
+            if (v < wave) ahead += sm.wave_sum[v];
+            all += sm.wave_sum[v];
+        }
+        const unsigned long long mine_through = ahead + scan;
+        if (w && mine_through - w < mark && mark <= mine_through) {
+            sm.nth_index = i;
+            sm.found_before = mine_through;
+        }
+        __syncthreads();
+        if (sm.nth_index >= 0) break;
+        run += all;
+        __syncthreads();
+    }
+    if (sm.nth_index >= 0) {
+        limit = sm.nth_index + 1;
+        through = sm.found_before;
+        token = sm.nth_index;
+    } else {                                                    // the mark lies past them all: all are kept, the last is drawn
+        limit = SM_NO_LIMIT;
+        through = before + in_bin;
+        token = lowest;
+    }
+    __syncthreads();
+    return key;
+}
+
+__global__ void __launch_bounds__(SM_THREADS)
+sample_rows_kernel(const float* __restrict__ logits, const float* __restrict__ temperature, const int* __restrict__ top_k,
+                   const float* __restrict__ top_p, const float* __restrict__ uniform, int* __restrict__ out, int V) {
+    __shared__ sm_shared sm;
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const float* x = logits + static_cast<size_t>(row) * V;
+    const float temp = temperature[row];
+    // the largest logit and its first index
+    float bv = -INFINITY;
+    int bi = SM_NO_LIMIT;
+    for (int i = tid; i < V; i += SM_THREADS) better(bv, bi, x[i], i);
+#pragma unroll
+    for (int off = PL_WAVE / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, PL_WAVE);
+        const int oi = __shfl_xor(bi, off, PL_WAVE);
+        better(bv, bi, ov, oi);
+    }
+    if (tid % PL_WAVE == 0) {
+        sm.red_v[tid / PL_WAVE] = bv;
+        sm.red_i[tid / PL_WAVE] = bi;
+    }
+    __syncthreads();
+    bv = sm.red_v[0];
+    bi = sm.red_i[0];
+    for (int w = 1; w < SM_THREADS / PL_WAVE; ++w) better(bv, bi, sm.red_v[w], sm.red_i[w]);
+    __syncthreads();
+    if (!(temp > 0.f) || bi == SM_NO_LIMIT) {                   // greedy, or a row of NaNs
+        if (tid == 0) out[row] = bi == SM_NO_LIMIT ? 0 : bi;
+        return;
+    }
+    const float inverse = 1.0f / temp;
+    const float top = bv * inverse;
+
+    sm_kept kept{(1u << 24), SM_NO_LIMIT};                      // everything
+    int limit, token;
+    unsigned long long through;
+    const int k = top_k[row];
+    if (k > 0 && k < V) {
+        const uint32_t key = sm_select<false>(sm, x, V, inverse, top, kept, static_cast<unsigned long long>(k), limit, through, token);
+        kept = sm_kept{key, limit};
+    }
+    // the mass of what is kept: the sum of a first pass over it
+    for (int b = tid; b < SM_BINS; b += SM_THREADS) sm.sum[b] = 0;
+    __syncthreads();
+    {
+        unsigned long long mine = 0;
+        for (int i = tid; i < V; i += SM_THREADS) {
+            const float y = x[i] * inverse;
+            if (kept.has(sm_key(y, top), i)) mine += sm_mass(y, top);
+        }
+#pragma unroll
+        for (int off = PL_WAVE / 2; off > 0; off >>= 1) mine += __shfl_xor(mine, off, PL_WAVE);
+        if (tid % PL_WAVE == 0) sm.wave_sum[tid / PL_WAVE] = mine;
+    }
+    __syncthreads();
+    unsigned long long total = 0;
+    for (int w = 0; w < SM_THREADS / PL_WAVE; ++w) total += sm.wave_sum[w];
+    __syncthreads();
+    const float p = top_p[row];
+    if (p < 1.f) {
+        unsigned long long mark = static_cast<unsigned long long>(static_cast<double>(p) * static_cast<double>(total));
+        mark = mark < 1 ? 1 : (mark > total ? total : mark);
+        const uint32_t key = sm_select<true>(sm, x, V, inverse, top, kept, mark, limit, through, token);
+        kept = sm_kept{key, limit};
+        total = through;                                        // the candidate that crosses the mark is kept
+    }
+    unsigned long long mark = static_cast<unsigned long long>(static_cast<double>(uniform[row]) * static_cast<double>(total));
+    mark = mark < 1 ? 1 : (mark > total ? total : mark);
+    sm_select<true>(sm, x, V, inverse, top, kept, mark, limit, through, token);
+    if (tid == 0) out[row] = token;
+}
+
+// One token a row.  temperature <= 0: the largest logit (the first of equals).  top_k <= 0 or >= V and
+// top_p >= 1 switch the cuts off.  uniform: a number in [0, 1) a row, the request's own draw.
+extern "C" int pl_sample(const float* logits, const float* temperature, const int* top_k, const float* top_p,
+                         const float* uniform, int* out, int m, int V, hipStream_t stream) {
+    PL_REQUIRE(m >= 0 && V > 0, "sampling: rows %d, vocabulary %d", m, V);
+    if (m == 0) return 0;
+    sample_rows_kernel<<<m, SM_THREADS, 0, stream>>>(logits, temperature, top_k, top_p, uniform, out, V);
+    PL_CHECK_LAUNCH("sample");
+    return 0;
+}

@@ -16,6 +16,7 @@ from typing import Optional
 
 import torch
 
+from .. import kernels
 from ..cache import PagedCache
 from ..config import GenerationConfig
 from ..errors import ConfigError, PagedLLMError
@@ -146,27 +147,26 @@ class Engine:
     # -- the loop ---------------------------------------------------------------------------
 
     def _choose(self, plan, output) -> list:
-        """One token per id of the plan.  Greedy rows are an argmax on the device;
-        the logits of the others go to the host sampler with the request's generator."""
+        """One token per id of the plan.  On the device (the default) greedy rows are an argmax and
+        the others are drawn by the sampling kernel with the next number of the request's generator;
+        with ``sampler="host"`` the logits go to the host sampler instead."""
         if not plan.ids:
             return []      # a portion in the middle of a prompt: the logits have no rows and are not touched
         logits = output.logits
         if logits.shape[0] != len(plan.ids):
             raise PagedLLMError(f"{logits.shape[0]} rows of logits for {len(plan.ids)} requests")
         greedy = [self._greedy.get(i, True) for i in plan.ids]
-        chosen = [0] * len(plan.ids)
-        if self.sampler == "device" and any(greedy):
-            picked = output.greedy_tokens().cpu().tolist()
-            for row, g in enumerate(greedy):
-                if g:
-                    chosen[row] = picked[row]
-        rows_on_host = [r for r, g in enumerate(greedy) if not (g and self.sampler == "device")]
-        if rows_on_host:
-            index = torch.tensor(rows_on_host, device=logits.device)
-            host = logits.index_select(0, index).cpu().numpy()
-            for k, row in enumerate(rows_on_host):
-                chosen[row] = self.scheduler.sample_on_host(plan.ids[row], host[k])
-        return chosen
+        if self.sampler == "device":
+            if all(greedy):
+                return output.greedy_tokens().cpu().tolist()
+            how = [self.scheduler.sampling_of(i) for i in plan.ids]     # draws the number of a request that samples
+            params = torch.tensor([[t, float(k), p, u] for t, k, p, u in how], dtype=torch.float32).pin_memory()
+            params = params.to(logits.device, non_blocking=True)
+            picked = kernels.sample(logits, params[:, 0].contiguous(), params[:, 1].to(torch.int32).contiguous(),
+                                    params[:, 2].contiguous(), params[:, 3].contiguous())
+            return picked.cpu().tolist()
+        host = logits.cpu().numpy()
+        return [self.scheduler.sample_on_host(i, host[row]) for row, i in enumerate(plan.ids)]
 
     def step(self):
         """One iteration.  Returns the outcome, or None when there is nothing to run."""

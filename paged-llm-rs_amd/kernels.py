@@ -35,6 +35,7 @@ def _signatures(lib) -> None:
         "pl_gemm_plain": [p, p, p, i, i, i, i, i, i, i, p],
         "pl_paged_attention_plain": [p, i, p, p, p, p, i, i, p, p, i, i, i, i, f, i, i, p],
         "pl_argmax": [p, p, p, p, i, i, p],
+        "pl_sample": [p, p, p, p, p, p, i, i, p],
         "pl_gemm_skinny": [p, p, p, p, f, p, i, i, i, i, i, p],
         "pl_paged_attention_decode": [p, i, p, p, p, p, p, p, i, p, i, i, p, p, i, i, i, i, f, i, i,
                                       i, p, p, i, f, p, p, i, p],
@@ -238,6 +239,26 @@ def argmax(logits: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tenso
     scratch_i = torch.empty((m * 64,), dtype=torch.int32, device=logits.device)
     _check(library().pl_argmax(logits.data_ptr(), out.data_ptr(), scratch_v.data_ptr(), scratch_i.data_ptr(),
                                m, V, _stream()))
+    return out
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+           uniform: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """One token a row: logits / temperature, the k most likely, of those the shortest head
+    whose mass reaches top_p, and of that the token on which the mass reaches uniform * total,
+    all in the order of falling logit and rising index (reference: crates/pagedllm/src/sampler.rs).
+    A row with temperature 0 takes its largest logit.  top_k 0 and top_p 1 cut nothing."""
+    m, V = logits.shape
+    _need(logits, "logits", None, torch.float32)
+    _need(temperature, "temperatures", (m,), torch.float32)
+    _need(top_k, "top_k", (m,), torch.int32)
+    _need(top_p, "top_p", (m,), torch.float32)
+    _need(uniform, "uniform numbers", (m,), torch.float32)
+    if out is None:
+        out = torch.empty((m,), dtype=torch.int32, device=logits.device)
+    _need(out, "chosen tokens", (m,), torch.int32)
+    _check(library().pl_sample(logits.data_ptr(), temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(),
+                               uniform.data_ptr(), out.data_ptr(), m, V, _stream()))
     return out
 
 

@@ -533,3 +533,99 @@ def test_argmax_first_maximum_wins():
     assert got[4] == int(torch.argmax(logits[4]))
     small = torch.tensor([[1.0, 3.0, 3.0, 2.0]], device=DEV)
     assert kernels.argmax(small).item() == 1
+
+
+def sampling_recipe(x, temperature, top_k, top_p, u, band=1e-5, slack=2e-5):
+    """The tokens the recipe allows (reference: crates/pagedllm/src/sampler.rs): scale, order by falling
+    logit and rising index, keep k, softmax, keep the head of mass top_p, walk it to u * total.  Logits
+    closer than `band` may stand in either order, and sums may differ by `slack` of the total."""
+    import numpy as np
+    y = (x.astype(np.float32) * np.float32(1.0 / temperature)).astype(np.float64)
+    order = np.lexsort((np.arange(y.size), -y))
+    if top_k and top_k < y.size:
+        order = order[:top_k]
+    mass = np.exp(y[order] - y[order[0]])
+    if top_p < 1.0:
+        running = np.cumsum(mass)
+        kept = int(np.searchsorted(running, top_p * running[-1], side="left")) + 1
+        order, mass = order[:kept], mass[:kept]
+    total = mass.sum()
+    point = float(np.float32(u)) * total
+    allowed = set()
+    ys = y[order]
+    for j, token in enumerate(order):
+        before = mass[ys > ys[j] + band].sum()          # what surely stands before it
+        through = mass[ys >= ys[j] - band].sum()        # what may stand before it, and itself
+        if before <= point + slack * total and point - slack * total <= through:
+            allowed.add(int(token))
+    return allowed, set(int(t) for t in order)
+
+
+def test_sampling_kernel_follows_the_recipe():
+    import numpy as np
+    from paged_llm_rs_amd import kernels
+    from paged_llm_rs_amd.sampling.sampler import Rng, Sampling, sample_host
+
+    g = torch.Generator().manual_seed(11)
+    V = 15193     # not a multiple of the workgroup
+    cases = [(0.7, 0, 1.0), (1.0, 50, 1.0), (1.3, 0, 0.9), (0.8, 40, 0.95), (2.0, 5, 0.5), (0.0, 0, 1.0),
+             (1.0, V + 5, 1.0), (0.05, 0, 0.3), (5.0, 3000, 0.999)]
+    rows, how = [], []
+    for rep in range(6):
+        for t, k, p in cases:
+            rows.append(torch.randn(V, generator=g) * (1.0 + rep))
+            how.append((t, k, p, float(torch.rand((), generator=g))))
+    logits = torch.stack(rows).to(DEV)
+    as_f = lambda col: torch.tensor([h[col] for h in how], dtype=torch.float32, device=DEV)
+    got = kernels.sample(logits, as_f(0), torch.tensor([h[1] for h in how], dtype=torch.int32, device=DEV), as_f(2),
+                         as_f(3)).cpu().tolist()
+    again = kernels.sample(logits, as_f(0), torch.tensor([h[1] for h in how], dtype=torch.int32, device=DEV), as_f(2),
+                           as_f(3)).cpu().tolist()
+    assert got == again, "a row and a number give the same token on every run"
+    same_as_host = 0
+    for row, (t, k, p, u) in enumerate(how):
+        x = logits[row].cpu().numpy()
+        if t == 0.0:
+            assert got[row] == int(np.argmax(x))
+            continue
+        allowed, kept = sampling_recipe(x, t, k, p, u)
+        assert got[row] in kept, f"row {row} {how[row]}: token {got[row]} had been cut"
+        assert got[row] in allowed, f"row {row} {how[row]}: token {got[row]}, the recipe allows {sorted(allowed)}"
+    # the host sampler and the kernel, fed the same numbers of the same generator
+    rng_a, rng_b = Rng(77), Rng(77)
+    us = [rng_a.next_f32() if h[0] > 0 else 0.0 for h in how]      # a greedy row draws nothing
+    got2 = kernels.sample(logits, as_f(0), torch.tensor([h[1] for h in how], dtype=torch.int32, device=DEV), as_f(2),
+                          torch.tensor(us, dtype=torch.float32, device=DEV)).cpu().tolist()
+    for row, (t, k, p, _) in enumerate(how):
+        if t == 0.0:
+            continue
+        host = sample_host(Sampling(t, k or None, p if p < 1.0 else None), logits[row].cpu().numpy(), rng_b)
+        same_as_host += int(host == got2[row])
+    drawn = sum(1 for h in how if h[0] > 0)
+    assert same_as_host >= drawn - 1, f"{same_as_host} of {drawn} tokens are the host sampler's"
+
+
+def test_sampling_kernel_on_rows_made_by_hand():
+    from paged_llm_rs_amd import kernels
+
+    V = 1000
+    probs = {17: 0.5, 900: 0.25, 3: 0.15, 512: 0.10}
+    row = torch.full((V,), -1000.0)
+    for token, p in probs.items():
+        row[token] = math.log(p)
+    flat = torch.zeros(V)             # all equal: the order is that of the indices
+    cases = [
+        (row, 1.0, 0, 1.0, 0.10, 17), (row, 1.0, 0, 1.0, 0.49, 17), (row, 1.0, 0, 1.0, 0.51, 900),
+        (row, 1.0, 0, 1.0, 0.76, 3), (row, 1.0, 0, 1.0, 0.95, 512), (row, 1.0, 0, 1.0, 0.0, 17),
+        (row, 1.0, 2, 1.0, 0.70, 900),          # of 0.75 kept: 0.525 > 0.5
+        (row, 1.0, 0, 0.6, 0.70, 900),          # 0.5 < 0.6: the second crosses and is kept
+        (row, 1.0, 0, 0.45, 0.99, 17),          # the first reaches 0.45 by itself
+        (row, 1.0, 3, 0.8, 0.99, 900),          # k keeps three (0.9), p two of them (0.72 of 0.9 is crossed at 0.75)
+        (flat, 1.0, 0, 1.0, 0.3705, 370), (flat, 0.5, 10, 1.0, 0.55, 5), (flat, 2.0, 0, 0.25, 0.5, 124),
+        (flat, 0.0, 0, 1.0, 0.9, 0),
+    ]
+    logits = torch.stack([c[0] for c in cases]).to(DEV)
+    col = lambda j, dt: torch.tensor([c[j] for c in cases], dtype=dt, device=DEV)
+    got = kernels.sample(logits, col(1, torch.float32), col(2, torch.int32), col(3, torch.float32),
+                         col(4, torch.float32)).cpu().tolist()
+    assert got == [c[5] for c in cases]
