@@ -37,6 +37,9 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 #ifndef AP_KS
 #define AP_KS 2    // waves a block of 32 tokens in the large tile
 #endif
+#ifndef AP_FEED
+#define AP_FEED 2  // how tiles reach LDS where pages are uniform and heads are 64 or 128 wide (see the kernel)
+#endif
 #define AP_BN 64   // keys a tile
 #define AP_KPAD 8  // padding of a row of keys in LDS, in elements
 
@@ -66,6 +69,15 @@ __device__ __forceinline__ ap_u32x2 ap_read_transposed(const uint16_t* at) {
     return __builtin_bit_cast(ap_u32x2, got);
 }
 
+// 16 bytes a lane from global memory straight into LDS: lane l's land at `lds_at` + 16 l (`lds_at`, the
+// same for the whole wave, travels in M0).  Written as assembly so that the compiler does not count
+// the load: it would make every later read of LDS wait for all such loads, the ones just issued for a
+// tile two rounds ahead included.  The waits are placed by hand (s_waitcnt vmcnt) where a tile is due.
+__device__ __forceinline__ void ap_load_to_lds(const void* from, const uint16_t* lds_at) {
+    const uint32_t at = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void*)lds_at));
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(at), "v"(from) : "memory");
+}
+
 typedef uint32_t ap_vec4 __attribute__((ext_vector_type(4)));   // 16 bytes on their way through registers
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -92,7 +104,14 @@ __host__ __device__ constexpr int ap_value_buffers(int ks) { return ks == 2 ? 3 
 // What is loaded is not masked on this path: scores of keys that do not exist are masked anyway, and
 // their values are multiplied by zero, so the pages have to hold finite numbers everywhere (the
 // pools are allocated zeroed).
-template <int DT, int NW, int KS, bool UP>
+//
+// FEED 0: any page size, tiles travel through registers and are masked.  1: uniform pages, through
+// registers.  2: uniform pages, and the loads write LDS themselves (global_load_lds_dwordx4: lane l of
+// a wave puts its 16 bytes at the wave's LDS base + 16 l), three tiles ahead of their use and with no
+// register or LDS write instruction spent on them.  Rows then lie unpadded in LDS, so their 16-byte
+// pieces are permuted instead (piece c of key r stands at c ^ (r & 7) for keys, c ^ 2 (r & 7) for
+// values: the reads of the matrix cores' operands fall on every bank equally); heads of 64 and 128.
+template <int DT, int NW, int KS, int FEED>
 __global__ void __launch_bounds__(64 * NW * KS, DT <= 4 ? AP_OCC : 1)
 paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
                                const int* __restrict__ q_start, const int* __restrict__ q_len,
@@ -105,16 +124,20 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     constexpr int BM = 32 * NW;
     constexpr int NT = 64 * NW * KS;
     constexpr int KT = 2 / KS;             // 32-key tiles of a 64-key tile a wave takes
-    constexpr int KROW = DP + AP_KPAD;     // elements a row of Ks
-    constexpr int VROW = DP + ap_vpad(DT); // elements a row of Vs
+    constexpr bool UP = FEED >= 1, DIRECT = FEED == 2;
+    static_assert(!DIRECT || ((DT == 2 || DT == 4) && KS == 2), "the direct feed is written for heads of 64 and 128");
+    constexpr int KROW = DIRECT ? DP : DP + AP_KPAD;       // elements a row of Ks
+    constexpr int VROW = DIRECT ? DP : DP + ap_vpad(DT);   // elements a row of Vs
     extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
     // Two tiles of keys [AP_BN][KROW], then NVB tiles of values [AP_BN][VROW].  The values of a tile
     // are read one round after its keys, and with two groups of waves half a round apart they live
     // for three rounds.
-    constexpr int NVB = ap_value_buffers(KS);
+    // (The direct feed asks for a tile two rounds before its keys are read: a buffer more of each.)
+    constexpr int NKB = DIRECT ? 3 : 2;
+    constexpr int NVB = DIRECT ? 4 : ap_value_buffers(KS);
     constexpr int KTILE = AP_BN * KROW, VTILE = AP_BN * VROW;
     uint16_t* const Kbase = lds;
-    uint16_t* const Vbase = lds + 2 * KTILE;
+    uint16_t* const Vbase = lds + NKB * KTILE;
 
     // Workgroups are dealt round-robin to the eight XCDs; consecutive pieces of
     // work (the token tiles of one head) go to one XCD, whose L2 then holds the
@@ -276,31 +299,76 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     };
 
     const int k_first = (first_pos / AP_BN) * AP_BN;
-    lookup(k_first);
-    fetch();
-    lookup(k_first + AP_BN);
-    stash(0, 0);
-    fetch();                         // the second tile, all zeros past the last key
-    lookup(k_first + 2 * AP_BN);
-
     int staged = 1, staged_v = 1;    // the tile that the registers hold, and the buffer its values go to
-    __syncthreads();
+    // The direct feed: the loads of tile j, this wave's share (KI instructions for the keys, KI for the
+    // values), into the buffers j % NKB and j % NVB.  The lane's place in the cache row differs between
+    // keys and values by the permutation of the pieces.
+    int asked = 0, asked_k = 0, asked_v = 0;   // the next tile to ask for and its buffers
+    uint32_t place_k = 0, place_v = 0;
+    if constexpr (DIRECT) {
+        const int r7 = ((64 * wave_id) / CP + lane / CP) & 7;
+        const int ck = (lane % CP) ^ (r7 & (CP - 1)), cv = (lane % CP) ^ ((2 * r7) & (CP - 1));
+        place_k = (lane / CP) * row_bytes + static_cast<uint32_t>(head_off + min(ck, cpr - 1) * 8) * 2;
+        place_v = (lane / CP) * row_bytes + static_cast<uint32_t>(head_off + min(cv, cpr - 1) * 8) * 2;
+    }
+    auto ask = [&]() {               // pages from kblk/kwithin, looked up before
+        if constexpr (DIRECT) {
+#pragma unroll
+            for (int i = 0; i < KI; ++i) {
+                const int first_row = (64 * wave_id + i * NT) / CP;
+                const int page = __builtin_amdgcn_readfirstlane(max(kblk[i], 0));
+                const size_t base = (static_cast<size_t>(page) * block_size + kwithin[i]) * row_bytes;
+                const char* gk = reinterpret_cast<const char*>(k_pool) + base + place_k;
+                const char* gv = reinterpret_cast<const char*>(v_pool) + base + place_v;
+                uint16_t* lk = Kbase + asked_k * KTILE + first_row * KROW;
+                uint16_t* lv = Vbase + asked_v * VTILE + first_row * VROW;
+                ap_load_to_lds(gk, lk);
+                ap_load_to_lds(gv, lv);
+            }
+            ++asked;
+            asked_k = asked_k + 1 == NKB ? 0 : asked_k + 1;
+            asked_v = asked_v + 1 == NVB ? 0 : asked_v + 1;
+        }
+    };
+    auto take_pages = [&]() {
+#pragma unroll
+        for (int i = 0; i < KI; ++i) {
+            kblk[i] = ahead_blk[i];
+            kwithin[i] = ahead_within[i];
+        }
+    };
+    if constexpr (DIRECT) {
+        lookup(k_first);
+        ask();
+        lookup(k_first + AP_BN);
+        ask();
+        lookup(k_first + 2 * AP_BN);             // for the first round's asking
+        __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): the first two tiles have landed
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    } else {
+        lookup(k_first);
+        fetch();
+        lookup(k_first + AP_BN);
+        stash(0, 0);
+        fetch();                         // the second tile, all zeros past the last key
+        lookup(k_first + 2 * AP_BN);
+        __syncthreads();
+    }
     // The registers hold tile `staged`: it goes into buffers that nobody reads now, the tile after it
     // is asked for and the one after that looked up.
     auto advance = [&]() {
-        stash(staged & 1, staged_v);
-        fetch();
-        if constexpr (UP) {
-#pragma unroll
-            for (int i = 0; i < KI; ++i) {
-                kblk[i] = ahead_blk[i];
-                kwithin[i] = ahead_within[i];
+        if constexpr (!DIRECT) {
+            stash(staged & 1, staged_v);
+            fetch();
+            if constexpr (UP) {
+                take_pages();
+            } else {
+                lookup(k_first + (staged + 2) * AP_BN);
             }
-        } else {
-            lookup(k_first + (staged + 2) * AP_BN);
+            ++staged;
+            staged_v = staged_v + 1 == NVB ? 0 : staged_v + 1;
         }
-        ++staged;
-        staged_v = staged_v + 1 == NVB ? 0 : staged_v + 1;
     };
 
     // A round has two halves with a barrier after each.  In the first a wave multiplies: the scores of
@@ -315,6 +383,18 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     f32x16 s[KT];
     ap_frag pb[KT][2];               // probabilities of the tile before, rounded: [kt][half] is 16 keys
     const int v_corner = (32 * kt0 + 4 * h + ((lane & 15) >> 2)) * VROW + (lane & 16) + 4 * (lane & 3);
+    // The direct feed's permuted pieces: where piece 2*kk + h of this lane's key stands, and where the
+    // block of head elements 32*dt .. of this lane's four keys begins.
+    int k_piece[2 * DT], v_piece[DT];
+    if constexpr (DIRECT) {
+        const int x7 = r32 & 7;
+#pragma unroll
+        for (int kk = 0; kk < 2 * DT; ++kk) k_piece[kk] = (((2 * kk + h) ^ x7) & (CP - 1)) * 8;
+        const int i16 = lane & 15, g = lane >> 4;
+        const int f = (2 * ((4 * h + (i16 >> 2)) & 7)) & (CP - 1);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) v_piece[dt] = ((4 * dt + 2 * (g & 1) + ((i16 & 3) >> 1)) ^ f) * 8 + 4 * (i16 & 1);
+    }
     // The multiplying half of a round: O^T += V^T . P^T for the tile before (sixteen keys a product:
     // pb[kt][half] holds the keys 32*(kt0+kt) + 16*half + {4h..4h+3} and + 8 + {4h..4h+3}; 16 lanes read a
     // block of 4 keys x 16 head elements transposed), and the scores of this tile, transposed:
@@ -325,8 +405,9 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         const uint16_t* Vs = Vbase + vbuf * VTILE + v_corner;
         if constexpr (DT <= 4 && KT == 1) {
             ap_frag va[2][DT], ka[2 * DT];
+            const uint16_t* Vrows = Vbase + vbuf * VTILE + (32 * kt0 + 4 * h + ((lane & 15) >> 2)) * VROW;
             auto ask_values = [&](int half, int dt) {
-                const uint16_t* block = Vs + 16 * half * VROW + 32 * dt;
+                const uint16_t* block = DIRECT ? Vrows + 16 * half * VROW + v_piece[dt] : Vs + 16 * half * VROW + 32 * dt;
                 va[half][dt].half[0] = ap_read_transposed(block);
                 va[half][dt].half[1] = ap_read_transposed(block + 8 * VROW);
             };
@@ -336,7 +417,8 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
             if (with_scores) {
 #pragma unroll
                 for (int kk = 0; kk < 2 * DT; ++kk)
-                    ka[kk].raw = *reinterpret_cast<const ap_u32x4*>(Ks + (32 * kt0 + r32) * KROW + 16 * kk + 8 * h);
+                    ka[kk].raw = *reinterpret_cast<const ap_u32x4*>(Ks + (32 * kt0 + r32) * KROW +
+                                                                    (DIRECT ? k_piece[kk] : 16 * kk + 8 * h));
 #pragma unroll
                 for (int r = 0; r < 16; ++r) s[0][r] = 0.f;
                 __builtin_amdgcn_sched_barrier(0);
@@ -440,9 +522,17 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
 
     // The end of half a round: the products stay on their side of the barrier (the compiler would let
     // them drift behind it, into the half that should run beside another wave's products).
+    // (The direct feed has no writes of its own to LDS to make visible, and the fence of __syncthreads
+    // would wait for every load on its way: there the bare barrier stands, between compiler fences.)
     auto half_done = [&]() {
         __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();
+        if constexpr (DIRECT) {
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        } else {
+            __syncthreads();
+        }
         __builtin_amdgcn_sched_barrier(0);
     };
     const bool behind_group = KS == 2 && kt0 != 0;
@@ -451,6 +541,23 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         advance();
         half_done();
     }
+    // The direct feed in the multiplying half of round t: ask for tile t + 2 (pages looked up a round
+    // before), look up the pages of tile t + 3, and at the end wait until this wave's loads of tile
+    // t + 1 have landed: two rounds of flight, and after the barrier every wave's have.
+    constexpr int LOADS_A_TILE = 2 * KI;
+    auto feed_before = [&]() {
+        if constexpr (DIRECT) {
+            ask();
+            look_ahead(k_first + asked * AP_BN);
+        }
+    };
+    auto feed_after = [&]() {
+        if constexpr (DIRECT) {
+            take_pages();
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(0x0F70 | LOADS_A_TILE);   // vmcnt(LOADS_A_TILE): all but the newest tile
+        }
+    };
     // First the tiles that every query of the workgroup sees whole: no masks, no wave stands idle
     // (a wave past the request's last token works on zero queries and stores nothing).  Then the
     // few tiles around the diagonal, where keys are hidden and waves of early tokens are done.
@@ -470,12 +577,14 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     auto next_tile = [&]() {
         if (k0 != k_first) vbuf_before = vbuf_before + 1 == NVB ? 0 : vbuf_before + 1;
         k0 += AP_BN;
-        kbuf ^= 1;
+        kbuf = kbuf + 1 == NKB ? 0 : kbuf + 1;
     };
     for (; k0 < open_end; next_tile()) {
+        feed_before();
         multiply(kbuf, vbuf_before, true);
+        feed_after();
         half_done();
-        look_ahead(k_first + (staged + 2) * AP_BN);
+        if constexpr (!DIRECT) look_ahead(k_first + (staged + 2) * AP_BN);
         soften(k0, false);
         advance();
         half_done();
@@ -484,9 +593,11 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         // a wave whose queries all stand before this tile, or that has no queries, has nothing to add
         const bool idle = !wave_active || k0 + 32 * kt0 > wave_last ||
                           (window > 0 && k0 + 32 * (kt0 + KT) - 1 <= wave_first - window);
+        feed_before();
         multiply(kbuf, vbuf_before, !idle);
+        feed_after();
         half_done();
-        look_ahead(k_first + (staged + 2) * AP_BN);
+        if constexpr (!DIRECT) look_ahead(k_first + (staged + 2) * AP_BN);
         if (!idle) soften(k0, true);
         else no_weights();
         advance();
@@ -494,6 +605,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     }
     multiply(kbuf, vbuf_before, false);
     if (KS == 2 && !behind_group) half_done();   // the later group is half a round behind
+    if constexpr (DIRECT) __builtin_amdgcn_s_waitcnt(0x0F70);   // nothing may still be on its way into LDS
     lsum += __shfl_xor(lsum, 32, PL_WAVE);
     if (KS == 2) {
         // The wave of the later keys hands its state to the wave of the earlier ones through LDS
@@ -539,26 +651,27 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         }
 }
 
-template <int DT, int NW, int KS, bool UP>
+template <int DT, int NW, int KS, int FEED>
 static int launch_prefill(const void* q, int q_stride, void* out, const int* q_start, const int* q_len,
                           const int* ctx_len, int short_limit, int num_seqs, int max_q_len, const int* block_table,
                           int max_blocks, int block_size, const void* k_pool, const void* v_pool, int nq, int nkv,
                           int d, float scale, int window, hipStream_t stream) {
     constexpr int DP = 32 * DT;
     constexpr int BM = 32 * NW;
-    const size_t tile_bytes = (2 * static_cast<size_t>(AP_BN) * (DP + AP_KPAD) +
-                               ap_value_buffers(KS) * static_cast<size_t>(AP_BN) * (DP + ap_vpad(DT))) * 2;
+    const size_t tile_bytes = FEED == 2 ? (3 + 4) * static_cast<size_t>(AP_BN) * DP * 2
+                                        : (2 * static_cast<size_t>(AP_BN) * (DP + AP_KPAD) +
+                                           ap_value_buffers(KS) * static_cast<size_t>(AP_BN) * (DP + ap_vpad(DT))) * 2;
     const size_t hand_bytes = KS == 2 ? static_cast<size_t>(NW) * (16 * DT + 2) * PL_WAVE * sizeof(float) : 0;
     const size_t lds_bytes = tile_bytes > hand_bytes ? tile_bytes : hand_bytes;
     if (lds_bytes > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_prefill_kernel<DT, NW, KS, UP>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_prefill_kernel<DT, NW, KS, FEED>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
         PL_REQUIRE(e == hipSuccess, "prefill attention: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
     }
     const int tiles = pl_ceil_div(max_q_len, BM);
     const long long total = static_cast<long long>(tiles) * nq * num_seqs;
     PL_REQUIRE(total > 0 && total < (1ll << 30), "prefill attention: %lld workgroups", total);
-    paged_attention_prefill_kernel<DT, NW, KS, UP><<<static_cast<int>(total), 64 * NW * KS, lds_bytes, stream>>>(
+    paged_attention_prefill_kernel<DT, NW, KS, FEED><<<static_cast<int>(total), 64 * NW * KS, lds_bytes, stream>>>(
         static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), q_start, q_len, ctx_len, short_limit, tiles,
         num_seqs, block_table, max_blocks, block_size, static_cast<const bf16_t*>(k_pool),
         static_cast<const bf16_t*>(v_pool), nq, nkv, d, scale * 1.4426950408889634f, window, static_cast<int>(total));
@@ -571,26 +684,27 @@ static int ap_dispatch(bool small, bool uniform_pages, const void* q, int q_stri
                        const int* q_len, const int* ctx_len, int short_limit, int num_seqs, int max_q_len,
                        const int* block_table, int max_blocks, int block_size, const void* k_pool, const void* v_pool,
                        int nq, int nkv, int d, float scale, int window, hipStream_t stream) {
-#define AP_LAUNCH(NW, KS, UP)                                                                                      \
-    launch_prefill<D, NW, KS, UP>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len,    \
+#define AP_LAUNCH(NW, KS, FEED)                                                                                    \
+    launch_prefill<D, NW, KS, FEED>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len,    \
                                   block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale, window, stream)
     constexpr bool can_fit = 64 % (4 * D) == 0;
+    constexpr int BEST = (D == 2 || D == 4) && AP_KS == 2 && AP_SMALL_KS == 2 ? AP_FEED : 1;   // the feed with uniform pages
     if constexpr (D <= 4) {
         if (small) {
             if constexpr (can_fit) {
-                if (uniform_pages) return AP_LAUNCH(2, AP_SMALL_KS, true);
+                if (uniform_pages) return AP_LAUNCH(2, AP_SMALL_KS, BEST);
             }
-            return AP_LAUNCH(2, AP_SMALL_KS, false);
+            return AP_LAUNCH(2, AP_SMALL_KS, 0);
         }
         if constexpr (can_fit) {
-            if (uniform_pages) return AP_LAUNCH(4, AP_KS, true);
+            if (uniform_pages) return AP_LAUNCH(4, AP_KS, BEST);
         }
-        return AP_LAUNCH(4, AP_KS, false);
+        return AP_LAUNCH(4, AP_KS, 0);
     } else {
         if constexpr (can_fit) {
-            if (uniform_pages) return AP_LAUNCH(4, 1, true);
+            if (uniform_pages) return AP_LAUNCH(4, 1, 1);
         }
-        return AP_LAUNCH(4, 1, false);
+        return AP_LAUNCH(4, 1, 0);
     }
 #undef AP_LAUNCH
 }
