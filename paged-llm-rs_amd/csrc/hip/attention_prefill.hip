@@ -81,6 +81,7 @@ __device__ __forceinline__ void ap_load_to_lds(const void* from, const uint16_t*
 typedef uint32_t ap_vec4 __attribute__((ext_vector_type(4)));   // 16 bytes on their way through registers
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // Two floats rounded to nearest-even bfloat16 in one word (the hardware's packed conversion).
 __device__ __forceinline__ uint32_t ap_pack2(float lo, float hi) {
@@ -119,7 +120,8 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
                                int num_seqs, const int* __restrict__ block_table, int max_blocks,
                                int block_size, const bf16_t* __restrict__ k_pool,
                                const bf16_t* __restrict__ v_pool, int nq, int nkv, int d, float scale_log2e,
-                               int window, int total_work) {
+                               int window, int total_work, int splits, float* __restrict__ part_acc,
+                               float* __restrict__ part_ml) {
     constexpr int DP = 32 * DT;
     constexpr int BM = 32 * NW;
     constexpr int NT = 64 * NW * KS;
@@ -144,7 +146,13 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     // keys and values they share.
     int work = blockIdx.x;
     if ((total_work & 7) == 0) work = (blockIdx.x & 7) * (total_work >> 3) + (blockIdx.x >> 3);
-    // work = (request * nq + head) * tiles + (tiles - 1 - tile): late tiles, which read the most keys, first
+    // work = ((request * nq + head) * tiles + (tiles - 1 - tile)) * splits + split: late tiles, which read
+    // the most keys, first.  With splits > 1 the key tiles of a token tile are dealt to that many
+    // workgroups (few token tiles over a long context would leave compute units idle, and the last
+    // token tiles of a prompt hold the others up); each leaves its unnormalised output, maximum and sum
+    // in the workspace and a second kernel puts them together.
+    const int split = work % splits;
+    work /= splits;
     const int tile = tiles_a_request - 1 - work % tiles_a_request;
     const int head = (work / tiles_a_request) % nq;
     const int seq = work / (tiles_a_request * nq);
@@ -298,7 +306,22 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         }
     };
 
-    const int k_first = (first_pos / AP_BN) * AP_BN;
+    // this workgroup's share of the key tiles
+    const int k_lowest = (first_pos / AP_BN) * AP_BN;
+    const int key_tiles = (last_pos - k_lowest) / AP_BN + 1;
+    const int tiles_a_split = (key_tiles + splits - 1) / splits;
+    const int k_first = k_lowest + split * tiles_a_split * AP_BN;
+    const int k_end = min(k_lowest + key_tiles * AP_BN, k_first + tiles_a_split * AP_BN);
+    if (k_first >= k_end) {          // more splits than key tiles: nothing to add
+        if (kt0 == 0 && q_ok) {
+            float* ml = part_ml + ((static_cast<size_t>(row0 + wq) * nq + head) * splits + split) * 2;
+            if (h == 0) {
+                ml[0] = -INFINITY;
+                ml[1] = 0.f;
+            }
+        }
+        return;
+    }
     int staged = 1, staged_v = 1;    // the tile that the registers hold, and the buffer its values go to
     // The direct feed: the loads of tile j, this wave's share (KI instructions for the keys, KI for the
     // values), into the buffers j % NKB and j % NVB.  The lane's place in the cache row differs between
@@ -579,7 +602,8 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         k0 += AP_BN;
         kbuf = kbuf + 1 == NKB ? 0 : kbuf + 1;
     };
-    for (; k0 < open_end; next_tile()) {
+    const int open_stop = min(open_end, k_end);
+    for (; k0 < open_stop; next_tile()) {
         feed_before();
         multiply(kbuf, vbuf_before, true);
         feed_after();
@@ -589,7 +613,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         advance();
         half_done();
     }
-    for (; k0 <= last_pos; next_tile()) {
+    for (; k0 < k_end; next_tile()) {
         // a wave whose queries all stand before this tile, or that has no queries, has nothing to add
         const bool idle = !wave_active || k0 + 32 * kt0 > wave_last ||
                           (window > 0 && k0 + 32 * (kt0 + KT) - 1 <= wave_first - window);
@@ -627,15 +651,32 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         const float use = big == -INFINITY ? 0.f : big;
         const float w0 = __builtin_amdgcn_exp2f((m - use) * scale_log2e), w1 = __builtin_amdgcn_exp2f((m1 - use) * scale_log2e);
         lsum = lsum * w0 + l1 * w1;
+        m = big;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int r = 0; r < 16; ++r) o[dt][r] = o[dt][r] * w0 + hand[(dt * 16 + r) * PL_WAVE + lane] * w1;
     }
     if (!q_ok) return;
+    // o[dt][4*j + i] is element 32*dt + 8*j + 4*h + i of query r32
+    if (splits > 1) {
+        const size_t at = (static_cast<size_t>(row0 + wq) * nq + head) * splits + split;
+        if (h == 0) {
+            part_ml[at * 2] = m * scale_log2e;     // in the exponent's own unit; -inf stays
+            part_ml[at * 2 + 1] = lsum;
+        }
+        float* arow = part_acc + at * d;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int e0 = 32 * dt + 8 * j + 4 * h;
+                if (e0 < d) *reinterpret_cast<f32x4*>(arow + e0) = f32x4{o[dt][4 * j], o[dt][4 * j + 1], o[dt][4 * j + 2], o[dt][4 * j + 3]};
+            }
+        return;
+    }
     const float total = lsum;
     const float inv = total > 0.f ? 1.f / total : 0.f;
-    // o[dt][4*j + i] is element 32*dt + 8*j + 4*h + i of query r32
     bf16_t* orow = out + (static_cast<size_t>(row0 + wq) * nq + head) * d;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
@@ -651,11 +692,66 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         }
 }
 
+// Puts the splits of a token tile together: out = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).
+// blockIdx.x names the token tile as in the kernel above (without the splits), blockIdx.y a stretch of
+// its tokens; a thread takes four head elements of one token and asks for all it needs at once.
+#define AP_MERGE_MAX 16
+__global__ void __launch_bounds__(256)
+paged_attention_prefill_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+                                     bf16_t* __restrict__ out, const int* __restrict__ q_start,
+                                     const int* __restrict__ q_len, int short_limit, int tiles_a_request, int num_seqs,
+                                     int nq, int d, int splits, int bm) {
+    const int work = blockIdx.x;
+    const int tile = work % tiles_a_request;
+    const int head = (work / tiles_a_request) % nq;
+    const int seq = work / (tiles_a_request * nq);
+    if (seq >= num_seqs) return;
+    const int count = q_len[seq];
+    if (count < short_limit) return;
+    const int quads = d / 4, rows = blockDim.x / quads;
+    const int r = tile * bm + blockIdx.y * rows + threadIdx.x / quads;
+    const int e0 = (threadIdx.x % quads) * 4;
+    if (static_cast<int>(threadIdx.x) >= rows * quads || r >= min(count, (tile + 1) * bm)) return;
+    const size_t row = static_cast<size_t>(q_start[seq]) + r;
+    const size_t at = (row * nq + head) * splits;
+    float ms[AP_MERGE_MAX], ls[AP_MERGE_MAX];
+    f32x4 os[AP_MERGE_MAX];
+#pragma unroll
+    for (int sp = 0; sp < AP_MERGE_MAX; ++sp) {
+        const int sc = min(sp, splits - 1);
+        ms[sp] = part_ml[(at + sc) * 2];
+        ls[sp] = part_ml[(at + sc) * 2 + 1];
+    }
+    float big = -INFINITY;
+#pragma unroll
+    for (int sp = 0; sp < AP_MERGE_MAX; ++sp) big = fmaxf(big, sp < splits ? ms[sp] : -INFINITY);
+#pragma unroll
+    for (int sp = 0; sp < AP_MERGE_MAX; ++sp) {
+        // a split that saw no key wrote no output: its place in the workspace holds anything
+        const bool live = sp < splits && ms[sp] != -INFINITY;
+        os[sp] = live ? *reinterpret_cast<const f32x4*>(part_acc + (at + sp) * d + e0) : f32x4{0.f, 0.f, 0.f, 0.f};
+        ms[sp] = live ? exp2f(ms[sp] - big) : 0.f;
+    }
+    float sum = 0.f;
+    f32x4 a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int sp = 0; sp < AP_MERGE_MAX; ++sp) {
+        sum = fmaf(ls[sp], ms[sp], sum);
+        a += os[sp] * ms[sp];
+    }
+    const float inv = sum > 0.f ? 1.f / sum : 0.f;
+    ap_u32x2 w;
+    w.v[0] = ap_pack2(a[0] * inv, a[1] * inv);
+    w.v[1] = ap_pack2(a[2] * inv, a[3] * inv);
+    *reinterpret_cast<ap_u32x2*>(out + (row * nq + head) * d + e0) = w;
+}
+
 template <int DT, int NW, int KS, int FEED>
 static int launch_prefill(const void* q, int q_stride, void* out, const int* q_start, const int* q_len,
                           const int* ctx_len, int short_limit, int num_seqs, int max_q_len, const int* block_table,
                           int max_blocks, int block_size, const void* k_pool, const void* v_pool, int nq, int nkv,
-                          int d, float scale, int window, hipStream_t stream) {
+                          int d, float scale, int window, int splits, float* part_acc, float* part_ml,
+                          hipStream_t stream) {
     constexpr int DP = 32 * DT;
     constexpr int BM = 32 * NW;
     const size_t tile_bytes = FEED == 2 ? (3 + 4) * static_cast<size_t>(AP_BN) * DP * 2
@@ -669,13 +765,20 @@ static int launch_prefill(const void* q, int q_stride, void* out, const int* q_s
         PL_REQUIRE(e == hipSuccess, "prefill attention: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
     }
     const int tiles = pl_ceil_div(max_q_len, BM);
-    const long long total = static_cast<long long>(tiles) * nq * num_seqs;
+    const long long whole = static_cast<long long>(tiles) * nq * num_seqs, total = whole * splits;
     PL_REQUIRE(total > 0 && total < (1ll << 30), "prefill attention: %lld workgroups", total);
     paged_attention_prefill_kernel<DT, NW, KS, FEED><<<static_cast<int>(total), 64 * NW * KS, lds_bytes, stream>>>(
         static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), q_start, q_len, ctx_len, short_limit, tiles,
         num_seqs, block_table, max_blocks, block_size, static_cast<const bf16_t*>(k_pool),
-        static_cast<const bf16_t*>(v_pool), nq, nkv, d, scale * 1.4426950408889634f, window, static_cast<int>(total));
+        static_cast<const bf16_t*>(v_pool), nq, nkv, d, scale * 1.4426950408889634f, window, static_cast<int>(total),
+        splits, part_acc, part_ml);
     PL_CHECK_LAUNCH("paged_attention_prefill");
+    if (splits > 1) {
+        const int rows = 256 / (d / 4);
+        paged_attention_prefill_merge_kernel<<<dim3(static_cast<int>(whole), pl_ceil_div(BM, rows)), 256, 0, stream>>>(
+            part_acc, part_ml, static_cast<bf16_t*>(out), q_start, q_len, short_limit, tiles, num_seqs, nq, d, splits, BM);
+        PL_CHECK_LAUNCH("paged_attention_prefill_merge");
+    }
     return 0;
 }
 
@@ -683,10 +786,12 @@ template <int D>
 static int ap_dispatch(bool small, bool uniform_pages, const void* q, int q_stride, void* out, const int* q_start,
                        const int* q_len, const int* ctx_len, int short_limit, int num_seqs, int max_q_len,
                        const int* block_table, int max_blocks, int block_size, const void* k_pool, const void* v_pool,
-                       int nq, int nkv, int d, float scale, int window, hipStream_t stream) {
+                       int nq, int nkv, int d, float scale, int window, int splits, float* part_acc, float* part_ml,
+                       hipStream_t stream) {
 #define AP_LAUNCH(NW, KS, FEED)                                                                                    \
     launch_prefill<D, NW, KS, FEED>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len,    \
-                                  block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale, window, stream)
+                                    block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale, window, \
+                                    splits, part_acc, part_ml, stream)
     constexpr bool can_fit = 64 % (4 * D) == 0;
     constexpr int BEST = (D == 2 || D == 4) && AP_KS == 2 && AP_SMALL_KS == 2 ? AP_FEED : 1;   // the feed with uniform pages
     if constexpr (D <= 4) {
@@ -712,11 +817,21 @@ static int ap_dispatch(bool small, bool uniform_pages, const void* q, int q_stri
 // bfloat16 only.  q rows begin with the nq*d rotated query values; request s brings the rows
 // q_start[s] .. q_start[s] + q_len[s] - 1, which stand at the positions ctx_len[s] - q_len[s] .. ctx_len[s] - 1.
 // Requests with q_len < short_limit are skipped.  max_q_len bounds q_len over the requests.
+// splits > 1 deals the keys of every token tile to that many workgroups; the workspace then needs
+// rows*nq*splits*d floats (part_acc) and rows*nq*splits*2 (part_ml), rows being the step's rows of q.
+// pl_paged_attention_prefill_tile says how many tokens a token tile will have.
+extern "C" int pl_paged_attention_prefill_tile(int max_q_len, int d) {
+    return (max_q_len <= 64 && d <= 128) ? 64 : 128;
+}
+
 extern "C" int pl_paged_attention_prefill(const void* q, int q_stride, void* out, const int* q_start,
                                           const int* q_len, const int* ctx_len, int short_limit, int num_seqs,
                                           int max_q_len, const int* block_table, int max_blocks, int block_size,
                                           const void* k_pool, const void* v_pool, int nq, int nkv, int d,
-                                          float scale, int window, hipStream_t stream) {
+                                          float scale, int window, int splits, float* part_acc, float* part_ml,
+                                          hipStream_t stream) {
+    PL_REQUIRE(splits >= 1 && splits <= AP_MERGE_MAX && (splits == 1 || (part_acc && part_ml)),
+               "prefill attention: %d splits%s", splits, splits > 1 ? " without a workspace" : "");
     PL_REQUIRE(d > 0 && d <= 256 && d % 16 == 0, "prefill attention: head size %d, which has to be a multiple of 16 up to 256", d);
     PL_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "prefill attention: %d query heads over %d key heads", nq, nkv);
     PL_REQUIRE(block_size > 0 && max_blocks > 0 && q_stride >= nq * d && q_stride % 8 == 0 && window >= 0,
@@ -736,7 +851,8 @@ extern "C" int pl_paged_attention_prefill(const void* q, int q_stride, void* out
     const bool pages_fit = (block_size & (block_size - 1)) == 0 && block_size * 4 * dt >= 64 && 64 % (4 * dt) == 0;
 #define AP_CALL(D)                                                                                                 \
     return ap_dispatch<D>(small, pages_fit, q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len, \
-                          block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale, window, stream)
+                          block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale, window, splits,   \
+                          part_acc, part_ml, stream)
     switch (dt) {
         case 1: AP_CALL(1);
         case 2: AP_CALL(2);

@@ -34,12 +34,13 @@ def _signatures(lib) -> None:
         "pl_swiglu": [p, p, i, i, i, p],
         "pl_gemm_plain": [p, p, p, i, i, i, i, i, i, i, p],
         "pl_paged_attention_plain": [p, i, p, p, p, p, i, i, p, p, i, i, i, i, f, i, i, p],
+        "pl_paged_attention_prefill_tile": [i, i],
         "pl_argmax": [p, p, p, p, i, i, p],
         "pl_sample": [p, p, p, p, p, p, i, i, p],
         "pl_gemm_skinny": [p, p, p, p, f, p, i, i, i, i, i, p],
         "pl_paged_attention_decode": [p, i, p, p, p, p, p, p, i, p, i, i, p, p, i, i, i, i, f, i, i,
                                       i, p, p, i, f, p, p, i, p],
-        "pl_paged_attention_prefill": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, p],
+        "pl_paged_attention_prefill": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, p],
     }
     for name, argtypes in table.items():
         fn = getattr(lib, name)
@@ -358,10 +359,13 @@ class QkFusion:
 def paged_attention_prefill(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, q_start: torch.Tensor,
                             q_len: torch.Tensor, ctx_len: torch.Tensor, max_q_len: int, block_table: torch.Tensor,
                             block_size: int, k_pool: torch.Tensor, v_pool: torch.Tensor, nq: int, nkv: int, d: int,
-                            scale: float, window: int = 0, short_limit: int = 0) -> torch.Tensor:
+                            scale: float, window: int = 0, short_limit: int = 0, max_ctx: int | None = None,
+                            splits: int | None = None) -> torch.Tensor:
     """bfloat16 attention of prompt portions on the matrix cores.  Request s brings the rows
     q_start[s] .. q_start[s]+q_len[s]-1 at the positions ctx_len[s]-q_len[s] .. ctx_len[s]-1;
-    requests with fewer than ``short_limit`` tokens are skipped."""
+    requests with fewer than ``short_limit`` tokens are skipped.  ``max_ctx`` (the longest context
+    of the step) lets the keys of a token tile be dealt to several workgroups where the tiles alone
+    would leave compute units idle; ``splits`` sets their number by hand."""
     n = q.shape[0]
     S = block_table.shape[0]
     _need(q, "query buffer", None, torch.bfloat16)
@@ -378,11 +382,49 @@ def paged_attention_prefill(q: torch.Tensor, q_row_stride: int, out: torch.Tenso
             raise TensorError(f"{what} has shape {tuple(pool.shape)}, expected [pages*{block_size}, {nkv * d}]")
     if not 0 < max_q_len <= n:
         raise TensorError(f"the longest portion is said to have {max_q_len} of the step's {n} tokens")
+    if splits is None:
+        splits = prefill_splits(S, int(max_q_len), nq, d, int(max_ctx or 0), n)
+    part_acc = part_ml = None
+    if splits > 1:
+        part_acc = torch.empty((n * nq * splits * d,), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((n * nq * splits * 2,), dtype=torch.float32, device=q.device)
     _check(library().pl_paged_attention_prefill(
         q.data_ptr(), q_row_stride, out.data_ptr(), q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(),
         int(short_limit), S, int(max_q_len), block_table.data_ptr(), block_table.shape[1], block_size,
-        k_pool.data_ptr(), v_pool.data_ptr(), nq, nkv, d, float(scale), int(window or 0), _stream()))
+        k_pool.data_ptr(), v_pool.data_ptr(), nq, nkv, d, float(scale), int(window or 0), int(splits),
+        part_acc.data_ptr() if splits > 1 else None, part_ml.data_ptr() if splits > 1 else None, _stream()))
     return out
+
+
+_compute_units = None
+
+
+def prefill_splits(requests: int, max_q_len: int, nq: int, d: int, max_ctx: int, rows: int | None = None) -> int:
+    """Into how many shares the keys of a token tile are cut.  A share more costs a trip of the
+    unnormalised outputs through memory (rows * nq * d floats written and read) and one launch;
+    it pays where few token tiles stand before a long context, as in a late portion of a long
+    prompt.  The shares that make the estimate below smallest are taken: a workgroup spends about
+    1.5 us on 64 keys, memory moves about 3 TB/s for this."""
+    global _compute_units
+    if max_ctx <= 0:
+        return 1
+    if _compute_units is None:
+        _compute_units = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
+    tile = library().pl_paged_attention_prefill_tile(max_q_len, d)
+    base = max(1, -(-max_q_len // tile) * nq * requests)
+    key_tiles = -(-max_ctx // 64)
+    rows = rows if rows is not None else requests * max_q_len
+    best, best_cost = 1, None
+    for s in (1, 2, 3, 4, 6, 8, 12, 16):
+        if s > 1 and key_tiles // s < 4:
+            break
+        turns = -(-base * s // _compute_units)
+        cost = turns * -(-key_tiles // s) * 1.5
+        if s > 1:
+            cost += 3.0 + rows * nq * d * 8.0 * s / 3e6
+        if best_cost is None or cost < best_cost:
+            best, best_cost = s, cost
+    return best
 
 
 def attention_step(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nkv: int, d: int, scale: float,
@@ -415,7 +457,7 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nk
     if batch.max_q_len >= SHORT_PORTION:
         paged_attention_prefill(qkv, stride, out, batch.q_start, batch.q_len, batch.ctx_len, batch.max_q_len,
                                 kv.block_table, kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window,
-                                short_limit=SHORT_PORTION)
+                                short_limit=SHORT_PORTION, max_ctx=batch.max_ctx_len)
         if batch.short_tokens == 0:
             return out
     mixed = batch.max_q_len >= SHORT_PORTION

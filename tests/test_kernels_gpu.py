@@ -445,10 +445,12 @@ PORTION_CASES = [
 ]
 
 
+@pytest.mark.parametrize("splits", [1, 3, 16])
 @pytest.mark.parametrize("nq,nkv,d,bs,requests,window", PORTION_CASES)
-def test_paged_attention_of_portions(nq, nkv, d, bs, requests, window):
+def test_paged_attention_of_portions(nq, nkv, d, bs, requests, window, splits):
     """The tiled kernel takes the requests that bring 16 tokens or more, the single-token kernel
-    the others; together they fill every row of the step."""
+    the others; together they fill every row of the step.  The keys of a token tile may be dealt to
+    several workgroups (more of them than there are key tiles, too)."""
     from paged_llm_rs_amd import kernels
 
     dtype = torch.bfloat16
@@ -469,7 +471,7 @@ def test_paged_attention_of_portions(nq, nkv, d, bs, requests, window):
     out = torch.full((n, nq * d), 7.0, dtype=dtype, device=DEV)
     limit = kernels.SHORT_PORTION
     kernels.paged_attention_prefill(q, stride, out, q_start_t, q_len_t, ctx_t, max(q_len), bt, bs, k_pool, v_pool,
-                                    nq, nkv, d, scale, window, short_limit=limit)
+                                    nq, nkv, d, scale, window, short_limit=limit, splits=splits)
     for s, (ctx, count) in enumerate(requests):
         if count < limit:
             rows = out[q_start[s]:q_start[s] + count]
