@@ -22,6 +22,13 @@
 //               them (rows c and N + c of w) and stores silu(gate) * up.
 //   EPI_ADD     the 32-bit residual stream takes the result: resid[r, c] += result.  Every
 //               element has one owner, so the sum does not depend on timing.
+//
+// With more than 16 rows a wave's registers fill with x (every 16 rows are another operand a K step), and
+// little of w is on its way at a time.  PANEL then brings the workgroup's 16 (or 32) rows of w into LDS
+// first: every wave asks for its share with loads that write LDS themselves (global_load_lds_dwordx4), so
+// the whole panel is on its way at once at no cost in registers, and the matrix cores take w from LDS
+// (16-byte pieces permuted within a row, piece p of row r at p ^ (r & 15), so that the 16 rows a read
+// touches fall on different banks).  K has to be a multiple of 512: a load of one wave fills 1 KB of a row.
 #pragma once
 #include "common.hpp"
 
@@ -70,7 +77,15 @@ __device__ __forceinline__ void sk_load_gain(const float* gain, int k, float* ou
 // The gain is 32-bit.
 // A workgroup walks the column tiles blockIdx.x, blockIdx.x + gridDim.x, ...; when a wave's share of
 // K fits one round of loads, its rows of x are loaded (and normalised) once and stay in registers.
-template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT>
+// 16 bytes a lane from global memory straight into LDS (lane l's land at lds_at + 16 l; lds_at, the same
+// for the wave, travels in M0).  Assembly, so that the compiler does not count the load and make every
+// later read of LDS wait for it; the wait is written by hand where the panel is due.
+__device__ __forceinline__ void sk_load_to_lds(const void* from, const void* lds_at) {
+    const uint32_t at = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void*)lds_at));
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(at), "v"(from) : "memory");
+}
+
+template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT, bool PANEL = false>
 __global__ void __launch_bounds__(64 * WV)
 gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OUT* __restrict__ y,
                    const float* __restrict__ gain, float eps, const int* __restrict__ rows, int n, int N_out,
@@ -78,8 +93,10 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
     const int nwaves = blockDim.x / PL_WAVE;
     extern __shared__ float sk_lds[];
+    // PANEL: [BT * 16][K] bfloat16, in the same place as the partial tiles (which are written when it is done with)
+    bf16_t* panel = reinterpret_cast<bf16_t*>(sk_lds);
     float* red = sk_lds;                                   // [nwaves][BT][MT][256] partial tiles
-    float* ssq_lds = sk_lds + nwaves * BT * MT * 256;      // [nwaves][MT * 16] partial sums of squares
+    float* ssq_lds = red + nwaves * BT * MT * 256;         // [nwaves][MT * 16] partial sums of squares
 
     const int lane = threadIdx.x % PL_WAVE;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PL_WAVE);
@@ -167,6 +184,18 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
         wrow[0] = w + static_cast<size_t>(col_ok ? n0 + c : 0) * K;
         if (BT == 2) wrow[BT - 1] = w + static_cast<size_t>(N_out + (col_ok ? n0 + c : 0)) * K;
 
+        if constexpr (PANEL) {
+            // the tile's rows of w, 1 KB (64 pieces of a row) a load, dealt to the waves in turn
+            const int chunks = K / 512, loads = BT * 16 * chunks;
+            for (int j = wave; j < loads; j += nwaves) {
+                const int prow = j / chunks, chunk = j - prow * chunks;
+                const int r = prow % 16;
+                const size_t grow = (prow >= 16 ? N_out : 0) + static_cast<size_t>(n0 + r < N_out ? n0 + r : 0);
+                const int piece = (chunk * 64 + lane) ^ r;
+                sk_load_to_lds(w + grow * K + piece * 8, panel + static_cast<size_t>(prow) * K + chunk * 512);
+            }
+        }
+
         f32x4 acc[BT][MT];
 #pragma unroll
         for (int m = 0; m < MT; ++m)
@@ -176,37 +205,66 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
 #pragma unroll
             for (int m = 0; m < MT; ++m) ssq[m] = 0.f;
         }
-
-        for (int k0 = kbeg; k0 < kend; k0 += SK_KSTEP * UNR) {
-            bf16x8 bw[BT][UNR];
-#pragma unroll
-            for (int u = 0; u < UNR; ++u) {
-                const int at = k0 + u * SK_KSTEP + g * 8;
-                const bool k_ok = at < kend;
-                const int kk = k_ok ? at : 0;
-#pragma unroll
-                for (int b = 0; b < BT; ++b) {
-                    const bf16x8 got = sk_load8(wrow[b] + kk);
-                    bw[b][u] = (k_ok && col_ok) ? got : sk_zero8();
-                }
-            }
-            // the weights are asked for first: they come from furthest away
-            if (!one_round) {
-                ask_x(k0);
-                take_x(k0);
-            } else if (x_asked) {
-                take_x(kbeg);
-                x_asked = false;
-            }
-#pragma unroll
-            for (int u = 0; u < UNR; ++u)
-#pragma unroll
-                for (int m = 0; m < MT; ++m)
-#pragma unroll
-                    for (int b = 0; b < BT; ++b)
-                        acc[b][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[m][u], bw[b][u], acc[b][m], 0, 0, 0);
+        if constexpr (PANEL) {
+            __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0): this wave's share of the panel has landed
+            __syncthreads();                               // and every wave's
         }
 
+        for (int k0 = kbeg; k0 < kend; k0 += SK_KSTEP * UNR) {
+            if constexpr (PANEL) {
+                // w waits in LDS: x is asked for (if it is not held from the start) and each step's
+                // piece of w is read just before its products
+                if (!one_round) {
+                    ask_x(k0);
+                    take_x(k0);
+                } else if (x_asked) {
+                    take_x(kbeg);
+                    x_asked = false;
+                }
+#pragma unroll
+                for (int u = 0; u < UNR; ++u) {
+                    const int at = k0 + u * SK_KSTEP + g * 8;
+                    const int kk = at < kend ? at : 0;          // past the end x is zero
+#pragma unroll
+                    for (int b = 0; b < BT; ++b) {
+                        const bf16x8 bw = sk_load8(panel + static_cast<size_t>(b * 16 + c) * K + (((kk >> 3) ^ c) << 3));
+#pragma unroll
+                        for (int m = 0; m < MT; ++m)
+                            acc[b][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[m][u], bw, acc[b][m], 0, 0, 0);
+                    }
+                }
+            } else {
+                bf16x8 bw[BT][UNR];
+#pragma unroll
+                for (int u = 0; u < UNR; ++u) {
+                    const int at = k0 + u * SK_KSTEP + g * 8;
+                    const bool k_ok = at < kend;
+                    const int kk = k_ok ? at : 0;
+#pragma unroll
+                    for (int b = 0; b < BT; ++b) {
+                        const bf16x8 got = sk_load8(wrow[b] + kk);
+                        bw[b][u] = (k_ok && col_ok) ? got : sk_zero8();
+                    }
+                }
+                // the weights are asked for first: they come from furthest away
+                if (!one_round) {
+                    ask_x(k0);
+                    take_x(k0);
+                } else if (x_asked) {
+                    take_x(kbeg);
+                    x_asked = false;
+                }
+#pragma unroll
+                for (int u = 0; u < UNR; ++u)
+#pragma unroll
+                    for (int m = 0; m < MT; ++m)
+#pragma unroll
+                        for (int b = 0; b < BT; ++b)
+                            acc[b][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[m][u], bw[b][u], acc[b][m], 0, 0, 0);
+            }
+        }
+
+        if constexpr (PANEL) __syncthreads();   // every wave has read its last of the panel
         // A lane holds rows (lane/16)*4 + i, i = 0..3, of column lane%16 of its 16x16 tile.
 #pragma unroll
         for (int b = 0; b < BT; ++b)
@@ -284,6 +342,28 @@ static int launch_one(int waves, const void* x, const void* w, void* y, const fl
     return 0;
 }
 
+// The panel variant: 8 waves (256 registers a lane); a wave holds 16 * MT rows of x for UNR K steps.
+template <int MT, int UNR, int PRO, int EPI, typename OUT>
+static int launch_panel(const void* x, const void* w, void* y, const float* gain, float eps,
+                        const int* rows, int n, int N_out, int K, hipStream_t stream) {
+    constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
+    constexpr int waves = 8;
+    const int grid = min(pl_ceil_div(N_out, SK_TILE_N), SK_MAX_GRID);
+    const size_t panel_bytes = static_cast<size_t>(BT) * 16 * K * 2;
+    const size_t red_bytes = static_cast<size_t>(waves) * (BT * MT * 256 + MT * 16) * sizeof(float);
+    const size_t lds_bytes = panel_bytes > red_bytes ? panel_bytes : red_bytes;
+    auto kernel = &gemm_skinny_kernel<MT, UNR, waves, PRO, EPI, OUT, true>;
+    if (lds_bytes > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           static_cast<int>(lds_bytes));
+        PL_REQUIRE(e == hipSuccess, "skinny product: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
+    }
+    kernel<<<grid, 64 * waves, lds_bytes, stream>>>(x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps,
+                                                   rows, n, N_out, K);
+    PL_CHECK_LAUNCH("gemm_skinny");
+    return 0;
+}
+
 // How many waves, and how many K steps each asks for at once.  What a wave holds in flight has to fit
 // its registers (512 a lane with four waves, 256 with eight, 128 with sixteen); within that, the
 // fewest waves whose one round of loads covers K are taken, so that the whole matrix is asked for at
@@ -301,6 +381,12 @@ template <int MT, int PRO, int EPI, typename OUT>
 static int launch_unr(const void* x, const void* w, void* y, const float* gain, float eps,
                       const int* rows, int n, int N_out, int K, hipStream_t stream) {
     using S = SkShape<MT, PRO, EPI>;
+    if constexpr (MT >= 2) {
+        constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
+        if (K % 512 == 0 && static_cast<size_t>(BT) * 16 * K * 2 <= 128 * 1024)
+            return launch_panel<MT, (PRO == PRO_NORM ? (MT == 4 ? 1 : 2) : (MT == 4 ? 4 : 8)), PRO, EPI, OUT>(
+                x, w, y, gain, eps, rows, n, N_out, K, stream);
+    }
     const int steps = pl_ceil_div(K, SK_KSTEP);
     const int most = max(4 * S::U4, max(8 * S::U8, 16 * S::U16));
     const int need = min(steps, most);     // beyond that, several rounds
