@@ -99,6 +99,13 @@ __device__ __forceinline__ uint32_t ap_pack2(float lo, float hi) {
 __host__ __device__ constexpr int ap_vpad(int dt) { return dt % 2 == 0 ? 32 : 0; }
 __host__ __device__ constexpr int ap_value_buffers(int ks) { return ks == 2 ? 3 : 2; }
 
+// The direct feed's permutation of the 16-byte pieces of an unpadded row in LDS (64 banks of 4 bytes: a row
+// of 128 elements covers them all once, of 64 elements half).  Piece c of the key with row number r (mod 16)
+// stands at c ^ shift.  Keys are read 16 rows at a time, one piece each: 16 different places.  Values are read
+// (transposed) four rows at a time, four neighbouring pieces each: four different groups of four.
+__device__ __forceinline__ int ap_key_shift(int r, int pieces) { return (pieces == 16 ? r : r >> 1) & (pieces - 1); }
+__device__ __forceinline__ int ap_value_shift(int r, int pieces) { return 4 * ((pieces == 16 ? r : r >> 1) & (pieces / 4 - 1)); }
+
 // UP (uniform pages): the 64 / (4*DT) keys whose pieces one wave loads with one instruction lie in one
 // page (the page size is a power of two and at least as many keys).  Page numbers then come through
 // the scalar unit and an address is a scalar base plus a lane's constant: no vector arithmetic a tile.
@@ -110,8 +117,8 @@ __host__ __device__ constexpr int ap_value_buffers(int ks) { return ks == 2 ? 3 
 // registers.  2: uniform pages, and the loads write LDS themselves (global_load_lds_dwordx4: lane l of
 // a wave puts its 16 bytes at the wave's LDS base + 16 l), three tiles ahead of their use and with no
 // register or LDS write instruction spent on them.  Rows then lie unpadded in LDS, so their 16-byte
-// pieces are permuted instead (piece c of key r stands at c ^ (r & 7) for keys, c ^ 2 (r & 7) for
-// values: the reads of the matrix cores' operands fall on every bank equally); heads of 64 and 128.
+// pieces are permuted instead (ap_key_shift, ap_value_shift: the reads of the matrix cores' operands
+// fall on every bank once); heads of 64 and 128.
 template <int DT, int NW, int KS, int FEED>
 __global__ void __launch_bounds__(64 * NW * KS, DT <= 4 ? AP_OCC : 1)
 paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
@@ -329,8 +336,8 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     int asked = 0, asked_k = 0, asked_v = 0;   // the next tile to ask for and its buffers
     uint32_t place_k = 0, place_v = 0;
     if constexpr (DIRECT) {
-        const int r7 = ((64 * wave_id) / CP + lane / CP) & 7;
-        const int ck = (lane % CP) ^ (r7 & (CP - 1)), cv = (lane % CP) ^ ((2 * r7) & (CP - 1));
+        const int r15 = ((64 * wave_id) / CP + lane / CP) & 15;
+        const int ck = (lane % CP) ^ ap_key_shift(r15, CP), cv = (lane % CP) ^ ap_value_shift(r15, CP);
         place_k = (lane / CP) * row_bytes + static_cast<uint32_t>(head_off + min(ck, cpr - 1) * 8) * 2;
         place_v = (lane / CP) * row_bytes + static_cast<uint32_t>(head_off + min(cv, cpr - 1) * 8) * 2;
     }
@@ -410,13 +417,13 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     // block of head elements 32*dt .. of this lane's four keys begins.
     int k_piece[2 * DT], v_piece[DT];
     if constexpr (DIRECT) {
-        const int x7 = r32 & 7;
+        const int fk = ap_key_shift(r32 & 15, CP);
 #pragma unroll
-        for (int kk = 0; kk < 2 * DT; ++kk) k_piece[kk] = (((2 * kk + h) ^ x7) & (CP - 1)) * 8;
+        for (int kk = 0; kk < 2 * DT; ++kk) k_piece[kk] = ((2 * kk + h) ^ fk) * 8;
         const int i16 = lane & 15, g = lane >> 4;
-        const int f = (2 * ((4 * h + (i16 >> 2)) & 7)) & (CP - 1);
+        const int fv = ap_value_shift(i16 >> 2, CP);     // of the lane's key 4h + i16/4 (+ 8, + 16: the same)
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) v_piece[dt] = ((4 * dt + 2 * (g & 1) + ((i16 & 3) >> 1)) ^ f) * 8 + 4 * (i16 & 1);
+        for (int dt = 0; dt < DT; ++dt) v_piece[dt] = ((4 * dt + 2 * (g & 1) + ((i16 & 3) >> 1)) ^ fv) * 8 + 4 * (i16 & 1);
     }
     // The multiplying half of a round: O^T += V^T . P^T for the tile before (sixteen keys a product:
     // pb[kt][half] holds the keys 32*(kt0+kt) + 16*half + {4h..4h+3} and + 8 + {4h..4h+3}; 16 lanes read a
