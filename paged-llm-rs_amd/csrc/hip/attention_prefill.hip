@@ -75,7 +75,7 @@ __device__ __forceinline__ ap_u32x2 ap_read_transposed(const uint16_t* at) {
 // tile two rounds ahead included.  The waits are placed by hand (s_waitcnt vmcnt) where a tile is due.
 __device__ __forceinline__ void ap_load_to_lds(const void* from, const uint16_t* lds_at) {
     const uint32_t at = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void*)lds_at));
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(at), "v"(from) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(at), "v"(from) : "memory", "m0");
 }
 
 typedef uint32_t ap_vec4 __attribute__((ext_vector_type(4)));   // 16 bytes on their way through registers

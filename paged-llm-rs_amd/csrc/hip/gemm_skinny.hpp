@@ -82,7 +82,7 @@ __device__ __forceinline__ void sk_load_gain(const float* gain, int k, float* ou
 // later read of LDS wait for it; the wait is written by hand where the panel is due.
 __device__ __forceinline__ void sk_load_to_lds(const void* from, const void* lds_at) {
     const uint32_t at = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void*)lds_at));
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(at), "v"(from) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(at), "v"(from) : "memory", "m0");
 }
 
 template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT, bool PANEL = false>
