@@ -130,6 +130,8 @@ def main() -> int:
                         help="fewer layers than the model has, where memory or time needs it; both numbers are reported")
     parser.add_argument("--no-graphs", action="store_true", help="run decode steps eagerly instead of as HIP graphs")
     parser.add_argument("--skip-points", action="store_true", help="leave out batch 1 and 64 and the prefill")
+    parser.add_argument("--prefill-eager", action="store_true",
+                        help="launch the prefill step kernel by kernel every time (a prompt length seen once)")
     parser.add_argument("--only", choices=["decode", "prefill"], default=None,
                         help="run one part alone (for a profiler): the decode steps at --batch, or the prefill")
     args = parser.parse_args()
@@ -181,10 +183,13 @@ def main() -> int:
             cache.manager.add_sequence(1000)
             assert cache.manager.reserve(1000, PREFILL_TOKENS)
             entry = [StepEntry(1000, prompt, 0, [PREFILL_TOKENS - 1])]
-            run_step(model, cache, entry)
+            if args.prefill_eager:
+                run_step(model, cache, entry)
+            else:
+                runner.run(entry)        # as the engine runs it: a shape of step that comes again is replayed from a graph
             cache.manager.free_sequence(1000)
 
-        seconds_prefill = timed(prefill, 5, 2)
+        seconds_prefill = timed(prefill, 5, 3)
         d, nq = cfg["head_dim"], cfg["num_attention_heads"]
         attention_flops = args.layers * 4 * nq * d * (PREFILL_TOKENS * (PREFILL_TOKENS + 1) // 2)
         flops = layer_flops * PREFILL_TOKENS + head_flops + attention_flops

@@ -37,6 +37,7 @@ class StepBatch:
                  num_logit_rows: int, max_q_len: int, max_ctx_len: int, seq_ids: list,
                  short_tokens: int | None = None):
         self.packed = packed
+        self.layout = layout
         self.num_tokens = num_tokens
         self.num_seqs = num_seqs
         self.num_logit_rows = num_logit_rows
@@ -61,9 +62,40 @@ class StepBatch:
         self.block_tables = [view(f"block_table_{g}", num_seqs, mb) for g, mb in enumerate(max_blocks)]
 
 
+def context_bound(longest: int) -> int:
+    """What a step reports as its longest context: the power of two (1024 at least) that holds it.  The
+    kernels size their launches and choose how to split the keys by it, so steps of one shape whose
+    contexts share a bound run the same launches, captured in a graph or not."""
+    bound = 1024
+    while bound < longest:
+        bound *= 2
+    return bound
+
+
+class CaptureOutgrown(Exception):
+    """A step no longer fits the fixed sizes it was to be laid out with."""
+
+
+class TableTooWide(CaptureOutgrown):
+    """A request has more pages than the rows of a fixed-width block table have room for."""
+
+    def __init__(self, group: int, pages: int):
+        super().__init__(f"group {group}: a table of {pages} pages")
+        self.group, self.pages = group, pages
+
+
+class ContextTooLong(CaptureOutgrown):
+    """A request's context is longer than the bound the step was to report."""
+
+
 def build_batch(entries, manager, num_groups: int, vocab_size: int, max_positions: int, device,
-                check_start: bool = True) -> StepBatch:
+                check_start: bool = True, widths: list | None = None, ctx_bound: int | None = None) -> StepBatch:
     """Validate the entries against the cache manager and lay the step out for the device.
+
+    ``widths`` fixes the pages a row of each group's block table has (TableTooWide if a request
+    has more) and ``ctx_bound`` what the batch reports as its longest context (ContextTooLong): a step laid out
+    so has the same layout, and gives the kernels the same launch sizes, as any other step with
+    the same tokens a request, whatever the requests' positions.
 
     Refused with ConfigError: an empty step, an entry without tokens, a token id
     outside the vocabulary, a position with no page or past the longest position
@@ -116,6 +148,11 @@ def build_batch(entries, manager, num_groups: int, vocab_size: int, max_position
         at += count
 
     max_blocks = [max(1, max(len(t) for t in tables[g])) for g in range(num_groups)]
+    if widths is not None:
+        for g in range(num_groups):
+            if max_blocks[g] > widths[g]:
+                raise TableTooWide(g, max_blocks[g])
+        max_blocks = list(widths)
     pieces = [("token_ids", token_ids), ("positions", positions), ("seq_of", seq_of), ("q_start", q_start),
               ("q_len", q_len), ("ctx_len", ctx_len), ("state_slots", state_slots),
               ("logit_rows", np.asarray(logit_rows, dtype=np.int32))]
@@ -135,5 +172,11 @@ def build_batch(entries, manager, num_groups: int, vocab_size: int, max_position
         host[begin:begin + count] = arr
     packed = torch.from_numpy(host).to(device)
     from ..kernels import SHORT_PORTION
-    return StepBatch(packed, layout, n, S, max_blocks, len(logit_rows), int(q_len.max()), int(ctx_len.max()),
+    longest = int(ctx_len.max())
+    if ctx_bound is None:
+        ctx_bound = context_bound(longest)
+    if longest > ctx_bound:
+        raise ContextTooLong(f"a context of {longest} tokens in a step laid out for {ctx_bound}")
+    longest = ctx_bound
+    return StepBatch(packed, layout, n, S, max_blocks, len(logit_rows), int(q_len.max()), longest,
                      [e.seq_id for e in entries], short_tokens=int(q_len[q_len < SHORT_PORTION].sum()))

@@ -7,8 +7,14 @@ A step in which every request brings exactly one token (plain decoding) is
 launch-bound: some two hundred small kernels.  Such steps are captured once as a
 HIP graph over static buffers, per (requests, pages a request) bucket, and
 replayed; the descriptor of the step is written into a pinned host buffer by the
-native cache manager and copied in with one transfer.  Every other step runs
-eagerly.  Both ways run the same model code and the same kernels.
+native cache manager and copied in with one transfer.
+
+Any other step costs the host some five milliseconds to launch, which is more
+than the GPU needs for a portion of a few hundred tokens.  A shape of step (the
+tokens each request brings and the places wanted, as when a long prompt is cut
+into equal portions) that comes a second time is captured too and replayed from
+then on; a few such graphs are kept.  A shape seen once runs eagerly.  All ways
+run the same model code and the same kernels.
 """
 
 from __future__ import annotations
@@ -21,9 +27,11 @@ import torch
 
 from .. import kernels
 from ..errors import ConfigError, PagedLLMError, TensorError
-from .batch import StepBatch, build_batch
+from .batch import CaptureOutgrown, StepBatch, TableTooWide, build_batch, context_bound
 
 GRAPH_MAX_REQUESTS = 64
+SHAPE_GRAPHS_KEPT = 6        # captured shapes of steps other than plain decoding, least recently used out first
+SHAPE_GRAPH_MAX_TOKENS = 8192
 
 
 def require_gpu(device) -> torch.device:
@@ -60,14 +68,6 @@ class StepOutput:
         return self.greedy
 
 
-class TableTooWide(Exception):
-    """A request has more pages than the rows of a captured graph's block table have room for."""
-
-    def __init__(self, group: int, pages: int):
-        super().__init__(f"group {group}: a table of {pages} pages")
-        self.group, self.pages = group, pages
-
-
 def _bucket(n: int, least: int = 1) -> int:
     b = least
     while b < n:
@@ -93,7 +93,7 @@ class DecodeGraph:
         self.device_buf = torch.zeros(offset, dtype=torch.int32, device=model.device)
         block_size = cache.block_size
         self.batch = StepBatch(self.device_buf, self.layout, cap, cap, list(widths), cap, 1,
-                               max(widths or [1]) * block_size, [])
+                               context_bound(max(widths or [1]) * block_size), [])
         h = self.host_np
         for name in ("seq_of", "q_start", "logit_rows"):
             b, c = self.layout[name]
@@ -167,19 +167,106 @@ class DecodeGraph:
         return StepOutput(self.logits[:live], self.tokens[:live])
 
 
+class ShapeGraph:
+    """A step of one shape (tokens a request, wanted places), with block tables of ``widths`` pages a
+    row and contexts up to ``ctx_bound``, captured."""
+
+    def __init__(self, model, cache, entries, widths: list, ctx_bound: int):
+        self.model, self.cache, self.widths, self.ctx_bound = model, cache, list(widths), ctx_bound
+        first = self._lay_out(entries)
+        self.size = first.packed.numel()
+        self.host = torch.zeros(self.size, dtype=torch.int32).pin_memory()
+        self.device_buf = torch.zeros(self.size, dtype=torch.int32, device=model.device)
+        self.host.copy_(first.packed)
+        self.layout = first.layout
+        self.batch = StepBatch(self.device_buf, first.layout, first.num_tokens, first.num_seqs, list(widths),
+                               first.num_logit_rows, first.max_q_len, ctx_bound, first.seq_ids,
+                               short_tokens=first.short_tokens)
+        self.graph = None
+        self.logits = None
+
+    def _lay_out(self, entries):
+        return build_batch(entries, self.cache.manager, len(self.cache.layout.groups), self.model.spec.vocab_size,
+                           self.model.spec.max_positions, "cpu", widths=self.widths, ctx_bound=self.ctx_bound)
+
+    def capture(self) -> None:
+        self.device_buf.copy_(self.host)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self.model.forward(self.batch, self.cache)     # lazy initialisation happens outside the capture
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.logits = self.model.forward(self.batch, self.cache)
+
+    def run(self, entries) -> StepOutput:
+        """Raises CaptureOutgrown when the step no longer fits what was captured."""
+        if self.graph is not None:
+            batch = self._lay_out(entries)
+            if batch.packed.numel() != self.size:
+                raise ConfigError("a step of another shape than the captured one")
+            self.host.copy_(batch.packed)
+        else:
+            self.capture()
+        self.device_buf.copy_(self.host, non_blocking=True)
+        self.graph.replay()
+        return StepOutput(self.logits)
+
+
 class StepRunner:
-    """Runs steps for one model and cache, keeping the captured decode graphs."""
+    """Runs steps for one model and cache, keeping the captured graphs."""
 
     def __init__(self, model, cache, graphs: bool = True):
         self.model, self.cache = model, cache
         self.use_graphs = graphs and getattr(model, "graph_safe", True)
         self._graphs: dict = {}
+        self._shapes: dict = {}          # shape of a step -> ShapeGraph, or None after its first (eager) run
         self.graph_steps = 0
         self.eager_steps = 0
 
     def _is_plain_decode(self, entries) -> bool:
         return (self.use_graphs and 0 < len(entries) <= GRAPH_MAX_REQUESTS
                 and all(len(e.tokens) == 1 and e.want == [0] for e in entries))
+
+    def _run_shaped(self, entries) -> StepOutput:
+        """A step other than plain decoding: eagerly the first time its shape comes, from a captured
+        graph from the second time on (while the requests' tables and contexts fit the capture)."""
+        tokens = sum(len(e.tokens) for e in entries)
+        if not self.use_graphs or tokens > SHAPE_GRAPH_MAX_TOKENS or len(entries) > GRAPH_MAX_REQUESTS:
+            self.eager_steps += 1
+            return StepOutput(run_step(self.model, self.cache, entries))
+        shape = tuple((len(e.tokens), tuple(e.want)) for e in entries)
+        known = shape in self._shapes
+        graph = self._shapes.pop(shape, None)
+        if not known:
+            self._shapes[shape] = None          # seen once
+            while len(self._shapes) > 4 * SHAPE_GRAPHS_KEPT:
+                self._shapes.pop(next(iter(self._shapes)))
+            self.eager_steps += 1
+            return StepOutput(run_step(self.model, self.cache, entries))
+        for e in entries:
+            if e.fresh_state and e.state_slot >= 0:
+                self.cache.clear_state_slot(e.state_slot)
+        if graph is not None:
+            try:
+                out = graph.run(entries)
+                self._shapes[shape] = graph     # most recently used last
+                self.graph_steps += 1
+                return out
+            except CaptureOutgrown:
+                pass                            # a request has outgrown the capture: a new one below
+        widths = [_bucket(w + 1, 32) for w in self._widths_needed(entries)]
+        longest = max(e.start + len(e.tokens) for e in entries)
+        graph = ShapeGraph(self.model, self.cache, entries, widths, context_bound(longest))
+        out = graph.run(entries)
+        self._shapes[shape] = graph
+        live = [k for k, g in self._shapes.items() if g is not None]
+        for k in live[:max(0, len(live) - SHAPE_GRAPHS_KEPT)]:
+            del self._shapes[k]
+        self.graph_steps += 1
+        return out
 
     def _widths_needed(self, entries) -> list:
         manager = self.cache.manager
@@ -190,8 +277,7 @@ class StepRunner:
         if not entries:
             raise ConfigError("an empty batch")
         if not self._is_plain_decode(entries):
-            self.eager_steps += 1
-            return StepOutput(run_step(self.model, self.cache, entries))
+            return self._run_shaped(entries)
         if len({e.seq_id for e in entries}) != len(entries):
             raise ConfigError("a request appears twice in one step")
         for e in entries:

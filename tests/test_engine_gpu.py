@@ -189,4 +189,40 @@ def test_a_captured_decode_step_replays_like_the_eager_one(model_dirs, dtype):
         assert np.array_equal(a[key], b[key]), f"{key}: a replay differs from the eager step"
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_shape_of_step_that_comes_again_is_captured_and_replays_like_the_eager_one(model_dirs, dtype):
+    """A long prompt cut into equal portions beside a request that decodes: from its second coming on a
+    shape of step is replayed from a graph.  Every replay is checked against the eager step, over
+    growing contexts (the tables outgrow the capture once) and with other shapes in between."""
+    from paged_llm_rs_amd.engine.replay import Replayer
+
+    d = model_dirs("B", dtype)
+    prompts = ru.make_prompts(384, [300, 60, 23], seed=33)
+    long_one, other, third = prompts["r0"], prompts["r1"], prompts["r2"]
+    steps, k = [], 0
+    steps.append({"step": k, "entries": [{"id": "r1", "tokens": other[:20], "want": [19]}], "end": []})
+    k += 1
+    fed, at = 20, 0
+    while at < 294:
+        entries = [{"id": "r0", "tokens": long_one[at:at + 21], "want": [20] if at + 21 >= 294 else []}]
+        if fed < len(other):
+            entries.append({"id": "r1", "tokens": [other[fed]], "want": [0]})
+            fed += 1
+        steps.append({"step": k, "entries": entries, "end": []})
+        at += 21
+        k += 1
+        if k == 6:      # another shape in between
+            steps.append({"step": k, "entries": [{"id": "r2", "tokens": third, "want": [len(third) - 1]}], "end": ["r2"]})
+            k += 1
+    steps.append({"step": k, "entries": [{"id": "r0", "tokens": long_one[294:], "want": [5]}], "end": ["r0", "r1"]})
+    eager = Replayer(d, dtype, max_tokens=64 * 8, block_size=8, graphs=False)
+    graph = Replayer(d, dtype, max_tokens=64 * 8, block_size=8, graphs=True)
+    a = ru.collect(eager, steps)
+    b = ru.collect(graph, steps)
+    assert graph.runner.graph_steps >= 10 and eager.runner.graph_steps == 0
+    assert a.keys() == b.keys() and len(a) >= 12
+    for key in a:
+        assert np.array_equal(a[key], b[key]), f"{key}: a replay differs from the eager step"
+
+
 import numpy as np  # noqa: E402
