@@ -166,7 +166,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     if (seq >= num_seqs) return;
 
     const int count = q_len[seq];
-    if (count < short_limit) return;
+    if (count < short_limit || ctx_len[seq] <= 0) return;   // a request of padding rows has no context
     const int q0 = tile * BM;
     if (q0 >= count) return;
     const int start = ctx_len[seq] - count;  // position of the request's first token in this step
@@ -706,15 +706,15 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
 __global__ void __launch_bounds__(256)
 paged_attention_prefill_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
                                      bf16_t* __restrict__ out, const int* __restrict__ q_start,
-                                     const int* __restrict__ q_len, int short_limit, int tiles_a_request, int num_seqs,
-                                     int nq, int d, int splits, int bm) {
+                                     const int* __restrict__ q_len, const int* __restrict__ ctx_len, int short_limit,
+                                     int tiles_a_request, int num_seqs, int nq, int d, int splits, int bm) {
     const int work = blockIdx.x;
     const int tile = work % tiles_a_request;
     const int head = (work / tiles_a_request) % nq;
     const int seq = work / (tiles_a_request * nq);
     if (seq >= num_seqs) return;
     const int count = q_len[seq];
-    if (count < short_limit) return;
+    if (count < short_limit || ctx_len[seq] <= 0) return;
     const int quads = d / 4, rows = blockDim.x / quads;
     const int r = tile * bm + blockIdx.y * rows + threadIdx.x / quads;
     const int e0 = (threadIdx.x % quads) * 4;
@@ -783,7 +783,8 @@ static int launch_prefill(const void* q, int q_stride, void* out, const int* q_s
     if (splits > 1) {
         const int rows = 256 / (d / 4);
         paged_attention_prefill_merge_kernel<<<dim3(static_cast<int>(whole), pl_ceil_div(BM, rows)), 256, 0, stream>>>(
-            part_acc, part_ml, static_cast<bf16_t*>(out), q_start, q_len, short_limit, tiles, num_seqs, nq, d, splits, BM);
+            part_acc, part_ml, static_cast<bf16_t*>(out), q_start, q_len, ctx_len, short_limit, tiles, num_seqs, nq, d,
+            splits, BM);
         PL_CHECK_LAUNCH("paged_attention_prefill_merge");
     }
     return 0;

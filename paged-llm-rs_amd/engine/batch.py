@@ -40,6 +40,7 @@ class StepBatch:
         self.layout = layout
         self.num_tokens = num_tokens
         self.num_seqs = num_seqs
+        self.live_seqs = num_seqs        # without the request of padding rows at the end, if there is one
         self.num_logit_rows = num_logit_rows
         self.max_q_len = max_q_len
         self.max_ctx_len = max_ctx_len
@@ -88,14 +89,31 @@ class ContextTooLong(CaptureOutgrown):
     """A request's context is longer than the bound the step was to report."""
 
 
+def token_bucket(tokens: int) -> int:
+    """The number of rows a step of so many tokens is padded to: steps of many lengths then have few
+    shapes, and a shape that comes again replays from a graph."""
+    for small in (16, 32, 64):
+        if tokens <= small:
+            return small
+    step = 64 if tokens <= 1024 else 256
+    return (tokens + step - 1) // step * step
+
+
 def build_batch(entries, manager, num_groups: int, vocab_size: int, max_positions: int, device,
-                check_start: bool = True, widths: list | None = None, ctx_bound: int | None = None) -> StepBatch:
+                check_start: bool = True, widths: list | None = None, ctx_bound: int | None = None,
+                pad_to: int | None = None) -> StepBatch:
     """Validate the entries against the cache manager and lay the step out for the device.
 
     ``widths`` fixes the pages a row of each group's block table has (TableTooWide if a request
     has more) and ``ctx_bound`` what the batch reports as its longest context (ContextTooLong): a step laid out
     so has the same layout, and gives the kernels the same launch sizes, as any other step with
     the same tokens a request, whatever the requests' positions.
+
+    ``pad_to`` adds one more request after the others that holds the rows up to that many: padding
+    (token 0, position -1, no pages, no context, state slot -1; it has no rows when none are
+    missing).  The batch then reports bounds instead of counts (every row might belong to one
+    request, or to short ones), so that steps with the same rows, requests and wanted places give
+    the kernels the same launch sizes.
 
     Refused with ConfigError: an empty step, an entry without tokens, a token id
     outside the vocabulary, a position with no page or past the longest position
@@ -106,11 +124,14 @@ def build_batch(entries, manager, num_groups: int, vocab_size: int, max_position
     if not entries:
         raise ConfigError("an empty batch")
     seen = set()
-    n = sum(len(e.tokens) for e in entries)
-    S = len(entries)
-    token_ids = np.empty(n, np.int32)
-    positions = np.empty(n, np.int32)
-    seq_of = np.empty(n, np.int32)
+    live = sum(len(e.tokens) for e in entries)
+    if pad_to is not None and pad_to < live:
+        raise ConfigError(f"{live} tokens in a step padded to {pad_to}")
+    n = live if pad_to is None else pad_to
+    S = len(entries) + (0 if pad_to is None else 1)
+    token_ids = np.zeros(n, np.int32)
+    positions = np.full(n, -1, np.int32)
+    seq_of = np.full(n, S - 1, np.int32)
     q_start = np.empty(S, np.int32)
     q_len = np.empty(S, np.int32)
     ctx_len = np.empty(S, np.int32)
@@ -146,6 +167,10 @@ def build_batch(entries, manager, num_groups: int, vocab_size: int, max_position
         for g in range(num_groups):
             tables[g].append(manager.table(e.seq_id, g))
         at += count
+    if pad_to is not None:
+        q_start[S - 1], q_len[S - 1], ctx_len[S - 1], state_slots[S - 1] = live, n - live, 0, -1
+        for g in range(num_groups):
+            tables[g].append([])
 
     max_blocks = [max(1, max(len(t) for t in tables[g])) for g in range(num_groups)]
     if widths is not None:
@@ -178,5 +203,12 @@ def build_batch(entries, manager, num_groups: int, vocab_size: int, max_position
     if longest > ctx_bound:
         raise ContextTooLong(f"a context of {longest} tokens in a step laid out for {ctx_bound}")
     longest = ctx_bound
+    if pad_to is not None:
+        # every row might belong to one request; if any request is short, every row might
+        any_short = bool((q_len[:S - 1] < SHORT_PORTION).any())
+        batch = StepBatch(packed, layout, n, S, max_blocks, len(logit_rows), n, longest,
+                          [e.seq_id for e in entries], short_tokens=n if any_short else 0)
+        batch.live_seqs = S - 1
+        return batch
     return StepBatch(packed, layout, n, S, max_blocks, len(logit_rows), int(q_len.max()), longest,
                      [e.seq_id for e in entries], short_tokens=int(q_len[q_len < SHORT_PORTION].sum()))

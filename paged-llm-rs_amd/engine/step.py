@@ -10,10 +10,11 @@ replayed; the descriptor of the step is written into a pinned host buffer by the
 native cache manager and copied in with one transfer.
 
 Any other step costs the host some five milliseconds to launch, which is more
-than the GPU needs for a portion of a few hundred tokens.  A shape of step (the
-tokens each request brings and the places wanted, as when a long prompt is cut
-into equal portions) that comes a second time is captured too and replayed from
-then on; a few such graphs are kept.  A shape seen once runs eagerly.  All ways
+than the GPU needs for a portion of a few hundred tokens.  Such steps are
+padded with rows that belong to no request up to a bucket of tokens, so that
+steps of many lengths have few shapes (rows, requests, wanted places); a shape
+that comes a second time is captured too and replayed from then on, and a few
+such graphs are kept.  A shape seen once runs eagerly, padded alike.  All ways
 run the same model code and the same kernels.
 """
 
@@ -27,10 +28,11 @@ import torch
 
 from .. import kernels
 from ..errors import ConfigError, PagedLLMError, TensorError
-from .batch import CaptureOutgrown, StepBatch, TableTooWide, build_batch, context_bound
+from .batch import CaptureOutgrown, StepBatch, TableTooWide, build_batch, context_bound, token_bucket
 
 GRAPH_MAX_REQUESTS = 64
-SHAPE_GRAPHS_KEPT = 6        # captured shapes of steps other than plain decoding, least recently used out first
+SHAPE_GRAPH_ROWS_KEPT = 32768    # rows over all captured shapes of steps other than plain decoding (the
+                                 # least recently used go first): their buffers stay allocated
 SHAPE_GRAPH_MAX_TOKENS = 8192
 
 
@@ -41,10 +43,10 @@ def require_gpu(device) -> torch.device:
     return device
 
 
-def run_step(model, cache, entries, check_start: bool = True) -> torch.Tensor:
+def run_step(model, cache, entries, check_start: bool = True, pad_to: int | None = None) -> torch.Tensor:
     """32-bit logits [wanted places, vocabulary], in the order of the entries and of their ``want``."""
     batch = build_batch(entries, cache.manager, len(cache.layout.groups), model.spec.vocab_size,
-                        model.spec.max_positions, model.device, check_start=check_start)
+                        model.spec.max_positions, model.device, check_start=check_start, pad_to=pad_to)
     for e in entries:
         if e.fresh_state and e.state_slot >= 0:
             cache.clear_state_slot(e.state_slot)
@@ -168,11 +170,11 @@ class DecodeGraph:
 
 
 class ShapeGraph:
-    """A step of one shape (tokens a request, wanted places), with block tables of ``widths`` pages a
-    row and contexts up to ``ctx_bound``, captured."""
+    """A step of one shape (rows after padding, requests, wanted places), with block tables of
+    ``widths`` pages a row and contexts up to ``ctx_bound``, captured."""
 
-    def __init__(self, model, cache, entries, widths: list, ctx_bound: int):
-        self.model, self.cache, self.widths, self.ctx_bound = model, cache, list(widths), ctx_bound
+    def __init__(self, model, cache, entries, widths: list, ctx_bound: int, rows: int):
+        self.model, self.cache, self.widths, self.ctx_bound, self.rows = model, cache, list(widths), ctx_bound, rows
         first = self._lay_out(entries)
         self.size = first.packed.numel()
         self.host = torch.zeros(self.size, dtype=torch.int32).pin_memory()
@@ -180,14 +182,16 @@ class ShapeGraph:
         self.host.copy_(first.packed)
         self.layout = first.layout
         self.batch = StepBatch(self.device_buf, first.layout, first.num_tokens, first.num_seqs, list(widths),
-                               first.num_logit_rows, first.max_q_len, ctx_bound, first.seq_ids,
+                               first.num_logit_rows, first.max_q_len, ctx_bound, [],
                                short_tokens=first.short_tokens)
+        self.batch.live_seqs = first.live_seqs
         self.graph = None
         self.logits = None
 
     def _lay_out(self, entries):
         return build_batch(entries, self.cache.manager, len(self.cache.layout.groups), self.model.spec.vocab_size,
-                           self.model.spec.max_positions, "cpu", widths=self.widths, ctx_bound=self.ctx_bound)
+                           self.model.spec.max_positions, "cpu", widths=self.widths, ctx_bound=self.ctx_bound,
+                           pad_to=self.rows)
 
     def capture(self) -> None:
         self.device_buf.copy_(self.host)
@@ -221,6 +225,9 @@ class StepRunner:
     def __init__(self, model, cache, graphs: bool = True):
         self.model, self.cache = model, cache
         self.use_graphs = graphs and getattr(model, "graph_safe", True)
+        # A model whose parts all take padding rows gets its steps padded whether graphs are on or not,
+        # so that a step launches the same kernels either way.
+        self.pads = getattr(model, "graph_safe", True)
         self._graphs: dict = {}
         self._shapes: dict = {}          # shape of a step -> ShapeGraph, or None after its first (eager) run
         self.graph_steps = 0
@@ -234,18 +241,20 @@ class StepRunner:
         """A step other than plain decoding: eagerly the first time its shape comes, from a captured
         graph from the second time on (while the requests' tables and contexts fit the capture)."""
         tokens = sum(len(e.tokens) for e in entries)
-        if not self.use_graphs or tokens > SHAPE_GRAPH_MAX_TOKENS or len(entries) > GRAPH_MAX_REQUESTS:
+        rows = token_bucket(tokens) if self.pads and tokens <= SHAPE_GRAPH_MAX_TOKENS else None
+        if not self.use_graphs or rows is None or len(entries) > GRAPH_MAX_REQUESTS:
             self.eager_steps += 1
-            return StepOutput(run_step(self.model, self.cache, entries))
-        shape = tuple((len(e.tokens), tuple(e.want)) for e in entries)
+            return StepOutput(run_step(self.model, self.cache, entries, pad_to=rows))
+        short = any(len(e.tokens) < kernels.SHORT_PORTION for e in entries)
+        shape = (rows, len(entries), sum(len(e.want) for e in entries), short)
         known = shape in self._shapes
         graph = self._shapes.pop(shape, None)
         if not known:
             self._shapes[shape] = None          # seen once
-            while len(self._shapes) > 4 * SHAPE_GRAPHS_KEPT:
+            while len(self._shapes) > 256:
                 self._shapes.pop(next(iter(self._shapes)))
             self.eager_steps += 1
-            return StepOutput(run_step(self.model, self.cache, entries))
+            return StepOutput(run_step(self.model, self.cache, entries, pad_to=rows))
         for e in entries:
             if e.fresh_state and e.state_slot >= 0:
                 self.cache.clear_state_slot(e.state_slot)
@@ -259,11 +268,15 @@ class StepRunner:
                 pass                            # a request has outgrown the capture: a new one below
         widths = [_bucket(w + 1, 32) for w in self._widths_needed(entries)]
         longest = max(e.start + len(e.tokens) for e in entries)
-        graph = ShapeGraph(self.model, self.cache, entries, widths, context_bound(longest))
+        graph = ShapeGraph(self.model, self.cache, entries, widths, context_bound(longest), rows)
         out = graph.run(entries)
         self._shapes[shape] = graph
         live = [k for k, g in self._shapes.items() if g is not None]
-        for k in live[:max(0, len(live) - SHAPE_GRAPHS_KEPT)]:
+        held = sum(k[0] for k in live)
+        for k in live[:-1]:
+            if held <= SHAPE_GRAPH_ROWS_KEPT:
+                break
+            held -= k[0]
             del self._shapes[k]
         self.graph_steps += 1
         return out

@@ -63,7 +63,13 @@ def _check(code: int) -> None:
         raise TensorError(library().pl_last_error().decode())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    """The handle of torch's current stream on the current device (asked for once a launch: the short way)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -360,12 +366,13 @@ def paged_attention_prefill(q: torch.Tensor, q_row_stride: int, out: torch.Tenso
                             q_len: torch.Tensor, ctx_len: torch.Tensor, max_q_len: int, block_table: torch.Tensor,
                             block_size: int, k_pool: torch.Tensor, v_pool: torch.Tensor, nq: int, nkv: int, d: int,
                             scale: float, window: int = 0, short_limit: int = 0, max_ctx: int | None = None,
-                            splits: int | None = None) -> torch.Tensor:
+                            splits: int | None = None, live_seqs: int | None = None) -> torch.Tensor:
     """bfloat16 attention of prompt portions on the matrix cores.  Request s brings the rows
     q_start[s] .. q_start[s]+q_len[s]-1 at the positions ctx_len[s]-q_len[s] .. ctx_len[s]-1;
     requests with fewer than ``short_limit`` tokens are skipped.  ``max_ctx`` (the longest context
     of the step) lets the keys of a token tile be dealt to several workgroups where the tiles alone
-    would leave compute units idle; ``splits`` sets their number by hand."""
+    would leave compute units idle; ``splits`` sets their number by hand.  ``live_seqs``: only so many
+    of the requests, the first ones, bring tokens (the rest is padding and gets no workgroups)."""
     n = q.shape[0]
     S = block_table.shape[0]
     _need(q, "query buffer", None, torch.bfloat16)
@@ -382,15 +389,18 @@ def paged_attention_prefill(q: torch.Tensor, q_row_stride: int, out: torch.Tenso
             raise TensorError(f"{what} has shape {tuple(pool.shape)}, expected [pages*{block_size}, {nkv * d}]")
     if not 0 < max_q_len <= n:
         raise TensorError(f"the longest portion is said to have {max_q_len} of the step's {n} tokens")
+    live = S if live_seqs is None else int(live_seqs)
+    if not 0 < live <= S:
+        raise TensorError(f"{live} requests with tokens of {S}")
     if splits is None:
-        splits = prefill_splits(S, int(max_q_len), nq, d, int(max_ctx or 0), n)
+        splits = prefill_splits(live, int(max_q_len), nq, d, int(max_ctx or 0), n)
     part_acc = part_ml = None
     if splits > 1:
         part_acc = torch.empty((n * nq * splits * d,), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((n * nq * splits * 2,), dtype=torch.float32, device=q.device)
     _check(library().pl_paged_attention_prefill(
         q.data_ptr(), q_row_stride, out.data_ptr(), q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(),
-        int(short_limit), S, int(max_q_len), block_table.data_ptr(), block_table.shape[1], block_size,
+        int(short_limit), live, int(max_q_len), block_table.data_ptr(), block_table.shape[1], block_size,
         k_pool.data_ptr(), v_pool.data_ptr(), nq, nkv, d, float(scale), int(window or 0), int(splits),
         part_acc.data_ptr() if splits > 1 else None, part_ml.data_ptr() if splits > 1 else None, _stream()))
     return out
@@ -457,7 +467,8 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nk
     if batch.max_q_len >= SHORT_PORTION:
         paged_attention_prefill(qkv, stride, out, batch.q_start, batch.q_len, batch.ctx_len, batch.max_q_len,
                                 kv.block_table, kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window,
-                                short_limit=SHORT_PORTION, max_ctx=batch.max_ctx_len)
+                                short_limit=SHORT_PORTION, max_ctx=batch.max_ctx_len,
+                                live_seqs=getattr(batch, "live_seqs", None))
         if batch.short_tokens == 0:
             return out
     mixed = batch.max_q_len >= SHORT_PORTION
