@@ -98,10 +98,32 @@ TINY_C = {
     "tie_word_embeddings": False,
 }
 
+# The layer sizes of Qwen3-0.6B (the sizes the kernels are tuned for: heads of 128, pages of 16), two
+# layers of them, with a vocabulary that is no multiple of anything.
+LAYERS_0P6B = {
+    "architectures": ["Qwen3ForCausalLM"],
+    "model_type": "qwen3",
+    "hidden_act": "silu",
+    "attention_bias": False,
+    "sliding_window": None,
+    "hidden_size": 1024,
+    "intermediate_size": 3072,
+    "num_hidden_layers": 2,
+    "num_attention_heads": 16,
+    "num_key_value_heads": 8,
+    "head_dim": 128,
+    "rms_norm_eps": 1e-6,
+    "rope_theta": 1000000.0,
+    "vocab_size": 4099,
+    "max_position_embeddings": 4096,
+    "tie_word_embeddings": True,
+}
+
 TINY_INIT = {
     "A": dict(config=TINY_A, seed=0, std=0.02, gain_std=0.1),
     "B": dict(config=TINY_B, seed=1, std=0.05, gain_std=0.2),
     "C": dict(config=TINY_C, seed=2, std=0.08, gain_std=0.2),
+    "D": dict(config=LAYERS_0P6B, seed=3, std=0.02, gain_std=0.1),
 }
 
 
