@@ -132,8 +132,10 @@ def main() -> int:
     parser.add_argument("--skip-points", action="store_true", help="leave out batch 1 and 64 and the prefill")
     parser.add_argument("--prefill-eager", action="store_true",
                         help="launch the prefill step kernel by kernel every time (a prompt length seen once)")
-    parser.add_argument("--only", choices=["decode", "prefill"], default=None,
-                        help="run one part alone (for a profiler): the decode steps at --batch, or the prefill")
+    parser.add_argument("--only", choices=["decode", "prefill", "engine"], default=None,
+                        help="run one part alone: the decode steps at --batch, the prefill, or (not part of the "
+                             "default line) the whole engine on 1/4/16/32/64 requests at once, 16 prompt tokens and "
+                             "128 generated each, as the reference's own table of clients does")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU; this engine has no multi-GPU path (N must be 1)")
@@ -199,6 +201,27 @@ def main() -> int:
 
     if args.only == "prefill":
         print(json.dumps({"prefill": prefill_point()}), flush=True)
+        tmp.cleanup()
+        return 0
+    if args.only == "engine":
+        # scheduler, cache manager, step function, sampling and the read-back of every token: generate()
+        from paged_llm_rs_amd.engine.engine import Engine
+
+        del runner, cache
+        engine = Engine(folder, dtype="bf16", block_size=BLOCK_SIZE, num_blocks=64 * 12 + 64, max_batch=64, chunk=128)
+        rng = random.Random(7)
+        result = {}
+        for clients in (1, 4, 16, 32, 64):
+            prompts = [[rng.randrange(cfg["vocab_size"]) for _ in range(16)] for _ in range(clients)]
+            for timed_run in (False, False, True):      # a shape of step is captured when it comes the second time
+                torch.cuda.synchronize()
+                start = time.perf_counter()
+                out = engine.generate(prompts, max_tokens=128, temperature=0.0, stop_tokens=[])
+                seconds = time.perf_counter() - start
+            made = sum(len(o["tokens"]) for o in out)
+            result[f"clients_{clients}"] = {"tokens_per_s": round(made / seconds, 1), "seconds": round(seconds, 3)}
+            say(f"engine, {clients} requests: {made / seconds:.0f} tokens/s")
+        print(json.dumps({"engine": result}), flush=True)
         tmp.cleanup()
         return 0
 
