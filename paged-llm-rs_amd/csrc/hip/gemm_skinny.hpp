@@ -342,6 +342,196 @@ static int launch_one(int waves, const void* x, const void* w, void* y, const fl
     return 0;
 }
 
+// ---------------------------------------------------------------------------
+// More than 16 rows, K a multiple of 512: every wave takes ONE tile of 16 rows and one stretch of K.
+// The workgroup's rows of w come into LDS first (as with PANEL above, and the norm's gains beside
+// them), so that w costs the waves no registers; a wave then asks for its whole share of x at once,
+// STEPS K steps of 16 bytes a lane (32 with the 32-bit stream), and multiplies as they arrive.  With MT
+// tiles of rows there are WV / MT stretches of K.  The partial tiles and sums of squares meet in LDS
+// (where the panel was) and every thread finishes one element of one tile.
+// ---------------------------------------------------------------------------
+template <int MT, int WV, int STEPS, int PRO, int EPI, typename OUT>
+__global__ void __launch_bounds__(64 * WV)
+gemm_skinny_rows_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OUT* __restrict__ y,
+                        const float* __restrict__ gain, float eps, const int* __restrict__ rows, int n, int N_out,
+                        int K) {
+    constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
+    constexpr int NKS = WV / MT;                                // stretches of K
+    extern __shared__ float sk_lds[];
+    bf16_t* panel = reinterpret_cast<bf16_t*>(sk_lds);          // [BT * 16][K], pieces permuted
+    float* gain_lds = sk_lds + BT * 16 * K / 2;                 // [K] (PRO_NORM)
+    float* red = sk_lds;                                        // [NKS][MT][BT][256], once the panel is done with
+    float* ssq_lds = sk_lds + NKS * MT * BT * 256;              // [NKS][MT][16]
+
+    const int lane = threadIdx.x % PL_WAVE;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PL_WAVE);
+    const int c = lane % 16, g = lane / 16;
+    const int mt = wave % MT, ks = wave / MT;
+    const bool working = ks < NKS;                              // WV need not be a multiple of MT
+    const int num_tiles = pl_ceil_div(N_out, SK_TILE_N);
+    const int per_slice = K / SK_KSTEP / NKS * SK_KSTEP;        // K is a multiple of 512, NKS of 16 at most... see the launcher
+    const int kbeg = ks * per_slice;
+
+    // the wave's rows of x, asked for once: they serve every tile of columns
+    const int row = mt * 16 + c;
+    const bool row_ok = working && row < n;
+    int src = row_ok ? row : 0;
+    if (PRO == PRO_NORM && rows) src = rows[src];
+    const size_t xrow = static_cast<size_t>(src) * K;
+    const bf16_t* xb = static_cast<const bf16_t*>(x_);
+    const float* xf = static_cast<const float*>(x_);
+    bf16x8 ax[PRO == PRO_BF16 ? STEPS : 1];
+    sk_f32x4 raw[PRO == PRO_NORM ? STEPS : 1][2];
+#pragma unroll
+    for (int u = 0; u < STEPS; ++u) {
+        const int at = kbeg + u * SK_KSTEP + g * 8;
+        const int kk = (u * SK_KSTEP < per_slice) ? at : 0;
+        if (PRO == PRO_BF16) {
+            ax[u] = sk_load8(xb + xrow + kk);
+        } else {
+            raw[u][0] = *reinterpret_cast<const sk_f32x4*>(xf + xrow + kk);
+            raw[u][1] = *reinterpret_cast<const sk_f32x4*>(xf + xrow + kk + 4);
+        }
+    }
+    if (PRO == PRO_NORM)
+        for (int k = threadIdx.x * 4; k < K; k += blockDim.x * 4)
+            *reinterpret_cast<sk_f32x4*>(gain_lds + k) = *reinterpret_cast<const sk_f32x4*>(gain + k);
+
+    for (int tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
+        const int n0 = tile * SK_TILE_N;
+        {
+            const int chunks = K / 512, loads = BT * 16 * chunks;
+            for (int j = wave; j < loads; j += WV) {
+                const int prow = j / chunks, chunk = j - prow * chunks;
+                const int r = prow % 16;
+                const size_t grow = (prow >= 16 ? N_out : 0) + static_cast<size_t>(n0 + r < N_out ? n0 + r : 0);
+                const int piece = (chunk * 64 + lane) ^ r;
+                sk_load_to_lds(w + grow * K + piece * 8, panel + static_cast<size_t>(prow) * K + chunk * 512);
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);                     // vmcnt(0): x and this wave's share of the panel
+        __syncthreads();
+
+        f32x4 acc[BT];
+#pragma unroll
+        for (int b = 0; b < BT; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+        float ssq = 0.f;
+        // Rows past n and steps past the stretch are not branched around: a row past n gives outputs that
+        // are not stored, and a step past the stretch multiplies by zeros instead of w (x is only looked
+        // at here, after the panel has been asked for, so nothing waits for it earlier).
+        const int nsteps = per_slice / SK_KSTEP;
+        // four steps' pieces of w are read from LDS before their products, so that LDS is waited for once in four
+        static_assert(STEPS % 4 == 0, "steps are taken four at a time");
+#pragma unroll
+        for (int u0 = 0; u0 < STEPS; u0 += 4) {
+            bf16x8 bw[4][BT];
+            int kk[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bool live = u0 + j < nsteps;
+                kk[j] = kbeg + (live ? u0 + j : 0) * SK_KSTEP + g * 8;
+#pragma unroll
+                for (int b = 0; b < BT; ++b) {
+                    const bf16x8 got = sk_load8(panel + static_cast<size_t>(b * 16 + c) * K + (((kk[j] >> 3) ^ c) << 3));
+                    bw[j][b] = live ? got : sk_zero8();
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int u = u0 + j;
+                bf16x8 a;
+                if (PRO == PRO_BF16) {
+                    a = ax[u];
+                } else {
+                    const bool live = u < nsteps;
+                    const sk_f32x4 g0 = *reinterpret_cast<const sk_f32x4*>(gain_lds + kk[j]);
+                    const sk_f32x4 g1 = *reinterpret_cast<const sk_f32x4*>(gain_lds + kk[j] + 4);
+                    f32x8 v;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float xv = raw[u][e / 4].v[e % 4];
+                        ssq = live ? fmaf(xv, xv, ssq) : ssq;
+                        v[e] = xv * (e < 4 ? g0.v[e % 4] : g1.v[e % 4]);
+                    }
+                    a = __builtin_convertvector(v, bf16x8);
+                }
+#pragma unroll
+                for (int b = 0; b < BT; ++b)
+                    acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bw[j][b], acc[b], 0, 0, 0);
+            }
+        }
+        __syncthreads();                                        // every wave has read its last of the panel
+        if (working) {
+#pragma unroll
+            for (int b = 0; b < BT; ++b)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) red[((ks * MT + mt) * BT + b) * 256 + lane * 4 + i] = acc[b][i];
+            if (PRO == PRO_NORM) {
+                float s = ssq;
+                s += __shfl_xor(s, 16, PL_WAVE);
+                s += __shfl_xor(s, 32, PL_WAVE);
+                if (g == 0) ssq_lds[(ks * MT + mt) * 16 + c] = s;
+            }
+        }
+        __syncthreads();
+        // one element of one tile a thread: element t of tile m is row (t/64)*4 + t%4 of the tile, column (t/4)%16
+        for (int e = threadIdx.x; e < MT * 256; e += blockDim.x) {
+            const int m = e / 256, t = e % 256;
+            const int src_lane = t / 4, i = t % 4;
+            const int row_in_tile = (src_lane / 16) * 4 + i;
+            const int out_row = m * 16 + row_in_tile, col = n0 + src_lane % 16;
+            float v[BT];
+#pragma unroll
+            for (int b = 0; b < BT; ++b) {
+                float s = 0.f;
+#pragma unroll
+                for (int k = 0; k < NKS; ++k) s += red[((k * MT + m) * BT + b) * 256 + t];
+                v[b] = s;
+            }
+            if (PRO == PRO_NORM) {
+                float total = 0.f;
+#pragma unroll
+                for (int k = 0; k < NKS; ++k) total += ssq_lds[(k * MT + m) * 16 + row_in_tile];
+                const float rinv = 1.f / sqrtf(total / static_cast<float>(K) + eps);
+#pragma unroll
+                for (int b = 0; b < BT; ++b) v[b] *= rinv;
+            }
+            if (out_row < n && col < N_out) {
+                float r = v[0];
+                if (EPI == EPI_SWIGLU) r = v[0] / (1.f + __expf(-v[0])) * v[BT - 1];
+                const size_t at = static_cast<size_t>(out_row) * N_out + col;
+                if (EPI == EPI_ADD)
+                    y[at] = from_float<OUT>(to_float(y[at]) + r);
+                else
+                    y[at] = from_float<OUT>(r);
+            }
+        }
+        __syncthreads();  // the next tile's panel lands where the partial tiles are
+    }
+}
+
+// The rows variant's launch: WV waves, MT tiles of rows, WV / MT stretches of K of at most STEPS steps.
+template <int MT, int WV, int STEPS, int PRO, int EPI, typename OUT>
+static int launch_rows(const void* x, const void* w, void* y, const float* gain, float eps,
+                       const int* rows, int n, int N_out, int K, hipStream_t stream) {
+    constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
+    constexpr int NKS = WV / MT;
+    const int grid = min(pl_ceil_div(N_out, SK_TILE_N), SK_MAX_GRID);
+    const size_t panel_bytes = static_cast<size_t>(BT) * 16 * K * 2 + (PRO == PRO_NORM ? static_cast<size_t>(K) * 4 : 0);
+    const size_t red_bytes = static_cast<size_t>(NKS) * MT * (BT * 256 + 16) * sizeof(float);
+    const size_t lds_bytes = panel_bytes > red_bytes ? panel_bytes : red_bytes;
+    auto kernel = &gemm_skinny_rows_kernel<MT, WV, STEPS, PRO, EPI, OUT>;
+    if (lds_bytes > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           static_cast<int>(lds_bytes));
+        PL_REQUIRE(e == hipSuccess, "skinny product: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
+    }
+    kernel<<<grid, 64 * WV, lds_bytes, stream>>>(x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps,
+                                                rows, n, N_out, K);
+    PL_CHECK_LAUNCH("gemm_skinny");
+    return 0;
+}
+
 // The panel variant: 8 waves (256 registers a lane); a wave holds 16 * MT rows of x for UNR K steps.
 template <int MT, int UNR, int PRO, int EPI, typename OUT>
 static int launch_panel(const void* x, const void* w, void* y, const float* gain, float eps,
@@ -381,6 +571,20 @@ template <int MT, int PRO, int EPI, typename OUT>
 static int launch_unr(const void* x, const void* w, void* y, const float* gain, float eps,
                       const int* rows, int n, int N_out, int K, hipStream_t stream) {
     using S = SkShape<MT, PRO, EPI>;
+    if constexpr (MT == 2 || MT == 4) {
+        // 16 waves: 16 / MT stretches of K, each a whole number of K steps that a wave can hold at once
+        constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
+        constexpr int NKS = 16 / MT;
+        const size_t panel = static_cast<size_t>(BT) * 16 * K * 2 + (PRO == PRO_NORM ? static_cast<size_t>(K) * 4 : 0);
+        const int need = K / SK_KSTEP / NKS;             // K steps a wave holds at once
+        if (K % 512 == 0 && K / SK_KSTEP % NKS == 0 && panel <= 144 * 1024) {
+            if (need <= 8) return launch_rows<MT, 16, 8, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, stream);
+            if constexpr (PRO == PRO_BF16) {             // the 32-bit stream takes twice the registers a step
+                // (24 steps would fit the registers of 16 waves only with spills: such a K goes the way below)
+                if (need <= 16) return launch_rows<MT, 16, 16, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, stream);
+            }
+        }
+    }
     if constexpr (MT >= 2) {
         constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
         if (K % 512 == 0 && static_cast<size_t>(BT) * 16 * K * 2 <= 128 * 1024)
