@@ -87,9 +87,11 @@ extern "C" int pl_argmax(const float* logits, int* out, float* scratch_v, int* s
 // downward order at which a running sum crosses a mark: the k-th candidate (a
 // sum of ones), the candidate at which the mass reaches top_p of the total,
 // the candidate at which it reaches the drawn point.  Such a place is found by
-// two histogram passes over a 24-bit key that falls as the logit rises:
+// histogram passes over a 24-bit key that falls as the logit rises:
 //     key = min(2^26 - 1, (max - y) * 2^20) >> 2,   y = logit / temperature,
-// 12 bits a pass.  Logits closer than 4e-6 share a key and count as equal: they
+// 12 bits a pass; the second pass is left out when the bin that the first one
+// finds holds a single candidate, which is the usual case near the top of a
+// row.  Logits closer than 4e-6 share a key and count as equal: they
 // are ordered by index, as equal logits are in the recipe.  Logits more than 64
 // below the maximum share the last key; their mass is zero.
 //
@@ -127,9 +129,16 @@ __device__ __forceinline__ unsigned long long sm_mass(float y, float top) {
     return (y == y) ? static_cast<unsigned long long>(p) : 0ull;
 }
 
-// The first bin, going up, at which the running sum of sm.sum reaches `mark` (mark >= 1; the last bin
-// that holds anything if the sum never gets there).  Leaves found_bin, found_before, found_in.
-__device__ void sm_find(sm_shared& sm, unsigned long long before, unsigned long long mark) {
+// The mark that is `fraction` of `total`, at least one and at most all of it.
+__device__ __forceinline__ unsigned long long sm_mark_of(double fraction, unsigned long long total) {
+    const unsigned long long mark = static_cast<unsigned long long>(fraction * static_cast<double>(total));
+    return mark < 1 ? 1 : (mark > total ? total : mark);
+}
+
+// The first bin, going up, at which the running sum of sm.sum reaches the mark (the last bin that holds
+// anything if the sum never gets there).  The mark is `mark` (>= 1), or, with fraction >= 0, that fraction
+// of the sum over all bins.  Leaves found_bin, found_before, found_in and returns the mark it used.
+__device__ unsigned long long sm_find(sm_shared& sm, unsigned long long before, unsigned long long mark, double fraction) {
     constexpr int PER = SM_BINS / SM_THREADS;                  // bins a thread
     const int tid = threadIdx.x, lane = tid % PL_WAVE, wave = tid / PL_WAVE;
     unsigned long long mine = 0;
@@ -145,8 +154,13 @@ __device__ void sm_find(sm_shared& sm, unsigned long long before, unsigned long 
     if (lane == PL_WAVE - 1) sm.wave_sum[wave] = run;
     if (tid == 0) sm.found_bin = -1;
     __syncthreads();
-    unsigned long long ahead = before;
-    for (int w = 0; w < wave; ++w) ahead += sm.wave_sum[w];
+    unsigned long long ahead = before, total = before;
+    for (int w = 0; w < SM_THREADS / PL_WAVE; ++w) {
+        const unsigned long long v = sm.wave_sum[w];
+        if (w < wave) ahead += v;
+        total += v;
+    }
+    if (fraction >= 0.0) mark = sm_mark_of(fraction, total);
     const unsigned long long through = ahead + run, upto = through - mine;   // sums through / before this thread's bins
     if (upto < mark && mark <= through) {
         unsigned long long at = upto;
@@ -164,7 +178,6 @@ __device__ void sm_find(sm_shared& sm, unsigned long long before, unsigned long 
     __syncthreads();
     if (sm.found_bin < 0) {                                     // the mark lies past the total: the last bin in use
         if (tid == SM_THREADS - 1) {
-            unsigned long long total = through;
             int b = SM_BINS - 1;
             while (b > 0 && sm.sum[b] == 0) --b;
             sm.found_bin = b;
@@ -175,6 +188,7 @@ __device__ void sm_find(sm_shared& sm, unsigned long long before, unsigned long 
         }
         __syncthreads();
     }
+    return mark;
 }
 
 // Which candidates are still in: keys below `key`, and of that key the indices below `limit`.
@@ -185,53 +199,68 @@ struct sm_kept {
 };
 
 // The place, in the order of key then index, at which the running sum of `weight` over the kept
-// candidates reaches `mark`.  Returns the key found; `limit` becomes the index after the candidate at
-// which the mark is reached, `before` the sum over the kept candidates of lower keys, `through` the sum
-// up to and with that candidate, and `token` that candidate.  WEIGHTED: masses, else ones.
+// candidates reaches the mark: `mark`, or with fraction >= 0 that fraction of the sum over all of them.
+// Returns the key found; `limit` becomes the index after the candidate at which the mark is reached,
+// `through` the sum up to and with that candidate, and `token` that candidate.  WEIGHTED: masses, else
+// ones.  A first pass over the upper 12 bits of the keys; a second over the lower 12 only if the bin
+// found holds more than one candidate.
 template <bool WEIGHTED>
 __device__ uint32_t sm_select(sm_shared& sm, const float* __restrict__ x, int V, float inverse, float top, sm_kept kept,
-                              unsigned long long mark, int& limit, unsigned long long& through, int& token) {
+                              unsigned long long mark, double fraction, int& limit, unsigned long long& through, int& token) {
     const int tid = threadIdx.x;
-    // first pass: the upper 12 bits
-    for (int b = tid; b < SM_BINS; b += SM_THREADS) sm.sum[b] = 0;
-    __syncthreads();
+    auto clear = [&]() {
+        for (int b = tid; b < SM_BINS; b += SM_THREADS) {
+            sm.sum[b] = 0;
+            sm.count[b] = 0;
+            sm.first[b] = SM_NO_LIMIT;
+        }
+        __syncthreads();
+    };
+    clear();
     for (int i = tid; i < V; i += SM_THREADS) {
         const float y = x[i] * inverse;
         const uint32_t k = sm_key(y, top);
         if (!kept.has(k, i)) continue;
         const unsigned long long w = WEIGHTED ? sm_mass(y, top) : 1ull;
-        if (w) atomicAdd(&sm.sum[k >> 12], w);
-    }
-    __syncthreads();
-    sm_find(sm, 0, mark);
-    const uint32_t upper = sm.found_bin;
-    const unsigned long long before_upper = sm.found_before;
-    __syncthreads();
-    // second pass: the lower 12 bits of the candidates of that bin
-    for (int b = tid; b < SM_BINS; b += SM_THREADS) {
-        sm.sum[b] = 0;
-        sm.count[b] = 0;
-        sm.first[b] = SM_NO_LIMIT;
-    }
-    __syncthreads();
-    for (int i = tid; i < V; i += SM_THREADS) {
-        const float y = x[i] * inverse;
-        const uint32_t k = sm_key(y, top);
-        if ((k >> 12) != upper || !kept.has(k, i)) continue;
-        const unsigned long long w = WEIGHTED ? sm_mass(y, top) : 1ull;
-        if (!WEIGHTED || w) {
-            atomicAdd(&sm.sum[k & 0xfff], w);
-            atomicAdd(&sm.count[k & 0xfff], 1u);
-            atomicMin(&sm.first[k & 0xfff], i);
+        if (w) {
+            atomicAdd(&sm.sum[k >> 12], w);
+            atomicAdd(&sm.count[k >> 12], 1u);
+            atomicMin(&sm.first[k >> 12], i);
         }
     }
     __syncthreads();
-    sm_find(sm, before_upper, mark);
-    const uint32_t key = (upper << 12) | static_cast<uint32_t>(sm.found_bin);
-    const unsigned long long before = sm.found_before, in_bin = sm.found_in;
-    const unsigned int many = sm.count[sm.found_bin];
-    const int lowest = sm.first[sm.found_bin];
+    mark = sm_find(sm, 0, mark, fraction);
+    const uint32_t upper = sm.found_bin;
+    uint32_t key;
+    unsigned long long before = sm.found_before, in_bin = sm.found_in;
+    unsigned int many = sm.count[upper];
+    int lowest = sm.first[upper];
     __syncthreads();
+    if (many == 1) {
+        key = sm_key(x[lowest] * inverse, top);
+    } else {
+        const unsigned long long before_upper = before;
+        clear();
+        for (int i = tid; i < V; i += SM_THREADS) {
+            const float y = x[i] * inverse;
+            const uint32_t k = sm_key(y, top);
+            if ((k >> 12) != upper || !kept.has(k, i)) continue;
+            const unsigned long long w = WEIGHTED ? sm_mass(y, top) : 1ull;
+            if (w) {
+                atomicAdd(&sm.sum[k & 0xfff], w);
+                atomicAdd(&sm.count[k & 0xfff], 1u);
+                atomicMin(&sm.first[k & 0xfff], i);
+            }
+        }
+        __syncthreads();
+        sm_find(sm, before_upper, mark, -1.0);
+        key = (upper << 12) | static_cast<uint32_t>(sm.found_bin);
+        before = sm.found_before;
+        in_bin = sm.found_in;
+        many = sm.count[sm.found_bin];
+        lowest = sm.first[sm.found_bin];
+        __syncthreads();
+    }
     if (many <= 1) {                                            // the usual case: one candidate has this key
         limit = many == 1 ? lowest + 1 : SM_NO_LIMIT;
         through = before + in_bin;
@@ -326,37 +355,19 @@ sample_rows_kernel(const float* __restrict__ logits, const float* __restrict__ t
     unsigned long long through;
     const int k = top_k[row];
     if (k > 0 && k < V) {
-        const uint32_t key = sm_select<false>(sm, x, V, inverse, top, kept, static_cast<unsigned long long>(k), limit, through, token);
+        const uint32_t key = sm_select<false>(sm, x, V, inverse, top, kept, static_cast<unsigned long long>(k), -1.0, limit, through, token);
         kept = sm_kept{key, limit};
     }
-    // the mass of what is kept: the sum of a first pass over it
-    for (int b = tid; b < SM_BINS; b += SM_THREADS) sm.sum[b] = 0;
-    __syncthreads();
-    {
-        unsigned long long mine = 0;
-        for (int i = tid; i < V; i += SM_THREADS) {
-            const float y = x[i] * inverse;
-            if (kept.has(sm_key(y, top), i)) mine += sm_mass(y, top);
-        }
-#pragma unroll
-        for (int off = PL_WAVE / 2; off > 0; off >>= 1) mine += __shfl_xor(mine, off, PL_WAVE);
-        if (tid % PL_WAVE == 0) sm.wave_sum[tid / PL_WAVE] = mine;
-    }
-    __syncthreads();
-    unsigned long long total = 0;
-    for (int w = 0; w < SM_THREADS / PL_WAVE; ++w) total += sm.wave_sum[w];
-    __syncthreads();
     const float p = top_p[row];
+    double fraction = static_cast<double>(uniform[row]);       // of everything kept
+    unsigned long long mark = 0;
     if (p < 1.f) {
-        unsigned long long mark = static_cast<unsigned long long>(static_cast<double>(p) * static_cast<double>(total));
-        mark = mark < 1 ? 1 : (mark > total ? total : mark);
-        const uint32_t key = sm_select<true>(sm, x, V, inverse, top, kept, mark, limit, through, token);
+        const uint32_t key = sm_select<true>(sm, x, V, inverse, top, kept, 0, static_cast<double>(p), limit, through, token);
         kept = sm_kept{key, limit};
-        total = through;                                        // the candidate that crosses the mark is kept
+        mark = sm_mark_of(fraction, through);                   // the candidate that crosses the mark is kept
+        fraction = -1.0;
     }
-    unsigned long long mark = static_cast<unsigned long long>(static_cast<double>(uniform[row]) * static_cast<double>(total));
-    mark = mark < 1 ? 1 : (mark > total ? total : mark);
-    sm_select<true>(sm, x, V, inverse, top, kept, mark, limit, through, token);
+    sm_select<true>(sm, x, V, inverse, top, kept, mark, fraction, limit, through, token);
     if (tid == 0) out[row] = token;
 }
 
