@@ -209,24 +209,42 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
     };
     const int first_base = s_begin + wave * KPW * U;
     lookup(first_base);
+    // The keys and values of a round are asked for a round ahead, while those of the round before are
+    // worked on: what comes back is held raw and masked only where it is used, so nothing waits early.
+    u32x4 knext[U], vnext[U];
+    bool oknext[U];
+    auto ask = [&]() {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            oknext[u] = blk[u] >= 0;
+            const size_t off = (static_cast<size_t>(max(blk[u], 0)) * block_size + within[u]) * row_stride + head_off;
+            knext[u] = *reinterpret_cast<const u32x4*>(k_pool + off);
+            vnext[u] = *reinterpret_cast<const u32x4*>(v_pool + off);
+        }
+    };
+    ask();
+    lookup(first_base + ROUND);
 
     for (int base = first_base; base < s_end; base += ROUND) {
         u32x4 kraw[U], vraw[U];
         bool ok[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            ok[u] = blk[u] >= 0;
-            const size_t off = (static_cast<size_t>(max(blk[u], 0)) * block_size + within[u]) * row_stride + head_off;
-            const u32x4 kgot = *reinterpret_cast<const u32x4*>(k_pool + off);
-            const u32x4 vgot = *reinterpret_cast<const u32x4*>(v_pool + off);
+            ok[u] = oknext[u];
+            kraw[u] = knext[u];
+            vraw[u] = vnext[u];
+        }
+        ask();
+        lookup(base + 2 * ROUND);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
             const uint32_t keep = (ok[u] && d_ok) ? 0xffffffffu : 0u;
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
-                kraw[u].v[w] = kgot.v[w] & keep;
-                vraw[u].v[w] = vgot.v[w] & keep;
+                kraw[u].v[w] &= keep;
+                vraw[u].v[w] &= keep;
             }
         }
-        lookup(base + ROUND);
         if (!q_ready) prepare_q();
         float s[U][GT];
 #pragma unroll
@@ -415,7 +433,7 @@ static int launch_decode(const void* q, int q_stride, void* out, float* part_acc
                          const ad_fuse_t& fuse, hipStream_t stream) {
     constexpr int KPW = PL_WAVE / LPK;
     constexpr int GROUPS = AD_WAVES * KPW;
-    constexpr int U = GT <= 2 ? 8 : 4;   // fewer heads a workgroup leave registers for more keys in flight
+    constexpr int U = GT <= 2 ? 4 : 2;   // keys a round; as many again are in flight for the round after
     const int g = nq / nkv;
     const int tiles = pl_ceil_div(g, GT);
     const size_t lds_bytes = (static_cast<size_t>(GROUPS) * GT * 2 + static_cast<size_t>(GROUPS) * GT * d) * sizeof(float);
