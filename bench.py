@@ -1,16 +1,17 @@
 #!/usr/bin/env python3
 """The headline measurement: Qwen3-0.6B-shape decoding and prefill on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--shape 0.6b|8b|32b]
 
 A step is one decode step of the engine's own step function on a batch of
-requests, each with a context of 512 tokens at the start: the cache write, the
+requests, each with a context of 512 tokens at the start (2,048 and 4,096 for
+the larger shapes): the cache write, the
 attention over the pages, every projection, the output projection and the greedy
 choice of the next token, which is what the next step is fed.  Weights are random
 (the random-weights mode writes the model folder, the loader reads it back),
 prompts are seeded uniform token ids.  One JSON line is printed.
 
-The sizes are those of BASELINE.json's third configuration.  Peaks are the
+The default sizes are those of BASELINE.json's third configuration.  Peaks are the
 published ones of the MI355X: 8 TB/s of HBM, 2.5 PFLOP/s dense bf16.
 """
 
@@ -31,18 +32,28 @@ sys.path.insert(0, str(ROOT))
 HBM_PEAK = 8.0e12            # bytes a second
 MFMA_PEAK = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}
 
-# Qwen3-0.6B shape (BASELINE.json, configs[2]).
-CONFIG = {
+COMMON = {
     "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "hidden_act": "silu",
-    "attention_bias": False, "sliding_window": None, "hidden_size": 1024, "intermediate_size": 3072,
-    "num_hidden_layers": 28, "num_attention_heads": 16, "num_key_value_heads": 8, "head_dim": 128,
+    "attention_bias": False, "sliding_window": None, "head_dim": 128, "num_key_value_heads": 8,
     "rms_norm_eps": 1e-6, "rope_theta": 1000000.0, "vocab_size": 151936,
-    "max_position_embeddings": 4096, "tie_word_embeddings": True,
 }
-FULL_LAYERS = 28
-CONTEXT = 512
+# The default is the Qwen3-0.6B shape (BASELINE.json, configs[2]); --shape 8b and 32b are configs[3] and [4]:
+# (config.json keys, the context a decode step starts from, layers that the default run of that shape loads).
+SHAPES = {
+    "0.6b": ("Qwen3-0.6B", dict(COMMON, hidden_size=1024, intermediate_size=3072, num_hidden_layers=28,
+                                num_attention_heads=16, max_position_embeddings=4096, tie_word_embeddings=True),
+             512, 28),
+    "8b": ("Qwen3-8B", dict(COMMON, hidden_size=4096, intermediate_size=12288, num_hidden_layers=36,
+                            num_attention_heads=32, max_position_embeddings=8192, tie_word_embeddings=False),
+           2048, 36),
+    "32b": ("Qwen3-32B", dict(COMMON, hidden_size=5120, intermediate_size=25600, num_hidden_layers=64,
+                              num_attention_heads=64, max_position_embeddings=16384, tie_word_embeddings=False),
+            4096, 16),
+}
 PREFILL_TOKENS = 2048
 BLOCK_SIZE = 16
+MIXED_SLICE = 512            # --only mixed: a slice of a prompt this long beside 63 decoded tokens
+MIXED_DECODES = 63
 
 
 def say(message: str) -> None:
@@ -126,16 +137,19 @@ def main() -> int:
     parser.add_argument("--steps", type=int, default=50)
     parser.add_argument("--warmup", type=int, default=10)
     parser.add_argument("--batch", type=int, default=8)
-    parser.add_argument("--layers", type=int, default=FULL_LAYERS,
+    parser.add_argument("--shape", choices=sorted(SHAPES), default="0.6b",
+                        help="layer sizes: the headline 0.6b, or the 8b and 32b shapes of BASELINE.json")
+    parser.add_argument("--layers", type=int, default=None,
                         help="fewer layers than the model has, where memory or time needs it; both numbers are reported")
     parser.add_argument("--no-graphs", action="store_true", help="run decode steps eagerly instead of as HIP graphs")
     parser.add_argument("--skip-points", action="store_true", help="leave out batch 1 and 64 and the prefill")
     parser.add_argument("--prefill-eager", action="store_true",
                         help="launch the prefill step kernel by kernel every time (a prompt length seen once)")
-    parser.add_argument("--only", choices=["decode", "prefill", "engine"], default=None,
+    parser.add_argument("--only", choices=["decode", "prefill", "engine", "mixed"], default=None,
                         help="run one part alone: the decode steps at --batch, the prefill, or (not part of the "
                              "default line) the whole engine on 1/4/16/32/64 requests at once, 16 prompt tokens and "
-                             "128 generated each, as the reference's own table of clients does")
+                             "128 generated each, as the reference's own table of clients does; mixed: one step of a "
+                             "512-token slice of a prompt beside 63 decoded tokens")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU; this engine has no multi-GPU path (N must be 1)")
@@ -150,6 +164,10 @@ def main() -> int:
     from paged_llm_rs_amd.parts.model import load_model
 
     device = require_gpu("cuda:0")
+    model_name, CONFIG, CONTEXT, default_layers = SHAPES[args.shape]
+    FULL_LAYERS = CONFIG["num_hidden_layers"]
+    if args.layers is None:
+        args.layers = default_layers
     cfg = dict(CONFIG)
     cfg["num_hidden_layers"] = args.layers
     tmp = tempfile.TemporaryDirectory()
@@ -203,6 +221,38 @@ def main() -> int:
         print(json.dumps({"prefill": prefill_point()}), flush=True)
         tmp.cleanup()
         return 0
+    if args.only == "mixed":
+        # 63 requests with CONTEXT tokens each bring one token; one more brings the third slice of a prompt.
+        # The step is not committed, so every run of it writes the same places of the cache again.
+        say(f"mixed step: {MIXED_DECODES} decoded tokens at context {CONTEXT} beside a slice of {MIXED_SLICE}")
+        bench = DecodeBench(model, cache, runner, MIXED_DECODES, CONTEXT, seed=3)
+        rng = random.Random(512)
+        long_prompt = [rng.randrange(cfg["vocab_size"]) for _ in range(PREFILL_TOKENS)]
+        behind = 2 * MIXED_SLICE
+        cache.manager.add_sequence(1000)
+        assert cache.manager.reserve(1000, behind)
+        first = [StepEntry(1000, long_prompt[:behind], 0, [])]
+        run_step(model, cache, first)
+        commit_step(cache, first)
+        assert cache.manager.reserve(1000, MIXED_SLICE)
+        entries = [StepEntry(1000, long_prompt[behind:behind + MIXED_SLICE], behind, [])]
+        for i, tok in zip(bench.ids, bench.tokens):
+            assert cache.manager.reserve(i, 1)
+            entries.append(StepEntry(i, [tok], cache.manager.tokens(i), [0]))
+        seconds = timed(lambda: runner.run(entries).greedy_tokens(), args.steps, args.warmup)
+        rows = MIXED_SLICE + MIXED_DECODES
+        d, nq = cfg["head_dim"], cfg["num_attention_heads"]
+        attention_flops = args.layers * 4 * nq * d * (MIXED_SLICE * (behind + (MIXED_SLICE + 1) // 2) + MIXED_DECODES * CONTEXT)
+        flops = layer_flops * rows + head_flops * MIXED_DECODES + attention_flops
+        step_bytes = weight_bytes + (MIXED_DECODES * CONTEXT + behind + MIXED_SLICE) * kv_token
+        print(json.dumps({"mixed": {
+            "model": f"{model_name} shape", "layers": args.layers, "layers_full": FULL_LAYERS, "rows": rows,
+            "decode_context": CONTEXT, "ms": round(seconds * 1e3, 3), "tokens_per_s": round(rows / seconds, 1),
+            "hbm_floor_ms": round(step_bytes / HBM_PEAK * 1e3, 3), "mfma_floor_ms": round(flops / MFMA_PEAK["bf16"] * 1e3, 3),
+            "frac_hbm": round(step_bytes / seconds / HBM_PEAK, 4), "frac_mfma": round(flops / seconds / MFMA_PEAK["bf16"], 4),
+        }}), flush=True)
+        tmp.cleanup()
+        return 0
     if args.only == "engine":
         # scheduler, cache manager, step function, sampling and the read-back of every token: generate()
         from paged_llm_rs_amd.engine.engine import Engine
@@ -228,16 +278,16 @@ def main() -> int:
     say(f"decode, batch {args.batch}")
     seconds, value, step_bytes = decode_point(args.batch, args.steps, args.warmup)
     line = {
-        "metric": f"Qwen3-0.6B bf16: decode tok/s @ batch {args.batch}, ctx 512",
+        "metric": f"{model_name} bf16: decode tok/s @ batch {args.batch}, ctx {CONTEXT}",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(seconds * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic: random weights, uniform random token ids",
         "config": {
-            "model": "Qwen3-0.6B shape", "global_batch": args.batch, "seq_len": CONTEXT, "parallelism": "none",
+            "model": f"{model_name} shape", "global_batch": args.batch, "seq_len": CONTEXT, "parallelism": "none",
             "layers": args.layers, "layers_full": FULL_LAYERS, "hidden": cfg["hidden_size"],
             "q_heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
             "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
-            "tied": True, "block_size": BLOCK_SIZE, "max_context": cfg["max_position_embeddings"],
+            "tied": cfg["tie_word_embeddings"], "block_size": BLOCK_SIZE, "max_context": cfg["max_position_embeddings"],
             "prefill_tokens": PREFILL_TOKENS,
         },
         "roofline": {"bound": "hbm", "achieved": round(step_bytes / seconds / 1e9, 1), "peak": HBM_PEAK / 1e9,

@@ -94,16 +94,19 @@ def is_current(kind: str) -> bool:
 
 def _run_all(commands: list, what: str) -> None:
     """Run compile commands side by side, saying now and then that they still run."""
-    procs = [(name, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True))
-             for name, cmd in commands]
+    # What a compiler prints goes to a file: a pipe that nobody reads while the compiler runs holds 64 KB,
+    # and a compiler with more warnings than that would wait for ever.
+    logs = {name: tempfile.TemporaryFile(mode="w+") for name, _ in commands}
+    pending = {name: subprocess.Popen(cmd, stdout=logs[name], stderr=subprocess.STDOUT) for name, cmd in commands}
     started = time.time()
     last = started
-    pending = dict(procs)
     outputs = {}
     while pending:
         for name, proc in list(pending.items()):
             if proc.poll() is not None:
-                outputs[name] = (proc.returncode, proc.stdout.read())
+                logs[name].seek(0)
+                outputs[name] = (proc.returncode, logs[name].read())
+                logs[name].close()
                 del pending[name]
         if pending:
             time.sleep(0.2)

@@ -119,7 +119,13 @@ __device__ __forceinline__ int ap_value_shift(int r, int pieces) { return 4 * ((
 // register or LDS write instruction spent on them.  Rows then lie unpadded in LDS, so their 16-byte
 // pieces are permuted instead (ap_key_shift, ap_value_shift: the reads of the matrix cores' operands
 // fall on every bank once); heads of 64 and 128.
-template <int DT, int NW, int KS, int FEED>
+//
+// GR (grouped): the 32*NW rows of a workgroup are not consecutive tokens of one query head but the query
+// heads of ONE token that share a key head (rows past the group's size stand idle): a single token, or
+// each token of a short portion, then reads its keys once for the whole group, on the matrix cores.
+// The token tile of the work index is then a token, its head a key head, and requests with
+// short_limit or more tokens are the ones left out.
+template <int DT, int NW, int KS, int FEED, bool GR = false>
 __global__ void __launch_bounds__(64 * NW * KS, DT <= 4 ? AP_OCC : 1)
 paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
                                const int* __restrict__ q_start, const int* __restrict__ q_len,
@@ -160,14 +166,16 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     // in the workspace and a second kernel puts them together.
     const int split = work % splits;
     work /= splits;
+    const int heads_n = GR ? nkv : nq;
     const int tile = tiles_a_request - 1 - work % tiles_a_request;
-    const int head = (work / tiles_a_request) % nq;
-    const int seq = work / (tiles_a_request * nq);
+    const int head = (work / tiles_a_request) % heads_n;
+    const int seq = work / (tiles_a_request * heads_n);
     if (seq >= num_seqs) return;
 
     const int count = q_len[seq];
-    if (count < short_limit || ctx_len[seq] <= 0) return;   // a request of padding rows has no context
-    const int q0 = tile * BM;
+    if (ctx_len[seq] <= 0) return;                           // a request of padding rows has no context
+    if (GR ? (short_limit > 0 && count >= short_limit) : count < short_limit) return;
+    const int q0 = GR ? tile : tile * BM;                    // the tile's first token
     if (q0 >= count) return;
     const int start = ctx_len[seq] - count;  // position of the request's first token in this step
     const int row0 = q_start[seq];
@@ -180,25 +188,28 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     const int kt0 = (wave_id / NW) * KT;                         // the wave's first 32-key tile of a 64-key tile
     const int r32 = lane & 31;
     const int h = lane >> 5;
-    const int kvh = head / (nq / nkv);
+    const int group = nq / nkv;
+    const int kvh = GR ? head : head / group;
 
     // the wave's queries: lane holds query wq = q0 + wave*32 + r32, elements 16*kk + 8*h .. +8
-    const int wq = q0 + wave * 32 + r32;
-    const bool q_ok = wq < count;
+    // (grouped: the lane's query is head kvh * group + wave*32 + r32 of token q0)
+    const int wq = GR ? q0 : q0 + wave * 32 + r32;
+    const int q_head = GR ? kvh * group + min(wave * 32 + r32, group - 1) : head;
+    const bool q_ok = GR ? wave * 32 + r32 < group : wq < count;
     ap_frag qf[2 * DT];
 #pragma unroll
     for (int kk = 0; kk < 2 * DT; ++kk) {
         const int e0 = 16 * kk + 8 * h;
         if (q_ok && e0 < d)
             qf[kk].raw = *reinterpret_cast<const ap_u32x4*>(q + static_cast<size_t>(row0 + wq) * q_stride +
-                                                            static_cast<size_t>(head) * d + e0);
+                                                            static_cast<size_t>(q_head) * d + e0);
         else
             qf[kk].raw = ap_u32x4{{0u, 0u, 0u, 0u}};
     }
     const int q_pos = start + wq;                               // position of this lane's query
-    const int wave_first = start + q0 + wave * 32;              // position of the wave's first query
-    const int wave_last = start + min(q0 + wave * 32 + 31, count - 1);
-    const bool wave_active = q0 + wave * 32 < count;
+    const int wave_first = GR ? q_pos : start + q0 + wave * 32; // position of the wave's first query
+    const int wave_last = GR ? q_pos : start + min(q0 + wave * 32 + 31, count - 1);
+    const bool wave_active = GR ? wave * 32 < group : q0 + wave * 32 < count;
 
     f32x16 o[DT];
 #pragma unroll
@@ -207,7 +218,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         for (int r = 0; r < 16; ++r) o[dt][r] = 0.f;
     float m = -INFINITY, lsum = 0.f;
 
-    const int last_pos = start + min(q0 + BM, count) - 1;       // the last key any query of the tile sees
+    const int last_pos = GR ? start + q0 : start + min(q0 + BM, count) - 1;   // the last key any query of the tile sees
     const int first_pos = (window > 0 && start + q0 + 1 > window) ? start + q0 + 1 - window : 0;
     const int* table = block_table + static_cast<size_t>(seq) * max_blocks;
     const size_t row_stride = static_cast<size_t>(nkv) * d;
@@ -321,7 +332,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     const int k_end = min(k_lowest + key_tiles * AP_BN, k_first + tiles_a_split * AP_BN);
     if (k_first >= k_end) {          // more splits than key tiles: nothing to add
         if (kt0 == 0 && q_ok) {
-            float* ml = part_ml + ((static_cast<size_t>(row0 + wq) * nq + head) * splits + split) * 2;
+            float* ml = part_ml + ((static_cast<size_t>(row0 + wq) * nq + q_head) * splits + split) * 2;
             if (h == 0) {
                 ml[0] = -INFINITY;
                 ml[1] = 0.f;
@@ -334,12 +345,19 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     // values), into the buffers j % NKB and j % NVB.  The lane's place in the cache row differs between
     // keys and values by the permutation of the pieces.
     int asked = 0, asked_k = 0, asked_v = 0;   // the next tile to ask for and its buffers
-    uint32_t place_k = 0, place_v = 0;
+    // (A wave's loads of one tile are NT / CP rows apart: where that is no multiple of 16, the row number
+    // mod 16, and with it the permutation, alternates between two values from one load to the next.)
+    constexpr bool ROWS_ALTERNATE = DIRECT && (NT / CP) % 16 != 0;
+    static_assert(!DIRECT || (2 * NT / CP) % 16 == 0, "the rows of a wave's loads repeat mod 16 after two loads at most");
+    uint32_t place_k[2] = {0, 0}, place_v[2] = {0, 0};
     if constexpr (DIRECT) {
-        const int r15 = ((64 * wave_id) / CP + lane / CP) & 15;
-        const int ck = (lane % CP) ^ ap_key_shift(r15, CP), cv = (lane % CP) ^ ap_value_shift(r15, CP);
-        place_k = (lane / CP) * row_bytes + static_cast<uint32_t>(head_off + min(ck, cpr - 1) * 8) * 2;
-        place_v = (lane / CP) * row_bytes + static_cast<uint32_t>(head_off + min(cv, cpr - 1) * 8) * 2;
+#pragma unroll
+        for (int odd = 0; odd < 2; ++odd) {
+            const int r15 = ((64 * wave_id + odd * NT) / CP + lane / CP) & 15;
+            const int ck = (lane % CP) ^ ap_key_shift(r15, CP), cv = (lane % CP) ^ ap_value_shift(r15, CP);
+            place_k[odd] = (lane / CP) * row_bytes + static_cast<uint32_t>(head_off + min(ck, cpr - 1) * 8) * 2;
+            place_v[odd] = (lane / CP) * row_bytes + static_cast<uint32_t>(head_off + min(cv, cpr - 1) * 8) * 2;
+        }
     }
     auto ask = [&]() {               // pages from kblk/kwithin, looked up before
         if constexpr (DIRECT) {
@@ -348,8 +366,8 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
                 const int first_row = (64 * wave_id + i * NT) / CP;
                 const int page = __builtin_amdgcn_readfirstlane(max(kblk[i], 0));
                 const size_t base = (static_cast<size_t>(page) * block_size + kwithin[i]) * row_bytes;
-                const char* gk = reinterpret_cast<const char*>(k_pool) + base + place_k;
-                const char* gv = reinterpret_cast<const char*>(v_pool) + base + place_v;
+                const char* gk = reinterpret_cast<const char*>(k_pool) + base + place_k[ROWS_ALTERNATE ? i & 1 : 0];
+                const char* gv = reinterpret_cast<const char*>(v_pool) + base + place_v[ROWS_ALTERNATE ? i & 1 : 0];
                 uint16_t* lk = Kbase + asked_k * KTILE + first_row * KROW;
                 uint16_t* lv = Vbase + asked_v * VTILE + first_row * VROW;
                 ap_load_to_lds(gk, lk);
@@ -585,7 +603,8 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         if constexpr (DIRECT) {
             take_pages();
             __builtin_amdgcn_sched_barrier(0);
-            __builtin_amdgcn_s_waitcnt(0x0F70 | LOADS_A_TILE);   // vmcnt(LOADS_A_TILE): all but the newest tile
+            // vmcnt(LOADS_A_TILE): all but the newest tile (the count's bits 4 and 5 stand at bits 14 and 15)
+            __builtin_amdgcn_s_waitcnt(0x0F70 | (LOADS_A_TILE & 15) | ((LOADS_A_TILE >> 4) << 14));
         }
     };
     // First the tiles that every query of the workgroup sees whole: no masks, no wave stands idle
@@ -667,7 +686,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     if (!q_ok) return;
     // o[dt][4*j + i] is element 32*dt + 8*j + 4*h + i of query r32
     if (splits > 1) {
-        const size_t at = (static_cast<size_t>(row0 + wq) * nq + head) * splits + split;
+        const size_t at = (static_cast<size_t>(row0 + wq) * nq + q_head) * splits + split;
         if (h == 0) {
             part_ml[at * 2] = m * scale_log2e;     // in the exponent's own unit; -inf stays
             part_ml[at * 2 + 1] = lsum;
@@ -684,7 +703,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     }
     const float total = lsum;
     const float inv = total > 0.f ? 1.f / total : 0.f;
-    bf16_t* orow = out + (static_cast<size_t>(row0 + wq) * nq + head) * d;
+    bf16_t* orow = out + (static_cast<size_t>(row0 + wq) * nq + q_head) * d;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -707,14 +726,15 @@ __global__ void __launch_bounds__(256)
 paged_attention_prefill_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
                                      bf16_t* __restrict__ out, const int* __restrict__ q_start,
                                      const int* __restrict__ q_len, const int* __restrict__ ctx_len, int short_limit,
-                                     int tiles_a_request, int num_seqs, int nq, int d, int splits, int bm) {
+                                     int tiles_a_request, int num_seqs, int nq, int d, int splits, int bm, int grouped) {
     const int work = blockIdx.x;
     const int tile = work % tiles_a_request;
     const int head = (work / tiles_a_request) % nq;
     const int seq = work / (tiles_a_request * nq);
     if (seq >= num_seqs) return;
     const int count = q_len[seq];
-    if (count < short_limit || ctx_len[seq] <= 0) return;
+    if (ctx_len[seq] <= 0) return;
+    if (grouped ? (short_limit > 0 && count >= short_limit) : count < short_limit) return;
     const int quads = d / 4, rows = blockDim.x / quads;
     const int r = tile * bm + blockIdx.y * rows + threadIdx.x / quads;
     const int e0 = (threadIdx.x % quads) * 4;
@@ -753,7 +773,7 @@ paged_attention_prefill_merge_kernel(const float* __restrict__ part_acc, const f
     *reinterpret_cast<ap_u32x2*>(out + (row * nq + head) * d + e0) = w;
 }
 
-template <int DT, int NW, int KS, int FEED>
+template <int DT, int NW, int KS, int FEED, bool GR = false>
 static int launch_prefill(const void* q, int q_stride, void* out, const int* q_start, const int* q_len,
                           const int* ctx_len, int short_limit, int num_seqs, int max_q_len, const int* block_table,
                           int max_blocks, int block_size, const void* k_pool, const void* v_pool, int nq, int nkv,
@@ -767,14 +787,14 @@ static int launch_prefill(const void* q, int q_stride, void* out, const int* q_s
     const size_t hand_bytes = KS == 2 ? static_cast<size_t>(NW) * (16 * DT + 2) * PL_WAVE * sizeof(float) : 0;
     const size_t lds_bytes = tile_bytes > hand_bytes ? tile_bytes : hand_bytes;
     if (lds_bytes > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_prefill_kernel<DT, NW, KS, FEED>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_prefill_kernel<DT, NW, KS, FEED, GR>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
         PL_REQUIRE(e == hipSuccess, "prefill attention: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
     }
-    const int tiles = pl_ceil_div(max_q_len, BM);
-    const long long whole = static_cast<long long>(tiles) * nq * num_seqs, total = whole * splits;
+    const int tiles = GR ? max_q_len : pl_ceil_div(max_q_len, BM);
+    const long long whole = static_cast<long long>(tiles) * (GR ? nkv : nq) * num_seqs, total = whole * splits;
     PL_REQUIRE(total > 0 && total < (1ll << 30), "prefill attention: %lld workgroups", total);
-    paged_attention_prefill_kernel<DT, NW, KS, FEED><<<static_cast<int>(total), 64 * NW * KS, lds_bytes, stream>>>(
+    paged_attention_prefill_kernel<DT, NW, KS, FEED, GR><<<static_cast<int>(total), 64 * NW * KS, lds_bytes, stream>>>(
         static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), q_start, q_len, ctx_len, short_limit, tiles,
         num_seqs, block_table, max_blocks, block_size, static_cast<const bf16_t*>(k_pool),
         static_cast<const bf16_t*>(v_pool), nq, nkv, d, scale * 1.4426950408889634f, window, static_cast<int>(total),
@@ -782,9 +802,14 @@ static int launch_prefill(const void* q, int q_stride, void* out, const int* q_s
     PL_CHECK_LAUNCH("paged_attention_prefill");
     if (splits > 1) {
         const int rows = 256 / (d / 4);
-        paged_attention_prefill_merge_kernel<<<dim3(static_cast<int>(whole), pl_ceil_div(BM, rows)), 256, 0, stream>>>(
-            part_acc, part_ml, static_cast<bf16_t*>(out), q_start, q_len, ctx_len, short_limit, tiles, num_seqs, nq, d,
-            splits, BM);
+        if (GR)     // a request's tokens as one tile of the merge, every query head
+            paged_attention_prefill_merge_kernel<<<dim3(num_seqs * nq, pl_ceil_div(max_q_len, rows)), 256, 0, stream>>>(
+                part_acc, part_ml, static_cast<bf16_t*>(out), q_start, q_len, ctx_len, short_limit, 1, num_seqs, nq, d,
+                splits, max_q_len, 1);
+        else
+            paged_attention_prefill_merge_kernel<<<dim3(static_cast<int>(whole), pl_ceil_div(BM, rows)), 256, 0, stream>>>(
+                part_acc, part_ml, static_cast<bf16_t*>(out), q_start, q_len, ctx_len, short_limit, tiles, num_seqs, nq, d,
+                splits, BM, 0);
         PL_CHECK_LAUNCH("paged_attention_prefill_merge");
     }
     return 0;
@@ -872,4 +897,38 @@ extern "C" int pl_paged_attention_prefill(const void* q, int q_stride, void* out
         default: AP_CALL(8);
     }
 #undef AP_CALL
+}
+
+// One token's query heads of a key-head group as the rows of a tile (see GR above): for single tokens and the
+// tokens of short portions where a group has four heads or more, so that the keys are read once a group and
+// multiplied on the matrix cores.  Same arguments as pl_paged_attention_prefill, but requests with
+// short_limit tokens or more are the ones left out (0: none is), and max_q_len bounds the tokens of those
+// that are served.  Heads of 64 or 128, groups of up to 32, pages of a power of two of at least
+// 64 / (head size / 8) tokens; pl_paged_attention_grouped_applies says whether a shape is served.
+extern "C" int pl_paged_attention_grouped_applies(int nq, int nkv, int d, int block_size) {
+    if (nq <= 0 || nkv <= 0 || nq % nkv || nq / nkv > 32 || (d != 64 && d != 128)) return 0;
+    const int rows_a_load = 64 / (d / 8);
+    return block_size >= rows_a_load && (block_size & (block_size - 1)) == 0 ? 1 : 0;
+}
+
+extern "C" int pl_paged_attention_grouped(const void* q, int q_stride, void* out, const int* q_start,
+                                          const int* q_len, const int* ctx_len, int short_limit, int num_seqs,
+                                          int max_q_len, const int* block_table, int max_blocks, int block_size,
+                                          const void* k_pool, const void* v_pool, int nq, int nkv, int d,
+                                          float scale, int window, int splits, float* part_acc, float* part_ml,
+                                          hipStream_t stream) {
+    PL_REQUIRE(pl_paged_attention_grouped_applies(nq, nkv, d, block_size),
+               "grouped attention: %d query heads over %d key heads of %d, pages of %d", nq, nkv, d, block_size);
+    PL_REQUIRE(splits >= 1 && splits <= AP_MERGE_MAX && (splits == 1 || (part_acc && part_ml)),
+               "grouped attention: %d splits%s", splits, splits > 1 ? " without a workspace" : "");
+    PL_REQUIRE(max_blocks > 0 && q_stride >= nq * d && q_stride % 8 == 0 && window >= 0,
+               "grouped attention: %d blocks a row, query stride %d, window %d", max_blocks, q_stride, window);
+    if (num_seqs <= 0 || max_q_len <= 0) return 0;
+    if (d == 64)
+        return launch_prefill<2, 1, 2, 2, true>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len,
+                                                block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale,
+                                                window, splits, part_acc, part_ml, stream);
+    return launch_prefill<4, 1, 2, 2, true>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len,
+                                            block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale,
+                                            window, splits, part_acc, part_ml, stream);
 }

@@ -85,7 +85,7 @@ __device__ __forceinline__ void sk_load_to_lds(const void* from, const void* lds
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(at), "v"(from) : "memory", "m0");
 }
 
-template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT, bool PANEL = false>
+template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT, bool PANEL = false, bool AHEAD = false>
 __global__ void __launch_bounds__(64 * WV)
 gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OUT* __restrict__ y,
                    const float* __restrict__ gain, float eps, const int* __restrict__ rows, int n, int N_out,
@@ -205,6 +205,21 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
 #pragma unroll
             for (int m = 0; m < MT; ++m) ssq[m] = 0.f;
         }
+        // AHEAD (a wave's share of K takes several rounds of loads): the weights of a round are asked for
+        // while the round before is multiplied, held as they come and masked when they are used.
+        bf16x8 ahead[AHEAD ? BT : 1][AHEAD ? UNR : 1];
+        auto ask_w = [&](int k0) {
+            if constexpr (AHEAD) {
+#pragma unroll
+                for (int u = 0; u < UNR; ++u) {
+                    const int at = k0 + u * SK_KSTEP + g * 8;
+                    const int kk = at < kend ? at : 0;
+#pragma unroll
+                    for (int b = 0; b < BT; ++b) ahead[b][u] = sk_load8(wrow[b] + kk);
+                }
+            }
+        };
+        ask_w(kbeg);
         if constexpr (PANEL) {
             __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0): this wave's share of the panel has landed
             __syncthreads();                               // and every wave's
@@ -235,15 +250,26 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
                 }
             } else {
                 bf16x8 bw[BT][UNR];
+                if constexpr (AHEAD) {
+                    // this round's weights were asked for a round ago; the next round's are asked for now
 #pragma unroll
-                for (int u = 0; u < UNR; ++u) {
-                    const int at = k0 + u * SK_KSTEP + g * 8;
-                    const bool k_ok = at < kend;
-                    const int kk = k_ok ? at : 0;
+                    for (int u = 0; u < UNR; ++u) {
+                        const bool k_ok = k0 + u * SK_KSTEP + g * 8 < kend;
 #pragma unroll
-                    for (int b = 0; b < BT; ++b) {
-                        const bf16x8 got = sk_load8(wrow[b] + kk);
-                        bw[b][u] = (k_ok && col_ok) ? got : sk_zero8();
+                        for (int b = 0; b < BT; ++b) bw[b][u] = (k_ok && col_ok) ? ahead[b][u] : sk_zero8();
+                    }
+                    ask_w(k0 + SK_KSTEP * UNR);
+                } else {
+#pragma unroll
+                    for (int u = 0; u < UNR; ++u) {
+                        const int at = k0 + u * SK_KSTEP + g * 8;
+                        const bool k_ok = at < kend;
+                        const int kk = k_ok ? at : 0;
+#pragma unroll
+                        for (int b = 0; b < BT; ++b) {
+                            const bf16x8 got = sk_load8(wrow[b] + kk);
+                            bw[b][u] = (k_ok && col_ok) ? got : sk_zero8();
+                        }
                     }
                 }
                 // the weights are asked for first: they come from furthest away
@@ -329,15 +355,26 @@ template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT>
 static int launch_one(int waves, const void* x, const void* w, void* y, const float* gain, float eps,
                       const int* rows, int n, int N_out, int K, hipStream_t stream) {
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
+    constexpr int UA = (WV == 16 && UNR >= 2) ? UNR / 2 : UNR;   // K steps a round when rounds overlap
     const int grid = min(pl_ceil_div(N_out, SK_TILE_N), SK_MAX_GRID);
     const size_t lds_bytes = static_cast<size_t>(waves) * (BT * MT * 256 + MT * 16) * sizeof(float);
     if (lds_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny_kernel<MT, UNR, WV, PRO, EPI, OUT>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
         PL_REQUIRE(e == hipSuccess, "skinny product: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny_kernel<MT, UA, WV, PRO, EPI, OUT, false, true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+        PL_REQUIRE(e == hipSuccess, "skinny product: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
     }
-    gemm_skinny_kernel<MT, UNR, WV, PRO, EPI, OUT><<<grid, 64 * waves, lds_bytes, stream>>>(
-        x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps, rows, n, N_out, K);
+    // A wave's share of K in more rounds of loads than one: the rounds overlap, two of them on their way at
+    // a time (of half the steps each where sixteen waves leave a lane 128 registers).
+    const bool several = pl_ceil_div(pl_ceil_div(K, SK_KSTEP), waves) > UNR;
+    if (several)
+        gemm_skinny_kernel<MT, UA, WV, PRO, EPI, OUT, false, true><<<grid, 64 * waves, lds_bytes, stream>>>(
+            x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps, rows, n, N_out, K);
+    else
+        gemm_skinny_kernel<MT, UNR, WV, PRO, EPI, OUT><<<grid, 64 * waves, lds_bytes, stream>>>(
+            x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps, rows, n, N_out, K);
     PL_CHECK_LAUNCH("gemm_skinny");
     return 0;
 }

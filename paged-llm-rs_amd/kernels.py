@@ -41,6 +41,8 @@ def _signatures(lib) -> None:
         "pl_paged_attention_decode": [p, i, p, p, p, p, p, p, i, p, i, i, p, p, i, i, i, i, f, i, i,
                                       i, p, p, i, f, p, p, i, p],
         "pl_paged_attention_prefill": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, p],
+        "pl_paged_attention_grouped": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, p],
+        "pl_paged_attention_grouped_applies": [i, i, i, i],
     }
     for name, argtypes in table.items():
         fn = getattr(lib, name)
@@ -409,17 +411,83 @@ def paged_attention_prefill(q: torch.Tensor, q_row_stride: int, out: torch.Tenso
 _compute_units = None
 
 
+def compute_units() -> int:
+    global _compute_units
+    if _compute_units is None:
+        _compute_units = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
+    return _compute_units
+
+
+# From this many query heads a key head on, single tokens go to the tiled kernel with a group's heads as
+# its rows: the kernel for single tokens multiplies on the vector units, once a query head, and at eight
+# heads a key that work, not the memory, bounds it (at four the two are as fast as each other).
+GROUPED_FROM = 8
+
+
+def grouped_applies(nq: int, nkv: int, d: int, block_size: int) -> bool:
+    return nq >= GROUPED_FROM * nkv and bool(library().pl_paged_attention_grouped_applies(nq, nkv, d, block_size))
+
+
+def grouped_splits(tokens: int, nkv: int, max_ctx: int) -> int:
+    """Into how many shares the keys of a token are cut for the grouped kernel: a workgroup a compute
+    unit if the tokens and key heads alone do not give that many, every share two tiles of keys at least."""
+    base = max(tokens * nkv, 1)
+    key_tiles = -(-max(max_ctx, 1) // 64)
+    return max(1, min(16, key_tiles // 2, -(-compute_units() // base)))
+
+
+def paged_attention_grouped(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, q_start: torch.Tensor,
+                            q_len: torch.Tensor, ctx_len: torch.Tensor, max_q_len: int, block_table: torch.Tensor,
+                            block_size: int, k_pool: torch.Tensor, v_pool: torch.Tensor, nq: int, nkv: int, d: int,
+                            scale: float, window: int = 0, short_limit: int = 0, max_ctx: int | None = None,
+                            splits: int | None = None, live_seqs: int | None = None,
+                            tokens: int | None = None) -> torch.Tensor:
+    """bfloat16 attention for single tokens and the tokens of short portions, the query heads of a
+    key-head group as the rows of a tile of the tiled kernel.  Arguments as for
+    ``paged_attention_prefill``, but requests with ``short_limit`` tokens or more are the ones skipped
+    (0: none), and ``max_q_len`` bounds the tokens of those that are served.  ``tokens``: how many
+    tokens those requests bring together (for the choice of ``splits``)."""
+    n = q.shape[0]
+    S = block_table.shape[0]
+    _need(q, "query buffer", None, torch.bfloat16)
+    if q.dim() != 2 or q.shape[1] != q_row_stride or q_row_stride < nq * d:
+        raise TensorError(f"query buffer has shape {tuple(q.shape)} for row stride {q_row_stride}")
+    _need(out, "attention output", (n, nq * d), torch.bfloat16)
+    _need(block_table, "block table", None, torch.int32)
+    for t, what in ((q_start, "first row of each request"), (q_len, "tokens of each request"),
+                    (ctx_len, "context length of each request")):
+        _need(t, what, (S,), torch.int32)
+    for pool, what in ((k_pool, "key pool"), (v_pool, "value pool")):
+        _need(pool, what, None, torch.bfloat16)
+        if pool.dim() != 2 or pool.shape[1] != nkv * d or pool.shape[0] % block_size != 0:
+            raise TensorError(f"{what} has shape {tuple(pool.shape)}, expected [pages*{block_size}, {nkv * d}]")
+    if not 0 < max_q_len <= n:
+        raise TensorError(f"the longest portion is said to have {max_q_len} of the step's {n} tokens")
+    live = S if live_seqs is None else int(live_seqs)
+    if not 0 < live <= S:
+        raise TensorError(f"{live} requests with tokens of {S}")
+    if splits is None:
+        splits = grouped_splits(n if tokens is None else int(tokens), nkv, int(max_ctx or 0))
+    part_acc = part_ml = None
+    if splits > 1:
+        part_acc = torch.empty((n * nq * splits * d,), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((n * nq * splits * 2,), dtype=torch.float32, device=q.device)
+    _check(library().pl_paged_attention_grouped(
+        q.data_ptr(), q_row_stride, out.data_ptr(), q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(),
+        int(short_limit), live, int(max_q_len), block_table.data_ptr(), block_table.shape[1], block_size,
+        k_pool.data_ptr(), v_pool.data_ptr(), nq, nkv, d, float(scale), int(window or 0), int(splits),
+        part_acc.data_ptr() if splits > 1 else None, part_ml.data_ptr() if splits > 1 else None, _stream()))
+    return out
+
+
 def prefill_splits(requests: int, max_q_len: int, nq: int, d: int, max_ctx: int, rows: int | None = None) -> int:
     """Into how many shares the keys of a token tile are cut.  A share more costs a trip of the
     unnormalised outputs through memory (rows * nq * d floats written and read) and one launch;
     it pays where few token tiles stand before a long context, as in a late portion of a long
     prompt.  The shares that make the estimate below smallest are taken: a workgroup spends about
     1.5 us on 64 keys, memory moves about 3 TB/s for this."""
-    global _compute_units
     if max_ctx <= 0:
         return 1
-    if _compute_units is None:
-        _compute_units = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
     tile = library().pl_paged_attention_prefill_tile(max_q_len, d)
     base = max(1, -(-max_q_len // tile) * nq * requests)
     key_tiles = -(-max_ctx // 64)
@@ -428,7 +496,7 @@ def prefill_splits(requests: int, max_q_len: int, nq: int, d: int, max_ctx: int,
     for s in (1, 2, 3, 4, 6, 8, 12, 16):
         if s > 1 and key_tiles // s < 4:
             break
-        turns = -(-base * s // _compute_units)
+        turns = -(-base * s // compute_units())
         cost = turns * -(-key_tiles // s) * 1.5
         if s > 1:
             cost += 3.0 + rows * nq * d * 8.0 * s / 3e6
@@ -444,7 +512,7 @@ def attention_step(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nkv
     which every request brings one token (in bfloat16) does all of it in the attention kernel;
     any other step runs the stand-alone kernel for the first three and then attention."""
     if (qkv.dtype == torch.bfloat16 and _attention_mode == "kernel" and batch.max_q_len == 1
-            and prepare.rot % 16 == 0):
+            and prepare.rot % 16 == 0 and not grouped_applies(nq, nkv, d, kv.block_size)):
         splits = decode_splits(batch.num_tokens, nq, nkv, batch.max_ctx_len)
         return paged_attention_decode(qkv, qkv.shape[1], out, batch.positions, batch.seq_of, kv.block_table,
                                       kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window, splits,
@@ -459,7 +527,8 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nk
                     scale: float, window: int = 0) -> torch.Tensor:
     """Attention for every token of a step.  ``qkv`` rows begin with the rotated queries.
     In bfloat16 the long portions go to the tiled kernel and the tokens of short ones
-    (decoded tokens among them) to the kernel for single tokens; both read the same pages."""
+    (decoded tokens among them) to the kernel for single tokens, or, where many query heads share a key
+    head, to the tiled kernel with a group's heads as its rows; all read the same pages."""
     if qkv.dtype != torch.bfloat16 or _attention_mode != "kernel":
         return paged_attention_plain(qkv, qkv.shape[1], out, batch.positions, batch.seq_of, kv.block_table,
                                      kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window)
@@ -472,6 +541,13 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nk
         if batch.short_tokens == 0:
             return out
     mixed = batch.max_q_len >= SHORT_PORTION
+    if grouped_applies(nq, nkv, d, kv.block_size):
+        # many query heads a key head: a token's group of heads as the rows of a tile of the tiled kernel
+        return paged_attention_grouped(qkv, stride, out, batch.q_start, batch.q_len, batch.ctx_len,
+                                       min(batch.max_q_len, SHORT_PORTION - 1), kv.block_table, kv.block_size,
+                                       kv.k_pool, kv.v_pool, nq, nkv, d, scale, window,
+                                       short_limit=SHORT_PORTION if mixed else 0, max_ctx=batch.max_ctx_len,
+                                       live_seqs=getattr(batch, "live_seqs", None), tokens=batch.short_tokens)
     splits = decode_splits(batch.short_tokens, nq, nkv, batch.max_ctx_len)
     return paged_attention_decode(qkv, stride, out, batch.positions, batch.seq_of, kv.block_table,
                                   kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window, splits,
@@ -522,18 +598,44 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
     return out
 
 
-def skinny_applies(x: torch.Tensor) -> bool:
-    return x.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_ROWS and x.shape[1] % 8 == 0
+# Where the hand-written product beats the library's on this chip (both timed over weights that come from
+# memory, not from a cache).  It streams a weight matrix of up to a few tens of megabytes faster than
+# the library starts, and fuses what stands before and after the product; a larger matrix the library
+# streams at a higher rate, except a very deep one (K several times N), which it cuts badly.  With more
+# than 16 rows the rows of x no longer stay in a wave's registers and only a shallow product is worth it.
+SKINNY_WEIGHT_BYTES = 48 << 20
+SKINNY_DEEP = 4
+SKINNY_SHALLOW_K = 2048
+
+
+def skinny_wins(rows: int, weight_rows: int, width: int) -> bool:
+    if not 0 < rows <= SKINNY_ROWS or width % 8:
+        return False
+    if rows <= 16:
+        return weight_rows * width * 2 <= SKINNY_WEIGHT_BYTES or width >= SKINNY_DEEP * weight_rows
+    return width <= SKINNY_SHALLOW_K
+
+
+def skinny_applies(x: torch.Tensor, w: torch.Tensor | None = None) -> bool:
+    """Whether the product of ``x`` goes to the hand-written kernel: whether it can, and, given the
+    weight, whether it is the faster of the two."""
+    if x.dtype != torch.bfloat16 or x.shape[0] > SKINNY_ROWS or x.shape[1] % 8:
+        return False
+    return w is None or skinny_wins(x.shape[0], w.shape[0], x.shape[1])
 
 
 # A product with more columns than this walks its column tiles in a loop; the norm as its first stage
 # then costs the registers that keep enough waves resident, and a norm kernel of its own is cheaper.
 FUSED_NORM_MAX_COLUMNS = 32768
+# The norm as the product's first stage is done again by every workgroup; beyond this width a norm kernel
+# of its own, once, is cheaper.
+FUSED_NORM_MAX_WIDTH = 2048
 
 
 def fused_norm_applies(rows_out: int, width: int, weight: torch.Tensor) -> bool:
-    """Whether norm and product run as one kernel: few rows of a bfloat16 model."""
-    return weight.dtype == torch.bfloat16 and 0 < rows_out <= SKINNY_ROWS and width % 8 == 0
+    """Whether norm and product run as one kernel: few rows of a bfloat16 model, a stream that is not wide."""
+    return (weight.dtype == torch.bfloat16 and width <= FUSED_NORM_MAX_WIDTH
+            and skinny_wins(rows_out, weight.shape[0], width))
 
 
 def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
@@ -541,9 +643,11 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> tor
     weights through the hand-written kernel, many rows go to the library's product."""
     _need(x, "matrix product input", None, torch.bfloat16)
     _need(w, "weight", None, torch.bfloat16)
-    if skinny_applies(x):
+    if skinny_applies(x, w):
         return gemm_skinny(x, w, out_dtype)
     if out_dtype == torch.float32:
+        if skinny_applies(x):
+            return gemm_skinny(x, w, torch.float32)
         if x.shape[1] % 8 == 0:
             # more wanted rows than one skinny launch takes: 64 at a time
             return torch.cat([gemm_skinny(x[i:i + SKINNY_ROWS].contiguous(), w, torch.float32)

@@ -50,7 +50,7 @@ class Linear:
             # the true 32-bit path: vector-unit multiply-add only
             y = kernels.gemm_plain(x, self.weight, out_dtype=torch.float32)
             return kernels.swiglu(y) if swiglu else y
-        if kernels.skinny_applies(x):
+        if kernels.skinny_applies(x, self.weight):
             if add_into is not None and not swiglu:
                 kernels.gemm_skinny(x, self.weight, add_into=add_into)
                 return None

@@ -119,11 +119,35 @@ LAYERS_0P6B = {
     "tie_word_embeddings": True,
 }
 
+# Layer sizes in the manner of the family's larger models, two layers of them: eight query heads a key
+# head (single tokens then go through the tiled attention kernel, a group's heads as its rows), a width
+# beyond what the product kernel normalises on the way in, and weights large enough that products of
+# few rows go to the library.
+LAYERS_WIDE = {
+    "architectures": ["Qwen3ForCausalLM"],
+    "model_type": "qwen3",
+    "hidden_act": "silu",
+    "attention_bias": False,
+    "sliding_window": None,
+    "hidden_size": 2560,
+    "intermediate_size": 6912,
+    "num_hidden_layers": 2,
+    "num_attention_heads": 16,
+    "num_key_value_heads": 2,
+    "head_dim": 128,
+    "rms_norm_eps": 1e-5,
+    "rope_theta": 1000000.0,
+    "vocab_size": 3001,
+    "max_position_embeddings": 4096,
+    "tie_word_embeddings": False,
+}
+
 TINY_INIT = {
     "A": dict(config=TINY_A, seed=0, std=0.02, gain_std=0.1),
     "B": dict(config=TINY_B, seed=1, std=0.05, gain_std=0.2),
     "C": dict(config=TINY_C, seed=2, std=0.08, gain_std=0.2),
     "D": dict(config=LAYERS_0P6B, seed=3, std=0.02, gain_std=0.1),
+    "E": dict(config=LAYERS_WIDE, seed=4, std=0.02, gain_std=0.1),
 }
 
 

@@ -488,6 +488,68 @@ def test_paged_attention_of_portions(nq, nkv, d, bs, requests, window, splits):
         assert err < 1e-2, f"token {i} (request {s}, position {p}): {err:.3e}"
 
 
+GROUPED_CASES = [
+    # nq, nkv, d, block size, [(context length after the step, tokens of the step)], window
+    (32, 8, 128, 16, [(513, 1), (40, 1), (2100, 1), (1, 1)], 0),
+    (16, 4, 64, 8, [(300, 3), (70, 1), (64, 15)], 0),
+    (64, 8, 128, 16, [(777, 2)], 0),
+    (32, 1, 128, 32, [(200, 1), (65, 4)], 0),
+    (8, 2, 64, 16, [(300, 5), (31, 1)], 48),
+    (16, 4, 128, 16, [(150, 64), (90, 2), (129, 1)], 0),
+    (10, 2, 128, 4, [(97, 1), (130, 2)], 0),
+]
+
+
+@pytest.mark.parametrize("splits", [1, 3, 16])
+@pytest.mark.parametrize("nq,nkv,d,bs,requests,window", GROUPED_CASES)
+def test_paged_attention_with_a_group_of_heads_as_the_rows_of_a_tile(nq, nkv, d, bs, requests, window, splits):
+    """Single tokens and short portions through the tiled kernel, the query heads that share a key head as
+    its rows; requests of 16 tokens or more are left out and their rows untouched."""
+    from paged_llm_rs_amd import kernels
+
+    assert kernels.library().pl_paged_attention_grouped_applies(nq, nkv, d, bs)
+    dtype = torch.bfloat16
+    ctx_lens = [c for c, _ in requests]
+    bt, k_pool, v_pool, keys, values = build_paged(nkv, d, bs, ctx_lens, dtype, seed=nq + bs + len(requests))
+    n = sum(c for _, c in requests)
+    stride = (nq + 2 * nkv) * d
+    q = torch.randn(n, stride, device=DEV).to(dtype)
+    q_start, q_len, positions, seq_of = [], [], [], []
+    for s, (ctx, count) in enumerate(requests):
+        q_start.append(len(positions))
+        q_len.append(count)
+        positions += list(range(ctx - count, ctx))
+        seq_of += [s] * count
+    as_i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    limit = kernels.SHORT_PORTION
+    short = [c for c in q_len if c < limit]
+    out = torch.full((n, nq * d), 7.0, dtype=dtype, device=DEV)
+    scale = 1 / math.sqrt(d)
+    kernels.paged_attention_grouped(q, stride, out, as_i32(q_start), as_i32(q_len), as_i32(ctx_lens), max(short), bt, bs,
+                                    k_pool, v_pool, nq, nkv, d, scale, window, short_limit=limit, splits=splits)
+    g = nq // nkv
+    for i in range(n):
+        s, p = seq_of[i], positions[i]
+        if q_len[s] >= limit:
+            assert bool((out[i] == 7.0).all()), "a long request is left to the other launch"
+            continue
+        want = attention_ref(q[i, :nq * d].double().cpu().reshape(nq, d), keys[s], values[s], p, g, scale, window)
+        err = rel(out[i].reshape(nq, d), want)
+        assert err < 1e-2, f"token {i} (request {s}, position {p}): {err:.3e}"
+
+
+def test_grouped_attention_refuses_what_it_does_not_serve():
+    from paged_llm_rs_amd import kernels
+
+    applies = kernels.library().pl_paged_attention_grouped_applies
+    assert not applies(16, 8, 96, 16)      # a head that is neither 64 nor 128
+    assert not applies(66, 2, 128, 16)     # more heads a group than a tile has rows
+    assert not applies(32, 8, 128, 2)      # pages smaller than one load of a wave
+    assert not applies(32, 8, 128, 24)     # no power of two
+    assert not kernels.grouped_applies(32, 8, 128, 16)   # four heads a key: the vector kernel is as fast
+    assert kernels.grouped_applies(64, 8, 128, 16)
+
+
 def test_a_far_key_is_found_from_inside_a_portion():
     """One key carries nearly all the weight of one query in the middle of a long portion: a key of an
     earlier step across a page edge, a key of the same step, the query's own key, and keys at a window's edge."""

@@ -25,7 +25,7 @@ pytestmark = pytest.mark.gpu
 # or three layers and a head that is a few times 1e-3 of the largest logit.
 TOLERANCE = {"float32": 1e-5, "bfloat16": 2e-2}
 LENGTHS = {"A": [5, 17, 33, 70, 100, 41], "B": [1, 9, 24, 40, 129, 66], "C": [3, 50, 97, 64, 20, 35],
-           "D": [300, 70, 33, 150]}
+           "D": [300, 70, 33, 150], "E": [260, 70, 33, 150]}
 
 
 @pytest.fixture(scope="module")
@@ -64,7 +64,7 @@ def test_whole_requests(setups, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,block_size", [("A", 16), ("B", 8), ("C", 4), ("D", 16)])
+@pytest.mark.parametrize("name,block_size", [("A", 16), ("B", 8), ("C", 4), ("D", 16), ("E", 16)])
 def test_last_tokens_decoded_one_by_one(setups, name, dtype, block_size):
     d, prompts, want = setups(name, dtype)
     got = replay(d, dtype, prompts, ru.tail_decoded(prompts, 32), max_live=1, block_size=block_size)
@@ -73,18 +73,19 @@ def test_last_tokens_decoded_one_by_one(setups, name, dtype, block_size):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,block_size", [("A", 16), ("B", 8), ("C", 4), ("D", 16)])
+@pytest.mark.parametrize("name,block_size", [("A", 16), ("B", 8), ("C", 4), ("D", 16), ("E", 16)])
 def test_portions_of_changing_size(setups, name, dtype, block_size):
     d, prompts, want = setups(name, dtype)
     # the large model gets portions of more than one tile of the attention kernel as well
-    steps = ru.portions(prompts, sizes=(130, 2, 64, 7, 33, 16)) if name == "D" else ru.portions(prompts)
+    steps = ru.portions(prompts, sizes=(130, 2, 64, 7, 33, 16)) if name in "DE" else ru.portions(prompts)
     got = replay(d, dtype, prompts, steps, max_live=1, block_size=block_size)
     worst, where = ru.worst_error(got, want)
     assert worst <= TOLERANCE[dtype], f"{worst:.3e} at {where}"
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,block_size,seed", [("A", 16, 1), ("B", 8, 2), ("C", 4, 3), ("B", 16, 4), ("D", 16, 5)])
+@pytest.mark.parametrize("name,block_size,seed", [("A", 16, 1), ("B", 8, 2), ("C", 4, 3), ("B", 16, 4), ("D", 16, 5),
+                                                    ("E", 16, 6)])
 def test_mixed_requests_with_pages_used_again(setups, name, dtype, block_size, seed):
     d, prompts, want = setups(name, dtype)
     steps = ru.mixed(prompts, seed=seed, max_live=4)
