@@ -606,6 +606,7 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
 SKINNY_WEIGHT_BYTES = 48 << 20
 SKINNY_DEEP = 4
 SKINNY_SHALLOW_K = 2048
+SKINNY_F32_FEW_K = 4096     # the widest stream whose projection onto a large vocabulary it wins, up to 16 rows
 
 
 def skinny_wins(rows: int, weight_rows: int, width: int) -> bool:
@@ -643,14 +644,13 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> tor
     weights through the hand-written kernel, many rows go to the library's product."""
     _need(x, "matrix product input", None, torch.bfloat16)
     _need(w, "weight", None, torch.bfloat16)
-    if skinny_applies(x, w):
-        return gemm_skinny(x, w, out_dtype)
     if out_dtype == torch.float32:
-        if skinny_applies(x):
+        # the projection onto the vocabulary: 32-bit out of the 32-bit sums, from either product
+        if skinny_applies(x) and x.shape[1] <= (SKINNY_F32_FEW_K if x.shape[0] <= 16 else SKINNY_SHALLOW_K):
             return gemm_skinny(x, w, torch.float32)
         if x.shape[1] % 8 == 0:
-            # more wanted rows than one skinny launch takes: 64 at a time
-            return torch.cat([gemm_skinny(x[i:i + SKINNY_ROWS].contiguous(), w, torch.float32)
-                              for i in range(0, x.shape[0], SKINNY_ROWS)], dim=0)
+            return torch.mm(x, w.t(), out_dtype=torch.float32)
         return gemm_plain(x, w, out_dtype=torch.float32)
+    if skinny_applies(x, w):
+        return gemm_skinny(x, w, out_dtype)
     return torch.mm(x, w.t())
