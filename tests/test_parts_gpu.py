@@ -276,6 +276,160 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path, dtype)
             tokens.append(produced)
 
 
+# --- a toy feed-forward with routing and a toy position encoding, defined here ----------------------------------------------
+
+@dataclass(frozen=True)
+class RoutedSpec:
+    kind: str = "routed_mlp"
+    experts: int = 3
+    intermediate_size: int = 0
+    top_k: int = 1
+
+
+class RoutedMlp:
+    """Experts of the gated form behind a router: the router's logits and their softmax in 32-bit, the
+    ``top_k`` largest weights kept and scaled to sum to one, the experts' outputs mixed by them."""
+
+    @staticmethod
+    def declare(spec, hidden):
+        from paged_llm_rs_amd.weights.loader import ParamDecl
+        decls = [ParamDecl("router.weight", (spec.experts, hidden))]
+        for e in range(spec.experts):
+            decls += [ParamDecl(f"experts.{e}.gate_proj.weight", (spec.intermediate_size, hidden)),
+                      ParamDecl(f"experts.{e}.up_proj.weight", (spec.intermediate_size, hidden)),
+                      ParamDecl(f"experts.{e}.down_proj.weight", (hidden, spec.intermediate_size))]
+        return decls
+
+    def __init__(self, spec, hidden, params, dtype, device, shared):
+        self.spec, self.params = spec, params
+
+    def forward(self, x):
+        spec, w = self.spec, self.params
+        weights = torch.softmax(x.float() @ w["router.weight"].float().t(), dim=-1)
+        if spec.top_k < spec.experts:
+            kept = torch.zeros_like(weights).scatter_(1, weights.topk(spec.top_k, dim=-1).indices, 1.0)
+            weights = weights * kept
+            weights = weights / weights.sum(-1, keepdim=True)
+        out = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
+        for e in range(spec.experts):
+            gate = x @ w[f"experts.{e}.gate_proj.weight"].t()
+            up = x @ w[f"experts.{e}.up_proj.weight"].t()
+            y = (torch.nn.functional.silu(gate.float()) * up.float()).to(x.dtype) @ w[f"experts.{e}.down_proj.weight"].t()
+            out += weights[:, e:e + 1] * y.float()
+        return out.to(x.dtype)
+
+
+class LinearAngles:
+    """Angles that grow linearly with the pair's index instead of geometrically, over part of a head:
+    position p turns pair i (elements i and i + dim/2 of the first ``dim``) by p * theta * (i + 1)."""
+
+    def __init__(self, spec, device):
+        self.dim, self.max_positions = spec.dim, spec.max_positions
+        angle = (torch.arange(spec.max_positions, dtype=torch.float64)[:, None]
+                 * spec.theta * torch.arange(1, spec.dim // 2 + 1, dtype=torch.float64)[None, :])
+        self.cos = angle.cos().float().to(device).contiguous()
+        self.sin = angle.sin().float().to(device).contiguous()
+
+
+class RoutedConfig:
+    """Two layers of attention with the linear angles over half of each head; the feed-forward of layer 0
+    is routed, that of layer 1 the plain gated one."""
+
+    def __init__(self, d):
+        self.d = d
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls(dict(d))
+
+    def to_dict(self):
+        return dict(self.d)
+
+    def model_spec(self):
+        from paged_llm_rs_amd.config import (AttentionSpec, GatedMlpSpec, LayerSpec, ModelSpec, NormSpec, PositionSpec,
+                                             ScheduleEntry)
+        d = self.d
+        norm = NormSpec("rms_norm", d["rms_norm_eps"])
+        position = PositionSpec("linear_angles", d["rotated"], d["angle_step"], d["max_position_embeddings"])
+        attention = AttentionSpec("paged_attention", d["num_attention_heads"], d["num_key_value_heads"], d["head_dim"],
+                                  norm, position, None, None)
+        routed = RoutedSpec("routed_mlp", d["num_experts"], d["expert_intermediate_size"], d["experts_per_token"])
+        layers = (LayerSpec("pre_norm", attention, routed, norm, "model.layers.0"),
+                  LayerSpec("pre_norm", attention, GatedMlpSpec("gated_mlp", d["intermediate_size"], "silu"), norm,
+                            "model.layers.1"))
+        return ModelSpec(d["hidden_size"], d["vocab_size"], layers, (ScheduleEntry(0), ScheduleEntry(1)), norm,
+                         d["tie_word_embeddings"], d["max_position_embeddings"])
+
+
+ROUTED = {"architectures": ["RoutedToyForCausalLM"], "model_type": "routed_toy", "hidden_size": 40, "intermediate_size": 72,
+          "num_experts": 3, "expert_intermediate_size": 24, "experts_per_token": 1, "num_attention_heads": 3,
+          "num_key_value_heads": 1, "head_dim": 32, "rotated": 16, "angle_step": 0.013, "rms_norm_eps": 1e-6,
+          "vocab_size": 113, "max_position_embeddings": 192, "tie_word_embeddings": False}
+
+
+def routed_plain(weights, cfg, tokens):
+    w = {k: v.double() for k, v in weights.items()}
+    n, eps = len(tokens), cfg["rms_norm_eps"]
+    nq, nkv, d, rot = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"], cfg["rotated"]
+    positions = torch.arange(n, dtype=torch.float64)
+    angle = positions[:, None] * cfg["angle_step"] * torch.arange(1, rot // 2 + 1, dtype=torch.float64)[None, :]
+    cos, sin = angle.cos()[:, None, :], angle.sin()[:, None, :]
+
+    def turn(t):   # [n, heads, d]
+        a, b, rest = t[..., :rot // 2], t[..., rot // 2:rot], t[..., rot:]
+        return torch.cat([a * cos - b * sin, b * cos + a * sin, rest], dim=-1)
+
+    def attend(x, prefix):
+        q = plain.rms_norm((x @ w[f"{prefix}.q_proj.weight"].T).reshape(n, nq, d), w[f"{prefix}.q_norm.weight"], eps)
+        k = plain.rms_norm((x @ w[f"{prefix}.k_proj.weight"].T).reshape(n, nkv, d), w[f"{prefix}.k_norm.weight"], eps)
+        v = (x @ w[f"{prefix}.v_proj.weight"].T).reshape(n, nkv, d)
+        k, v = plain.repeat_kv(turn(k), nq // nkv), plain.repeat_kv(v, nq // nkv)
+        return plain.attention_core(turn(q), k, v, 1.0 / math.sqrt(d)).reshape(n, nq * d) @ w[f"{prefix}.o_proj.weight"].T
+
+    def routed(x, prefix):
+        weight = plain.softmax_last(x @ w[f"{prefix}.router.weight"].T)
+        if cfg["experts_per_token"] < cfg["num_experts"]:
+            kept = torch.zeros_like(weight).scatter_(1, weight.topk(cfg["experts_per_token"], dim=-1).indices, 1.0)
+            weight = weight * kept / (weight * kept).sum(-1, keepdim=True)
+        return sum(weight[:, e:e + 1] * plain.swiglu_mlp(x, w, f"{prefix}.experts.{e}") for e in range(cfg["num_experts"]))
+
+    x = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+    for layer, feed in ((0, routed), (1, lambda t, prefix: plain.swiglu_mlp(t, w, prefix))):
+        p = f"model.layers.{layer}"
+        x = x + attend(plain.rms_norm(x, w[f"{p}.input_layernorm.weight"], eps), f"{p}.self_attn")
+        x = x + feed(plain.rms_norm(x, w[f"{p}.post_attention_layernorm.weight"], eps), f"{p}.mlp")
+    return plain.rms_norm(x, w["model.norm.weight"], eps) @ w["lm_head.weight"].T
+
+
+@pytest.mark.parametrize("dtype,experts_per_token", [("float32", 1), ("float32", 2), ("bfloat16", 3)])
+def test_a_toy_feed_forward_with_routing_and_a_toy_position_encoding(tmp_path, dtype, experts_per_token):
+    """A routed feed-forward in one layer beside the framework's own in the other, and angles of another
+    law over half of each head: registered here, built, replayed whole, decoded and mixed.  (In bfloat16
+    every expert keeps its weight: a router that cuts experts off is not continuous, and a rounding
+    that flips its choice at a near tie is no fault of the engine's.)"""
+    from safetensors.torch import load_file
+
+    from paged_llm_rs_amd import register_architecture, write_random_model
+    from paged_llm_rs_amd.engine.replay import Replayer
+    from paged_llm_rs_amd.parts import register_feed_forward, register_position
+
+    register_feed_forward("routed_mlp", RoutedMlp)
+    register_position("linear_angles", LinearAngles)
+    register_architecture("RoutedToyForCausalLM", RoutedConfig, model_type="routed_toy")
+    cfg = dict(ROUTED, experts_per_token=experts_per_token)
+    folder = write_random_model(tmp_path / "routed", cfg, seed=8, std=0.15, gain_std=0.2, dtype=dtype)
+    weights = load_file(str(folder / "model.safetensors"))
+    assert "model.layers.0.mlp.experts.2.down_proj.weight" in weights and "model.layers.1.mlp.gate_proj.weight" in weights
+    prompts = ru.make_prompts(cfg["vocab_size"], [40, 7, 66, 21], seed=4)
+    want = {name: routed_plain(weights, cfg, toks) for name, toks in prompts.items()}
+    tolerance = 1e-5 if dtype == "float32" else 2e-2
+    for steps, live in ((ru.whole(prompts), 1), (ru.tail_decoded(prompts, 12), 1), (ru.mixed(prompts, seed=2, max_live=3), 3)):
+        r = Replayer(folder, dtype, max_tokens=ru.pool_tokens(prompts, live), block_size=8, max_live=4)
+        got = ru.collect(r, steps)
+        worst, where = ru.worst_error(got, want)
+        assert worst <= tolerance, f"{worst:.3e} at {where}"
+
+
 # --- long decoding, first tokens, long portions -----------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
