@@ -38,6 +38,8 @@ def _signatures(lib) -> None:
         "pl_argmax": [p, p, p, p, i, i, p],
         "pl_sample": [p, p, p, p, p, p, i, i, p],
         "pl_gemm_skinny": [p, p, p, p, f, p, i, i, i, i, i, p],
+        "pl_gemm_tiled": [p, p, p, i, i, i, i, p],
+        "pl_gemm_tiled_applies": [i, i, i, i],
         "pl_paged_attention_decode": [p, i, p, p, p, p, p, p, i, p, i, i, p, p, i, i, i, i, f, i, i,
                                       i, p, p, i, f, p, p, i, p],
         "pl_paged_attention_prefill": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, p],
@@ -615,6 +617,45 @@ def skinny_wins(rows: int, weight_rows: int, width: int) -> bool:
     if rows <= 16:
         return weight_rows * width * 2 <= SKINNY_WEIGHT_BYTES or width >= SKINNY_DEEP * weight_rows
     return width <= SKINNY_SHALLOW_K
+
+
+def gemm_tiled_applies(rows: int, columns: int, width: int, swiglu: bool = False, add: bool = False) -> bool:
+    return bool(library().pl_gemm_tiled_applies(rows, columns, width, 1 if swiglu else (2 if add else 0)))
+
+
+# The tiled product reads LDS once a matrix instruction (a wave's tile is 64 x 64) and levels off at about
+# 0.7 PFLOP/s, below the library's best; what it saves is the trip of gate and up through memory and a
+# launch.  That wins for the gated feed-forward of a narrow model in portions of a prompt (512 rows of
+# width 1,024: 12.6 us against 20 for product plus activation; 2,048 rows: 38 against 39, no better inside
+# a step), and loses from a width of 4,096 on, as do the plain and the adding product at every size measured.
+TILED_SWIGLU_MAX_ROWS = 1024
+TILED_SWIGLU_MAX_WIDTH = 2048
+
+
+def tiled_swiglu_wins(rows: int, columns: int, width: int) -> bool:
+    return (SKINNY_ROWS < rows <= TILED_SWIGLU_MAX_ROWS and width <= TILED_SWIGLU_MAX_WIDTH
+            and gemm_tiled_applies(rows, columns, width, swiglu=True))
+
+
+def gemm_tiled(x: torch.Tensor, w: torch.Tensor, swiglu: bool = False, add_into: torch.Tensor | None = None) -> torch.Tensor:
+    """y = x . w^T for many rows of bfloat16 on the matrix cores, 32-bit sums, with SwiGLU (``w`` is
+    [gate | up] stacked, silu(gate) * up comes back) or the sum into the 32-bit residual stream
+    (``add_into``, which is returned) as the product's last stage."""
+    _need(x, "matrix product input", None, torch.bfloat16)
+    _need(w, "weight", None, torch.bfloat16)
+    if x.dim() != 2 or w.dim() != 2 or w.shape[1] != x.shape[1]:
+        raise TensorError(f"weight has shape {tuple(w.shape)} for an input of shape {tuple(x.shape)}")
+    M, K = x.shape
+    if swiglu and (w.shape[0] % 2 or add_into is not None):
+        raise TensorError("the activation needs an even number of weight rows and is not added into the stream")
+    N = w.shape[0] // 2 if swiglu else w.shape[0]
+    if add_into is not None:
+        _need(add_into, "residual stream", (M, N), torch.float32)
+        out, epilogue = add_into, 2
+    else:
+        out, epilogue = torch.empty((M, N), dtype=torch.bfloat16, device=x.device), (1 if swiglu else 0)
+    _check(library().pl_gemm_tiled(x.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, epilogue, _stream()))
+    return out
 
 
 def skinny_applies(x: torch.Tensor, w: torch.Tensor | None = None) -> bool:

@@ -56,5 +56,7 @@ class Linear:
                 return None
             return kernels.gemm_skinny(x, self.weight, out_dtype, swiglu=swiglu)
         if swiglu:
+            if kernels.tiled_swiglu_wins(x.shape[0], self.out_features // 2, self.in_features):
+                return kernels.gemm_tiled(x, self.weight, swiglu=True)
             return kernels.swiglu(kernels.linear_bf16(x, self.weight, x.dtype))
         return kernels.linear_bf16(x, self.weight, out_dtype)

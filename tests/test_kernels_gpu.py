@@ -259,6 +259,44 @@ def test_gemm_skinny_with_the_norm_before_and_the_residual_after(n, N, K):
     assert rel(resid, want) < 1e-5
 
 
+@pytest.mark.parametrize("M", [1, 127, 128, 300, 2048])
+@pytest.mark.parametrize("N,K", [(128, 32), (256, 96), (1024, 1024), (384, 2080)])
+@pytest.mark.parametrize("kind", ["store", "swiglu", "add"])
+def test_gemm_tiled(M, N, K, kind):
+    """The product for many rows, with its fused last stages, against 64-bit products of the same bfloat16 numbers."""
+    from paged_llm_rs_amd import kernels
+
+    x = (torch.randn(M, K, device=DEV) * 0.5).bfloat16()
+    if kind == "swiglu":
+        w = (torch.randn(2 * N, K, device=DEV) / math.sqrt(K)).bfloat16()
+        both = x.double() @ w.double().t()
+        want = torch.nn.functional.silu(both[:, :N]) * both[:, N:]
+        got = kernels.gemm_tiled(x, w, swiglu=True)
+        assert got.dtype == torch.bfloat16 and got.shape == (M, N)
+        assert rel(got, want) < 6e-3
+        return
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).bfloat16()
+    want = x.double() @ w.double().t()
+    if kind == "store":
+        assert rel(kernels.gemm_tiled(x, w), want) < 4e-3      # one rounding to bfloat16
+    else:
+        stream = torch.randn(M, N, device=DEV)
+        before = stream.clone()
+        assert kernels.gemm_tiled(x, w, add_into=stream) is stream
+        assert rel(stream.double() - before.double(), want) < 1e-5
+
+
+def test_gemm_tiled_refusals():
+    from paged_llm_rs_amd import kernels
+    from paged_llm_rs_amd.errors import TensorError
+
+    assert not kernels.gemm_tiled_applies(64, 100, 64) and not kernels.gemm_tiled_applies(64, 128, 40)
+    assert kernels.gemm_tiled_applies(64, 192, 64, swiglu=True) and not kernels.gemm_tiled_applies(64, 192, 64)
+    x = torch.zeros(4, 40, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(TensorError):
+        kernels.gemm_tiled(x, torch.zeros(128, 40, device=DEV, dtype=torch.bfloat16))
+
+
 def test_gemm_skinny_refusals():
     from paged_llm_rs_amd import kernels
     from paged_llm_rs_amd.errors import TensorError
