@@ -430,6 +430,90 @@ def test_a_toy_feed_forward_with_routing_and_a_toy_position_encoding(tmp_path, d
         assert worst <= tolerance, f"{worst:.3e} at {where}"
 
 
+# --- layers that see all keys beside layers that see a window of them ----------------------------------------------------
+
+class WindowedConfig:
+    """Layer 0 attends to every key, layers 1 and 2 to the last ``window`` keys: two groups of pages."""
+
+    def __init__(self, d):
+        self.d = d
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls(dict(d))
+
+    def to_dict(self):
+        return dict(self.d)
+
+    def model_spec(self):
+        from paged_llm_rs_amd.config import (AttentionSpec, GatedMlpSpec, LayerSpec, ModelSpec, NormSpec, PositionSpec,
+                                             ScheduleEntry)
+        d = self.d
+        norm = NormSpec("rms_norm", d["rms_norm_eps"])
+        ffn = GatedMlpSpec("gated_mlp", d["intermediate_size"], "silu")
+        position = PositionSpec("rotary_half", d["head_dim"], d["rope_theta"], d["max_position_embeddings"])
+
+        def attention(window):
+            return AttentionSpec("paged_attention", d["num_attention_heads"], d["num_key_value_heads"], d["head_dim"],
+                                 norm, position, window, None)
+
+        layers = tuple(LayerSpec("pre_norm", attention(None if i == 0 else d["window"]), ffn, norm, f"model.layers.{i}")
+                       for i in range(3))
+        return ModelSpec(d["hidden_size"], d["vocab_size"], layers, tuple(ScheduleEntry(i) for i in range(3)), norm,
+                         d["tie_word_embeddings"], d["max_position_embeddings"])
+
+
+WINDOWED = {"architectures": ["WindowedToyForCausalLM"], "model_type": "windowed_toy", "hidden_size": 64,
+            "intermediate_size": 96, "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 32, "window": 21,
+            "rms_norm_eps": 1e-6, "rope_theta": 1e4, "vocab_size": 101, "max_position_embeddings": 512,
+            "tie_word_embeddings": True}
+
+
+def windowed_plain(weights, tokens):
+    w = {k: v.double() for k, v in weights.items()}
+    x = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+    positions = torch.arange(len(tokens))
+    for i in range(3):
+        x = plain.decoder_block(x, w, f"model.layers.{i}", WINDOWED, positions, window=None if i == 0 else WINDOWED["window"])
+    return plain.rms_norm(x, w["model.norm.weight"], WINDOWED["rms_norm_eps"]) @ w["model.embed_tokens.weight"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_layers_with_a_window_beside_layers_without(tmp_path, dtype):
+    """Two groups of pages in one model: the windowed layers give pages back while a request still runs,
+    the others keep theirs; replayed whole, decoded, in portions and mixed with so few pages that they are
+    used again, against the plain implementation with the window in its mask."""
+    from safetensors.torch import load_file
+
+    from paged_llm_rs_amd import register_architecture, write_random_model
+    from paged_llm_rs_amd.engine.replay import Replayer
+
+    register_architecture("WindowedToyForCausalLM", WindowedConfig, model_type="windowed_toy")
+    folder = write_random_model(tmp_path / "windowed", WINDOWED, seed=12, std=0.12, gain_std=0.2, dtype=dtype)
+    weights = load_file(str(folder / "model.safetensors"))
+    prompts = ru.make_prompts(WINDOWED["vocab_size"], [90, 23, 141, 60], seed=6)
+    want = {name: windowed_plain(weights, toks) for name, toks in prompts.items()}
+    tolerance = 1e-5 if dtype == "float32" else 2e-2
+    schedules = ((ru.whole(prompts), 1), (ru.tail_decoded(prompts, 32), 1), (ru.portions(prompts), 1),
+                 (ru.mixed(prompts, seed=3, max_live=3), 3))
+    for steps, live in schedules:
+        r = Replayer(folder, dtype, max_tokens=ru.pool_tokens(prompts, live), block_size=8, max_live=4)
+        assert len(r.cache.layout.groups) == 2, "the windowed layers have pages of their own"
+        got = ru.collect(r, steps)
+        worst, where = ru.worst_error(got, want)
+        assert worst <= tolerance, f"{worst:.3e} at {where}"
+        assert r.cache.manager.live_sequences == 0 and r.cache.manager.available() == r.cache.manager.total()
+    # while a request runs, the windowed group holds the window and no more; the other group holds everything
+    r = Replayer(folder, dtype, max_tokens=256, block_size=8, max_live=4)
+    longest = prompts[max(prompts, key=lambda n: len(prompts[n]))]
+    r.step([{"id": "x", "tokens": longest[:100], "want": []}], [])
+    r.step([{"id": "x", "tokens": longest[100:], "want": [0]}], [])
+    assert r.cache.manager.in_use(0) == -(-len(longest) // 8)
+    assert r.cache.manager.in_use(1) <= -(-WINDOWED["window"] // 8) + 2
+    r.step([], ["x"])
+    assert r.cache.manager.in_use(0) == 0 and r.cache.manager.in_use(1) == 0
+
+
 # --- long decoding, first tokens, long portions -----------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
