@@ -14,6 +14,8 @@ from typing import Optional
 
 import torch
 
+from ..errors import ConfigError
+
 
 @dataclass(frozen=True)
 class KVCacheSpec:
@@ -45,7 +47,31 @@ class CacheLayout:
 
     @classmethod
     def from_blocks(cls, blocks, schedule) -> "CacheLayout":
-        owners = sorted({e.layer for e in schedule if e.cache_from is None})
+        # A run of a layer either owns its cache or reads the one another run has written earlier in the
+        # same pass.  Two owning runs of one layer would write the same pages twice, and what a later step
+        # reads there would depend on how the tokens were cut into steps: refused.
+        def spec_of(index):
+            mixer = getattr(blocks[index], "mixer", None)
+            return (mixer.cache_spec(), mixer.state_spec()) if mixer is not None else (None, None)
+
+        written: set = set()
+        for at, e in enumerate(schedule):
+            kv, state = spec_of(e.layer)
+            if e.cache_from is None:
+                if e.layer in written and (kv is not None or state is not None):
+                    raise ConfigError(f"the schedule runs layer {e.layer} twice with a cache of its own; the second run "
+                                      f"can read what the first wrote (cache_from={e.layer})")
+                written.add(e.layer)
+            else:
+                if e.cache_from not in written:
+                    raise ConfigError(f"run {at} of the schedule reads the cache of layer {e.cache_from}, which no "
+                                      "earlier run of the pass has written")
+                if state is not None:
+                    raise ConfigError(f"layer {e.layer} keeps a state of its own and cannot read another layer's cache")
+                if spec_of(e.cache_from)[0] != kv:
+                    raise ConfigError(f"layer {e.layer} reads the cache of layer {e.cache_from}, whose keys and values "
+                                      "have another shape or window")
+        owners = sorted(written)
         groups: list = []
         layer_group: dict = {}
         states: dict = {}

@@ -395,3 +395,31 @@ def test_shared_pages_are_counted_right_under_random_orders(seed):
     for sid in list(live):
         m.free_sequence(sid)
     assert m.available() == total
+
+
+# --- the order of layers and whose cache a run uses ---------------------------------------------------------
+
+def test_schedules_that_would_write_a_cache_twice_or_read_an_unwritten_one_are_refused():
+    import types
+
+    from paged_llm_rs_amd.cache import CacheLayout
+    from paged_llm_rs_amd.cache.layout import KVCacheSpec
+    from paged_llm_rs_amd.config import ScheduleEntry
+    from paged_llm_rs_amd.errors import ConfigError
+
+    def block(kv_heads, head_dim, window=None):
+        mixer = types.SimpleNamespace(cache_spec=lambda: KVCacheSpec(kv_heads, head_dim, window), state_spec=lambda: None)
+        return types.SimpleNamespace(mixer=mixer)
+
+    blocks = [block(2, 16), block(2, 16), block(1, 16), block(2, 16, 8)]
+    ok = CacheLayout.from_blocks(blocks, [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(1, cache_from=1),
+                                          ScheduleEntry(0, cache_from=1)])
+    assert len(ok.groups) == 1 and ok.groups[0].layers == [0, 1]
+    with pytest.raises(ConfigError, match="twice"):
+        CacheLayout.from_blocks(blocks, [ScheduleEntry(0), ScheduleEntry(0)])
+    with pytest.raises(ConfigError, match="no earlier run"):
+        CacheLayout.from_blocks(blocks, [ScheduleEntry(0, cache_from=1), ScheduleEntry(1)])
+    with pytest.raises(ConfigError, match="another shape"):
+        CacheLayout.from_blocks(blocks, [ScheduleEntry(0), ScheduleEntry(2, cache_from=0)])
+    with pytest.raises(ConfigError, match="another shape"):
+        CacheLayout.from_blocks(blocks, [ScheduleEntry(0), ScheduleEntry(3, cache_from=0)])

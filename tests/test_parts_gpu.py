@@ -514,6 +514,94 @@ def test_layers_with_a_window_beside_layers_without(tmp_path, dtype):
     assert r.cache.manager.in_use(0) == 0 and r.cache.manager.in_use(1) == 0
 
 
+# --- a layer that runs twice, and layers that read another layer's keys and values --------------------------------------
+
+class SharingConfig:
+    """Three layers run as 0, 1, 2 (with the keys and values of layer 0), 1 again (with what its first run wrote)."""
+
+    def __init__(self, d):
+        self.d = d
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls(dict(d))
+
+    def to_dict(self):
+        return dict(self.d)
+
+    def model_spec(self):
+        from paged_llm_rs_amd.config import (AttentionSpec, GatedMlpSpec, LayerSpec, ModelSpec, NormSpec, PositionSpec,
+                                             ScheduleEntry)
+        d = self.d
+        norm = NormSpec("rms_norm", d["rms_norm_eps"])
+        ffn = GatedMlpSpec("gated_mlp", d["intermediate_size"], "silu")
+        attention = AttentionSpec("paged_attention", d["num_attention_heads"], d["num_key_value_heads"], d["head_dim"], norm,
+                                  PositionSpec("rotary_half", d["head_dim"], d["rope_theta"], d["max_position_embeddings"]),
+                                  None, None)
+        layers = tuple(LayerSpec("pre_norm", attention, ffn, norm, f"model.layers.{i}") for i in range(3))
+        schedule = (ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2, cache_from=0), ScheduleEntry(1, cache_from=1))
+        return ModelSpec(d["hidden_size"], d["vocab_size"], layers, schedule, norm, d["tie_word_embeddings"],
+                         d["max_position_embeddings"])
+
+
+SHARING = {"architectures": ["SharingToyForCausalLM"], "model_type": "sharing_toy", "hidden_size": 48, "intermediate_size": 64,
+           "num_attention_heads": 6, "num_key_value_heads": 2, "head_dim": 16, "rms_norm_eps": 1e-5, "rope_theta": 1e4,
+           "vocab_size": 89, "max_position_embeddings": 256, "tie_word_embeddings": True}
+
+
+def sharing_plain(weights, tokens):
+    cfg = SHARING
+    w = {k: v.double() for k, v in weights.items()}
+    n, eps = len(tokens), cfg["rms_norm_eps"]
+    nq, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    positions = torch.arange(n)
+    held = {}       # layer -> the rotated keys and the values its own run computed
+
+    def attend(x, layer, source):
+        p = f"model.layers.{layer}.self_attn"
+        q = plain.rms_norm((x @ w[f"{p}.q_proj.weight"].T).reshape(n, nq, d), w[f"{p}.q_norm.weight"], eps)
+        q = plain.apply_rope(q, positions, cfg["rope_theta"])
+        if source is None:
+            k = plain.rms_norm((x @ w[f"{p}.k_proj.weight"].T).reshape(n, nkv, d), w[f"{p}.k_norm.weight"], eps)
+            held[layer] = (plain.apply_rope(k, positions, cfg["rope_theta"]), (x @ w[f"{p}.v_proj.weight"].T).reshape(n, nkv, d))
+            source = layer
+        k, v = held[source]
+        out = plain.attention_core(q, plain.repeat_kv(k, nq // nkv), plain.repeat_kv(v, nq // nkv), 1.0 / math.sqrt(d))
+        return out.reshape(n, nq * d) @ w[f"{p}.o_proj.weight"].T
+
+    x = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+    for layer, source in ((0, None), (1, None), (2, 0), (1, 1)):
+        p = f"model.layers.{layer}"
+        x = x + attend(plain.rms_norm(x, w[f"{p}.input_layernorm.weight"], eps), layer, source)
+        x = x + plain.swiglu_mlp(plain.rms_norm(x, w[f"{p}.post_attention_layernorm.weight"], eps), w, f"{p}.mlp")
+    return plain.rms_norm(x, w["model.norm.weight"], eps) @ w["model.embed_tokens.weight"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_layer_that_runs_twice_and_layers_that_read_another_layers_cache(tmp_path, dtype):
+    """The order of layers is data: layer 2 has no pages and attends over what layer 0 wrote, layer 1 runs a
+    second time over what its first run wrote.  Two layers own pages; every schedule of replay agrees with the
+    plain implementation."""
+    from safetensors.torch import load_file
+
+    from paged_llm_rs_amd import register_architecture, write_random_model
+    from paged_llm_rs_amd.engine.replay import Replayer
+
+    register_architecture("SharingToyForCausalLM", SharingConfig, model_type="sharing_toy")
+    folder = write_random_model(tmp_path / "sharing", SHARING, seed=21, std=0.15, gain_std=0.2, dtype=dtype)
+    weights = load_file(str(folder / "model.safetensors"))
+    prompts = ru.make_prompts(SHARING["vocab_size"], [50, 13, 77, 34], seed=9)
+    want = {name: sharing_plain(weights, toks) for name, toks in prompts.items()}
+    tolerance = 1e-5 if dtype == "float32" else 2e-2
+    for steps, live in ((ru.whole(prompts), 1), (ru.tail_decoded(prompts, 20), 1), (ru.portions(prompts), 1),
+                        (ru.mixed(prompts, seed=5, max_live=3), 3)):
+        r = Replayer(folder, dtype, max_tokens=ru.pool_tokens(prompts, live), block_size=8, max_live=4)
+        assert [g.layers for g in r.cache.layout.groups] == [[0, 1]], "two layers own pages, the third borrows"
+        got = ru.collect(r, steps)
+        worst, where = ru.worst_error(got, want)
+        assert worst <= tolerance, f"{worst:.3e} at {where}"
+
+
 # --- long decoding, first tokens, long portions -----------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
