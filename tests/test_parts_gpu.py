@@ -602,6 +602,132 @@ def test_a_layer_that_runs_twice_and_layers_that_read_another_layers_cache(tmp_p
         assert worst <= tolerance, f"{worst:.3e} at {where}"
 
 
+# --- a toy norm and a toy arrangement of a layer ----------------------------------------------------------------------------
+
+class CenteredNorm:
+    """(x - mean) / sqrt(var + eps) * weight + bias over the last axis, in 32-bit."""
+
+    @staticmethod
+    def declare(spec, width):
+        from paged_llm_rs_amd.weights.loader import ParamDecl
+        return [ParamDecl("weight", (width,), "gain"), ParamDecl("bias", (width,), "matrix")]
+
+    def __init__(self, spec, width, params, dtype, device):
+        self.eps, self.weight, self.bias = float(spec.eps), params["weight"].float(), params["bias"].float()
+
+    def apply(self, resid, delta, out_dtype, rows=None):
+        if delta is not None:
+            resid += delta.float()                       # the residual sum: into the 32-bit stream, in place
+        x = resid if rows is None else resid[rows.long()]
+        centred = x - x.mean(-1, keepdim=True)
+        return (centred * torch.rsqrt(centred.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight + self.bias).to(out_dtype)
+
+
+class ParallelBlock:
+    """One norm, then mixer and feed-forward side by side on the same rows: x + mix(n(x)) + ff(n(x))."""
+
+    @classmethod
+    def declare(cls, layer, hidden):
+        from paged_llm_rs_amd.parts.registry import FEED_FORWARDS, MIXERS, NORMS, lookup, prefixed
+        return (prefixed(lookup(NORMS, layer.norm.kind, "norm").declare(layer.norm, hidden), "ln")
+                + prefixed(lookup(MIXERS, layer.mixer.kind, "mixer").declare(layer.mixer, hidden), "attn")
+                + prefixed(lookup(FEED_FORWARDS, layer.feed_forward.kind, "feed-forward").declare(layer.feed_forward, hidden), "ffn"))
+
+    def __init__(self, layer, hidden, params, dtype, device, shared):
+        from paged_llm_rs_amd.parts.registry import FEED_FORWARDS, MIXERS, NORMS, lookup, scoped
+        self.dtype = dtype
+        self.norm = lookup(NORMS, layer.norm.kind, "norm")(layer.norm, hidden, scoped(params, "ln"), dtype, device)
+        self.mixer = lookup(MIXERS, layer.mixer.kind, "mixer")(layer.mixer, hidden, scoped(params, "attn"), dtype, device, shared)
+        self.feed_forward = lookup(FEED_FORWARDS, layer.feed_forward.kind, "feed-forward")(
+            layer.feed_forward, hidden, scoped(params, "ffn"), dtype, device, shared)
+
+    def forward(self, resid, delta, ctx):
+        x = self.norm.apply(resid, delta, self.dtype)
+        return self.mixer.forward(x, ctx) + self.feed_forward.forward(x)
+
+
+class ParallelConfig:
+    def __init__(self, d):
+        self.d = d
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls(dict(d))
+
+    def to_dict(self):
+        return dict(self.d)
+
+    def model_spec(self):
+        from paged_llm_rs_amd.config import (AttentionSpec, GatedMlpSpec, LayerSpec, ModelSpec, NormSpec, PositionSpec,
+                                             ScheduleEntry)
+        d = self.d
+        norm = NormSpec("centered_norm", d["layer_norm_eps"])
+        attention = AttentionSpec("paged_attention", d["num_attention_heads"], d["num_key_value_heads"], d["head_dim"], None,
+                                  PositionSpec("rotary_half", d["rotary_dim"], d["rope_theta"], d["max_position_embeddings"]),
+                                  None, d["attention_scale"])
+        ffn = GatedMlpSpec("gated_mlp", d["intermediate_size"], "silu")
+        layers = tuple(LayerSpec("parallel", attention, ffn, norm, f"transformer.h.{i}") for i in range(d["num_hidden_layers"]))
+        return ModelSpec(d["hidden_size"], d["vocab_size"], layers, tuple(ScheduleEntry(i) for i in range(len(layers))), norm,
+                         False, d["max_position_embeddings"], embed_name="transformer.wte.weight",
+                         final_norm_name="transformer.ln_f.weight", head_name="lm_head.weight")
+
+
+PARALLEL = {"architectures": ["ParallelToyForCausalLM"], "model_type": "parallel_toy", "hidden_size": 56, "intermediate_size": 88,
+            "num_hidden_layers": 2, "num_attention_heads": 4, "num_key_value_heads": 4, "head_dim": 16, "rotary_dim": 16,
+            "attention_scale": 0.3, "layer_norm_eps": 1e-5, "rope_theta": 1e4, "vocab_size": 71,
+            "max_position_embeddings": 256}
+
+
+def parallel_plain(weights, tokens):
+    cfg = PARALLEL
+    w = {k: v.double() for k, v in weights.items()}
+    n, nh, d = len(tokens), cfg["num_attention_heads"], cfg["head_dim"]
+    positions = torch.arange(n)
+
+    def norm(x, prefix):
+        c = x - x.mean(-1, keepdim=True)
+        return c / torch.sqrt(c.pow(2).mean(-1, keepdim=True) + cfg["layer_norm_eps"]) * w[f"{prefix}.weight"] + w[f"{prefix}.bias"]
+
+    x = w["transformer.wte.weight"][torch.tensor(tokens)]
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"transformer.h.{i}"
+        y = norm(x, f"{p}.ln")
+        q = plain.apply_rope((y @ w[f"{p}.attn.q_proj.weight"].T).reshape(n, nh, d), positions, cfg["rope_theta"])
+        k = plain.apply_rope((y @ w[f"{p}.attn.k_proj.weight"].T).reshape(n, nh, d), positions, cfg["rope_theta"])
+        v = (y @ w[f"{p}.attn.v_proj.weight"].T).reshape(n, nh, d)
+        mixed = plain.attention_core(q, k, v, cfg["attention_scale"]).reshape(n, nh * d) @ w[f"{p}.attn.o_proj.weight"].T
+        x = x + mixed + plain.swiglu_mlp(y, w, f"{p}.ffn")
+    return norm(x, "transformer.ln_f") @ w["lm_head.weight"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_toy_norm_and_a_toy_arrangement_of_a_layer(tmp_path, dtype):
+    """A norm with a mean and a bias, and a layer whose mixer and feed-forward read the same normalised rows,
+    under tensor names of another family, with attention that has no q/k norm, one key head a query head and
+    a scale of its own: registered here, built, replayed whole, decoded, in portions and mixed."""
+    from safetensors.torch import load_file
+
+    from paged_llm_rs_amd import register_architecture, write_random_model
+    from paged_llm_rs_amd.engine.replay import Replayer
+    from paged_llm_rs_amd.parts import register_block, register_norm
+
+    register_norm("centered_norm", CenteredNorm)
+    register_block("parallel", ParallelBlock)
+    register_architecture("ParallelToyForCausalLM", ParallelConfig, model_type="parallel_toy")
+    folder = write_random_model(tmp_path / "parallel", PARALLEL, seed=31, std=0.15, gain_std=0.2, dtype=dtype)
+    weights = load_file(str(folder / "model.safetensors"))
+    assert "transformer.h.1.ln.bias" in weights and "transformer.ln_f.bias" in weights and "lm_head.weight" in weights
+    prompts = ru.make_prompts(PARALLEL["vocab_size"], [33, 8, 58, 19], seed=13)
+    want = {name: parallel_plain(weights, toks) for name, toks in prompts.items()}
+    tolerance = 1e-5 if dtype == "float32" else 2e-2
+    for steps, live in ((ru.whole(prompts), 1), (ru.tail_decoded(prompts, 12), 1), (ru.portions(prompts), 1),
+                        (ru.mixed(prompts, seed=4, max_live=3), 3)):
+        r = Replayer(folder, dtype, max_tokens=ru.pool_tokens(prompts, live), block_size=8, max_live=4)
+        got = ru.collect(r, steps)
+        worst, where = ru.worst_error(got, want)
+        assert worst <= tolerance, f"{worst:.3e} at {where}"
+
+
 # --- long decoding, first tokens, long portions -----------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
