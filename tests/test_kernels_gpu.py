@@ -394,7 +394,7 @@ def test_paged_attention_of_single_tokens(kernel, nq, nkv, d, bs, ctx_lens, wind
     assert bool((out[-1] == 7.0).all()), "a padding row is not written"
 
 
-@pytest.mark.parametrize("kernel", ["plain", "decode"])
+@pytest.mark.parametrize("kernel", ["plain", "decode", "grouped-1", "grouped-4"])
 def test_a_far_key_among_hundreds_is_found(kernel):
     """Random scores hide a lost key; here one key far back (just across a page edge,
     then just inside a window's edge) carries nearly all the weight, and its value is the answer."""
@@ -417,9 +417,13 @@ def test_a_far_key_among_hundreds_is_found(kernel):
         scale = 1 / math.sqrt(d)
         if kernel == "plain":
             kernels.paged_attention_plain(q, stride, out, positions, seq_of, bt, bs, k_pool, v_pool, nq, nkv, d, scale, window)
-        else:
+        elif kernel == "decode":
             kernels.paged_attention_decode(q, stride, out, positions, seq_of, bt, bs, k_pool, v_pool, nq, nkv, d,
                                            scale, window, splits=4)
+        else:
+            one = torch.ones(1, dtype=torch.int32, device=DEV)
+            kernels.paged_attention_grouped(q, stride, out, seq_of, one, one * ctx, 1, bt, bs, k_pool, v_pool, nq, nkv, d,
+                                            scale, window, splits=int(kernel.split("-")[1]))
         want = attention_ref(q[0, :nq * d].double().cpu().reshape(nq, d), keys[0], values[0], ctx - 1, 2, scale, window)
         assert rel(out[0].reshape(nq, d), want) < 1e-2, (ctx, target, window)
         inside = window == 0 or target > ctx - 1 - window
