@@ -359,6 +359,8 @@ ATTENTION_CASES = [
     (4, 2, 256, 16, [77, 150], 0),
     (4, 2, 64, 16, [300, 31], 48),
     (2, 2, 16, 4, [50], 7),
+    (16, 8, 128, 128, [513, 40], 0),
+    (8, 2, 64, 64, [300], 100),
 ]
 
 
@@ -484,6 +486,8 @@ PORTION_CASES = [
     (4, 2, 64, 16, [(300, 140), (31, 31)], 48),
     (2, 2, 16, 4, [(90, 70)], 7),
     (2, 2, 32, 16, [(500, 200)], 64),
+    (16, 8, 128, 64, [(513, 300), (129, 129)], 0),
+    (8, 2, 64, 256, [(700, 200), (40, 17)], 0),
 ]
 
 
@@ -539,6 +543,8 @@ GROUPED_CASES = [
     (8, 2, 64, 16, [(300, 5), (31, 1)], 48),
     (16, 4, 128, 16, [(150, 64), (90, 2), (129, 1)], 0),
     (10, 2, 128, 4, [(97, 1), (130, 2)], 0),
+    (32, 4, 128, 64, [(513, 1), (300, 2)], 0),
+    (16, 2, 64, 256, [(700, 3)], 100),
 ]
 
 
