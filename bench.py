@@ -145,11 +145,13 @@ def main() -> int:
     parser.add_argument("--skip-points", action="store_true", help="leave out batch 1 and 64 and the prefill")
     parser.add_argument("--prefill-eager", action="store_true",
                         help="launch the prefill step kernel by kernel every time (a prompt length seen once)")
-    parser.add_argument("--only", choices=["decode", "prefill", "engine", "mixed"], default=None,
+    parser.add_argument("--only", choices=["decode", "prefill", "engine", "mixed", "serving"], default=None,
                         help="run one part alone: the decode steps at --batch, the prefill, or (not part of the "
                              "default line) the whole engine on 1/4/16/32/64 requests at once, 16 prompt tokens and "
                              "128 generated each, as the reference's own table of clients does; mixed: one step of a "
-                             "512-token slice of a prompt beside 63 decoded tokens")
+                             "512-token slice of a prompt beside 63 decoded tokens; serving: the reference's two other "
+                             "tables, first tokens behind a shared preamble with the prefix cache off and on, and the "
+                             "gaps between the tokens of four running requests when a long prompt arrives, by --chunk")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU; this engine has no multi-GPU path (N must be 1)")
@@ -251,6 +253,76 @@ def main() -> int:
             "hbm_floor_ms": round(step_bytes / HBM_PEAK * 1e3, 3), "mfma_floor_ms": round(flops / MFMA_PEAK["bf16"] * 1e3, 3),
             "frac_hbm": round(step_bytes / seconds / HBM_PEAK, 4), "frac_mfma": round(flops / seconds / MFMA_PEAK["bf16"], 4),
         }}), flush=True)
+        tmp.cleanup()
+        return 0
+    if args.only == "serving":
+        from paged_llm_rs_amd.engine.engine import Engine
+
+        del runner, cache
+        vocab = cfg["vocab_size"]
+
+        def drive(engine, arrivals):
+            """Submit the (step, prompt, max_tokens) arrivals when their step comes, run to the end; per request
+            the times of its tokens, counted from its arrival."""
+            pending = sorted(arrivals, key=lambda a: a[0])
+            arrived, stamps, step = {}, {}, 0
+            while pending or engine.open_requests:
+                while pending and pending[0][0] <= step:
+                    _, prompt, budget = pending.pop(0)
+                    arrived[engine.submit(prompt, max_tokens=budget, temperature=0.0, stop_tokens=[])] = time.perf_counter()
+                outcome = engine.step()
+                step += 1
+                if outcome is None:
+                    continue
+                now = time.perf_counter()
+                for seq_id, _ in outcome.tokens:
+                    stamps.setdefault(seq_id, []).append(now - arrived[seq_id])
+            for seq_id in stamps:
+                engine.take_result(seq_id)
+            return [stamps[k] for k in sorted(stamps)]
+
+        def percentile(values, q):
+            ordered = sorted(values)
+            return ordered[min(len(ordered) - 1, int(q * len(ordered)))]
+
+        result = {"prefix_cache": {}, "chunk": {}}
+        rng = random.Random(11)
+        preamble = [rng.randrange(vocab) for _ in range(384)]
+        shared = [preamble + [rng.randrange(vocab) for _ in range(16)] for _ in range(16)]
+        apart = [[rng.randrange(vocab) for _ in range(400)] for _ in range(16)]
+        for workload, prompts in (("one shared preamble", shared), ("nothing in common", apart)):
+            for cache_on in (False, True):
+                engine = Engine(folder, dtype="bf16", block_size=BLOCK_SIZE, num_blocks=2048, max_batch=16, chunk=128,
+                                prefix_cache=cache_on)
+                for run, timed_run in enumerate((False, False, True)):   # shapes of step are captured when they come again
+                    # other tokens every run: what an earlier run left in the cache must not make this one a hit
+                    prompts_run = [[(t + 7 * run) % vocab for t in p] for p in prompts]
+                    before = engine.metrics().get("cached_tokens", 0)
+                    torch.cuda.synchronize()
+                    start = time.perf_counter()
+                    times = drive(engine, [(0, p, 64) for p in prompts_run])
+                    seconds = time.perf_counter() - start
+                firsts = [t[0] for t in times]
+                result["prefix_cache"][f"{workload}, cache {'on' if cache_on else 'off'}"] = {
+                    "ttft_ms": round(sum(firsts) / len(firsts) * 1e3, 2), "p95_ttft_ms": round(percentile(firsts, 0.95) * 1e3, 2),
+                    "tokens_per_s": round(sum(len(t) for t in times) / seconds, 1),
+                    "cached_tokens": engine.metrics().get("cached_tokens", 0) - before}
+                say(f"prefix cache, {workload}, {'on' if cache_on else 'off'}: {result['prefix_cache'][f'{workload}, cache ' + ('on' if cache_on else 'off')]}")
+                del engine
+        long_prompt = [rng.randrange(vocab) for _ in range(1100)]
+        residents = [[rng.randrange(vocab) for _ in range(12)] for _ in range(4)]
+        for chunk in ("off", 512, 128, 64, 32):
+            engine = Engine(folder, dtype="bf16", block_size=BLOCK_SIZE, num_blocks=1024, max_batch=16, chunk=chunk,
+                            prefix_cache=False)
+            for timed_run in (False, False, True):
+                times = drive(engine, [(0, p, 160) for p in residents] + [(40, long_prompt, 16)])
+            gaps = [b - a for t in times[:4] for a, b in zip(t, t[1:])]
+            result["chunk"][str(chunk)] = {
+                "median_gap_ms": round(percentile(gaps, 0.5) * 1e3, 3), "worst_gap_ms": round(max(gaps) * 1e3, 3),
+                "newcomer_first_token_ms": round(times[4][0] * 1e3, 2)}
+            say(f"chunk {chunk}: {result['chunk'][str(chunk)]}")
+            del engine
+        print(json.dumps({"serving": result}), flush=True)
         tmp.cleanup()
         return 0
     if args.only == "engine":

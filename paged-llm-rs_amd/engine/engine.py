@@ -205,6 +205,11 @@ class Engine:
             self._greedy.pop(f.id, None)
             self._results[f.id] = done
 
+    @property
+    def open_requests(self) -> int:
+        """Requests that were submitted and have not finished."""
+        return len(self._open)
+
     def run(self) -> None:
         """Run until every submitted request has finished."""
         while self._open:
