@@ -674,9 +674,14 @@ FUSED_NORM_MAX_COLUMNS = 32768
 FUSED_NORM_MAX_WIDTH = 2048
 
 
+# ... and every workgroup reads the rows of the 32-bit stream, twice the bytes of normalised bfloat16 rows; a
+# compute unit takes in some 30 GB/s, and beyond this many rows that costs more than a norm kernel.
+FUSED_NORM_MAX_ROWS = 32
+
+
 def fused_norm_applies(rows_out: int, width: int, weight: torch.Tensor) -> bool:
     """Whether norm and product run as one kernel: few rows of a bfloat16 model, a stream that is not wide."""
-    return (weight.dtype == torch.bfloat16 and width <= FUSED_NORM_MAX_WIDTH
+    return (weight.dtype == torch.bfloat16 and width <= FUSED_NORM_MAX_WIDTH and rows_out <= FUSED_NORM_MAX_ROWS
             and skinny_wins(rows_out, weight.shape[0], width))
 
 
