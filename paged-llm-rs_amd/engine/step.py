@@ -78,10 +78,13 @@ def _bucket(n: int, least: int = 1) -> int:
 
 
 class DecodeGraph:
-    """One decode step for up to ``cap`` requests with up to ``widths[g]`` pages each, captured."""
+    """One decode step for up to ``cap`` requests with up to ``widths[g]`` pages each, captured; or, with
+    ``captured=False``, launched kernel by kernel over the same buffers with the same idle rows, so that a
+    runner without graphs computes what one with graphs replays."""
 
-    def __init__(self, model, cache, cap: int, widths: list):
+    def __init__(self, model, cache, cap: int, widths: list, captured: bool = True):
         self.model, self.cache, self.cap, self.widths = model, cache, cap, list(widths)
+        self.captured = captured
         pieces = [("token_ids", cap), ("positions", cap), ("seq_of", cap), ("q_start", cap), ("q_len", cap),
                   ("ctx_len", cap), ("state_slots", cap), ("logit_rows", cap)]
         pieces += [(f"block_table_{g}", cap * w) for g, w in enumerate(widths)]
@@ -162,6 +165,10 @@ class DecodeGraph:
     def run(self, entries) -> StepOutput:
         live = len(entries)
         self.fill(entries)
+        if not self.captured:
+            self.device_buf.copy_(self.host, non_blocking=True)
+            logits, tokens = self._forward()
+            return StepOutput(logits[:live], tokens[:live])
         if self.graph is None:
             self.capture()
         self.device_buf.copy_(self.host, non_blocking=True)
@@ -234,7 +241,7 @@ class StepRunner:
         self.eager_steps = 0
 
     def _is_plain_decode(self, entries) -> bool:
-        return (self.use_graphs and 0 < len(entries) <= GRAPH_MAX_REQUESTS
+        return ((self.use_graphs or self.pads) and 0 < len(entries) <= GRAPH_MAX_REQUESTS
                 and all(len(e.tokens) == 1 and e.want == [0] for e in entries))
 
     def _run_shaped(self, entries) -> StepOutput:
@@ -301,14 +308,20 @@ class StepRunner:
         if graph is not None:
             try:
                 out = graph.run(entries)
-                self.graph_steps += 1
+                self._count(graph)
                 return out
             except TableTooWide:
                 pass
         # no graph for this many requests yet, or a request has outgrown the bucket's table
         widths = [_bucket(w + 1, 32) for w in self._widths_needed(entries)]
-        graph = DecodeGraph(self.model, self.cache, cap, widths)
+        graph = DecodeGraph(self.model, self.cache, cap, widths, captured=self.use_graphs)
         self._graphs[cap] = graph
         out = graph.run(entries)
-        self.graph_steps += 1
+        self._count(graph)
         return out
+
+    def _count(self, graph) -> None:
+        if graph.captured:
+            self.graph_steps += 1
+        else:
+            self.eager_steps += 1
