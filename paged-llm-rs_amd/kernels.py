@@ -525,6 +525,10 @@ def attention_step(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nkv
     return paged_attention(qkv, out, batch, kv, nq, nkv, d, scale, window)
 
 
+# Up to this many workgroups (requests times query heads) the tiled kernel takes a mixed step's short requests too.
+TILED_TAKES_SHORT_WORKGROUPS = 512
+
+
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nkv: int, d: int,
                     scale: float, window: int = 0) -> torch.Tensor:
     """Attention for every token of a step.  ``qkv`` rows begin with the rotated queries.
@@ -536,11 +540,15 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nk
                                      kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window)
     stride = qkv.shape[1]
     if batch.max_q_len >= SHORT_PORTION:
+        # A few short requests beside a long portion ride along in the tiled kernel, a token tile each: their
+        # workgroups run beside the portion's and finish sooner, which saves the other kernel's launch and
+        # its merge.  (Counted by requests, which a step's shape fixes; the tokens of short ones it does not.)
+        all_tiled = batch.short_tokens > 0 and batch.num_seqs * nq <= TILED_TAKES_SHORT_WORKGROUPS
         paged_attention_prefill(qkv, stride, out, batch.q_start, batch.q_len, batch.ctx_len, batch.max_q_len,
                                 kv.block_table, kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window,
-                                short_limit=SHORT_PORTION, max_ctx=batch.max_ctx_len,
+                                short_limit=0 if all_tiled else SHORT_PORTION, max_ctx=batch.max_ctx_len,
                                 live_seqs=getattr(batch, "live_seqs", None))
-        if batch.short_tokens == 0:
+        if batch.short_tokens == 0 or all_tiled:
             return out
     mixed = batch.max_q_len >= SHORT_PORTION
     if grouped_applies(nq, nkv, d, kv.block_size):

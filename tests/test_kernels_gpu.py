@@ -598,6 +598,38 @@ def test_grouped_attention_refuses_what_it_does_not_serve():
     assert kernels.grouped_applies(64, 8, 128, 16)
 
 
+@pytest.mark.parametrize("splits", [1, 4])
+@pytest.mark.parametrize("nq,nkv,d,bs,requests,window", PORTION_CASES)
+def test_the_tiled_kernel_takes_short_requests_too(nq, nkv, d, bs, requests, window, splits):
+    """With no lower limit the tiled kernel serves every request of the step, those of one token as well."""
+    from paged_llm_rs_amd import kernels
+
+    dtype = torch.bfloat16
+    requests = list(requests) + [(37, 1), (9, 3)]
+    ctx_lens = [c for c, _ in requests]
+    bt, k_pool, v_pool, keys, values = build_paged(nkv, d, bs, ctx_lens, dtype, seed=d + bs + len(requests))
+    n = sum(c for _, c in requests)
+    stride = (nq + 2 * nkv) * d
+    q = torch.randn(n, stride, device=DEV).to(dtype)
+    q_start, q_len, positions, seq_of = [], [], [], []
+    for s, (ctx, count) in enumerate(requests):
+        q_start.append(len(positions))
+        q_len.append(count)
+        positions += list(range(ctx - count, ctx))
+        seq_of += [s] * count
+    as_i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    scale = 1 / math.sqrt(d)
+    out = torch.full((n, nq * d), 7.0, dtype=dtype, device=DEV)
+    kernels.paged_attention_prefill(q, stride, out, as_i32(q_start), as_i32(q_len), as_i32(ctx_lens), max(q_len), bt, bs,
+                                    k_pool, v_pool, nq, nkv, d, scale, window, short_limit=0, splits=splits)
+    g = nq // nkv
+    for i in range(n):
+        s, p = seq_of[i], positions[i]
+        want = attention_ref(q[i, :nq * d].double().cpu().reshape(nq, d), keys[s], values[s], p, g, scale, window)
+        err = rel(out[i].reshape(nq, d), want)
+        assert err < 1e-2, f"token {i} (request {s}, position {p}): {err:.3e}"
+
+
 def test_a_far_key_is_found_from_inside_a_portion():
     """One key carries nearly all the weight of one query in the middle of a long portion: a key of an
     earlier step across a page edge, a key of the same step, the query's own key, and keys at a window's edge."""

@@ -489,7 +489,7 @@ def test_layers_with_a_window_beside_layers_without(tmp_path, dtype):
     from paged_llm_rs_amd.engine.replay import Replayer
 
     register_architecture("WindowedToyForCausalLM", WindowedConfig, model_type="windowed_toy")
-    folder = write_random_model(tmp_path / "windowed", WINDOWED, seed=12, std=0.12, gain_std=0.2, dtype=dtype)
+    folder = write_random_model(tmp_path / "windowed", WINDOWED, seed=12, std=0.08, gain_std=0.2, dtype=dtype)
     weights = load_file(str(folder / "model.safetensors"))
     prompts = ru.make_prompts(WINDOWED["vocab_size"], [90, 23, 141, 60], seed=6)
     want = {name: windowed_plain(weights, toks) for name, toks in prompts.items()}
