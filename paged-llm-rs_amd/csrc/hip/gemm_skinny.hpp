@@ -115,9 +115,11 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
     const float* xf = static_cast<const float*>(x_);
     size_t xrow[MT];
     bool row_ok[MT];
+    // (blockIdx.y: with few tiles of columns the rows are dealt to workgroups too, 16 * MT to each)
+    const int row0 = blockIdx.y * 16 * MT;
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
-        const int row = m * 16 + c;
+        const int row = row0 + m * 16 + c;
         row_ok[m] = row < n;
         int src = row_ok[m] ? row : 0;
         if (PRO == PRO_NORM && rows) src = rows[src];
@@ -316,7 +318,7 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
         const int col = n0 + src_lane % 16;
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
-            const int row = m * 16 + row_in_tile;
+            const int row = row0 + m * 16 + row_in_tile;
             float v[BT];
 #pragma unroll
             for (int b = 0; b < BT; ++b) {
@@ -350,10 +352,13 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
 // More column tiles than this many workgroups are walked in a loop, which keeps a wave's rows of x
 // in its registers from tile to tile: eight workgroups a compute unit are as many as stay resident.
 #define SK_MAX_GRID 2048
+// Up to this many workgroups (column tiles times row tiles) a product of 17 to 64 rows is dealt out by row tiles too.
+#define SK_ROW_TILES_GRID 512
 
 template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT>
 static int launch_one(int waves, const void* x, const void* w, void* y, const float* gain, float eps,
                       const int* rows, int n, int N_out, int K, hipStream_t stream) {
+    const int row_tiles = pl_ceil_div(n, 16 * MT);   // more than one where launch_mt deals the rows out
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
     constexpr int UA = (WV == 16 && UNR >= 2) ? UNR / 2 : UNR;   // K steps a round when rounds overlap
     const int grid = min(pl_ceil_div(N_out, SK_TILE_N), SK_MAX_GRID);
@@ -370,10 +375,10 @@ static int launch_one(int waves, const void* x, const void* w, void* y, const fl
     // a time (of half the steps each where sixteen waves leave a lane 128 registers).
     const bool several = pl_ceil_div(pl_ceil_div(K, SK_KSTEP), waves) > UNR;
     if (several)
-        gemm_skinny_kernel<MT, UA, WV, PRO, EPI, OUT, false, true><<<grid, 64 * waves, lds_bytes, stream>>>(
+        gemm_skinny_kernel<MT, UA, WV, PRO, EPI, OUT, false, true><<<dim3(grid, row_tiles), 64 * waves, lds_bytes, stream>>>(
             x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps, rows, n, N_out, K);
     else
-        gemm_skinny_kernel<MT, UNR, WV, PRO, EPI, OUT><<<grid, 64 * waves, lds_bytes, stream>>>(
+        gemm_skinny_kernel<MT, UNR, WV, PRO, EPI, OUT><<<dim3(grid, row_tiles), 64 * waves, lds_bytes, stream>>>(
             x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps, rows, n, N_out, K);
     PL_CHECK_LAUNCH("gemm_skinny");
     return 0;
@@ -646,6 +651,12 @@ static int launch_unr(const void* x, const void* w, void* y, const float* gain, 
 template <int PRO, int EPI, typename OUT>
 static int launch_mt(const void* x, const void* w, void* y, const float* gain, float eps,
                      const int* rows, int n, int N_out, int K, hipStream_t stream) {
+    // Few tiles of columns (a narrow output, as of the projections back into the stream): the tiles of 16 rows
+    // go to workgroups of their own, the kernel for up to 16 rows on a grid of (column tiles, row tiles), so that
+    // the launch has workgroups for every compute unit; each reads its rows of x only, and w comes from L2
+    // from the second row tile on.
+    if (n > 16 && pl_ceil_div(N_out, SK_TILE_N) * pl_ceil_div(n, 16) <= SK_ROW_TILES_GRID)
+        return launch_unr<1, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, stream);
     switch (pl_ceil_div(n, 16)) {
         case 1: return launch_unr<1, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, stream);
         case 2: return launch_unr<2, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, stream);
