@@ -543,7 +543,8 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nk
         # A few short requests beside a long portion ride along in the tiled kernel, a token tile each: their
         # workgroups run beside the portion's and finish sooner, which saves the other kernel's launch and
         # its merge.  (Counted by requests, which a step's shape fixes; the tokens of short ones it does not.)
-        all_tiled = batch.short_tokens > 0 and batch.num_seqs * nq <= TILED_TAKES_SHORT_WORKGROUPS
+        all_tiled = (batch.short_tokens > 0 and batch.num_seqs * nq <= TILED_TAKES_SHORT_WORKGROUPS
+                     and not grouped_applies(nq, nkv, d, kv.block_size))   # (grouped, a token reads its keys once for all its heads)
         paged_attention_prefill(qkv, stride, out, batch.q_start, batch.q_len, batch.ctx_len, batch.max_q_len,
                                 kv.block_table, kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window,
                                 short_limit=0 if all_tiled else SHORT_PORTION, max_ctx=batch.max_ctx_len,
