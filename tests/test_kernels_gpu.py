@@ -297,6 +297,39 @@ def test_gemm_tiled_refusals():
         kernels.gemm_tiled(x, torch.zeros(128, 40, device=DEV, dtype=torch.bfloat16))
 
 
+@pytest.mark.parametrize("M,N,K,out_dtype", [(576, 6144, 4096, None), (2048, 24576, 4096, None), (2048, 4096, 12288, None),
+                                             (40, 151936, 1024, torch.float32), (300, 3001, 2560, torch.float32)])
+def test_library_products_in_a_captured_graph_replay_like_the_eager_ones(M, N, K, out_dtype):
+    """The library's products stand inside captured steps (large weights, many rows, the projection onto the
+    vocabulary).  Some of its kernels clear a workspace first, and a clearing node in a graph is what has
+    given wrong replays on this chip: every replay, with eager work and a synchronisation between, has to
+    give the bits of the eager product."""
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).bfloat16()
+    x = torch.randn(M, K, device=DEV).bfloat16()
+    other = torch.randn(512, 512, device=DEV)
+
+    def product():
+        return torch.mm(x, w.t()) if out_dtype is None else torch.mm(x, w.t(), out_dtype=out_dtype)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        product()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = product()
+    for replay in range(4):
+        x.copy_(torch.randn(M, K, device=DEV).bfloat16())
+        float((other @ other).sum())
+        want = product().clone()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want), f"replay {replay} differs from the eager product"
+
+
 def test_gemm_skinny_refusals():
     from paged_llm_rs_amd import kernels
     from paged_llm_rs_amd.errors import TensorError
