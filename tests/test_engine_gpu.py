@@ -189,15 +189,16 @@ def test_a_captured_decode_step_replays_like_the_eager_one(model_dirs, dtype):
         assert np.array_equal(a[key], b[key]), f"{key}: a replay differs from the eager step"
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_a_shape_of_step_that_comes_again_is_captured_and_replays_like_the_eager_one(model_dirs, dtype):
+@pytest.mark.parametrize("name,dtype,block_size", [("B", "float32", 8), ("B", "bfloat16", 8), ("E", "bfloat16", 16)])
+def test_a_shape_of_step_that_comes_again_is_captured_and_replays_like_the_eager_one(model_dirs, name, dtype, block_size):
     """A long prompt cut into equal portions beside a request that decodes: from its second coming on a
     shape of step is replayed from a graph.  Every replay is checked against the eager step, over
-    growing contexts (the tables outgrow the capture once) and with other shapes in between."""
+    growing contexts (the tables outgrow the capture once) and with other shapes in between.  (The wide
+    model's captured steps hold the library's products and the grouped attention kernel.)"""
     from paged_llm_rs_amd.engine.replay import Replayer
 
-    d = model_dirs("B", dtype)
-    prompts = ru.make_prompts(384, [300, 60, 23], seed=33)
+    d = model_dirs(name, dtype)
+    prompts = ru.make_prompts(TINY_INIT[name]["config"]["vocab_size"], [300, 60, 23], seed=33)
     long_one, other, third = prompts["r0"], prompts["r1"], prompts["r2"]
     steps, k = [], 0
     steps.append({"step": k, "entries": [{"id": "r1", "tokens": other[:20], "want": [19]}], "end": []})
@@ -215,8 +216,8 @@ def test_a_shape_of_step_that_comes_again_is_captured_and_replays_like_the_eager
             steps.append({"step": k, "entries": [{"id": "r2", "tokens": third, "want": [len(third) - 1]}], "end": ["r2"]})
             k += 1
     steps.append({"step": k, "entries": [{"id": "r0", "tokens": long_one[294:], "want": [5]}], "end": ["r0", "r1"]})
-    eager = Replayer(d, dtype, max_tokens=64 * 8, block_size=8, graphs=False)
-    graph = Replayer(d, dtype, max_tokens=64 * 8, block_size=8, graphs=True)
+    eager = Replayer(d, dtype, max_tokens=64 * 8, block_size=block_size, graphs=False)
+    graph = Replayer(d, dtype, max_tokens=64 * 8, block_size=block_size, graphs=True)
     a = ru.collect(eager, steps)
     b = ru.collect(graph, steps)
     assert graph.runner.graph_steps >= 10 and eager.runner.graph_steps == 0
