@@ -799,3 +799,36 @@ def test_long_portions_over_earlier_context(model_dirs, name, dtype, block_size)
     r = Replayer(d, dtype, max_tokens=ru.pool_tokens(prompts, 2), block_size=block_size)
     worst, where = ru.worst_error(ru.collect(r, steps), want)
     assert worst <= (1e-5 if dtype == "float32" else 2e-2), f"{worst:.3e} at {where}"
+
+
+def test_a_context_of_thousands_of_tokens_in_portions_and_decoded(model_dirs):
+    """The 0.6B layer sizes over 2,600 tokens in bfloat16: portions of 512 whose keys are dealt to several
+    workgroups a token tile, block tables that outgrow their first width, then single tokens whose keys are
+    cut into many shares, beside a second request that decodes all along."""
+    from paged_llm_rs_amd.engine.replay import Replayer
+
+    d = model_dirs("D", "bfloat16")
+    prompts = ru.make_prompts(TINY_INIT["D"]["config"]["vocab_size"], [2600, 90], seed=41)
+    want = ru.plain_logits(d, prompts)
+    long, short = prompts["r0"], prompts["r1"]
+    steps = [{"step": 0, "entries": [{"id": "r1", "tokens": short[:40], "want": [39]}], "end": []}]
+    fed, at = 40, 0
+    while at < 2560:
+        entries = [{"id": "r0", "tokens": long[at:at + 512], "want": [0, 511]}]
+        if fed < len(short):
+            entries.append({"id": "r1", "tokens": [short[fed]], "want": [0]})
+            fed += 1
+        steps.append({"step": len(steps), "entries": entries, "end": []})
+        at += 512
+    for i in range(2560, 2600):
+        entries = [{"id": "r0", "tokens": [long[i]], "want": [0]}]
+        if fed < len(short):
+            entries.append({"id": "r1", "tokens": [short[fed]], "want": [0]})
+            fed += 1
+        steps.append({"step": len(steps), "entries": entries, "end": ["r0"] if i == 2599 else []})
+    steps.append({"step": len(steps), "entries": [{"id": "r1", "tokens": short[fed:], "want": [0]}], "end": ["r1"]})
+    r = Replayer(d, "bfloat16", max_tokens=ru.pool_tokens(prompts, 2), block_size=16)
+    got = ru.collect(r, steps)
+    assert len(got) >= 2 * 5 + 40 + 40
+    worst, where = ru.worst_error(got, want)
+    assert worst <= 2e-2, f"{worst:.3e} at {where}"
