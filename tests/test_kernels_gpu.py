@@ -48,7 +48,7 @@ def test_embed(dtype, V, H):
 # --- residual add + norm -----------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("n,H", [(1, 24), (7, 100), (33, 1024), (5, 5120), (3, 33), (2, 9000), (4, 4096), (2, 8192), (3, 2050)])
+@pytest.mark.parametrize("n,H", [(1, 24), (7, 100), (33, 1024), (5, 5120), (3, 33), (2, 9000), (4, 4096), (2, 8192), (3, 2050), (300, 1024), (257, 100), (513, 4096), (260, 5120)])
 def test_add_rmsnorm(dtype, n, H):
     from paged_llm_rs_amd import kernels
 
