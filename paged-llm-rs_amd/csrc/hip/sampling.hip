@@ -102,6 +102,7 @@ extern "C" int pl_argmax(const float* logits, int* out, float* scratch_v, int* s
 #define SM_THREADS 1024
 #define SM_BINS 4096
 #define SM_NO_LIMIT 0x7fffffff
+#define SM_LIST 256                    // the most candidates that top-k may keep for the short way (see sm_few)
 
 struct sm_shared {
     unsigned long long sum[SM_BINS];   // mass, or count, a bin
@@ -114,6 +115,14 @@ struct sm_shared {
     unsigned long long found_in;       // sum of the bin found
     int found_bin;
     int nth_index;
+    // the short way after top-k: the candidates kept, as they are found and in order
+    uint32_t list_key[SM_LIST];
+    int list_idx[SM_LIST];
+    unsigned long long list_mass[SM_LIST];
+    int list_order[SM_LIST];           // list_order[r]: which entry stands at place r of the order (key, then index)
+    uint32_t maybe_key[SM_LIST];       // the candidates of the bin in which the k-th stands
+    int maybe_idx[SM_LIST];
+    int list_n, maybe_n;
 };
 
 __device__ __forceinline__ uint32_t sm_key(float y, float top) {
@@ -127,6 +136,22 @@ __device__ __forceinline__ unsigned long long sm_mass(float y, float top) {
     // 2^40 * exp(y - top): zero from about 28 below the maximum on
     const float p = __builtin_amdgcn_exp2f((y - top) * 1.4426950408889634f + 40.f);
     return (y == y) ? static_cast<unsigned long long>(p) : 0ull;
+}
+
+// f(value, index) for every element of a row that falls to this thread, in rising order.  Eight loads are asked
+// for before the first is used: a pass over a row is one workgroup's and lives on what it has in flight.
+template <class F>
+__device__ __forceinline__ void sm_each(const float* __restrict__ x, int V, F&& f) {
+    constexpr int AHEAD = 8;
+    int i = threadIdx.x;
+    for (; i + (AHEAD - 1) * SM_THREADS < V; i += AHEAD * SM_THREADS) {
+        float v[AHEAD];
+#pragma unroll
+        for (int j = 0; j < AHEAD; ++j) v[j] = x[i + j * SM_THREADS];
+#pragma unroll
+        for (int j = 0; j < AHEAD; ++j) f(v[j], i + j * SM_THREADS);
+    }
+    for (; i < V; i += SM_THREADS) f(x[i], i);
 }
 
 // The mark that is `fraction` of `total`, at least one and at most all of it.
@@ -217,17 +242,17 @@ __device__ uint32_t sm_select(sm_shared& sm, const float* __restrict__ x, int V,
         __syncthreads();
     };
     clear();
-    for (int i = tid; i < V; i += SM_THREADS) {
-        const float y = x[i] * inverse;
+    sm_each(x, V, [&](float v, int i) {
+        const float y = v * inverse;
         const uint32_t k = sm_key(y, top);
-        if (!kept.has(k, i)) continue;
+        if (!kept.has(k, i)) return;
         const unsigned long long w = WEIGHTED ? sm_mass(y, top) : 1ull;
         if (w) {
             atomicAdd(&sm.sum[k >> 12], w);
             atomicAdd(&sm.count[k >> 12], 1u);
             atomicMin(&sm.first[k >> 12], i);
         }
-    }
+    });
     __syncthreads();
     mark = sm_find(sm, 0, mark, fraction);
     const uint32_t upper = sm.found_bin;
@@ -241,17 +266,17 @@ __device__ uint32_t sm_select(sm_shared& sm, const float* __restrict__ x, int V,
     } else {
         const unsigned long long before_upper = before;
         clear();
-        for (int i = tid; i < V; i += SM_THREADS) {
-            const float y = x[i] * inverse;
+        sm_each(x, V, [&](float v, int i) {
+            const float y = v * inverse;
             const uint32_t k = sm_key(y, top);
-            if ((k >> 12) != upper || !kept.has(k, i)) continue;
+            if ((k >> 12) != upper || !kept.has(k, i)) return;
             const unsigned long long w = WEIGHTED ? sm_mass(y, top) : 1ull;
             if (w) {
                 atomicAdd(&sm.sum[k & 0xfff], w);
                 atomicAdd(&sm.count[k & 0xfff], 1u);
                 atomicMin(&sm.first[k & 0xfff], i);
             }
-        }
+        });
         __syncthreads();
         sm_find(sm, before_upper, mark, -1.0);
         key = (upper << 12) | static_cast<uint32_t>(sm.found_bin);
@@ -267,12 +292,49 @@ __device__ uint32_t sm_select(sm_shared& sm, const float* __restrict__ x, int V,
         token = many == 1 ? lowest : 0;
         return key;
     }
-    // Several candidates share the key: they are walked in the order of their indices, a stretch of
-    // SM_THREADS indices at a time, until the running sum reaches the mark.
+    // Several candidates share the key.  A few of them are gathered in one pass and one thread walks them
+    // in the order of their indices; more than SM_LIST are walked where they lie, a stretch of SM_THREADS
+    // indices at a time, until the running sum reaches the mark.
     unsigned long long run = before;
-    if (tid == 0) sm.nth_index = -1;
+    if (tid == 0) {
+        sm.nth_index = -1;
+        sm.maybe_n = 0;
+    }
     __syncthreads();
     const int lane = tid % PL_WAVE, wave = tid / PL_WAVE;
+    if (many <= SM_LIST) {
+        sm_each(x, V, [&](float v, int i) {
+            const float y = v * inverse;
+            const uint32_t k = sm_key(y, top);
+            if (k != key || !kept.has(k, i)) return;
+            const unsigned long long w = WEIGHTED ? sm_mass(y, top) : 1ull;
+            if (w) {
+                const int at = atomicAdd(&sm.maybe_n, 1);
+                sm.maybe_idx[at] = i;
+                sm.list_mass[at] = w;
+            }
+        });
+        __syncthreads();
+        const int n = sm.maybe_n;                               // == many: the same candidates were counted
+        if (tid < n) {
+            int place = 0;
+            for (int j = 0; j < n; ++j) place += sm.maybe_idx[j] < sm.maybe_idx[tid] ? 1 : 0;
+            sm.list_order[place] = tid;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            for (int r = 0; r < n; ++r) {
+                const int e = sm.list_order[r];
+                run += sm.list_mass[e];
+                if (run >= mark) {
+                    sm.nth_index = sm.maybe_idx[e];
+                    sm.found_before = run;
+                    break;
+                }
+            }
+        }
+        __syncthreads();
+    } else
     for (int base = 0; base < V; base += SM_THREADS) {
         const int i = base + tid;
         unsigned long long w = 0;
@@ -317,6 +379,98 @@ __device__ uint32_t sm_select(sm_shared& sm, const float* __restrict__ x, int V,
     return key;
 }
 
+// Top-k with few candidates kept (k <= SM_LIST), and everything after it: one pass finds the bin of the upper
+// 12 key bits in which the k-th candidate stands, a second gathers the candidates of the bins before it (kept for
+// certain) and those of that bin, of which the first k - (kept so far) in the order (key, index) are kept too.
+// The k candidates are then ordered and one thread walks them: the mass up to top_p of the total, and in what
+// is left the drawn point.  Three passes over the row with the one for the maximum, where the general way
+// takes five to seven.  Returns false (the same in every thread, nothing decided) when the k-th candidate's
+// bin holds more than SM_LIST candidates: the general way then serves the row.
+__device__ bool sm_few(sm_shared& sm, const float* __restrict__ x, int V, float inverse, float top, int k, float p,
+                       float u, int& token) {
+    const int tid = threadIdx.x;
+    for (int b = tid; b < SM_BINS; b += SM_THREADS) sm.sum[b] = 0;
+    if (tid == 0) sm.list_n = sm.maybe_n = 0;
+    __syncthreads();
+    sm_each(x, V, [&](float v, int) { atomicAdd(&sm.sum[sm_key(v * inverse, top) >> 12], 1ull); });
+    __syncthreads();
+    sm_find(sm, 0, static_cast<unsigned long long>(k), -1.0);
+    const uint32_t upper = sm.found_bin;
+    const int sure = static_cast<int>(sm.found_before), in_bin = static_cast<int>(sm.found_in);
+    __syncthreads();
+    if (in_bin > SM_LIST) return false;
+    sm_each(x, V, [&](float v, int i) {
+        const uint32_t key = sm_key(v * inverse, top);
+        if ((key >> 12) < upper) {
+            const int at = atomicAdd(&sm.list_n, 1);
+            sm.list_key[at] = key;
+            sm.list_idx[at] = i;
+        } else if ((key >> 12) == upper) {
+            const int at = atomicAdd(&sm.maybe_n, 1);
+            sm.maybe_key[at] = key;
+            sm.maybe_idx[at] = i;
+        }
+    });
+    __syncthreads();
+    // of the k-th candidate's bin, the first k - sure in the order
+    if (tid < in_bin) {
+        const uint32_t key = sm.maybe_key[tid];
+        const int idx = sm.maybe_idx[tid];
+        int before = 0;
+        for (int j = 0; j < in_bin; ++j)
+            before += (sm.maybe_key[j] < key || (sm.maybe_key[j] == key && sm.maybe_idx[j] < idx)) ? 1 : 0;
+        if (before < k - sure) {
+            sm.list_key[sure + before] = key;
+            sm.list_idx[sure + before] = idx;
+        }
+    }
+    __syncthreads();
+    // masses, and the place of every kept candidate in the order
+    if (tid < k) {
+        const uint32_t key = sm.list_key[tid];
+        const int idx = sm.list_idx[tid];
+        sm.list_mass[tid] = sm_mass(x[idx] * inverse, top);
+        int before = 0;
+        for (int j = 0; j < k; ++j)
+            before += (sm.list_key[j] < key || (sm.list_key[j] == key && sm.list_idx[j] < idx)) ? 1 : 0;
+        sm.list_order[before] = tid;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        unsigned long long total = 0;
+        for (int r = 0; r < k; ++r) total += sm.list_mass[sm.list_order[r]];
+        int last = k - 1;                                       // the last candidate that top_p keeps
+        if (p < 1.f) {
+            const unsigned long long mark = sm_mark_of(static_cast<double>(p), total);
+            unsigned long long run = 0;
+            for (int r = 0; r < k; ++r) {
+                run += sm.list_mass[sm.list_order[r]];
+                if (run >= mark) {
+                    last = r;
+                    break;
+                }
+            }
+            total = run;
+        }
+        const unsigned long long mark = sm_mark_of(static_cast<double>(u), total);
+        unsigned long long run = 0;
+        int chosen = sm.list_order[0];
+        for (int r = 0; r <= last; ++r) {
+            const int e = sm.list_order[r];
+            run += sm.list_mass[e];
+            if (sm.list_mass[e] && run >= mark) {
+                chosen = e;
+                break;
+            }
+        }
+        sm.nth_index = sm.list_idx[chosen];
+    }
+    __syncthreads();
+    token = sm.nth_index;
+    __syncthreads();
+    return true;
+}
+
 __global__ void __launch_bounds__(SM_THREADS)
 sample_rows_kernel(const float* __restrict__ logits, const float* __restrict__ temperature, const int* __restrict__ top_k,
                    const float* __restrict__ top_p, const float* __restrict__ uniform, int* __restrict__ out, int V) {
@@ -327,7 +481,7 @@ sample_rows_kernel(const float* __restrict__ logits, const float* __restrict__ t
     // the largest logit and its first index
     float bv = -INFINITY;
     int bi = SM_NO_LIMIT;
-    for (int i = tid; i < V; i += SM_THREADS) better(bv, bi, x[i], i);
+    sm_each(x, V, [&](float v, int i) { better(bv, bi, v, i); });
 #pragma unroll
     for (int off = PL_WAVE / 2; off > 0; off >>= 1) {
         const float ov = __shfl_xor(bv, off, PL_WAVE);
@@ -354,6 +508,10 @@ sample_rows_kernel(const float* __restrict__ logits, const float* __restrict__ t
     int limit, token;
     unsigned long long through;
     const int k = top_k[row];
+    if (k > 0 && k < V && k <= SM_LIST && sm_few(sm, x, V, inverse, top, k, top_p[row], uniform[row], token)) {
+        if (tid == 0) out[row] = token;
+        return;
+    }
     if (k > 0 && k < V) {
         const uint32_t key = sm_select<false>(sm, x, V, inverse, top, kept, static_cast<unsigned long long>(k), -1.0, limit, through, token);
         kept = sm_kept{key, limit};

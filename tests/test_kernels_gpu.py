@@ -782,6 +782,47 @@ def test_sampling_kernel_follows_the_recipe():
     assert same_as_host >= drawn - 1, f"{same_as_host} of {drawn} tokens are the host sampler's"
 
 
+def test_sampling_kernel_with_few_candidates_kept():
+    """top_k up to 256 takes a way of its own (the kept candidates are gathered and walked by one thread);
+    above it, or when more than 256 candidates stand in the k-th one's bin, the general way.  Logits rounded
+    to bfloat16 make equal values, so that the index decides who is kept."""
+    import numpy as np
+    from paged_llm_rs_amd import kernels
+
+    g = torch.Generator().manual_seed(23)
+    V = 151936
+    cases = [(1.0, 1, 1.0), (0.6, 20, 0.95), (0.6, 20, 1.0), (1.0, 255, 0.8), (1.0, 256, 0.8), (1.0, 257, 0.8),
+             (3.0, 64, 0.99), (0.3, 100, 0.5)]
+    rows, how = [], []
+    for rep in range(4):
+        for t, k, p in cases:
+            x = torch.randn(V, generator=g) * (1.0 + rep)
+            if rep % 2:
+                x = x.bfloat16().float()
+            rows.append(x)
+            how.append((t, k, p, float(torch.rand((), generator=g))))
+    logits = torch.stack(rows).to(DEV)
+    as_f = lambda col: torch.tensor([h[col] for h in how], dtype=torch.float32, device=DEV)
+    got = kernels.sample(logits, as_f(0), torch.tensor([h[1] for h in how], dtype=torch.int32, device=DEV), as_f(2),
+                         as_f(3)).cpu().tolist()
+    for row, (t, k, p, u) in enumerate(how):
+        allowed, kept = sampling_recipe(logits[row].cpu().numpy(), t, k, p, u)
+        assert got[row] in kept, f"row {row} {how[row]}: token {got[row]} had been cut"
+        assert got[row] in allowed, f"row {row} {how[row]}: token {got[row]}, the recipe allows {sorted(allowed)}"
+    # equal logits: the lowest indices are kept, whether the k-th one's bin holds few candidates or many
+    few, many = torch.zeros(200), torch.zeros(5000)
+    few[150:] = -3.0
+    hand = [(few, 10, 1.0, 0.55, 5), (few, 10, 0.5, 0.99, 4), (few, 160, 1.0, 0.99, 148), (few, 160, 1.0, 0.9995, 158),
+            (few, 1, 1.0, 0.99, 0), (many[:200], 10, 1.0, 0.95, 9), (many[:200], 256, 1.0, 0.5025, 100)]
+    for x, k, p, u, want in hand:
+        one = kernels.sample(x[None].to(DEV), torch.ones(1, device=DEV), torch.tensor([k], dtype=torch.int32, device=DEV),
+                             torch.tensor([p], device=DEV), torch.tensor([u], device=DEV)).item()
+        assert one == want, (k, p, u, one, want)
+    wide = kernels.sample(many[None].to(DEV), torch.ones(1, device=DEV), torch.tensor([10], dtype=torch.int32, device=DEV),
+                          torch.ones(1, device=DEV), torch.tensor([0.95], device=DEV)).item()
+    assert wide == 9
+
+
 def test_sampling_kernel_on_rows_made_by_hand():
     from paged_llm_rs_amd import kernels
 
