@@ -16,17 +16,23 @@ from .step import StepRunner, commit_step, require_gpu
 
 
 class Replayer:
+    LIVE_AT_MOST = 4        # requests that a trace holds at a time
+
     def __init__(self, model_dir, dtype: str, max_tokens: int, block_size: int = 16, device="cuda:0",
                  max_live: int = 64, graphs: bool = True):
         device = require_gpu(device)
         self.config, self.model = load_model(model_dir, dtype, device)
         if max_tokens < 1:
             raise ConfigError(f"--max-tokens {max_tokens}")
-        # Each live request's tokens are counted rounded up to 64, so a pool of
-        # max_tokens/block_size pages holds them whatever the page size (a divisor of 64).
+        # Each live request's tokens are counted rounded up to 64, so a pool of max_tokens/block_size pages
+        # holds them when the page size divides 64.  With any other page size a request's last page may
+        # reach past its multiple of 64: one page more for each of the requests that a trace may hold.
         tokens = (max_tokens + 63) // 64 * 64
-        self.cache = PagedCache(self.model.cache_layout, block_size, max(tokens // block_size, 1),
-                                DTYPES[dtype], device, max_seqs=max_live)
+        pages = -(-tokens // block_size)
+        if 64 % block_size:
+            pages += self.LIVE_AT_MOST
+        self.cache = PagedCache(self.model.cache_layout, block_size, max(pages, 1), DTYPES[dtype], device,
+                                max_seqs=max_live)
         self.runner = StepRunner(self.model, self.cache, graphs=graphs)
         self.ids: dict = {}
         self.next_id = 1

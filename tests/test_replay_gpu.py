@@ -133,3 +133,45 @@ def test_trace_run_program(setups, tmp_path):
             fed[e["id"]] = start + len(e["tokens"])
     worst, where = ru.worst_error(got, want)
     assert worst <= TOLERANCE["float32"], f"{worst:.3e} at {where}"
+
+
+def drawn_configuration(case: int):
+    """A configuration, a page size and four prompt lengths drawn from the sizes kernels have to take: heads
+    of every multiple of 16, groups of one to sixteen, widths and vocabularies that are no multiple of eight."""
+    import random
+
+    rng = random.Random(case)
+    d = rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 144, 160, 192, 256])
+    nkv = rng.choice([1, 2, 3, 5, 8])
+    group = min(rng.choice([1, 2, 3, 4, 7, 8, 16]), max(1, 4096 // (nkv * d)))
+    config = {
+        "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "hidden_act": "silu", "attention_bias": False,
+        "hidden_size": rng.choice([64, 72, 100, 136, 200, 520, 1000, 2056, 2304]),
+        "intermediate_size": rng.choice([96, 130, 212, 500, 1030, 2500]),
+        "num_hidden_layers": rng.choice([1, 2, 3]), "num_attention_heads": nkv * group, "num_key_value_heads": nkv,
+        "head_dim": d, "rms_norm_eps": rng.choice([1e-6, 1e-5, 3e-4]), "rope_theta": rng.choice([10000.0, 1e6]),
+        "vocab_size": rng.choice([97, 256, 331, 1001, 5003]), "max_position_embeddings": 4096,
+        "tie_word_embeddings": rng.choice([True, False]),
+    }
+    block_size = rng.choice([1, 2, 4, 8, 16, 32, 64, 128, 24, 3])
+    lengths = [rng.randint(1, 40), rng.randint(300, 900) if case % 3 == 0 else rng.randint(30, 140), rng.randint(60, 300),
+               rng.randint(2, 90)]
+    return config, block_size, lengths
+
+
+@pytest.mark.parametrize("case", range(12))
+def test_drawn_configurations_mixed_and_decoded(tmp_path, case):
+    """Sizes that no other test has: every one is served right, in 32-bit and in bfloat16, or refused."""
+    from paged_llm_rs_amd.weights import write_random_model
+
+    config, block_size, lengths = drawn_configuration(case)
+    prompts = ru.make_prompts(config["vocab_size"], lengths, seed=case)
+    for dtype in ("float32", "bfloat16"):
+        folder = tmp_path / dtype
+        write_random_model(folder, config, seed=case, std=0.05 if config["hidden_size"] <= 200 else 0.02, gain_std=0.1,
+                           dtype=dtype)
+        want = ru.plain_logits(folder, prompts)
+        for steps, live in ((ru.mixed(prompts, seed=case, max_live=4), 4), (ru.tail_decoded(prompts, 32), 1)):
+            got = replay(folder, dtype, prompts, steps, max_live=live, block_size=block_size)
+            worst, where = ru.worst_error(got, want)
+            assert worst <= TOLERANCE[dtype], f"{config} pages of {block_size}, {dtype}: {worst:.3e} at {where}"
