@@ -77,6 +77,25 @@ def _bucket(n: int, least: int = 1) -> int:
     return b
 
 
+class _Sent:
+    """Guards a pinned descriptor that is copied to the device without waiting: the copy of one step has to
+    have left the buffer before the next step is written into it.  A caller that reads every step's result
+    has waited already; one that does not (a portion in the middle of a prompt gives nothing to read) would
+    overwrite a descriptor that the device has not yet fetched."""
+
+    def __init__(self):
+        self.event = None
+
+    def mark(self) -> None:
+        if self.event is None:
+            self.event = torch.cuda.Event()
+        self.event.record()
+
+    def wait(self) -> None:
+        if self.event is not None:
+            self.event.synchronize()
+
+
 class DecodeGraph:
     """One decode step for up to ``cap`` requests with up to ``widths[g]`` pages each, captured; or, with
     ``captured=False``, launched kernel by kernel over the same buffers with the same idle rows, so that a
@@ -109,6 +128,7 @@ class DecodeGraph:
         self.graph = None
         self.logits = None
         self.tokens = None
+        self.sent = _Sent()
 
     def _view(self, name):
         b, c = self.layout[name]
@@ -164,14 +184,17 @@ class DecodeGraph:
 
     def run(self, entries) -> StepOutput:
         live = len(entries)
+        self.sent.wait()
         self.fill(entries)
         if not self.captured:
             self.device_buf.copy_(self.host, non_blocking=True)
+            self.sent.mark()
             logits, tokens = self._forward()
             return StepOutput(logits[:live], tokens[:live])
         if self.graph is None:
             self.capture()
         self.device_buf.copy_(self.host, non_blocking=True)
+        self.sent.mark()
         self.graph.replay()
         return StepOutput(self.logits[:live], self.tokens[:live])
 
@@ -194,6 +217,7 @@ class ShapeGraph:
         self.batch.live_seqs = first.live_seqs
         self.graph = None
         self.logits = None
+        self.sent = _Sent()
 
     def _lay_out(self, entries):
         return build_batch(entries, self.cache.manager, len(self.cache.layout.groups), self.model.spec.vocab_size,
@@ -218,10 +242,12 @@ class ShapeGraph:
             batch = self._lay_out(entries)
             if batch.packed.numel() != self.size:
                 raise ConfigError("a step of another shape than the captured one")
+            self.sent.wait()
             self.host.copy_(batch.packed)
         else:
             self.capture()
         self.device_buf.copy_(self.host, non_blocking=True)
+        self.sent.mark()
         self.graph.replay()
         return StepOutput(self.logits)
 

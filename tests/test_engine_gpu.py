@@ -226,4 +226,76 @@ def test_a_shape_of_step_that_comes_again_is_captured_and_replays_like_the_eager
         assert np.array_equal(a[key], b[key]), f"{key}: a replay differs from the eager step"
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_portions_that_return_nothing_replay_like_eager_ones(model_dirs, dtype):
+    """Equal portions in the middle of a prompt give nothing to read, so nothing makes the host wait for
+    the device between them: each replay still has to run on its own step's descriptor, not on the next
+    one's, which the host is already writing."""
+    from paged_llm_rs_amd.engine.replay import Replayer
+
+    d = model_dirs("C", dtype)
+    prompt = ru.make_prompts(TINY_INIT["C"]["config"]["vocab_size"], [150], seed=41)["r0"]
+    results = {}
+    for portion in (7, 2):
+        steps = []
+        for k, at in enumerate(range(0, len(prompt), portion)):
+            tokens = prompt[at:at + portion]
+            last = at + portion >= len(prompt)
+            steps.append({"step": k, "entries": [{"id": "r0", "tokens": tokens, "want": [len(tokens) - 1] if last else []}],
+                          "end": ["r0"] if last else []})
+        for graphs in (False, True):
+            r = Replayer(d, dtype, max_tokens=256, block_size=4, graphs=graphs)
+            results[(portion, graphs)] = ru.collect(r, steps)
+            if graphs:
+                assert r.runner.graph_steps >= 10
+        a, b = results[(portion, False)], results[(portion, True)]
+        assert a.keys() == b.keys() and len(a) == 1
+        for key in a:
+            assert np.array_equal(a[key], b[key]), f"portions of {portion}: a replay differs from the eager step"
+
+
+def drawn_engine_case(case: int):
+    import random
+
+    rng = random.Random(case)
+    name = rng.choice("ABC")
+    vocab = TINY_INIT[name]["config"]["vocab_size"]
+    head = [rng.randrange(vocab) for _ in range(rng.choice([0, 8, 16, 33]))]
+    prompts = []
+    for _ in range(rng.randint(2, 9)):
+        body = [rng.randrange(vocab) for _ in range(rng.randint(1, 60))]
+        prompts.append((head if rng.random() < 0.6 else []) + body)
+    if rng.random() < 0.3:
+        prompts.append(list(prompts[0]))
+    max_tokens = rng.randint(1, 40)
+    block_size = rng.choice([1, 2, 4, 8, 16])
+    one = -(-(max(len(p) for p in prompts) + max_tokens) // block_size)      # pages of the longest request
+    settings = dict(block_size=block_size, num_blocks=rng.choice([one + 1, one * 2, one * 4, 10 * one]),
+                    max_batch=rng.choice([1, 2, 3, 4, 6, 8]), chunk=rng.choice([None, 2, 3, 7, 16, 64]),
+                    prefix_cache=rng.random() < 0.5, sampler=rng.choice(["device", "host"]))
+    sampling = rng.choice([dict(temperature=0.0), dict(temperature=0.8, seed=case),
+                           dict(temperature=1.2, top_k=20, top_p=0.9, seed=case)])
+    return name, prompts, max_tokens, settings, sampling
+
+
+@pytest.mark.parametrize("case", range(16))
+def test_the_engines_settings_change_no_token(model_dirs, case):
+    """Page size, pool (down to one request's worth and a page), requests a step, portion size, prefix
+    sharing and the sampler's place, all drawn: in 32-bit the tokens are those of an engine that runs the
+    requests one by one, whole, with room to spare; greedy and drawn with a seed."""
+    from paged_llm_rs_amd import Engine
+
+    name, prompts, max_tokens, settings, sampling = drawn_engine_case(case)
+    d = model_dirs(name, "float32")
+    roomy = Engine(d, dtype="f32", block_size=16, num_blocks=64 * len(prompts), max_batch=1, chunk=None,
+                   prefix_cache=False, sampler=settings["sampler"])
+    want = roomy.generate(prompts, max_tokens=max_tokens, stop_tokens=[], **sampling)
+    engine = Engine(d, dtype="f32", **settings)
+    got = engine.generate(prompts, max_tokens=max_tokens, stop_tokens=[], **sampling)
+    assert [g["tokens"] for g in got] == [w["tokens"] for w in want], f"{settings} {sampling}"
+    m = engine.metrics()
+    if not settings["prefix_cache"]:
+        assert m["available"] == m["total"]
+
+
 import numpy as np  # noqa: E402
