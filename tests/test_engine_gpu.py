@@ -298,4 +298,59 @@ def test_the_engines_settings_change_no_token(model_dirs, case):
         assert m["available"] == m["total"]
 
 
+@pytest.mark.parametrize("case", range(8))
+def test_requests_that_arrive_and_are_cancelled_while_others_run(model_dirs, case):
+    """Requests are submitted at drawn steps, some are cancelled a few steps later, the pool is drawn from
+    tight to roomy: every request that finishes has the tokens it has alone in an engine with room to
+    spare, and without prefix sharing every page is free again at the end."""
+    import random
+
+    from paged_llm_rs_amd import Engine
+
+    rng = random.Random(1000 + case)
+    name = rng.choice("ABC")
+    vocab = TINY_INIT[name]["config"]["vocab_size"]
+    head = [rng.randrange(vocab) for _ in range(rng.choice([0, 8, 16, 33]))]
+    requests = []
+    for i in range(rng.randint(3, 14)):
+        prompt = (head if rng.random() < 0.6 else []) + [rng.randrange(vocab) for _ in range(rng.randint(1, 60))]
+        sampling = rng.choice([dict(temperature=0.0), dict(temperature=0.8, seed=case * 100 + i),
+                               dict(temperature=1.2, top_k=20, top_p=0.9, seed=case * 100 + i)])
+        requests.append(dict(prompt=prompt, max_tokens=rng.randint(1, 30), sampling=sampling, arrives=rng.randint(0, 40),
+                             cancelled_after=rng.randint(1, 25) if rng.random() < 0.2 else None))
+    block_size = rng.choice([1, 2, 4, 8, 16])
+    one = -(-max(len(r["prompt"]) + r["max_tokens"] for r in requests) // block_size)
+    settings = dict(block_size=block_size, num_blocks=rng.choice([one + 1, one * 2, one * 4, 10 * one]),
+                    max_batch=rng.choice([1, 2, 3, 4, 6, 8]), chunk=rng.choice([None, 2, 3, 7, 16, 64]),
+                    prefix_cache=rng.random() < 0.5, sampler=rng.choice(["device", "host"]))
+    d = model_dirs(name, "float32")
+    roomy = Engine(d, dtype="f32", block_size=16, num_blocks=64 * len(requests), max_batch=1, chunk=None,
+                   prefix_cache=False, sampler=settings["sampler"])
+    for r in requests:
+        i = roomy.submit(r["prompt"], r["max_tokens"], stop_tokens=[], **r["sampling"])
+        roomy.run()
+        r["want"] = roomy.take_result(i).tokens
+    engine = Engine(d, dtype="f32", **settings)
+    step = 0
+    while any("id" not in r for r in requests) or engine.open_requests:
+        for r in requests:
+            if "id" not in r and r["arrives"] <= step:
+                r["id"] = engine.submit(r["prompt"], r["max_tokens"], stop_tokens=[], **r["sampling"])
+                r["submitted"] = step
+            if (r.get("cancelled_after") is not None and "id" in r and not r.get("gone")
+                    and r["submitted"] + r["cancelled_after"] <= step):
+                engine.cancel(r["id"])
+                r["gone"] = True
+        if engine.open_requests:
+            assert engine.step() is not None or not engine.open_requests, "the scheduler idles while requests are open"
+        step += 1
+        assert step < 5000
+    for r in requests:
+        if not r.get("gone"):
+            assert engine.take_result(r["id"]).tokens == r["want"], f"{settings}"
+    m = engine.metrics()
+    if not settings["prefix_cache"]:
+        assert m["available"] == m["total"]
+
+
 import numpy as np  # noqa: E402
