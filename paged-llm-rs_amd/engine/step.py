@@ -77,23 +77,43 @@ def _bucket(n: int, least: int = 1) -> int:
     return b
 
 
-class _Sent:
-    """Guards a pinned descriptor that is copied to the device without waiting: the copy of one step has to
-    have left the buffer before the next step is written into it.  A caller that reads every step's result
-    has waited already; one that does not (a portion in the middle of a prompt gives nothing to read) would
-    overwrite a descriptor that the device has not yet fetched."""
+class _DescriptorRing:
+    """Pinned buffers for a graph's step descriptor, used in turn.  A descriptor travels to the device without
+    the host waiting, so the copy of one step has to have left its buffer before that buffer is written again.
+    A caller that reads every step's result has waited already; one that does not (a portion in the middle of
+    a prompt gives nothing to read) would overwrite a descriptor that the device has not yet fetched.  An
+    event after every copy would guard that, at some microseconds a step; here an event is recorded after the
+    copy from the last buffer of a lap and waited for before the first buffer is written again: copies run
+    in the order of the stream, so all of the lap's copies are done by then."""
 
-    def __init__(self):
+    LAP = 8
+
+    def __init__(self, size: int):
+        self.buffers = [torch.zeros(size, dtype=torch.int32).pin_memory() for _ in range(self.LAP)]
+        self.views = [b.numpy() for b in self.buffers]
+        self.at = 0
         self.event = None
 
-    def mark(self) -> None:
-        if self.event is None:
-            self.event = torch.cuda.Event()
-        self.event.record()
-
-    def wait(self) -> None:
-        if self.event is not None:
+    def advance(self) -> None:
+        """Go on to the buffer that the next step is written into."""
+        self.at = (self.at + 1) % self.LAP
+        if self.at == 0 and self.event is not None:
             self.event.synchronize()
+
+    @property
+    def host(self) -> torch.Tensor:
+        return self.buffers[self.at]
+
+    @property
+    def view(self):
+        return self.views[self.at]
+
+    def sent(self) -> None:
+        """After the copy of the current buffer has been put on the stream."""
+        if self.at == self.LAP - 1:
+            if self.event is None:
+                self.event = torch.cuda.Event()
+            self.event.record()
 
 
 class DecodeGraph:
@@ -111,28 +131,28 @@ class DecodeGraph:
         for name, count in pieces:
             self.layout[name] = (offset, count)
             offset += (count + 3) // 4 * 4
-        self.host = torch.zeros(offset, dtype=torch.int32).pin_memory()
-        self.host_np = self.host.numpy()
+        self.ring = _DescriptorRing(offset)
         self.ids = np.zeros(cap, dtype=np.uint64)
         self.device_buf = torch.zeros(offset, dtype=torch.int32, device=model.device)
         block_size = cache.block_size
         self.batch = StepBatch(self.device_buf, self.layout, cap, cap, list(widths), cap, 1,
                                context_bound(max(widths or [1]) * block_size), [])
-        h = self.host_np
-        for name in ("seq_of", "q_start", "logit_rows"):
-            b, c = self.layout[name]
-            h[b:b + c] = np.arange(cap, dtype=np.int32)
-        b, c = self.layout["q_len"]
-        h[b:b + c] = 1
-        self._idle_rows(0)
+        for _ in range(self.ring.LAP):         # what no step changes, in every buffer
+            h = self.ring.view
+            for name in ("seq_of", "q_start", "logit_rows"):
+                b, c = self.layout[name]
+                h[b:b + c] = np.arange(cap, dtype=np.int32)
+            b, c = self.layout["q_len"]
+            h[b:b + c] = 1
+            self._idle_rows(0)
+            self.ring.advance()
         self.graph = None
         self.logits = None
         self.tokens = None
-        self.sent = _Sent()
 
     def _view(self, name):
         b, c = self.layout[name]
-        return self.host_np[b:b + c]
+        return self.ring.view[b:b + c]
 
     def _idle_rows(self, live: int) -> None:
         """Rows past the live requests are padding: position -1, no pages."""
@@ -148,7 +168,7 @@ class DecodeGraph:
         return logits, kernels.argmax(logits)
 
     def capture(self) -> None:
-        self.device_buf.copy_(self.host)
+        self.device_buf.copy_(self.ring.host)
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -184,17 +204,17 @@ class DecodeGraph:
 
     def run(self, entries) -> StepOutput:
         live = len(entries)
-        self.sent.wait()
+        self.ring.advance()
         self.fill(entries)
         if not self.captured:
-            self.device_buf.copy_(self.host, non_blocking=True)
-            self.sent.mark()
+            self.device_buf.copy_(self.ring.host, non_blocking=True)
+            self.ring.sent()
             logits, tokens = self._forward()
             return StepOutput(logits[:live], tokens[:live])
         if self.graph is None:
             self.capture()
-        self.device_buf.copy_(self.host, non_blocking=True)
-        self.sent.mark()
+        self.device_buf.copy_(self.ring.host, non_blocking=True)
+        self.ring.sent()
         self.graph.replay()
         return StepOutput(self.logits[:live], self.tokens[:live])
 
@@ -207,9 +227,9 @@ class ShapeGraph:
         self.model, self.cache, self.widths, self.ctx_bound, self.rows = model, cache, list(widths), ctx_bound, rows
         first = self._lay_out(entries)
         self.size = first.packed.numel()
-        self.host = torch.zeros(self.size, dtype=torch.int32).pin_memory()
+        self.ring = _DescriptorRing(self.size)
         self.device_buf = torch.zeros(self.size, dtype=torch.int32, device=model.device)
-        self.host.copy_(first.packed)
+        self.ring.host.copy_(first.packed)
         self.layout = first.layout
         self.batch = StepBatch(self.device_buf, first.layout, first.num_tokens, first.num_seqs, list(widths),
                                first.num_logit_rows, first.max_q_len, ctx_bound, [],
@@ -217,7 +237,6 @@ class ShapeGraph:
         self.batch.live_seqs = first.live_seqs
         self.graph = None
         self.logits = None
-        self.sent = _Sent()
 
     def _lay_out(self, entries):
         return build_batch(entries, self.cache.manager, len(self.cache.layout.groups), self.model.spec.vocab_size,
@@ -225,7 +244,7 @@ class ShapeGraph:
                            pad_to=self.rows)
 
     def capture(self) -> None:
-        self.device_buf.copy_(self.host)
+        self.device_buf.copy_(self.ring.host)
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -242,12 +261,12 @@ class ShapeGraph:
             batch = self._lay_out(entries)
             if batch.packed.numel() != self.size:
                 raise ConfigError("a step of another shape than the captured one")
-            self.sent.wait()
-            self.host.copy_(batch.packed)
+            self.ring.advance()
+            self.ring.host.copy_(batch.packed)
         else:
             self.capture()
-        self.device_buf.copy_(self.host, non_blocking=True)
-        self.sent.mark()
+        self.device_buf.copy_(self.ring.host, non_blocking=True)
+        self.ring.sent()
         self.graph.replay()
         return StepOutput(self.logits)
 

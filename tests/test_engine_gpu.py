@@ -226,12 +226,17 @@ def test_a_shape_of_step_that_comes_again_is_captured_and_replays_like_the_eager
         assert np.array_equal(a[key], b[key]), f"{key}: a replay differs from the eager step"
 
 
+@pytest.mark.parametrize("lap", [1, 8])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_portions_that_return_nothing_replay_like_eager_ones(model_dirs, dtype):
+def test_portions_that_return_nothing_replay_like_eager_ones(model_dirs, dtype, lap, monkeypatch):
     """Equal portions in the middle of a prompt give nothing to read, so nothing makes the host wait for
     the device between them: each replay still has to run on its own step's descriptor, not on the next
-    one's, which the host is already writing."""
+    one's, which the host is already writing.  (The pinned descriptors are used in turn; with a lap of one
+    buffer every step waits for the copy before it, with the usual lap only every eighth.)"""
+    from paged_llm_rs_amd.engine import step
     from paged_llm_rs_amd.engine.replay import Replayer
+
+    monkeypatch.setattr(step._DescriptorRing, "LAP", lap)
 
     d = model_dirs("C", dtype)
     prompt = ru.make_prompts(TINY_INIT["C"]["config"]["vocab_size"], [150], seed=41)["r0"]
