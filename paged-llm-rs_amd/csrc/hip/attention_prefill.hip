@@ -125,6 +125,44 @@ __device__ __forceinline__ int ap_value_shift(int r, int pieces) { return 4 * ((
 // each token of a short portion, then reads its keys once for the whole group, on the matrix cores.
 // The token tile of the work index is then a token, its head a key head, and requests with
 // short_limit or more tokens are the ones left out.
+// Token tiles counted over the requests that a launch serves (those with `short_limit` tokens or more, and a
+// context; grouped: those with fewer, a tile being one token), one request after the other: which request and
+// which of its tiles is number `slot`?  Late tiles, which read the most keys, come first within a request.  A step of one long portion beside many single
+// tokens then has workgroups for the portion's tiles only, and not tiles-of-the-longest times requests of
+// them, nearly all of which would find nothing to do.  Every thread of the workgroup calls this, with all
+// lanes of its wave; false: there is no such tile.
+__device__ __forceinline__ bool ap_find_tile(int slot, const int* __restrict__ q_len, const int* __restrict__ ctx_len,
+                                             int num_seqs, int short_limit, int bm, bool grouped, int& seq, int& tile) {
+    const int lane = threadIdx.x & 63;
+    int before = 0;                                             // tiles of the requests before this stretch of 64
+    for (int base = 0; base < num_seqs; base += 64) {
+        const int s = base + lane;
+        int mine = 0;
+        if (s < num_seqs) {
+            const int c = q_len[s];
+            const bool served = grouped ? (short_limit <= 0 || c < short_limit) : c >= short_limit;
+            if (c > 0 && served && ctx_len[s] > 0) mine = (c + bm - 1) / bm;
+        }
+        int through = mine;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int other = __shfl_up(through, off, 64);
+            if (lane >= off) through += other;
+        }
+        const int total = __builtin_amdgcn_readfirstlane(__shfl(through, 63, 64));   // uniform, and known to be
+        if (slot < before + total) {
+            const bool here = mine > 0 && slot >= before + through - mine && slot < before + through;
+            const int l = __ffsll(static_cast<unsigned long long>(__ballot(here))) - 1;   // one lane says so
+            // (the same in every lane: said so to the compiler, which keeps what follows from them in scalar registers)
+            seq = __builtin_amdgcn_readfirstlane(base + l);
+            tile = __builtin_amdgcn_readfirstlane(__shfl(mine, l, 64) - 1 - (slot - before - __shfl(through - mine, l, 64)));
+            return true;
+        }
+        before += total;
+    }
+    return false;
+}
+
 template <int DT, int NW, int KS, int FEED, bool GR = false>
 __global__ void __launch_bounds__(64 * NW * KS, DT <= 4 ? AP_OCC : 1)
 paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
@@ -134,7 +172,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
                                int block_size, const bf16_t* __restrict__ k_pool,
                                const bf16_t* __restrict__ v_pool, int nq, int nkv, int d, float scale_log2e,
                                int window, int total_work, int splits, float* __restrict__ part_acc,
-                               float* __restrict__ part_ml) {
+                               float* __restrict__ part_ml, int compact) {
     constexpr int DP = 32 * DT;
     constexpr int BM = 32 * NW;
     constexpr int NT = 64 * NW * KS;
@@ -158,18 +196,26 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     // work (the token tiles of one head) go to one XCD, whose L2 then holds the
     // keys and values they share.
     int work = blockIdx.x;
-    if ((total_work & 7) == 0) work = (blockIdx.x & 7) * (total_work >> 3) + (blockIdx.x >> 3);
+    // (compact: only the first slots have tiles, and a stretch of them must not fall to one XCD; workgroups
+    // that follow each other go to XCDs that follow each other, so with heads times splits a multiple of eight
+    // a head's tiles still meet in one XCD.)
+    if (!compact && (total_work & 7) == 0) work = (blockIdx.x & 7) * (total_work >> 3) + (blockIdx.x >> 3);
     // work = ((request * nq + head) * tiles + (tiles - 1 - tile)) * splits + split: late tiles, which read
     // the most keys, first.  With splits > 1 the key tiles of a token tile are dealt to that many
     // workgroups (few token tiles over a long context would leave compute units idle, and the last
     // token tiles of a prompt hold the others up); each leaves its unnormalised output, maximum and sum
     // in the workspace and a second kernel puts them together.
+    // (compact: work = (slot * heads + head) * splits + split, the slot being a token tile as ap_find_tile counts them)
     const int split = work % splits;
     work /= splits;
     const int heads_n = GR ? nkv : nq;
-    const int tile = tiles_a_request - 1 - work % tiles_a_request;
-    const int head = (work / tiles_a_request) % heads_n;
-    const int seq = work / (tiles_a_request * heads_n);
+    int tile = tiles_a_request - 1 - work % tiles_a_request;
+    int head = (work / tiles_a_request) % heads_n;
+    int seq = work / (tiles_a_request * heads_n);
+    if (compact) {
+        head = work % heads_n;
+        if (!ap_find_tile(work / heads_n, q_len, ctx_len, num_seqs, short_limit, GR ? 1 : 32 * NW, GR, seq, tile)) return;
+    }
     if (seq >= num_seqs) return;
 
     const int count = q_len[seq];
@@ -719,28 +765,30 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
 }
 
 // Puts the splits of a token tile together: out = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).
-// blockIdx.x names the token tile as in the kernel above (without the splits), blockIdx.y a stretch of
-// its tokens; a thread takes four head elements of one token and asks for all it needs at once.
+// The step's rows are its grid: blockIdx.x names a stretch of rows of q, blockIdx.y a query head; a thread takes
+// four head elements of one row, finds the request the row belongs to (the requests' rows follow each other in
+// q) and asks for all it needs at once.  A step of one portion beside many single tokens so has no workgroups
+// for token tiles that do not exist.
 #define AP_MERGE_MAX 16
 __global__ void __launch_bounds__(256)
 paged_attention_prefill_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
-                                     bf16_t* __restrict__ out, const int* __restrict__ q_start,
-                                     const int* __restrict__ q_len, const int* __restrict__ ctx_len, int short_limit,
-                                     int tiles_a_request, int num_seqs, int nq, int d, int splits, int bm, int grouped) {
-    const int work = blockIdx.x;
-    const int tile = work % tiles_a_request;
-    const int head = (work / tiles_a_request) % nq;
-    const int seq = work / (tiles_a_request * nq);
-    if (seq >= num_seqs) return;
-    const int count = q_len[seq];
-    if (ctx_len[seq] <= 0) return;
-    if (grouped ? (short_limit > 0 && count >= short_limit) : count < short_limit) return;
+                                          bf16_t* __restrict__ out, const int* __restrict__ q_start,
+                                          const int* __restrict__ q_len, const int* __restrict__ ctx_len,
+                                          int short_limit, int num_seqs, int nq, int d, int splits, int total_rows,
+                                          int grouped) {
     const int quads = d / 4, rows = blockDim.x / quads;
-    const int r = tile * bm + blockIdx.y * rows + threadIdx.x / quads;
+    const int r = blockIdx.x * rows + threadIdx.x / quads;
+    const int head = blockIdx.y;
     const int e0 = (threadIdx.x % quads) * 4;
-    if (static_cast<int>(threadIdx.x) >= rows * quads || r >= min(count, (tile + 1) * bm)) return;
-    const size_t row = static_cast<size_t>(q_start[seq]) + r;
-    const size_t at = (row * nq + head) * splits;
+    if (static_cast<int>(threadIdx.x) >= rows * quads || r >= total_rows) return;
+    bool served = false;
+    for (int s = 0; s < num_seqs; ++s) {
+        const int first = q_start[s], count = q_len[s];
+        if (r >= first && r < first + count)
+            served = ctx_len[s] > 0 && (grouped ? (short_limit <= 0 || count < short_limit) : count >= short_limit);
+    }
+    if (!served) return;
+    const size_t at = (static_cast<size_t>(r) * nq + head) * splits;
     float ms[AP_MERGE_MAX], ls[AP_MERGE_MAX];
     f32x4 os[AP_MERGE_MAX];
 #pragma unroll
@@ -770,7 +818,7 @@ paged_attention_prefill_merge_kernel(const float* __restrict__ part_acc, const f
     ap_u32x2 w;
     w.v[0] = ap_pack2(a[0] * inv, a[1] * inv);
     w.v[1] = ap_pack2(a[2] * inv, a[3] * inv);
-    *reinterpret_cast<ap_u32x2*>(out + (row * nq + head) * d + e0) = w;
+    *reinterpret_cast<ap_u32x2*>(out + (static_cast<size_t>(r) * nq + head) * d + e0) = w;
 }
 
 template <int DT, int NW, int KS, int FEED, bool GR = false>
@@ -778,7 +826,7 @@ static int launch_prefill(const void* q, int q_stride, void* out, const int* q_s
                           const int* ctx_len, int short_limit, int num_seqs, int max_q_len, const int* block_table,
                           int max_blocks, int block_size, const void* k_pool, const void* v_pool, int nq, int nkv,
                           int d, float scale, int window, int splits, float* part_acc, float* part_ml,
-                          hipStream_t stream) {
+                          int total_rows, hipStream_t stream) {
     constexpr int DP = 32 * DT;
     constexpr int BM = 32 * NW;
     const size_t tile_bytes = FEED == 2 ? (3 + 4) * static_cast<size_t>(AP_BN) * DP * 2
@@ -792,24 +840,33 @@ static int launch_prefill(const void* q, int q_stride, void* out, const int* q_s
         PL_REQUIRE(e == hipSuccess, "prefill attention: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
     }
     const int tiles = GR ? max_q_len : pl_ceil_div(max_q_len, BM);
-    const long long whole = static_cast<long long>(tiles) * (GR ? nkv : nq) * num_seqs, total = whole * splits;
+    long long whole = static_cast<long long>(tiles) * (GR ? nkv : nq) * num_seqs;
+    // The requests served bring total_rows tokens at most, and each of them short_limit at least: so many token
+    // tiles there can be.  Where that is fewer than tiles of the longest times requests, workgroups are dealt
+    // to the tiles that there are (ap_find_tile).
+    // (Grouped, a tile is a token: there are total_rows of them at most.)
+    int compact = 0;
+    {
+        const long long served = short_limit > 0 ? (total_rows / short_limit < num_seqs ? total_rows / short_limit : num_seqs) : num_seqs;
+        const long long bound = GR ? total_rows : (total_rows + served * (BM - 1)) / BM;
+        if (bound < static_cast<long long>(tiles) * num_seqs) {
+            compact = 1;
+            whole = bound * (GR ? nkv : nq);
+        }
+    }
+    const long long total = whole * splits;
     PL_REQUIRE(total > 0 && total < (1ll << 30), "prefill attention: %lld workgroups", total);
     paged_attention_prefill_kernel<DT, NW, KS, FEED, GR><<<static_cast<int>(total), 64 * NW * KS, lds_bytes, stream>>>(
         static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), q_start, q_len, ctx_len, short_limit, tiles,
         num_seqs, block_table, max_blocks, block_size, static_cast<const bf16_t*>(k_pool),
         static_cast<const bf16_t*>(v_pool), nq, nkv, d, scale * 1.4426950408889634f, window, static_cast<int>(total),
-        splits, part_acc, part_ml);
+        splits, part_acc, part_ml, compact);
     PL_CHECK_LAUNCH("paged_attention_prefill");
     if (splits > 1) {
         const int rows = 256 / (d / 4);
-        if (GR)     // a request's tokens as one tile of the merge, every query head
-            paged_attention_prefill_merge_kernel<<<dim3(num_seqs * nq, pl_ceil_div(max_q_len, rows)), 256, 0, stream>>>(
-                part_acc, part_ml, static_cast<bf16_t*>(out), q_start, q_len, ctx_len, short_limit, 1, num_seqs, nq, d,
-                splits, max_q_len, 1);
-        else
-            paged_attention_prefill_merge_kernel<<<dim3(static_cast<int>(whole), pl_ceil_div(BM, rows)), 256, 0, stream>>>(
-                part_acc, part_ml, static_cast<bf16_t*>(out), q_start, q_len, ctx_len, short_limit, tiles, num_seqs, nq, d,
-                splits, BM, 0);
+        paged_attention_prefill_merge_kernel<<<dim3(pl_ceil_div(total_rows, rows), nq), 256, 0, stream>>>(
+            part_acc, part_ml, static_cast<bf16_t*>(out), q_start, q_len, ctx_len, short_limit, num_seqs, nq, d, splits,
+            total_rows, GR ? 1 : 0);
         PL_CHECK_LAUNCH("paged_attention_prefill_merge");
     }
     return 0;
@@ -820,11 +877,11 @@ static int ap_dispatch(bool small, bool uniform_pages, const void* q, int q_stri
                        const int* q_len, const int* ctx_len, int short_limit, int num_seqs, int max_q_len,
                        const int* block_table, int max_blocks, int block_size, const void* k_pool, const void* v_pool,
                        int nq, int nkv, int d, float scale, int window, int splits, float* part_acc, float* part_ml,
-                       hipStream_t stream) {
+                       int total_rows, hipStream_t stream) {
 #define AP_LAUNCH(NW, KS, FEED)                                                                                    \
     launch_prefill<D, NW, KS, FEED>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len,    \
                                     block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale, window, \
-                                    splits, part_acc, part_ml, stream)
+                                    splits, part_acc, part_ml, total_rows, stream)
     constexpr bool can_fit = 64 % (4 * D) == 0;
     constexpr int BEST = (D == 2 || D == 4) && AP_KS == 2 && AP_SMALL_KS == 2 ? AP_FEED : 1;   // the feed with uniform pages
     if constexpr (D <= 4) {
@@ -852,6 +909,8 @@ static int ap_dispatch(bool small, bool uniform_pages, const void* q, int q_stri
 // Requests with q_len < short_limit are skipped.  max_q_len bounds q_len over the requests.
 // splits > 1 deals the keys of every token tile to that many workgroups; the workspace then needs
 // rows*nq*splits*d floats (part_acc) and rows*nq*splits*2 (part_ml), rows being the step's rows of q.
+// total_rows: the rows of q (the requests bring so many together at most); workgroups are dealt to the token
+// tiles that can exist among them where that is fewer than tiles-of-the-longest for every request.
 // pl_paged_attention_prefill_tile says how many tokens a token tile will have.
 extern "C" int pl_paged_attention_prefill_tile(int max_q_len, int d) {
     return (max_q_len <= 64 && d <= 128) ? 64 : 128;
@@ -862,7 +921,7 @@ extern "C" int pl_paged_attention_prefill(const void* q, int q_stride, void* out
                                           int max_q_len, const int* block_table, int max_blocks, int block_size,
                                           const void* k_pool, const void* v_pool, int nq, int nkv, int d,
                                           float scale, int window, int splits, float* part_acc, float* part_ml,
-                                          hipStream_t stream) {
+                                          int total_rows, hipStream_t stream) {
     PL_REQUIRE(splits >= 1 && splits <= AP_MERGE_MAX && (splits == 1 || (part_acc && part_ml)),
                "prefill attention: %d splits%s", splits, splits > 1 ? " without a workspace" : "");
     PL_REQUIRE(d > 0 && d <= 256 && d % 16 == 0, "prefill attention: head size %d, which has to be a multiple of 16 up to 256", d);
@@ -872,6 +931,7 @@ extern "C" int pl_paged_attention_prefill(const void* q, int q_stride, void* out
                q_stride, window);
     PL_REQUIRE((nkv * d) % 8 == 0, "prefill attention: a cache row of %d elements is not read 16 bytes at a time", nkv * d);
     if (num_seqs <= 0 || max_q_len <= 0) return 0;
+    PL_REQUIRE(total_rows >= max_q_len, "prefill attention: %d rows for a portion of %d", total_rows, max_q_len);
     const int dt = pl_ceil_div(d, 32);
     // few tokens a request: 64-token tiles give twice the workgroups
 #ifdef AP_FORCE_SMALL
@@ -885,7 +945,7 @@ extern "C" int pl_paged_attention_prefill(const void* q, int q_stride, void* out
 #define AP_CALL(D)                                                                                                 \
     return ap_dispatch<D>(small, pages_fit, q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len, \
                           block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale, window, splits,   \
-                          part_acc, part_ml, stream)
+                          part_acc, part_ml, total_rows, stream)
     switch (dt) {
         case 1: AP_CALL(1);
         case 2: AP_CALL(2);
@@ -916,7 +976,7 @@ extern "C" int pl_paged_attention_grouped(const void* q, int q_stride, void* out
                                           int max_q_len, const int* block_table, int max_blocks, int block_size,
                                           const void* k_pool, const void* v_pool, int nq, int nkv, int d,
                                           float scale, int window, int splits, float* part_acc, float* part_ml,
-                                          hipStream_t stream) {
+                                          int total_rows, hipStream_t stream) {
     PL_REQUIRE(pl_paged_attention_grouped_applies(nq, nkv, d, block_size),
                "grouped attention: %d query heads over %d key heads of %d, pages of %d", nq, nkv, d, block_size);
     PL_REQUIRE(splits >= 1 && splits <= AP_MERGE_MAX && (splits == 1 || (part_acc && part_ml)),
@@ -924,11 +984,12 @@ extern "C" int pl_paged_attention_grouped(const void* q, int q_stride, void* out
     PL_REQUIRE(max_blocks > 0 && q_stride >= nq * d && q_stride % 8 == 0 && window >= 0,
                "grouped attention: %d blocks a row, query stride %d, window %d", max_blocks, q_stride, window);
     if (num_seqs <= 0 || max_q_len <= 0) return 0;
+    PL_REQUIRE(total_rows >= max_q_len, "grouped attention: %d rows for portions of %d", total_rows, max_q_len);
     if (d == 64)
         return launch_prefill<2, 1, 2, 2, true>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len,
                                                 block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale,
-                                                window, splits, part_acc, part_ml, stream);
+                                                window, splits, part_acc, part_ml, total_rows, stream);
     return launch_prefill<4, 1, 2, 2, true>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len,
                                             block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale,
-                                            window, splits, part_acc, part_ml, stream);
+                                            window, splits, part_acc, part_ml, total_rows, stream);
 }

@@ -42,8 +42,8 @@ def _signatures(lib) -> None:
         "pl_gemm_tiled_applies": [i, i, i, i],
         "pl_paged_attention_decode": [p, i, p, p, p, p, p, p, i, p, i, i, p, p, i, i, i, i, f, i, i,
                                       i, p, p, i, f, p, p, i, p],
-        "pl_paged_attention_prefill": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, p],
-        "pl_paged_attention_grouped": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, p],
+        "pl_paged_attention_prefill": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, i, p],
+        "pl_paged_attention_grouped": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, i, p],
         "pl_paged_attention_grouped_applies": [i, i, i, i],
     }
     for name, argtypes in table.items():
@@ -397,7 +397,7 @@ def paged_attention_prefill(q: torch.Tensor, q_row_stride: int, out: torch.Tenso
     if not 0 < live <= S:
         raise TensorError(f"{live} requests with tokens of {S}")
     if splits is None:
-        splits = prefill_splits(live, int(max_q_len), nq, d, int(max_ctx or 0), n)
+        splits = prefill_splits(live, int(max_q_len), nq, d, int(max_ctx or 0), n, int(short_limit))
     part_acc = part_ml = None
     if splits > 1:
         part_acc = torch.empty((n * nq * splits * d,), dtype=torch.float32, device=q.device)
@@ -406,7 +406,7 @@ def paged_attention_prefill(q: torch.Tensor, q_row_stride: int, out: torch.Tenso
         q.data_ptr(), q_row_stride, out.data_ptr(), q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(),
         int(short_limit), live, int(max_q_len), block_table.data_ptr(), block_table.shape[1], block_size,
         k_pool.data_ptr(), v_pool.data_ptr(), nq, nkv, d, float(scale), int(window or 0), int(splits),
-        part_acc.data_ptr() if splits > 1 else None, part_ml.data_ptr() if splits > 1 else None, _stream()))
+        part_acc.data_ptr() if splits > 1 else None, part_ml.data_ptr() if splits > 1 else None, n, _stream()))
     return out
 
 
@@ -478,11 +478,12 @@ def paged_attention_grouped(q: torch.Tensor, q_row_stride: int, out: torch.Tenso
         q.data_ptr(), q_row_stride, out.data_ptr(), q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(),
         int(short_limit), live, int(max_q_len), block_table.data_ptr(), block_table.shape[1], block_size,
         k_pool.data_ptr(), v_pool.data_ptr(), nq, nkv, d, float(scale), int(window or 0), int(splits),
-        part_acc.data_ptr() if splits > 1 else None, part_ml.data_ptr() if splits > 1 else None, _stream()))
+        part_acc.data_ptr() if splits > 1 else None, part_ml.data_ptr() if splits > 1 else None, n, _stream()))
     return out
 
 
-def prefill_splits(requests: int, max_q_len: int, nq: int, d: int, max_ctx: int, rows: int | None = None) -> int:
+def prefill_splits(requests: int, max_q_len: int, nq: int, d: int, max_ctx: int, rows: int | None = None,
+                   short_limit: int = 0) -> int:
     """Into how many shares the keys of a token tile are cut.  A share more costs a trip of the
     unnormalised outputs through memory (rows * nq * d floats written and read) and one launch;
     it pays where few token tiles stand before a long context, as in a late portion of a long
@@ -494,6 +495,12 @@ def prefill_splits(requests: int, max_q_len: int, nq: int, d: int, max_ctx: int,
     base = max(1, -(-max_q_len // tile) * nq * requests)
     key_tiles = -(-max_ctx // 64)
     rows = rows if rows is not None else requests * max_q_len
+    # Where the rows cannot fill that many token tiles the kernel deals its workgroups to the tiles there can
+    # be; most of those are empty too when the step is one portion beside single tokens, so the portion's
+    # own tiles are what is counted.
+    served = min(requests, rows // short_limit) if short_limit > 0 else requests
+    if (rows + served * (tile - 1)) // tile < -(-max_q_len // tile) * requests:
+        base = (rows // tile + 1) * nq
     best, best_cost = 1, None
     for s in (1, 2, 3, 4, 6, 8, 12, 16):
         if s > 1 and key_tiles // s < 4:
