@@ -769,7 +769,9 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
 // four head elements of one row, finds the request the row belongs to (the requests' rows follow each other in
 // q) and asks for all it needs at once.  A step of one portion beside many single tokens so has no workgroups
 // for token tiles that do not exist.
+// SP: the splits the registers are laid out for (every one of them is asked for, used or not).
 #define AP_MERGE_MAX 16
+template <int SP>
 __global__ void __launch_bounds__(256)
 paged_attention_prefill_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
                                           bf16_t* __restrict__ out, const int* __restrict__ q_start,
@@ -780,28 +782,41 @@ paged_attention_prefill_merge_kernel(const float* __restrict__ part_acc, const f
     const int r = blockIdx.x * rows + threadIdx.x / quads;
     const int head = blockIdx.y;
     const int e0 = (threadIdx.x % quads) * 4;
-    if (static_cast<int>(threadIdx.x) >= rows * quads || r >= total_rows) return;
+    // The requests are read 64 at a time, one a lane; each lane says for each of the few rows of its wave
+    // whether its request holds that row and is served here.
+    const int lane = threadIdx.x & 63, wave_first = threadIdx.x - lane;
+    const int row_first = blockIdx.x * rows + wave_first / quads, row_last = blockIdx.x * rows + (wave_first + 63) / quads;
     bool served = false;
-    for (int s = 0; s < num_seqs; ++s) {
-        const int first = q_start[s], count = q_len[s];
-        if (r >= first && r < first + count)
-            served = ctx_len[s] > 0 && (grouped ? (short_limit <= 0 || count < short_limit) : count >= short_limit);
+    for (int base = 0; base < num_seqs; base += 64) {
+        const int s = base + lane;
+        int first = 0, count = 0;
+        bool ok = false;
+        if (s < num_seqs) {
+            first = q_start[s];
+            count = q_len[s];
+            ok = ctx_len[s] > 0 && (grouped ? (short_limit <= 0 || count < short_limit) : count >= short_limit);
+        }
+        for (int row = row_first; row <= row_last; ++row) {
+            const bool holds = __ballot(ok && row >= first && row < first + count) != 0;
+            if (holds && row == r) served = true;
+        }
     }
-    if (!served) return;
+    if (static_cast<int>(threadIdx.x) >= rows * quads || r >= total_rows || !served) return;
     const size_t at = (static_cast<size_t>(r) * nq + head) * splits;
-    float ms[AP_MERGE_MAX], ls[AP_MERGE_MAX];
-    f32x4 os[AP_MERGE_MAX];
+    float ms[SP], ls[SP];
+    f32x4 os[SP];
 #pragma unroll
-    for (int sp = 0; sp < AP_MERGE_MAX; ++sp) {
+    for (int sp = 0; sp < SP; ++sp) {
         const int sc = min(sp, splits - 1);
-        ms[sp] = part_ml[(at + sc) * 2];
-        ls[sp] = part_ml[(at + sc) * 2 + 1];
+        const float2 ml = *reinterpret_cast<const float2*>(part_ml + (at + sc) * 2);
+        ms[sp] = ml.x;
+        ls[sp] = ml.y;
     }
     float big = -INFINITY;
 #pragma unroll
-    for (int sp = 0; sp < AP_MERGE_MAX; ++sp) big = fmaxf(big, sp < splits ? ms[sp] : -INFINITY);
+    for (int sp = 0; sp < SP; ++sp) big = fmaxf(big, sp < splits ? ms[sp] : -INFINITY);
 #pragma unroll
-    for (int sp = 0; sp < AP_MERGE_MAX; ++sp) {
+    for (int sp = 0; sp < SP; ++sp) {
         // a split that saw no key wrote no output: its place in the workspace holds anything
         const bool live = sp < splits && ms[sp] != -INFINITY;
         os[sp] = live ? *reinterpret_cast<const f32x4*>(part_acc + (at + sp) * d + e0) : f32x4{0.f, 0.f, 0.f, 0.f};
@@ -810,7 +825,7 @@ paged_attention_prefill_merge_kernel(const float* __restrict__ part_acc, const f
     float sum = 0.f;
     f32x4 a = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int sp = 0; sp < AP_MERGE_MAX; ++sp) {
+    for (int sp = 0; sp < SP; ++sp) {
         sum = fmaf(ls[sp], ms[sp], sum);
         a += os[sp] * ms[sp];
     }
@@ -864,9 +879,15 @@ static int launch_prefill(const void* q, int q_stride, void* out, const int* q_s
     PL_CHECK_LAUNCH("paged_attention_prefill");
     if (splits > 1) {
         const int rows = 256 / (d / 4);
-        paged_attention_prefill_merge_kernel<<<dim3(pl_ceil_div(total_rows, rows), nq), 256, 0, stream>>>(
-            part_acc, part_ml, static_cast<bf16_t*>(out), q_start, q_len, ctx_len, short_limit, num_seqs, nq, d, splits,
-            total_rows, GR ? 1 : 0);
+#define AP_MERGE(SP)                                                                                               \
+    paged_attention_prefill_merge_kernel<SP><<<dim3(pl_ceil_div(total_rows, rows), nq), 256, 0, stream>>>(         \
+        part_acc, part_ml, static_cast<bf16_t*>(out), q_start, q_len, ctx_len, short_limit, num_seqs, nq, d, splits, \
+        total_rows, GR ? 1 : 0)
+        if (splits <= 2) AP_MERGE(2);
+        else if (splits <= 4) AP_MERGE(4);
+        else if (splits <= 8) AP_MERGE(8);
+        else AP_MERGE(AP_MERGE_MAX);
+#undef AP_MERGE
         PL_CHECK_LAUNCH("paged_attention_prefill_merge");
     }
     return 0;
