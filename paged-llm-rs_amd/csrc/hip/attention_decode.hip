@@ -104,14 +104,53 @@ __device__ __forceinline__ void ad_norm_rope8(float* x, const void* gain, const 
     for (int i = 0; i < 8; ++i) x[i] = to_float(from_float<bf16_t>(x[i]));
 }
 
+// The tokens of the requests with fewer than `short_limit` tokens, counted through the requests in their
+// order: which row of the step is number `slot`?  (The requests' rows follow each other.)  A step of a long
+// portion beside single tokens then has workgroups for the single tokens only: one for every row of the
+// portion as well, each of which would leave at once, costs the launch some 7 ns apiece.  Every thread of the
+// workgroup calls this with all lanes of its wave; false: there is no such token.
+__device__ __forceinline__ bool ad_find_row(int slot, const int* __restrict__ q_len, int num_seqs, int short_limit,
+                                            int& row) {
+    const int lane = threadIdx.x % PL_WAVE;
+    int rows_before = 0, short_before = 0;
+    for (int base = 0; base < num_seqs; base += PL_WAVE) {
+        const int s = base + lane;
+        const int count = s < num_seqs ? q_len[s] : 0;
+        const int few = count < short_limit ? count : 0;
+        int rows_through = count, short_through = few;
+#pragma unroll
+        for (int off = 1; off < PL_WAVE; off <<= 1) {
+            const int a = __shfl_up(rows_through, off, PL_WAVE), b = __shfl_up(short_through, off, PL_WAVE);
+            if (lane >= off) {
+                rows_through += a;
+                short_through += b;
+            }
+        }
+        // (uniform, and said to be: what follows from them stays in scalar registers)
+        const int rows_here = __builtin_amdgcn_readfirstlane(__shfl(rows_through, PL_WAVE - 1, PL_WAVE));
+        const int short_here = __builtin_amdgcn_readfirstlane(__shfl(short_through, PL_WAVE - 1, PL_WAVE));
+        if (slot < short_before + short_here) {
+            const bool mine = few > 0 && slot >= short_before + short_through - few && slot < short_before + short_through;
+            const int l = __ffsll(static_cast<unsigned long long>(__ballot(mine))) - 1;   // one lane says so
+            row = __builtin_amdgcn_readfirstlane(rows_before + __shfl(rows_through - count, l, PL_WAVE) +
+                                                 (slot - short_before - __shfl(short_through - few, l, PL_WAVE)));
+            return true;
+        }
+        rows_before += rows_here;
+        short_before += short_here;
+    }
+    return false;
+}
+
 // LPK: lanes a key (a power of two, LPK*8 >= d).  GT: query heads a workgroup serves.
 // U: keys a lane group asks for at once.
+// num_seqs > 0: blockIdx.y counts the tokens of the short requests (ad_find_row) and not the step's rows.
 template <int LPK, int GT, int U>
 __global__ void __launch_bounds__(256)
 paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
                               float* __restrict__ part_acc, float* __restrict__ part_ml,
                               const int* __restrict__ positions, const int* __restrict__ seq_of,
-                              const int* __restrict__ q_len, int short_limit,
+                              const int* __restrict__ q_len, int short_limit, int num_seqs,
                               const int* __restrict__ block_table, int max_blocks, int block_size,
                               bf16_t* __restrict__ k_pool, bf16_t* __restrict__ v_pool, int nq,
                               int nkv, int d, float scale_log2e, int window, int splits, int tiles, ad_fuse_t fuse) {
@@ -119,7 +158,8 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
     constexpr int GROUPS = AD_WAVES * KPW;
     extern __shared__ float lds[];  // [GROUPS][GT][2] running max and sum, then [GROUPS][GT][d] accumulators
 
-    const int t = blockIdx.y;
+    int t = blockIdx.y;
+    if (num_seqs > 0 && !ad_find_row(blockIdx.y, q_len, num_seqs, short_limit, t)) return;
     const int pos = positions[t];
     if (pos < 0) return;
     const int seq = seq_of[t];
@@ -427,8 +467,8 @@ paged_attention_merge_kernel(const float* __restrict__ part_acc, const float* __
 
 template <int LPK, int GT>
 static int launch_decode(const void* q, int q_stride, void* out, float* part_acc, float* part_ml,
-                         const int* positions, const int* seq_of, const int* q_len, int short_limit,
-                         const int* block_table, int max_blocks, int block_size, void* k_pool,
+                         const int* positions, const int* seq_of, const int* q_len, int short_limit, int num_seqs,
+                         int short_rows, const int* block_table, int max_blocks, int block_size, void* k_pool,
                          void* v_pool, int n, int nq, int nkv, int d, float scale, int window, int splits,
                          const ad_fuse_t& fuse, hipStream_t stream) {
     constexpr int KPW = PL_WAVE / LPK;
@@ -443,11 +483,13 @@ static int launch_decode(const void* q, int q_stride, void* out, float* part_acc
                                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
         PL_REQUIRE(e == hipSuccess, "decode attention: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
     }
-    dim3 grid(nkv * tiles, n, splits);
+    // rows of the grid: the step's rows, or, where fewer, the tokens that the short requests can bring
+    const bool compact = q_len != nullptr && num_seqs > 0 && short_rows > 0 && short_rows < n;
+    dim3 grid(nkv * tiles, compact ? short_rows : n, splits);
     PL_REQUIRE(n <= 65535 && splits <= 65535, "decode attention: %d tokens or %d splits are more than one launch covers", n, splits);
     paged_attention_decode_kernel<LPK, GT, U><<<grid, 256, lds_bytes, stream>>>(
         static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), part_acc, part_ml, positions, seq_of,
-        q_len, short_limit, block_table, max_blocks, block_size, static_cast<bf16_t*>(k_pool),
+        q_len, short_limit, compact ? num_seqs : 0, block_table, max_blocks, block_size, static_cast<bf16_t*>(k_pool),
         static_cast<bf16_t*>(v_pool), nq, nkv, d, scale * 1.4426950408889634f, window, splits, tiles, fuse);
     PL_CHECK_LAUNCH("paged_attention_decode");
     if (splits > 1) {
@@ -468,13 +510,13 @@ static int launch_decode(const void* q, int q_stride, void* out, float* part_acc
 
 template <int LPK>
 static int dispatch_gt(int gt, const void* q, int q_stride, void* out, float* part_acc, float* part_ml,
-                       const int* positions, const int* seq_of, const int* q_len, int short_limit,
-                       const int* block_table, int max_blocks, int block_size, void* k_pool,
+                       const int* positions, const int* seq_of, const int* q_len, int short_limit, int num_seqs,
+                       int short_rows, const int* block_table, int max_blocks, int block_size, void* k_pool,
                        void* v_pool, int n, int nq, int nkv, int d, float scale, int window, int splits,
                        const ad_fuse_t& fuse, hipStream_t stream) {
 #define AD_CALL(G)                                                                                              \
     return launch_decode<LPK, G>(q, q_stride, out, part_acc, part_ml, positions, seq_of, q_len, short_limit,   \
-                                 block_table, max_blocks, block_size, k_pool, v_pool, n, nq, nkv, d, scale,    \
+                                 num_seqs, short_rows, block_table, max_blocks, block_size, k_pool, v_pool, n, nq, nkv, d, scale,    \
                                  window, splits, fuse, stream)
     switch (gt) {
         case 1: AD_CALL(1);
@@ -487,12 +529,16 @@ static int dispatch_gt(int gt, const void* q, int q_stride, void* out, float* pa
 
 // bfloat16 only.  With splits > 1 the workspace needs n*nq*splits*d floats (part_acc) and n*nq*splits*2 (part_ml).
 // q_len (may be null) and short_limit leave the tokens of requests with q_len >= short_limit to the tiled kernel.
+// With q_len: num_seqs, the requests whose rows follow each other in q from row 0 on, and short_rows, the most
+// tokens that the other requests bring together (0: not known); where that is fewer than the step's rows the
+// launch has workgroups for those tokens only.
 // fuse_mode 0: the rows of q are ready and the cache holds every key up to each token's own.  1: the rows of q are
 // the raw projection and are normalised (gains, eps) and rotated (tables, rot a multiple of 16) here.  2: as 1, and
 // each token's key and value are taken raw from its row [q | k | v], used, and written into the cache; every
 // request then has to bring exactly one token.
 extern "C" int pl_paged_attention_decode(const void* q, int q_stride, void* out, float* part_acc, float* part_ml,
                                          const int* positions, const int* seq_of, const int* q_len, int short_limit,
+                                         int num_seqs, int short_rows,
                                          const int* block_table, int max_blocks, int block_size, void* k_pool,
                                          void* v_pool, int n, int nq, int nkv, int d, float scale, int window,
                                          int splits, int fuse_mode, const void* q_gain, const void* k_gain,
@@ -520,7 +566,7 @@ extern "C" int pl_paged_attention_decode(const void* q, int q_stride, void* out,
     const int chunks = d / 8;
 #define AD_LPK(L)                                                                                                  \
     return dispatch_gt<L>(gt, q, q_stride, out, part_acc, part_ml, positions, seq_of, q_len, short_limit,        \
-                          block_table, max_blocks, block_size, k_pool, v_pool, n, nq, nkv, d, scale, window,      \
+                          num_seqs, short_rows, block_table, max_blocks, block_size, k_pool, v_pool, n, nq, nkv, d, scale, window,      \
                           splits, fuse, stream)
     if (chunks <= 2) AD_LPK(2);
     if (chunks <= 4) AD_LPK(4);

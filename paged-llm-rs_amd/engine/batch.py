@@ -89,6 +89,10 @@ class ContextTooLong(CaptureOutgrown):
     """A request's context is longer than the bound the step was to report."""
 
 
+class ShortTokensOutgrown(CaptureOutgrown):
+    """The requests of few tokens bring more tokens together than the bound the step was to report."""
+
+
 def token_bucket(tokens: int) -> int:
     """The number of rows a step of so many tokens is padded to: steps of many lengths then have few
     shapes, and a shape that comes again replays from a graph."""
@@ -101,7 +105,7 @@ def token_bucket(tokens: int) -> int:
 
 def build_batch(entries, manager, num_groups: int, vocab_size: int, max_positions: int, device,
                 check_start: bool = True, widths: list | None = None, ctx_bound: int | None = None,
-                pad_to: int | None = None) -> StepBatch:
+                pad_to: int | None = None, short_bound: int | None = None) -> StepBatch:
     """Validate the entries against the cache manager and lay the step out for the device.
 
     ``widths`` fixes the pages a row of each group's block table has (TableTooWide if a request
@@ -113,7 +117,9 @@ def build_batch(entries, manager, num_groups: int, vocab_size: int, max_position
     (token 0, position -1, no pages, no context, state slot -1; it has no rows when none are
     missing).  The batch then reports bounds instead of counts (every row might belong to one
     request, or to short ones), so that steps with the same rows, requests and wanted places give
-    the kernels the same launch sizes.
+    the kernels the same launch sizes.  ``short_bound`` says how many tokens the requests with fewer
+    than SHORT_PORTION tokens bring at most (ShortTokensOutgrown if they bring more); without it every
+    row might be one of theirs.
 
     Refused with ConfigError: an empty step, an entry without tokens, a token id
     outside the vocabulary, a position with no page or past the longest position
@@ -205,9 +211,12 @@ def build_batch(entries, manager, num_groups: int, vocab_size: int, max_position
     longest = ctx_bound
     if pad_to is not None:
         # every row might belong to one request; if any request is short, every row might
-        any_short = bool((q_len[:S - 1] < SHORT_PORTION).any())
+        short = int(q_len[:S - 1][q_len[:S - 1] < SHORT_PORTION].sum())
+        if short_bound is not None and short > short_bound:
+            raise ShortTokensOutgrown(f"{short} tokens of short requests in a step laid out for {short_bound}")
+        bound = n if short_bound is None else min(n, short_bound)
         batch = StepBatch(packed, layout, n, S, max_blocks, len(logit_rows), n, longest,
-                          [e.seq_id for e in entries], short_tokens=n if any_short else 0)
+                          [e.seq_id for e in entries], short_tokens=bound if short > 0 else 0)
         batch.live_seqs = S - 1
         return batch
     return StepBatch(packed, layout, n, S, max_blocks, len(logit_rows), int(q_len.max()), longest,

@@ -43,10 +43,12 @@ def require_gpu(device) -> torch.device:
     return device
 
 
-def run_step(model, cache, entries, check_start: bool = True, pad_to: int | None = None) -> torch.Tensor:
+def run_step(model, cache, entries, check_start: bool = True, pad_to: int | None = None,
+             short_bound: int | None = None) -> torch.Tensor:
     """32-bit logits [wanted places, vocabulary], in the order of the entries and of their ``want``."""
     batch = build_batch(entries, cache.manager, len(cache.layout.groups), model.spec.vocab_size,
-                        model.spec.max_positions, model.device, check_start=check_start, pad_to=pad_to)
+                        model.spec.max_positions, model.device, check_start=check_start, pad_to=pad_to,
+                        short_bound=short_bound)
     for e in entries:
         if e.fresh_state and e.state_slot >= 0:
             cache.clear_state_slot(e.state_slot)
@@ -223,8 +225,9 @@ class ShapeGraph:
     """A step of one shape (rows after padding, requests, wanted places), with block tables of
     ``widths`` pages a row and contexts up to ``ctx_bound``, captured."""
 
-    def __init__(self, model, cache, entries, widths: list, ctx_bound: int, rows: int):
+    def __init__(self, model, cache, entries, widths: list, ctx_bound: int, rows: int, short_bound: int):
         self.model, self.cache, self.widths, self.ctx_bound, self.rows = model, cache, list(widths), ctx_bound, rows
+        self.short_bound = short_bound
         first = self._lay_out(entries)
         self.size = first.packed.numel()
         self.ring = _DescriptorRing(self.size)
@@ -241,7 +244,7 @@ class ShapeGraph:
     def _lay_out(self, entries):
         return build_batch(entries, self.cache.manager, len(self.cache.layout.groups), self.model.spec.vocab_size,
                            self.model.spec.max_positions, "cpu", widths=self.widths, ctx_bound=self.ctx_bound,
-                           pad_to=self.rows)
+                           pad_to=self.rows, short_bound=self.short_bound)
 
     def capture(self) -> None:
         self.device_buf.copy_(self.ring.host)
@@ -294,11 +297,13 @@ class StepRunner:
         graph from the second time on (while the requests' tables and contexts fit the capture)."""
         tokens = sum(len(e.tokens) for e in entries)
         rows = token_bucket(tokens) if self.pads and tokens <= SHAPE_GRAPH_MAX_TOKENS else None
+        # the tokens of requests that bring few, rounded up: the kernel for single tokens gets so many workgroups
+        short = sum(len(e.tokens) for e in entries if len(e.tokens) < kernels.SHORT_PORTION)
+        short_bound = None if rows is None else min(rows, _bucket(short, 16)) if short else 0
         if not self.use_graphs or rows is None or len(entries) > GRAPH_MAX_REQUESTS:
             self.eager_steps += 1
-            return StepOutput(run_step(self.model, self.cache, entries, pad_to=rows))
-        short = any(len(e.tokens) < kernels.SHORT_PORTION for e in entries)
-        shape = (rows, len(entries), sum(len(e.want) for e in entries), short)
+            return StepOutput(run_step(self.model, self.cache, entries, pad_to=rows, short_bound=short_bound))
+        shape = (rows, len(entries), sum(len(e.want) for e in entries), short_bound)
         known = shape in self._shapes
         graph = self._shapes.pop(shape, None)
         if not known:
@@ -306,7 +311,7 @@ class StepRunner:
             while len(self._shapes) > 256:
                 self._shapes.pop(next(iter(self._shapes)))
             self.eager_steps += 1
-            return StepOutput(run_step(self.model, self.cache, entries, pad_to=rows))
+            return StepOutput(run_step(self.model, self.cache, entries, pad_to=rows, short_bound=short_bound))
         for e in entries:
             if e.fresh_state and e.state_slot >= 0:
                 self.cache.clear_state_slot(e.state_slot)
@@ -320,7 +325,7 @@ class StepRunner:
                 pass                            # a request has outgrown the capture: a new one below
         widths = [_bucket(w + 1, 32) for w in self._widths_needed(entries)]
         longest = max(e.start + len(e.tokens) for e in entries)
-        graph = ShapeGraph(self.model, self.cache, entries, widths, context_bound(longest), rows)
+        graph = ShapeGraph(self.model, self.cache, entries, widths, context_bound(longest), rows, short_bound)
         out = graph.run(entries)
         self._shapes[shape] = graph
         live = [k for k, g in self._shapes.items() if g is not None]

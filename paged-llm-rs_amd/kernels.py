@@ -40,7 +40,7 @@ def _signatures(lib) -> None:
         "pl_gemm_skinny": [p, p, p, p, f, p, i, i, i, i, i, p],
         "pl_gemm_tiled": [p, p, p, i, i, i, i, p],
         "pl_gemm_tiled_applies": [i, i, i, i],
-        "pl_paged_attention_decode": [p, i, p, p, p, p, p, p, i, p, i, i, p, p, i, i, i, i, f, i, i,
+        "pl_paged_attention_decode": [p, i, p, p, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, i, f, i, i,
                                       i, p, p, i, f, p, p, i, p],
         "pl_paged_attention_prefill": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, i, p],
         "pl_paged_attention_grouped": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, i, p],
@@ -308,8 +308,12 @@ def paged_attention_decode(q: torch.Tensor, q_row_stride: int, out: torch.Tensor
                            seq_of: torch.Tensor, block_table: torch.Tensor, block_size: int,
                            k_pool: torch.Tensor, v_pool: torch.Tensor, nq: int, nkv: int, d: int, scale: float,
                            window: int = 0, splits: int = 1, q_len: torch.Tensor | None = None,
-                           short_limit: int = 0, fuse: "QkFusion | None" = None) -> torch.Tensor:
+                           short_limit: int = 0, fuse: "QkFusion | None" = None, live_seqs: int | None = None,
+                           short_rows: int = 0) -> torch.Tensor:
     """bfloat16 attention of single tokens over their requests' pages, split along the context.
+    With ``q_len`` the tokens of requests with ``short_limit`` tokens or more are left out; ``short_rows``
+    then bounds the tokens that the other requests bring (0: not known) and ``live_seqs`` says how many
+    requests, the first ones, bring tokens, so that the launch has workgroups for those tokens only.
     With ``fuse`` the rows of ``q`` are the raw projection [q | k | v]: queries (and, when it says so, each
     token's key) are normalised and rotated inside the kernel, and key and value are written into the pages."""
     n = positions.numel()
@@ -349,7 +353,9 @@ def paged_attention_decode(q: torch.Tensor, q_row_stride: int, out: torch.Tensor
             raise TensorError(f"rows of {q_row_stride} values are not [q | k | v] of {nq}+2*{nkv} heads of {d}")
     _check(library().pl_paged_attention_decode(
         q.data_ptr(), q_row_stride, out.data_ptr(), _ptr(part_acc), _ptr(part_ml), positions.data_ptr(),
-        seq_of.data_ptr(), _ptr(q_len), int(short_limit), block_table.data_ptr(), block_table.shape[1], block_size,
+        seq_of.data_ptr(), _ptr(q_len), int(short_limit),
+        int(block_table.shape[0] if live_seqs is None else live_seqs), int(short_rows if q_len is not None else 0),
+        block_table.data_ptr(), block_table.shape[1], block_size,
         k_pool.data_ptr(), v_pool.data_ptr(), n, nq, nkv, d, float(scale), int(window or 0), int(splits),
         mode, _ptr(q_gain), _ptr(k_gain), gain_code, float(eps), _ptr(cos), _ptr(sin), int(rot), _stream()))
     return out
@@ -569,7 +575,8 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nk
     splits = decode_splits(batch.short_tokens, nq, nkv, batch.max_ctx_len)
     return paged_attention_decode(qkv, stride, out, batch.positions, batch.seq_of, kv.block_table,
                                   kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window, splits,
-                                  q_len=batch.q_len if mixed else None, short_limit=SHORT_PORTION if mixed else 0)
+                                  q_len=batch.q_len if mixed else None, short_limit=SHORT_PORTION if mixed else 0,
+                                  live_seqs=getattr(batch, "live_seqs", None), short_rows=batch.short_tokens)
 
 
 def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, swiglu: bool = False,

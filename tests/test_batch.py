@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 from paged_llm_rs_amd.cache import CacheManager, GroupGeometry
-from paged_llm_rs_amd.engine.batch import (ContextTooLong, StepEntry, TableTooWide, build_batch, context_bound,
+from paged_llm_rs_amd.engine.batch import (ContextTooLong, ShortTokensOutgrown, StepEntry, TableTooWide, build_batch, context_bound,
                                             token_bucket)
 from paged_llm_rs_amd.errors import ConfigError
 
@@ -58,6 +58,11 @@ def test_padding_adds_a_request_that_holds_nothing_and_bounds_instead_of_counts(
     assert piece(batch, "ctx_len").tolist() == [5, 23, 0] and piece(batch, "state_slots")[2] == -1
     table = piece(batch, "block_table_0").reshape(3, -1)
     assert (table[2] == -1).all() and table[1, 0] >= 0
+    # told how many tokens the short requests bring at most, the batch reports that bound; more of them are refused
+    bounded = build_batch(entries, m, 1, 100, 0, "cpu", pad_to=32, short_bound=16)
+    assert bounded.short_tokens == 16 and bounded.max_q_len == 32
+    with pytest.raises(ShortTokensOutgrown):
+        build_batch(entries, m, 1, 100, 0, "cpu", pad_to=32, short_bound=4)
     # the same step without short requests reports no short rows; a full bucket has a request of no rows
     m2 = manager()
     full = build_batch(requests(m2, [16, 16]), m2, 1, 100, 0, "cpu", pad_to=32)

@@ -555,8 +555,15 @@ def test_paged_attention_of_portions(nq, nkv, d, bs, requests, window, splits):
         if count < limit:
             rows = out[q_start[s]:q_start[s] + count]
             assert bool((rows == 7.0).all()), "a short request is left to the other kernel"
+    # the launch has workgroups for the tokens of the short requests only when it is told how many there are at most
+    few = sum(c for c in q_len if c < limit)
+    again = out.clone()
     kernels.paged_attention_decode(q, stride, out, as_i32(positions), as_i32(seq_of), bt, bs, k_pool, v_pool, nq, nkv, d,
                                    scale, window, splits=2, q_len=q_len_t, short_limit=limit)
+    kernels.paged_attention_decode(q, stride, again, as_i32(positions), as_i32(seq_of), bt, bs, k_pool, v_pool, nq, nkv, d,
+                                   scale, window, splits=2, q_len=q_len_t, short_limit=limit, live_seqs=len(requests),
+                                   short_rows=few + 2)
+    assert torch.equal(out, again)
     g = nq // nkv
     worst = 0.0
     for i in range(n):
