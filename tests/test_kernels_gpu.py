@@ -670,6 +670,64 @@ def test_the_tiled_kernel_takes_short_requests_too(nq, nkv, d, bs, requests, win
         assert err < 1e-2, f"token {i} (request {s}, position {p}): {err:.3e}"
 
 
+@pytest.mark.parametrize("nq,nkv,d,bs", [(4, 2, 64, 16), (16, 2, 128, 16)])
+def test_attention_of_a_step_with_more_requests_than_a_wave_has_lanes(nq, nkv, d, bs):
+    """150 requests, long portions at the start, in the middle and at the end among single tokens and short
+    portions: the kernels count their work through the requests 64 at a time, so the count has to carry over."""
+    from paged_llm_rs_amd import kernels
+
+    dtype = torch.bfloat16
+    requests = []
+    for i in range(150):
+        count = {0: 40, 5: 130, 70: 17, 149: 64}.get(i, 3 if i % 11 == 0 else 1)
+        requests.append((count + (i * 7) % 90, count))
+    ctx_lens = [c for c, _ in requests]
+    bt, k_pool, v_pool, keys, values = build_paged(nkv, d, bs, ctx_lens, dtype, seed=nq)
+    n = sum(c for _, c in requests)
+    stride = (nq + 2 * nkv) * d
+    q = torch.randn(n, stride, device=DEV).to(dtype)
+    q_start, q_len, positions, seq_of = [], [], [], []
+    for s, (ctx, count) in enumerate(requests):
+        q_start.append(len(positions))
+        q_len.append(count)
+        positions += list(range(ctx - count, ctx))
+        seq_of += [s] * count
+    as_i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    scale = 1 / math.sqrt(d)
+    limit = kernels.SHORT_PORTION
+    few = sum(c for c in q_len if c < limit)
+    g = nq // nkv
+    want = [attention_ref(q[i, :nq * d].double().cpu().reshape(nq, d), keys[seq_of[i]], values[seq_of[i]], positions[i], g,
+                          scale, 0) for i in range(n)]
+
+    def check(out, rows, what):
+        for i in rows:
+            err = rel(out[i].reshape(nq, d), want[i])
+            assert err < 1e-2, f"{what}: token {i} (request {seq_of[i]}, position {positions[i]}): {err:.3e}"
+
+    long_rows = [i for i in range(n) if q_len[seq_of[i]] >= limit]
+    short_rows = [i for i in range(n) if q_len[seq_of[i]] < limit]
+    for splits in (1, 3):
+        out = torch.full((n, nq * d), 7.0, dtype=dtype, device=DEV)
+        kernels.paged_attention_prefill(q, stride, out, as_i32(q_start), as_i32(q_len), as_i32(ctx_lens), max(q_len), bt, bs,
+                                        k_pool, v_pool, nq, nkv, d, scale, 0, short_limit=limit, splits=splits)
+        assert all(bool((out[i] == 7.0).all()) for i in short_rows), "short requests are left to the other kernel"
+        check(out, long_rows, f"tiled, {splits} splits")
+        kernels.paged_attention_decode(q, stride, out, as_i32(positions), as_i32(seq_of), bt, bs, k_pool, v_pool, nq, nkv, d,
+                                       scale, 0, splits=splits, q_len=as_i32(q_len), short_limit=limit, short_rows=few + 5)
+        check(out, range(n), f"tiled and single tokens, {splits} splits")
+        out = torch.full((n, nq * d), 7.0, dtype=dtype, device=DEV)
+        kernels.paged_attention_prefill(q, stride, out, as_i32(q_start), as_i32(q_len), as_i32(ctx_lens), max(q_len), bt, bs,
+                                        k_pool, v_pool, nq, nkv, d, scale, 0, short_limit=0, splits=splits)
+        check(out, range(n), f"tiled for all, {splits} splits")
+        if kernels.library().pl_paged_attention_grouped_applies(nq, nkv, d, bs):
+            out = torch.full((n, nq * d), 7.0, dtype=dtype, device=DEV)
+            kernels.paged_attention_grouped(q, stride, out, as_i32(q_start), as_i32(q_len), as_i32(ctx_lens), limit - 1, bt, bs,
+                                            k_pool, v_pool, nq, nkv, d, scale, 0, short_limit=limit, splits=splits)
+            check(out, short_rows, f"grouped, {splits} splits")
+            assert all(bool((out[i] == 7.0).all()) for i in long_rows)
+
+
 def test_a_far_key_is_found_from_inside_a_portion():
     """One key carries nearly all the weight of one query in the middle of a long portion: a key of an
     earlier step across a page edge, a key of the same step, the query's own key, and keys at a window's edge."""
