@@ -434,11 +434,21 @@ __global__ void __launch_bounds__(256)
 paged_attention_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
                              bf16_t* __restrict__ out, const int* __restrict__ positions,
                              const int* __restrict__ seq_of, const int* __restrict__ q_len, int short_limit,
-                             int nq, int d, int splits, int n) {
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+                             int nq, int d, int splits, int n, int num_seqs) {
     const int per_token = nq * d;
-    const int t = min(idx / per_token, n - 1);
-    const int rest = idx - t * per_token;
+    int t, rest;
+    bool inside;
+    if (num_seqs > 0) {      // blockIdx.y counts the tokens of the short requests, blockIdx.x a token's elements
+        if (!ad_find_row(blockIdx.y, q_len, num_seqs, short_limit, t)) return;
+        rest = blockIdx.x * blockDim.x + threadIdx.x;
+        inside = rest < per_token;
+        rest = min(rest, per_token - 1);
+    } else {
+        const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+        t = min(idx / per_token, n - 1);
+        rest = idx - t * per_token;
+        inside = idx < n * per_token;
+    }
     const int h = rest / d, dd = rest - h * d;
     const size_t base = (static_cast<size_t>(t) * nq + h) * splits;
     const int pos = positions[t];
@@ -451,7 +461,7 @@ paged_attention_merge_kernel(const float* __restrict__ part_acc, const float* __
         ls[s] = part_ml[(base + sc) * 2 + 1];
         as[s] = part_acc[(base + sc) * d + dd];
     }
-    if (idx >= n * per_token || pos < 0 || (q_len && len >= short_limit)) return;
+    if (!inside || pos < 0 || (q_len && len >= short_limit)) return;
     float big = -INFINITY;
 #pragma unroll
     for (int s = 0; s < SP; ++s) big = fmaxf(big, s < splits ? ms[s] : -INFINITY);
@@ -493,11 +503,11 @@ static int launch_decode(const void* q, int q_stride, void* out, float* part_acc
         static_cast<bf16_t*>(v_pool), nq, nkv, d, scale * 1.4426950408889634f, window, splits, tiles, fuse);
     PL_CHECK_LAUNCH("paged_attention_decode");
     if (splits > 1) {
-        const int mgrid = pl_ceil_div(n * nq * d, 256);
+        const dim3 mgrid = compact ? dim3(pl_ceil_div(nq * d, 256), short_rows) : dim3(pl_ceil_div(n * nq * d, 256));
 #define AD_MERGE(SP)                                                                                              \
     paged_attention_merge_kernel<SP><<<mgrid, 256, 0, stream>>>(part_acc, part_ml, static_cast<bf16_t*>(out),     \
                                                                 positions, seq_of, q_len, short_limit, nq, d,     \
-                                                                splits, n)
+                                                                splits, n, compact ? num_seqs : 0)
         if (splits <= 4) AD_MERGE(4);
         else if (splits <= 8) AD_MERGE(8);
         else if (splits <= 16) AD_MERGE(16);
