@@ -97,25 +97,38 @@ std::optional<Plan> Scheduler::mixed() {
     }
     const size_t decodes = step.entries.size();
 
-    // Whatever the decodes left goes to the prompt.
-    const size_t room = budget > decodes ? budget - decodes : 0;
+    // Whatever the decodes left goes to the prompt in flight; and where that prompt ends within the budget,
+    // to the next waiting ones, as long as tokens and rows are left.  (The reference's step carries a slice
+    // of one prompt; short prompts then enter one a step however large the budget, and a batch takes as many
+    // steps to fill as it has requests.)  At most one prompt is left part-way by a step, so the next step
+    // finds one prompt in flight, as the reference's does.
+    size_t room = budget > decodes ? budget - decodes : 0;
     if (room == 0) return std::nullopt;
-    // A new prompt joins only now, after the residents have taken their pages.
-    if (!index) {
-        start_next_prompt();
-        index = prompt_in_flight();
+    bool any = false;
+    while (room > 0 && (!any || step.entries.size() < cap)) {
+        // A new prompt joins only now, after the residents have taken their pages.
+        if (!index) {
+            const size_t before = running_.size();
+            start_next_prompt();
+            if (running_.size() == before) break;
+            index = before;
+        }
+        Sequence& s = running_[*index];
+        const size_t done = s.history.size() - s.prompt_left;
+        const size_t want = std::min(room, s.prompt_left);
+        const size_t take = cache_->reserve_up_to(s.id, want);
+        if (take == 0) break;
+        const bool last = take == s.prompt_left;
+        if (last) step.ids.push_back(s.id);  // only the last portion asks for logits
+        step.advanced.emplace_back(s.id, take);
+        step.entries.push_back(entry_for(
+            s, done, std::vector<uint32_t>(s.history.begin() + done, s.history.begin() + done + take), last));
+        any = true;
+        room -= take;
+        if (!last) break;
+        index.reset();
     }
-    if (!index) return std::nullopt;
-    Sequence& s = running_[*index];
-    const size_t done = s.history.size() - s.prompt_left;
-    const size_t want = std::min(room, s.prompt_left);
-    const size_t take = cache_->reserve_up_to(s.id, want);
-    if (take == 0) return std::nullopt;
-    const bool last = take == s.prompt_left;
-    if (last) step.ids.push_back(s.id);  // only the last portion asks for logits
-    step.advanced.emplace_back(s.id, take);
-    step.entries.push_back(entry_for(
-        s, done, std::vector<uint32_t>(s.history.begin() + done, s.history.begin() + done + take), last));
+    if (!any) return std::nullopt;
 
     metrics_.steps += 1;
     metrics_.mixed_steps += 1;

@@ -353,6 +353,33 @@ def test_a_prompt_that_is_admitted_gets_a_slice_in_the_pass_that_admitted_it():
 
 # --- beyond the reference's scenarios ---------------------------------------------------------------
 
+def test_short_prompts_share_a_step_while_the_budget_lasts():
+    """Not in the reference, whose step carries a slice of one prompt: here the tokens that the first prompt
+    leaves of the budget go to the next waiting ones, and at most one prompt is left part-way."""
+    s = scheduler(256, 4, 8, chunk=32)
+    for i, n in enumerate([10, 10, 10, 10, 50], start=1):
+        submit(s, i, n, 4, prompt=[i] * n)        # nothing in common: no pages are shared
+    plan, _ = step(s)
+    # 32 tokens: three prompts whole and two tokens of the fourth
+    assert [(e.seq_id, len(e.tokens), e.want) for e in plan.entries] == [(1, 10, [9]), (2, 10, [9]), (3, 10, [9]), (4, 2, [])]
+    assert plan.ids == [1, 2, 3] and plan.kind == sched.MIXED
+    plan, _ = step(s)
+    # three decodes first, then the prompt in flight, then the next one with what is left: 3 + 8 + 21
+    assert [(e.seq_id, len(e.tokens), e.start) for e in plan.entries] == [(1, 1, 10), (2, 1, 10), (3, 1, 10), (4, 8, 2), (5, 21, 0)]
+    assert plan.ids == [1, 2, 3, 4]
+    plan, _ = step(s)
+    assert [(e.seq_id, len(e.tokens), e.start) for e in plan.entries] == [(1, 1, 11), (2, 1, 11), (3, 1, 11), (4, 1, 10), (5, 28, 21)]
+    # the rows of a step are bounded by max_batch (a step always has room for one prompt)
+    t = scheduler(256, 4, 3, chunk=32)
+    for i in range(1, 7):
+        submit(t, i, 2, 4, prompt=[i, i])
+    assert [e.seq_id for e in step(t)[0].entries] == [1, 2, 3]
+    assert [e.seq_id for e in step(t)[0].entries] == [1, 2, 3, 4]
+    while t.running or t.waiting:
+        step(t)
+    assert t.manager.available() == t.manager.total()
+
+
 def test_bad_requests_are_refused_at_submission():
     """session/sampler refusals: scheduler.rs:68-70, sampler.rs:72-95"""
     s = scheduler(8, 4, 4)
