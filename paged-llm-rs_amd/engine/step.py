@@ -30,7 +30,7 @@ from .. import kernels
 from ..errors import ConfigError, PagedLLMError, TensorError
 from .batch import CaptureOutgrown, StepBatch, TableTooWide, build_batch, context_bound, token_bucket
 
-GRAPH_MAX_REQUESTS = 64
+GRAPH_MAX_REQUESTS = 256     # requests a captured step may have (steps of more run kernel by kernel)
 SHAPE_GRAPH_ROWS_KEPT = 32768    # rows over all captured shapes of steps other than plain decoding (the
                                  # least recently used go first): their buffers stay allocated
 SHAPE_GRAPH_MAX_TOKENS = 8192
