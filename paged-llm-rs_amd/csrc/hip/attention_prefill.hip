@@ -841,7 +841,7 @@ static int launch_prefill(const void* q, int q_stride, void* out, const int* q_s
                           const int* ctx_len, int short_limit, int num_seqs, int max_q_len, const int* block_table,
                           int max_blocks, int block_size, const void* k_pool, const void* v_pool, int nq, int nkv,
                           int d, float scale, int window, int splits, float* part_acc, float* part_ml,
-                          int total_rows, hipStream_t stream) {
+                          int total_rows, int short_rows, hipStream_t stream) {
     constexpr int DP = 32 * DT;
     constexpr int BM = 32 * NW;
     const size_t tile_bytes = FEED == 2 ? (3 + 4) * static_cast<size_t>(AP_BN) * DP * 2
@@ -859,11 +859,13 @@ static int launch_prefill(const void* q, int q_stride, void* out, const int* q_s
     // The requests served bring total_rows tokens at most, and each of them short_limit at least: so many token
     // tiles there can be.  Where that is fewer than tiles of the longest times requests, workgroups are dealt
     // to the tiles that there are (ap_find_tile).
-    // (Grouped, a tile is a token: there are total_rows of them at most.)
+    // (Grouped, a tile is a token: there are total_rows of them at most, or short_rows where the caller knows
+    // how many tokens the requests served here bring together.)
     int compact = 0;
     {
         const long long served = short_limit > 0 ? (total_rows / short_limit < num_seqs ? total_rows / short_limit : num_seqs) : num_seqs;
-        const long long bound = GR ? total_rows : (total_rows + served * (BM - 1)) / BM;
+        const long long bound = GR ? (short_rows > 0 && short_rows < total_rows ? short_rows : total_rows)
+                                   : (total_rows + served * (BM - 1)) / BM;
         if (bound < static_cast<long long>(tiles) * num_seqs) {
             compact = 1;
             whole = bound * (GR ? nkv : nq);
@@ -902,7 +904,7 @@ static int ap_dispatch(bool small, bool uniform_pages, const void* q, int q_stri
 #define AP_LAUNCH(NW, KS, FEED)                                                                                    \
     launch_prefill<D, NW, KS, FEED>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len,    \
                                     block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale, window, \
-                                    splits, part_acc, part_ml, total_rows, stream)
+                                    splits, part_acc, part_ml, total_rows, 0, stream)
     constexpr bool can_fit = 64 % (4 * D) == 0;
     constexpr int BEST = (D == 2 || D == 4) && AP_KS == 2 && AP_SMALL_KS == 2 ? AP_FEED : 1;   // the feed with uniform pages
     if constexpr (D <= 4) {
@@ -986,6 +988,7 @@ extern "C" int pl_paged_attention_prefill(const void* q, int q_stride, void* out
 // short_limit tokens or more are the ones left out (0: none is), and max_q_len bounds the tokens of those
 // that are served.  Heads of 64 or 128, groups of up to 32, pages of a power of two of at least
 // 64 / (head size / 8) tokens; pl_paged_attention_grouped_applies says whether a shape is served.
+// short_rows: the most tokens that the requests served bring together (0: not known, the step's rows then).
 extern "C" int pl_paged_attention_grouped_applies(int nq, int nkv, int d, int block_size) {
     if (nq <= 0 || nkv <= 0 || nq % nkv || nq / nkv > 32 || (d != 64 && d != 128)) return 0;
     const int rows_a_load = 64 / (d / 8);
@@ -997,7 +1000,7 @@ extern "C" int pl_paged_attention_grouped(const void* q, int q_stride, void* out
                                           int max_q_len, const int* block_table, int max_blocks, int block_size,
                                           const void* k_pool, const void* v_pool, int nq, int nkv, int d,
                                           float scale, int window, int splits, float* part_acc, float* part_ml,
-                                          int total_rows, hipStream_t stream) {
+                                          int total_rows, int short_rows, hipStream_t stream) {
     PL_REQUIRE(pl_paged_attention_grouped_applies(nq, nkv, d, block_size),
                "grouped attention: %d query heads over %d key heads of %d, pages of %d", nq, nkv, d, block_size);
     PL_REQUIRE(splits >= 1 && splits <= AP_MERGE_MAX && (splits == 1 || (part_acc && part_ml)),
@@ -1009,8 +1012,8 @@ extern "C" int pl_paged_attention_grouped(const void* q, int q_stride, void* out
     if (d == 64)
         return launch_prefill<2, 1, 2, 2, true>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len,
                                                 block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale,
-                                                window, splits, part_acc, part_ml, total_rows, stream);
+                                                window, splits, part_acc, part_ml, total_rows, short_rows, stream);
     return launch_prefill<4, 1, 2, 2, true>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len,
                                             block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale,
-                                            window, splits, part_acc, part_ml, total_rows, stream);
+                                            window, splits, part_acc, part_ml, total_rows, short_rows, stream);
 }

@@ -43,7 +43,7 @@ def _signatures(lib) -> None:
         "pl_paged_attention_decode": [p, i, p, p, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, i, f, i, i,
                                       i, p, p, i, f, p, p, i, p],
         "pl_paged_attention_prefill": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, i, p],
-        "pl_paged_attention_grouped": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, i, p],
+        "pl_paged_attention_grouped": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, i, i, p],
         "pl_paged_attention_grouped_applies": [i, i, i, i],
     }
     for name, argtypes in table.items():
@@ -484,7 +484,7 @@ def paged_attention_grouped(q: torch.Tensor, q_row_stride: int, out: torch.Tenso
         q.data_ptr(), q_row_stride, out.data_ptr(), q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(),
         int(short_limit), live, int(max_q_len), block_table.data_ptr(), block_table.shape[1], block_size,
         k_pool.data_ptr(), v_pool.data_ptr(), nq, nkv, d, float(scale), int(window or 0), int(splits),
-        part_acc.data_ptr() if splits > 1 else None, part_ml.data_ptr() if splits > 1 else None, n, _stream()))
+        part_acc.data_ptr() if splits > 1 else None, part_ml.data_ptr() if splits > 1 else None, n, int(tokens or 0), _stream()))
     return out
 
 
