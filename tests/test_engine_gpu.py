@@ -358,4 +358,45 @@ def test_requests_that_arrive_and_are_cancelled_while_others_run(model_dirs, cas
         assert m["available"] == m["total"]
 
 
+@pytest.mark.parametrize("name,seed", [("D", 0), ("E", 1)])
+def test_a_long_run_of_arrivals_gives_the_same_tokens_from_graphs_as_kernel_by_kernel(model_dirs, name, seed, monkeypatch):
+    """A hundred requests of drawn lengths arriving over some hundred steps, in bfloat16, greedy and drawn:
+    steps of many shapes are captured, dropped again (few rows of captured shapes are kept here) and
+    captured again, tables and contexts outgrow their captures; every token is the one that the same
+    engine gives when it launches every step kernel by kernel."""
+    import random
+
+    from paged_llm_rs_amd import Engine
+    from paged_llm_rs_amd.engine import step as step_module
+
+    monkeypatch.setattr(step_module, "SHAPE_GRAPH_ROWS_KEPT", 2048)
+    rng = random.Random(seed)
+    vocab = TINY_INIT[name]["config"]["vocab_size"]
+    head = [rng.randrange(vocab) for _ in range(48)]
+    requests, at = [], 0
+    for i in range(100):
+        at += rng.choice([0, 0, 1, 2, 5, 20])
+        body = [rng.randrange(vocab) for _ in range(rng.choice([rng.randint(1, 40), rng.randint(100, 400)]))]
+        sampling = rng.choice([dict(temperature=0.0), dict(temperature=0.9, top_k=40, top_p=0.95, seed=i)])
+        requests.append(((head if rng.random() < 0.3 else []) + body, rng.randint(1, 40), sampling, at))
+    settings = dict(block_size=16, num_blocks=400, max_batch=rng.choice([8, 24, 64]), chunk=rng.choice([64, 128, 512]))
+    d = model_dirs(name, "bfloat16")
+    tokens = {}
+    for graphs in (False, True):
+        engine = Engine(d, dtype="bf16", graphs=graphs, **settings)
+        ids, step = {}, 0
+        while len(ids) < len(requests) or engine.open_requests:
+            for r, (prompt, most, sampling, arrives) in enumerate(requests):
+                if r not in ids and arrives <= step:
+                    ids[r] = engine.submit(prompt, most, stop_tokens=[], **sampling)
+            if engine.open_requests:
+                engine.step()
+            step += 1
+            assert step < 5000
+        tokens[graphs] = [engine.take_result(ids[r]).tokens for r in range(len(requests))]
+        if graphs:
+            assert engine.runner.graph_steps > 5 * engine.runner.eager_steps
+    assert tokens[True] == tokens[False]
+
+
 import numpy as np  # noqa: E402
