@@ -299,7 +299,9 @@ class StepRunner:
         rows = token_bucket(tokens) if self.pads and tokens <= SHAPE_GRAPH_MAX_TOKENS else None
         # the tokens of requests that bring few, rounded up: the kernel for single tokens gets so many workgroups
         short = sum(len(e.tokens) for e in entries if len(e.tokens) < kernels.SHORT_PORTION)
-        short_bound = None if rows is None else min(rows, _bucket(short, 16)) if short else 0
+        short_bound = None
+        if rows is not None:
+            short_bound = min(rows, _bucket(short, 16)) if short else 0
         if not self.use_graphs or rows is None or len(entries) > GRAPH_MAX_REQUESTS:
             self.eager_steps += 1
             return StepOutput(run_step(self.model, self.cache, entries, pad_to=rows, short_bound=short_bound))
