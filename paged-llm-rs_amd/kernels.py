@@ -294,15 +294,17 @@ def set_attention(mode: str) -> None:
 
 def decode_splits(tokens: int, nq: int, nkv: int, max_ctx: int) -> int:
     """How many stretches the context is cut into, so that a launch fills the chip: none when the
-    tokens and heads alone give two workgroups a compute unit, else up to about that many
-    workgroups, each with at least 128 keys (two rounds of loads).  (Twice as many shares were slower
-    wherever they were measured: 8 tokens at context 4,096, 39.7 us with 16 shares against 34.0 with 4.)"""
+    tokens and heads alone give a workgroup a compute unit (two, with more than two query heads a key
+    head: a workgroup then has more arithmetic a key), else up to about that many workgroups, each with at
+    least 128 keys (two rounds of loads).  (More shares were slower wherever they were measured, 1 to 64
+    tokens at contexts of 512 to 4,096: 8 tokens at context 4,096 take 39.7 us with 16 shares and 34.0 with 4.)"""
     g = nq // nkv
     gt = 8 if g >= 8 else (4 if g > 2 else g)
     base = max(tokens * nkv * ((g + gt - 1) // gt), 1)
-    if base >= 512:
+    target = 256 if g <= 2 else 512
+    if base >= target:
         return 1
-    return max(1, min((512 + base - 1) // base, (max_ctx + 127) // 128, 64))
+    return max(1, min((target + base - 1) // base, (max_ctx + 127) // 128, 64))
 
 
 def paged_attention_decode(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, positions: torch.Tensor,
