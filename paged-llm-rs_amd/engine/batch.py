@@ -64,11 +64,15 @@ class StepBatch:
 
 
 def context_bound(longest: int) -> int:
-    """What a step reports as its longest context: the power of two (1024 at least) that holds it.  The
-    kernels size their launches and choose how to split the keys by it, so steps of one shape whose
-    contexts share a bound run the same launches, captured in a graph or not."""
+    """What a step reports as its longest context: the power of two (1024 at least), or one and a half
+    times a power of two, that holds it.  The kernels size their launches and choose how to split the keys
+    by it, so steps of one shape whose contexts share a bound run the same launches, captured in a graph or
+    not.  (Powers of two alone overstate a context by up to a factor of two, and the keys were then dealt
+    to more workgroups than paid.)"""
     bound = 1024
     while bound < longest:
+        if bound + bound // 2 >= longest:
+            return bound + bound // 2
         bound *= 2
     return bound
 

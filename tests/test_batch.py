@@ -34,7 +34,7 @@ def piece(batch, name):
 def test_buckets():
     assert [token_bucket(n) for n in (1, 16, 17, 33, 64, 65, 128, 1000, 1024, 1025, 2048, 2049)] == \
         [16, 16, 32, 64, 64, 128, 128, 1024, 1024, 1280, 2048, 2304]
-    assert [context_bound(n) for n in (1, 1024, 1025, 5000)] == [1024, 1024, 2048, 8192]
+    assert [context_bound(n) for n in (1, 1024, 1025, 1537, 5000, 6145)] == [1024, 1024, 1536, 2048, 6144, 8192]
 
 
 def test_a_step_without_padding_reports_what_it_holds():
