@@ -401,9 +401,11 @@ gemm_skinny_rows_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ 
     constexpr int NKS = WV / MT;                                // stretches of K
     extern __shared__ float sk_lds[];
     bf16_t* panel = reinterpret_cast<bf16_t*>(sk_lds);          // [BT * 16][K], pieces permuted
-    float* gain_lds = sk_lds + BT * 16 * K / 2;                 // [K] (PRO_NORM)
     float* red = sk_lds;                                        // [NKS][MT][BT][256], once the panel is done with
-    float* ssq_lds = sk_lds + NKS * MT * BT * 256;              // [NKS][MT][16]
+    // The gains are loaded once and read for every tile of columns, the sums of squares are written for
+    // every tile: both lie behind the larger of the panel and the partial tiles, which alone share a place.
+    float* gain_lds = sk_lds + max(BT * 16 * K / 2, NKS * MT * BT * 256);   // [K] (PRO_NORM)
+    float* ssq_lds = gain_lds + (PRO == PRO_NORM ? K : 0);      // [NKS][MT][16]
 
     const int lane = threadIdx.x % PL_WAVE;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PL_WAVE);
@@ -559,9 +561,11 @@ static int launch_rows(const void* x, const void* w, void* y, const float* gain,
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
     constexpr int NKS = WV / MT;
     const int grid = min(pl_ceil_div(N_out, SK_TILE_N), SK_MAX_GRID);
-    const size_t panel_bytes = static_cast<size_t>(BT) * 16 * K * 2 + (PRO == PRO_NORM ? static_cast<size_t>(K) * 4 : 0);
-    const size_t red_bytes = static_cast<size_t>(NKS) * MT * (BT * 256 + 16) * sizeof(float);
-    const size_t lds_bytes = panel_bytes > red_bytes ? panel_bytes : red_bytes;
+    const size_t panel_bytes = static_cast<size_t>(BT) * 16 * K * 2;
+    const size_t red_bytes = static_cast<size_t>(NKS) * MT * BT * 256 * sizeof(float);
+    const size_t lds_bytes = (panel_bytes > red_bytes ? panel_bytes : red_bytes)
+                             + (PRO == PRO_NORM ? static_cast<size_t>(K) * 4 : 0)      // the gains
+                             + static_cast<size_t>(NKS) * MT * 16 * sizeof(float);     // the sums of squares
     auto kernel = &gemm_skinny_rows_kernel<MT, WV, STEPS, PRO, EPI, OUT>;
     if (lds_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,

@@ -142,12 +142,17 @@ LAYERS_WIDE = {
     "tie_word_embeddings": False,
 }
 
+# The same two layers under the family's real vocabulary, tied: the projection onto it walks its column
+# tiles in a loop (few rows) or goes to the library (many), which no smaller vocabulary shows.
+LAYERS_0P6B_REAL_VOCAB = dict(LAYERS_0P6B, vocab_size=151936)
+
 TINY_INIT = {
     "A": dict(config=TINY_A, seed=0, std=0.02, gain_std=0.1),
     "B": dict(config=TINY_B, seed=1, std=0.05, gain_std=0.2),
     "C": dict(config=TINY_C, seed=2, std=0.08, gain_std=0.2),
     "D": dict(config=LAYERS_0P6B, seed=3, std=0.02, gain_std=0.1),
     "E": dict(config=LAYERS_WIDE, seed=4, std=0.02, gain_std=0.1),
+    "V": dict(config=LAYERS_0P6B_REAL_VOCAB, seed=5, std=0.02, gain_std=0.1),
 }
 
 

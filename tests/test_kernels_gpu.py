@@ -259,6 +259,84 @@ def test_gemm_skinny_with_the_norm_before_and_the_residual_after(n, N, K):
     assert rel(resid, want) < 1e-5
 
 
+def one_hot_rows(n, K):
+    """Rows that pick single columns of a weight matrix, and the columns they pick."""
+    eye = torch.zeros(n, K, device=DEV, dtype=torch.bfloat16)
+    idx = torch.randint(0, K, (n,), device=DEV)
+    eye[torch.arange(n, device=DEV), idx] = 1
+    return eye, idx
+
+
+@pytest.mark.parametrize("N", [32768, 32784, 151936])
+@pytest.mark.parametrize("K", [512, 1024, 4096, 5120])
+def test_gemm_skinny_against_more_columns_than_a_launch_has_workgroups(N, K):
+    """Beyond 32,768 columns a workgroup walks several tiles of columns and uses its LDS again for each:
+    the projection onto a real vocabulary does so in every decode step.  One-hot rows pick single
+    weights, so a tile that is dropped, written twice or mixed with its neighbour cannot pass."""
+    from paged_llm_rs_amd import kernels
+
+    w = torch.randn(N, K, device=DEV).to(torch.bfloat16)
+    w64 = w.double()
+    for n in (1, 8, 16, 17, 33, 64):
+        x = torch.randn(n, K, device=DEV).to(torch.bfloat16)
+        want = x.double() @ w64.T
+        assert rel(kernels.gemm_skinny(x, w, torch.float32), want) < 1e-5, f"{n} rows, 32-bit out"
+        assert rel(kernels.gemm_skinny(x, w, torch.bfloat16), want) < 6e-3, f"{n} rows, bfloat16 out"
+        eye, idx = one_hot_rows(n, K)
+        picked = w[:, idx].T.contiguous()
+        assert torch.equal(kernels.gemm_skinny(eye, w, torch.bfloat16), picked), f"{n} one-hot rows"
+        assert torch.equal(kernels.gemm_skinny(eye, w, torch.float32), picked.float()), f"{n} one-hot rows, 32-bit out"
+    # the gated product's tiles are pairs of column tiles: its loop starts at 65,536 rows of w
+    if N % 2 == 0:
+        for n in (1, 17, 64):
+            x = (torch.randn(n, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
+            both = x.double() @ w64.T
+            act = torch.nn.functional.silu(both[:, :N // 2]) * both[:, N // 2:]
+            assert rel(kernels.gemm_skinny(x, w, swiglu=True), act) < 6e-3, f"{n} rows, gated"
+
+
+@pytest.mark.parametrize("N", [32784, 151936])
+@pytest.mark.parametrize("K", [512, 1024, 4096])
+def test_gemm_skinny_with_the_norm_before_against_many_columns(N, K):
+    """The norm as the first stage of a product that walks its column tiles: the gains and the rows'
+    statistics have to outlast every tile (K = 512 is where gains and statistics once shared LDS)."""
+    from paged_llm_rs_amd import kernels
+
+    eps = 1e-5
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
+    w64 = w.double()
+    gain = 1 + 0.3 * torch.randn(K, device=DEV)
+    for n in (1, 8, 17, 33, 64):
+        stream = torch.randn(n + 3, K, device=DEV) * 3.0
+        stream[0] *= 50.0
+        picked = [(7 * i + 2) % (n + 3) for i in range(n)]
+        x = stream[picked].double()
+        normed = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * gain.double()
+        rows = torch.tensor(picked, dtype=torch.int32, device=DEV)
+        got = kernels.gemm_skinny(stream, w, torch.float32, norm_gain=gain, eps=eps, rows=rows)
+        # the kernel multiplies bf16(x * gain) and scales afterwards: compare with exactly that, tightly ...
+        exact = (x.float() * gain).to(torch.bfloat16).double() @ w64.T / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+        assert rel(got, exact) < 1e-5, f"{n} rows against the kernel's own rounding"
+        # ... and with the unrounded norm at bfloat16's precision
+        assert rel(got, normed @ w64.T) < 6e-3, f"{n} rows"
+
+
+@pytest.mark.parametrize("M,K", [(65, 1024), (300, 1024), (2048, 1024), (70, 4096), (300, 5120)])
+def test_the_librarys_projection_onto_a_real_vocabulary(M, K):
+    """More than 64 rows against 151,936 columns go to the library with 32-bit output
+    (``linear_bf16``): compared with 64-bit products, not with the library itself."""
+    from paged_llm_rs_amd import kernels
+
+    N = 151936
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
+    x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    got = kernels.linear_bf16(x, w, torch.float32)
+    assert got.dtype == torch.float32 and got.shape == (M, N)
+    assert rel(got, x.double() @ w.double().T) < 1e-5
+    eye, idx = one_hot_rows(M, K)
+    assert torch.equal(kernels.linear_bf16(eye, w, torch.float32), w[:, idx].T.float().contiguous())
+
+
 @pytest.mark.parametrize("M", [1, 127, 128, 300, 2048])
 @pytest.mark.parametrize("N,K", [(128, 32), (256, 96), (1024, 1024), (384, 2080)])
 @pytest.mark.parametrize("kind", ["store", "swiglu", "add"])

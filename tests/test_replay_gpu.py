@@ -25,7 +25,10 @@ pytestmark = pytest.mark.gpu
 # or three layers and a head that is a few times 1e-3 of the largest logit.
 TOLERANCE = {"float32": 1e-5, "bfloat16": 2e-2}
 LENGTHS = {"A": [5, 17, 33, 70, 100, 41], "B": [1, 9, 24, 40, 129, 66], "C": [3, 50, 97, 64, 20, 35],
-           "D": [300, 70, 33, 150], "E": [260, 70, 33, 150]}
+           "D": [300, 70, 33, 150], "E": [260, 70, 33, 150],
+           # whole requests of these lengths put 70 and 150 rows (the library), 33, 20 and 50 rows (the three
+           # shapes of the product for 17 to 64 rows) before the projection onto the vocabulary
+           "V": [70, 33, 150, 20, 50]}
 
 
 @pytest.fixture(scope="module")
@@ -54,7 +57,7 @@ def replay(model_dir, dtype, prompts, steps, max_live, block_size=16):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "V"])
 def test_whole_requests(setups, name, dtype):
     d, prompts, want = setups(name, dtype)
     got = replay(d, dtype, prompts, ru.whole(prompts), max_live=1)
@@ -64,7 +67,7 @@ def test_whole_requests(setups, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,block_size", [("A", 16), ("B", 8), ("C", 4), ("D", 16), ("E", 16)])
+@pytest.mark.parametrize("name,block_size", [("A", 16), ("B", 8), ("C", 4), ("D", 16), ("E", 16), ("V", 16)])
 def test_last_tokens_decoded_one_by_one(setups, name, dtype, block_size):
     d, prompts, want = setups(name, dtype)
     got = replay(d, dtype, prompts, ru.tail_decoded(prompts, 32), max_live=1, block_size=block_size)
@@ -85,7 +88,7 @@ def test_portions_of_changing_size(setups, name, dtype, block_size):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name,block_size,seed", [("A", 16, 1), ("B", 8, 2), ("C", 4, 3), ("B", 16, 4), ("D", 16, 5),
-                                                    ("E", 16, 6)])
+                                                    ("E", 16, 6), ("V", 16, 7)])
 def test_mixed_requests_with_pages_used_again(setups, name, dtype, block_size, seed):
     d, prompts, want = setups(name, dtype)
     steps = ru.mixed(prompts, seed=seed, max_live=4)
