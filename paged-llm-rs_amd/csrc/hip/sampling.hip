@@ -1,5 +1,8 @@
 // Choosing the next token on the device.
 #include "common.hpp"
+#include "no_alloc.h"
+
+#include <mutex>
 
 // ---------------------------------------------------------------------------
 // Greedy: the index of the largest logit of each row; the first maximum wins
@@ -74,6 +77,47 @@ extern "C" int pl_argmax(const float* logits, int* out, float* scratch_v, int* s
     argmax_stage1_kernel<<<dim3(ARGMAX_CHUNKS, m), 256, 0, stream>>>(logits, scratch_v, scratch_i, V);
     PL_CHECK_LAUNCH("argmax");
     argmax_stage2_kernel<<<m, 64, 0, stream>>>(scratch_v, scratch_i, out);
+    PL_CHECK_LAUNCH("argmax");
+    return 0;
+}
+
+// The same two kernels over scratch memory that the library owns, for callers that cannot allocate.
+// The array's name is only a handle on the host: what kernels are given is its address on the current
+// device, asked for once a device (every GPU holds its own copy at its own address).
+static __device__ __align__(256) unsigned char scratch[PL_ARGMAX_STATIC_MAX_ROWS * ARGMAX_CHUNKS * (sizeof(float) + sizeof(int))];
+
+#define PL_MAX_DEVICES 64
+static std::mutex scratch_lock;
+static void* scratch_on_device[PL_MAX_DEVICES];
+
+static int scratch_address(void** at) {
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    PL_REQUIRE(e == hipSuccess, "argmax: no current device: %s", hipGetErrorString(e));
+    PL_REQUIRE(device >= 0 && device < PL_MAX_DEVICES, "argmax: device %d is beyond the %d this library counts", device, PL_MAX_DEVICES);
+    std::lock_guard<std::mutex> hold(scratch_lock);
+    if (!scratch_on_device[device]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        PL_REQUIRE(e == hipSuccess && ptr, "argmax: the scratch array has no address on device %d: %s", device, hipGetErrorString(e));
+        scratch_on_device[device] = ptr;
+    }
+    *at = scratch_on_device[device];
+    return 0;
+}
+
+extern "C" int pl_argmax_static(const float* logits, int* out, int m, int V, hipStream_t stream) {
+    PL_REQUIRE(m >= 0 && V > 0, "argmax: rows %d, vocabulary %d", m, V);
+    PL_REQUIRE(m <= PL_ARGMAX_STATIC_MAX_ROWS, "argmax: %d rows, the scratch array of this entry point holds %d", m,
+               PL_ARGMAX_STATIC_MAX_ROWS);
+    if (m == 0) return 0;
+    void* base = nullptr;
+    if (int code = scratch_address(&base)) return code;
+    float* part_v = static_cast<float*>(base);
+    int* part_i = reinterpret_cast<int*>(part_v + PL_ARGMAX_STATIC_MAX_ROWS * ARGMAX_CHUNKS);
+    argmax_stage1_kernel<<<dim3(ARGMAX_CHUNKS, m), 256, 0, stream>>>(logits, part_v, part_i, V);
+    PL_CHECK_LAUNCH("argmax");
+    argmax_stage2_kernel<<<m, 64, 0, stream>>>(part_v, part_i, out);
     PL_CHECK_LAUNCH("argmax");
     return 0;
 }
