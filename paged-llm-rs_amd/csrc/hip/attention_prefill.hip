@@ -109,9 +109,13 @@ __device__ __forceinline__ int ap_value_shift(int r, int pieces) { return 4 * ((
 // UP (uniform pages): the 64 / (4*DT) keys whose pieces one wave loads with one instruction lie in one
 // page (the page size is a power of two and at least as many keys).  Page numbers then come through
 // the scalar unit and an address is a scalar base plus a lane's constant: no vector arithmetic a tile.
-// What is loaded is not masked on this path: scores of keys that do not exist are masked anyway, and
-// their values are multiplied by zero, so the pages have to hold finite numbers everywhere (the
-// pools are allocated zeroed).
+// What is loaded is not masked on this path.  Scores of keys that do not exist are replaced, not
+// multiplied, so whatever their rows of the key pool hold is never seen.  Their values are multiplied by
+// a probability of exactly zero, which only gives zero for a finite value: a page keeps what its last
+// owner left there, and that may be anything.  So a lane whose value row lies past the last key that the
+// tile's queries see, or before the first (a window's pages may have been given back), reads the last
+// key's row instead, a row that this request wrote; only the first and the last tile of keys of a
+// workgroup have such rows, and only there the addresses are chosen lane by lane.
 //
 // FEED 0: any page size, tiles travel through registers and are masked.  1: uniform pages, through
 // registers.  2: uniform pages, and the loads write LDS themselves (global_load_lds_dwordx4: lane l of
@@ -286,12 +290,20 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     // A lookup leaves the table's answer raw: what depends on it is computed by the fetch, one tile
     // later, so that the wait for the answer stands there and not in the middle of this tile.
     int kblk[KI], kwithin[KI];       // UP: the page of the wave's keys of piece i and their first row in it
+    int kj0[KI];                     // UP: the key that this row is
     bool kin[KI];
     uint32_t keep[KI];
     const int log2_bs = 31 - __builtin_clz(static_cast<unsigned>(block_size));
     const uint32_t row_bytes = static_cast<uint32_t>(nkv) * d * 2;
     // UP: this lane's place beside the wave's base: its row among the wave's rows, its piece of the row
-    const uint32_t lane_place = (lane / CP) * row_bytes + static_cast<uint32_t>(head_off + min(lane % CP, cpr - 1) * 8) * 2;
+    const uint32_t lane_piece = static_cast<uint32_t>(head_off + min(lane % CP, cpr - 1) * 8) * 2;
+    const uint32_t lane_place = (lane / CP) * row_bytes + lane_piece;
+    // UP: the row of the last key that the tile's queries see, where the values of later rows are read from
+    size_t last_base = 0;
+    if constexpr (UP) {
+        const int last_page = __builtin_amdgcn_readfirstlane(max(table[last_pos >> log2_bs], 0));
+        last_base = (static_cast<size_t>(last_page) * block_size + (last_pos & (block_size - 1))) * row_bytes;
+    }
     auto locate = [&](int j, int& blk, int& within, bool& in) {  // page and place in the page of key j
         in = j <= last_pos;
         const int jj = in ? j : last_pos;
@@ -309,6 +321,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
                 // the first key of the wave's rows; past the last key the page of the last key serves
                 // (its rows exist, and what they hold is never seen)
                 const int j0 = k0 + (64 * wave_id + i * NT) / CP;
+                kj0[i] = j0;
                 kwithin[i] = j0 & (block_size - 1);
                 kblk[i] = table[__builtin_amdgcn_readfirstlane(min(j0, last_pos) >> log2_bs)];
             } else {
@@ -318,12 +331,13 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     };
     // UP: the scalar unit answers slowly, so the pages of the tile after the next are asked for at the
     // start of the half round whose end needs them
-    int ahead_blk[KI], ahead_within[KI];
+    int ahead_blk[KI], ahead_within[KI], ahead_j0[KI];
     auto look_ahead = [&](int k0) {
         if constexpr (UP) {
 #pragma unroll
             for (int i = 0; i < KI; ++i) {
                 const int j0 = k0 + (64 * wave_id + i * NT) / CP;
+                ahead_j0[i] = j0;
                 ahead_within[i] = j0 & (block_size - 1);
                 ahead_blk[i] = table[__builtin_amdgcn_readfirstlane(min(j0, last_pos) >> log2_bs)];
             }
@@ -341,7 +355,12 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
                 const int page = __builtin_amdgcn_readfirstlane(max(kblk[i], 0));
                 const size_t base = (static_cast<size_t>(page) * block_size + kwithin[i]) * row_bytes;
                 kreg[i] = *reinterpret_cast<const ap_vec4*>(reinterpret_cast<const char*>(k_pool) + base + lane_place);
-                vreg[i] = *reinterpret_cast<const ap_vec4*>(reinterpret_cast<const char*>(v_pool) + base + lane_place);
+                size_t vat = base + lane_place;
+                if (kj0[i] + 64 / CP - 1 > last_pos || kj0[i] < first_pos) {   // (the same for the wave)
+                    const int j = kj0[i] + lane / CP;
+                    vat = (j > last_pos || j < first_pos) ? last_base + lane_piece : vat;
+                }
+                vreg[i] = *reinterpret_cast<const ap_vec4*>(reinterpret_cast<const char*>(v_pool) + vat);
             } else {
                 const int c = (tid + i * NT) % CP;
                 const size_t at = row_of(kblk[i], kwithin[i]) + head_off + min(c, cpr - 1) * 8;
@@ -395,14 +414,15 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     // mod 16, and with it the permutation, alternates between two values from one load to the next.)
     constexpr bool ROWS_ALTERNATE = DIRECT && (NT / CP) % 16 != 0;
     static_assert(!DIRECT || (2 * NT / CP) % 16 == 0, "the rows of a wave's loads repeat mod 16 after two loads at most");
-    uint32_t place_k[2] = {0, 0}, place_v[2] = {0, 0};
+    uint32_t place_k[2] = {0, 0}, place_v[2] = {0, 0}, piece_v[2] = {0, 0};
     if constexpr (DIRECT) {
 #pragma unroll
         for (int odd = 0; odd < 2; ++odd) {
             const int r15 = ((64 * wave_id + odd * NT) / CP + lane / CP) & 15;
             const int ck = (lane % CP) ^ ap_key_shift(r15, CP), cv = (lane % CP) ^ ap_value_shift(r15, CP);
             place_k[odd] = (lane / CP) * row_bytes + static_cast<uint32_t>(head_off + min(ck, cpr - 1) * 8) * 2;
-            place_v[odd] = (lane / CP) * row_bytes + static_cast<uint32_t>(head_off + min(cv, cpr - 1) * 8) * 2;
+            piece_v[odd] = static_cast<uint32_t>(head_off + min(cv, cpr - 1) * 8) * 2;
+            place_v[odd] = (lane / CP) * row_bytes + piece_v[odd];
         }
     }
     auto ask = [&]() {               // pages from kblk/kwithin, looked up before
@@ -414,6 +434,11 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
                 const size_t base = (static_cast<size_t>(page) * block_size + kwithin[i]) * row_bytes;
                 const char* gk = reinterpret_cast<const char*>(k_pool) + base + place_k[ROWS_ALTERNATE ? i & 1 : 0];
                 const char* gv = reinterpret_cast<const char*>(v_pool) + base + place_v[ROWS_ALTERNATE ? i & 1 : 0];
+                if (kj0[i] + 64 / CP - 1 > last_pos || kj0[i] < first_pos) {   // (the same for the wave)
+                    const int j = kj0[i] + lane / CP;
+                    if (j > last_pos || j < first_pos)
+                        gv = reinterpret_cast<const char*>(v_pool) + last_base + piece_v[ROWS_ALTERNATE ? i & 1 : 0];
+                }
                 uint16_t* lk = Kbase + asked_k * KTILE + first_row * KROW;
                 uint16_t* lv = Vbase + asked_v * VTILE + first_row * VROW;
                 ap_load_to_lds(gk, lk);
@@ -429,6 +454,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         for (int i = 0; i < KI; ++i) {
             kblk[i] = ahead_blk[i];
             kwithin[i] = ahead_within[i];
+            kj0[i] = ahead_j0[i];
         }
     };
     if constexpr (DIRECT) {

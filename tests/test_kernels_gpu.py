@@ -435,14 +435,46 @@ def build_paged(nkv, d, bs, ctx_lens, dtype, seed=0, pages_extra=7):
     v_pool = torch.randn(pages * bs, nkv * d, generator=g).to(dtype)
     keys, values = [], []
     at = 0
+    used = torch.zeros(pages * bs, dtype=torch.bool)
     for s, c in enumerate(ctx_lens):
         for b in range(need[s]):
             bt[s, b] = order[at]
             at += 1
         slots = [int(bt[s, p // bs]) * bs + p % bs for p in range(c)]
+        used[slots] = True
         keys.append(k_pool[slots].reshape(c, nkv, d).double())
         values.append(v_pool[slots].reshape(c, nkv, d).double())
+    # Every row that belongs to no request (the rest of a last page, pages that are free) holds what a
+    # page's last owner may have left there: infinities, NaNs and the largest finite numbers.
+    k_pool[~used] = poison_rows(int((~used).sum()), nkv * d, dtype)
+    v_pool[~used] = poison_rows(int((~used).sum()), nkv * d, dtype)
     return bt.to(DEV), k_pool.to(DEV), v_pool.to(DEV), keys, values
+
+
+def give_back_pages_behind_the_window(bt, k_pool, v_pool, bs, requests, window):
+    """What a windowed cache group does: the pages that lie wholly before the window of a request's first
+    token of the step are no longer the request's (-1 in its table) and hold anything."""
+    if not window:
+        return
+    for s, (ctx, count) in enumerate(requests):
+        first_needed = max(0, ctx - count + 1 - window)
+        for b in range(first_needed // bs):
+            page = int(bt[s, b])
+            for pool in (k_pool, v_pool):
+                pool[page * bs:(page + 1) * bs] = poison_rows(bs, pool.shape[1], pool.dtype).to(pool.device)
+            bt[s, b] = -1
+
+
+def same_bits(a, b):
+    """Equal bit for bit, NaNs included."""
+    as_int = torch.int16 if a.element_size() == 2 else torch.int32
+    return a.shape == b.shape and torch.equal(a.view(as_int), b.view(as_int))
+
+
+def poison_rows(rows, width, dtype):
+    pattern = torch.tensor([float("inf"), float("nan"), 3e38, float("-inf")])
+    at = (torch.arange(rows)[:, None] + torch.arange(width)[None]) % 4
+    return pattern[at].to(dtype)
 
 
 def attention_ref(q, keys, values, pos, g, scale, window):
@@ -575,7 +607,7 @@ def test_decode_attention_that_prepares_its_own_queries_and_keys(nq, nkv, d, bs,
     k_b, v_b = k_pool.clone(), v_pool.clone()
     kernels.paged_attention_decode(raw, stride, got, positions, seq_of, bt, bs, k_b, v_b, nq, nkv, d, scale, window, splits,
                                    fuse=kernels.QkFusion(q_gain, k_gain, 1e-5, cos, sin, rot, True))
-    assert torch.equal(k_a, k_b) and torch.equal(v_a, v_b), "the same keys and values in the same places"
+    assert same_bits(k_a, k_b) and same_bits(v_a, v_b), "the same keys and values in the same places"
     assert rel(got[:-1], want[:-1]) < 4e-3
     assert bool((got[-1] == 7.0).all()), "a padding row is not written"
     # queries only: a layer that reads pages another layer wrote
@@ -613,6 +645,7 @@ def test_paged_attention_of_portions(nq, nkv, d, bs, requests, window, splits):
     dtype = torch.bfloat16
     ctx_lens = [c for c, _ in requests]
     bt, k_pool, v_pool, keys, values = build_paged(nkv, d, bs, ctx_lens, dtype, seed=d + bs + len(requests))
+    give_back_pages_behind_the_window(bt, k_pool, v_pool, bs, requests, window)
     n = sum(c for _, c in requests)
     stride = (nq + 2 * nkv) * d
     q = torch.randn(n, stride, device=DEV).to(dtype)
@@ -677,6 +710,7 @@ def test_paged_attention_with_a_group_of_heads_as_the_rows_of_a_tile(nq, nkv, d,
     dtype = torch.bfloat16
     ctx_lens = [c for c, _ in requests]
     bt, k_pool, v_pool, keys, values = build_paged(nkv, d, bs, ctx_lens, dtype, seed=nq + bs + len(requests))
+    give_back_pages_behind_the_window(bt, k_pool, v_pool, bs, requests, window)
     n = sum(c for _, c in requests)
     stride = (nq + 2 * nkv) * d
     q = torch.randn(n, stride, device=DEV).to(dtype)
@@ -726,6 +760,7 @@ def test_the_tiled_kernel_takes_short_requests_too(nq, nkv, d, bs, requests, win
     requests = list(requests) + [(37, 1), (9, 3)]
     ctx_lens = [c for c, _ in requests]
     bt, k_pool, v_pool, keys, values = build_paged(nkv, d, bs, ctx_lens, dtype, seed=d + bs + len(requests))
+    give_back_pages_behind_the_window(bt, k_pool, v_pool, bs, requests, window)
     n = sum(c for _, c in requests)
     stride = (nq + 2 * nkv) * d
     q = torch.randn(n, stride, device=DEV).to(dtype)

@@ -46,11 +46,43 @@ def setups(model_dirs):
     return get
 
 
-def replay(model_dir, dtype, prompts, steps, max_live, block_size=16):
+class LeftoversInFreePages:
+    """A replayer whose free pages hold what a page's last owner may have left there (infinities, NaNs,
+    the largest finite numbers): all pages at the start, and a request's pages again when it ends."""
+
+    def __init__(self, replayer):
+        self.r = replayer
+        self.spoil(range(replayer.cache.num_blocks))
+
+    def spoil(self, pages, group=None):
+        cache = self.r.cache
+        bs = cache.block_size
+        pattern = torch.tensor([float("inf"), float("nan"), 3e38, float("-inf")], device=cache.device)
+        for g in cache.layout.groups if group is None else [group]:
+            for layer in g.layers:
+                for pool in cache.layer_pools(layer):
+                    at = (torch.arange(bs, device=cache.device)[:, None] + torch.arange(pool.shape[1], device=cache.device)[None]) % 4
+                    rows = pattern[at].to(pool.dtype)
+                    for page in pages:
+                        pool[page * bs:(page + 1) * bs] = rows
+
+    def step(self, entries, end=()):
+        out = self.r.step(entries, [])
+        manager = self.r.cache.manager
+        for name in end:
+            seq = self.r.ids.pop(name)
+            held = [[p for p in manager.table(seq, gi) if p >= 0] for gi in range(len(self.r.cache.layout.groups))]
+            manager.free_sequence(seq)
+            for gi, pages in enumerate(held):
+                self.spoil(pages, self.r.cache.layout.groups[gi])
+        return out
+
+
+def replay(model_dir, dtype, prompts, steps, max_live, block_size=16, leftovers=False):
     from paged_llm_rs_amd.engine.replay import Replayer
 
     r = Replayer(model_dir, dtype, max_tokens=ru.pool_tokens(prompts, max_live), block_size=block_size)
-    got = ru.collect(r, steps)
+    got = ru.collect(LeftoversInFreePages(r) if leftovers else r, steps)
     assert r.cache.manager.live_sequences == 0
     assert r.cache.manager.available() == r.cache.manager.total(), "every page came back"
     return got
@@ -96,6 +128,28 @@ def test_mixed_requests_with_pages_used_again(setups, name, dtype, block_size, s
     assert any(len(e["tokens"]) > 1 for s in steps for e in s["entries"] if len(s["entries"]) > 1)
     got = replay(d, dtype, prompts, steps, max_live=4, block_size=block_size)
     worst, where = ru.worst_error(got, want)
+    assert worst <= TOLERANCE[dtype], f"{worst:.3e} at {where}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,block_size", [("A", 16), ("B", 8), ("D", 16), ("E", 16)])
+@pytest.mark.parametrize("schedule", ["whole", "tail", "portions", "mixed"])
+def test_what_free_pages_hold_changes_no_logit(setups, name, dtype, block_size, schedule):
+    """A page keeps what its last owner wrote.  Whatever that is, numbers that are not finite among them,
+    the next owner's logits are the bits they are over pages of zeros: what a kernel reads beyond a
+    request's keys is replaced, never multiplied by zero."""
+    d, prompts, want = setups(name, dtype)
+    live = 4 if schedule == "mixed" else 1
+    steps = {"whole": lambda: ru.whole(prompts), "tail": lambda: ru.tail_decoded(prompts, 32),
+             "portions": lambda: ru.portions(prompts, sizes=(130, 2, 64, 7, 33, 16)) if name in "DE" else ru.portions(prompts),
+             "mixed": lambda: ru.mixed(prompts, seed=21, max_live=4)}[schedule]()
+    clean = replay(d, dtype, prompts, steps, max_live=live, block_size=block_size)
+    spoiled = replay(d, dtype, prompts, steps, max_live=live, block_size=block_size, leftovers=True)
+    assert clean.keys() == spoiled.keys()
+    for key, row in clean.items():
+        assert np.isfinite(spoiled[key]).all(), f"{key}: not finite"
+        assert np.array_equal(row, spoiled[key]), f"{key}: differs by {np.abs(row - spoiled[key]).max():.3e}"
+    worst, where = ru.worst_error(spoiled, want)
     assert worst <= TOLERANCE[dtype], f"{worst:.3e} at {where}"
 
 
