@@ -12,7 +12,7 @@ from ..cache import PagedCache
 from ..errors import ConfigError
 from ..parts.model import DTYPES, load_model
 from .batch import StepEntry
-from .step import StepRunner, commit_step, require_gpu
+from .step import StepRunner, commit_step, require_gpu, run_step
 
 
 class Replayer:
@@ -37,9 +37,11 @@ class Replayer:
         self.ids: dict = {}
         self.next_id = 1
 
-    def step(self, entries, end=()):
+    def step(self, entries, end=(), trace: dict | None = None):
         """Run one step.  Returns the logits at the wanted places as a numpy
-        array [wanted, vocabulary] of 32-bit floats, or None when nothing is wanted."""
+        array [wanted, vocabulary] of 32-bit floats, or None when nothing is wanted.
+        ``trace`` (32-bit models) receives the step's named activations, rows in the order of the
+        entries' tokens; such a step runs kernel by kernel."""
         manager = self.cache.manager
         step_entries = []
         for e in entries:
@@ -61,7 +63,10 @@ class Replayer:
                                           state_slot=slot, fresh_state=fresh and slot >= 0))
         logits = None
         if step_entries:
-            out = self.runner.run(step_entries).logits
+            if trace is not None:
+                out = run_step(self.model, self.cache, step_entries, trace=trace)
+            else:
+                out = self.runner.run(step_entries).logits
             commit_step(self.cache, step_entries)
             if out.shape[0] > 0:
                 logits = out.to(torch.float32).cpu().numpy().astype("<f4", copy=False)

@@ -44,14 +44,17 @@ def require_gpu(device) -> torch.device:
 
 
 def run_step(model, cache, entries, check_start: bool = True, pad_to: int | None = None,
-             short_bound: int | None = None) -> torch.Tensor:
-    """32-bit logits [wanted places, vocabulary], in the order of the entries and of their ``want``."""
+             short_bound: int | None = None, trace: dict | None = None) -> torch.Tensor:
+    """32-bit logits [wanted places, vocabulary], in the order of the entries and of their ``want``.
+    ``trace`` receives the named activations of the step (32-bit models; see ``DecoderModel.forward``)."""
     batch = build_batch(entries, cache.manager, len(cache.layout.groups), model.spec.vocab_size,
                         model.spec.max_positions, model.device, check_start=check_start, pad_to=pad_to,
                         short_bound=short_bound)
     for e in entries:
         if e.fresh_state and e.state_slot >= 0:
             cache.clear_state_slot(e.state_slot)
+    if trace is not None:
+        return model.forward(batch, cache, trace=trace)
     return model.forward(batch, cache)
 
 

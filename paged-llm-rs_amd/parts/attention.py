@@ -65,6 +65,8 @@ class PagedAttention:
 
     # forward takes a norm still to run in place of rows, and may add its result into ctx.residual
     fuses = True
+    # ... and records named activations into ctx.trace
+    records = True
 
     def forward(self, x, ctx):
         """``x``: normalised rows, or a PendingNorm.  Where ``ctx.residual`` is given and the output
@@ -77,8 +79,33 @@ class PagedAttention:
         rot = self.rotary.dim if self.rotary is not None else 0
         prepare = kernels.QkFusion(self.q_gain, self.k_gain, self.eps, cos, sin, rot, ctx.writes_cache)
         out = torch.empty((qkv.shape[0], self.nq * self.d), dtype=qkv.dtype, device=qkv.device)
+        if ctx.trace is not None:
+            self._record_projections(qkv, batch, kv, ctx.trace)
         kernels.attention_step(qkv, out, batch, kv, self.nq, self.nkv, self.d, self.scale, self.window, prepare)
+        if ctx.trace is not None:
+            ctx.trace.record("o_proj.in", out)
+            out = self.o_proj.forward(out)
+            ctx.trace.record("o_proj.out", out)
+            return out
         return self.o_proj.forward(out, add_into=ctx.residual)
+
+    def _record_projections(self, qkv, batch, kv, trace) -> None:
+        """q, k and v as projected, and q and k after their per-head norm (before the rotation).  The
+        norm, the rotation and the cache write are one kernel; for the record it runs once more on copies,
+        without rotation and without writing, the keys standing in the place of queries."""
+        q_width, kv_width = self.nq * self.d, self.nkv * self.d
+        q, k, v = qkv[:, :q_width], qkv[:, q_width:q_width + kv_width], qkv[:, q_width + kv_width:]
+        trace.record("q_proj.out", q)
+        trace.record("k_proj.out", k)
+        trace.record("v_proj.out", v)
+        if self.q_gain is None:
+            return
+        for name, heads, count, gain in (("q_norm.out", q, self.nq, self.q_gain), ("k_norm.out", k, self.nkv, self.k_gain)):
+            copy = torch.cat([heads, k, v], dim=1).contiguous()
+            kernels.qk_norm_rope_kv_write(copy, gain, gain, self.eps, None, None, 0, batch.positions, batch.seq_of,
+                                          kv.block_table, kv.block_size, kv.k_pool, kv.v_pool, count, self.nkv, self.d,
+                                          write_kv=False)
+            trace.record(name, copy[:, :count * self.d])
 
 
 register_mixer("paged_attention", PagedAttention)

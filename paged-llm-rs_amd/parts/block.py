@@ -50,6 +50,8 @@ class PreNormBlock:
     def forward(self, resid, delta, ctx):
         """``delta``: what the block before has not added to the stream yet, or None.  Returns this
         block's own unadded output, or None when the feed-forward added it itself."""
+        if ctx.trace is not None:
+            return self._forward_recorded(resid, delta, ctx)
         mixer_fuses = getattr(self.mixer, "fuses", False)
         ffn_fuses = getattr(self.feed_forward, "fuses", False)
         if delta is None and mixer_fuses:
@@ -66,6 +68,27 @@ class PreNormBlock:
         if ffn_fuses:
             return self.feed_forward.forward(x, residual=resid)
         return self.feed_forward.forward(x)
+
+    def _forward_recorded(self, resid, delta, ctx):
+        """The same layer with every module's output recorded under its name: nothing is fused, so
+        every norm runs as a kernel and no part adds into the stream itself.  A part whose class sets
+        ``records = True`` takes the recorder (``ctx.trace`` for a mixer, ``trace=`` for a feed-forward)
+        and records what happens inside it."""
+        n, trace = self.NAMES, ctx.trace
+        x = self.norm1.apply(resid, delta, self.dtype)
+        trace.record(f"{n['norm1']}.out", x)
+        ctx.trace = trace.child(n["mixer"]) if getattr(self.mixer, "records", False) else None
+        mixed = self.mixer.forward(x, ctx)
+        ctx.trace = trace
+        trace.record(f"{n['mixer']}.out", mixed)
+        x = self.norm2.apply(resid, mixed, self.dtype)
+        trace.record(f"{n['norm2']}.out", x)
+        if getattr(self.feed_forward, "records", False):
+            out = self.feed_forward.forward(x, trace=trace.child(n["feed_forward"]))
+        else:
+            out = self.feed_forward.forward(x)
+        trace.record(f"{n['feed_forward']}.out", out)
+        return out
 
 
 register_block("pre_norm", PreNormBlock)

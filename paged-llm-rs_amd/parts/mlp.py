@@ -28,10 +28,22 @@ class GatedMlp:
 
     # forward takes a norm still to run in place of rows, and may add its result into the stream
     fuses = True
+    # ... and a recorder of named activations
+    records = True
 
-    def forward(self, x, residual: torch.Tensor | None = None):
+    def forward(self, x, residual: torch.Tensor | None = None, trace=None):
         """``x``: normalised rows, or a PendingNorm.  With ``residual`` (the 32-bit stream) the
         result is added there where the product kernel can do it, and None comes back."""
+        if trace is not None:
+            both = self.gate_up_proj.forward(x)
+            inter = both.shape[1] // 2
+            trace.record("gate_proj.out", both[:, :inter])
+            trace.record("up_proj.out", both[:, inter:])
+            act = kernels.swiglu(both)
+            trace.record("down_proj.in", act)
+            out = self.down_proj.forward(act)
+            trace.record("down_proj.out", out)
+            return out
         act = self.gate_up_proj.forward(x, swiglu=True)      # few rows: the activation is the product's epilogue
         return self.down_proj.forward(act, add_into=residual)
 

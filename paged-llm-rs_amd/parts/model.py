@@ -20,6 +20,7 @@ from . import attention, block, mlp, norm  # noqa: F401  (register the built-in 
 from .linear import Linear
 from .norm import PendingNorm
 from .registry import BLOCKS, NORMS, lookup, prefixed, scoped
+from .trace import ActivationTrace
 
 DTYPES = {"float32": torch.float32, "f32": torch.float32, "bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
           torch.float32: torch.float32, torch.bfloat16: torch.bfloat16}
@@ -43,7 +44,7 @@ class LayerContext:
     """What one run of one layer sees of the step: the batch, its own pages (or
     the pages of the layer it reads from) and its state slots."""
 
-    __slots__ = ("batch", "cache", "layer", "cache_layer", "writes_cache", "residual")
+    __slots__ = ("batch", "cache", "layer", "cache_layer", "writes_cache", "residual", "trace")
 
     def __init__(self, batch, cache, layer: int, cache_layer: int, writes_cache: bool):
         self.batch = batch
@@ -53,6 +54,8 @@ class LayerContext:
         self.writes_cache = writes_cache
         # the 32-bit stream, while a mixer that adds its own output runs; None otherwise
         self.residual = None
+        # an ActivationTrace for the part that runs, when named activations are recorded; None otherwise
+        self.trace = None
 
     def kv(self):
         return self.cache.layer_view(self.cache_layer, self.batch)
@@ -94,15 +97,34 @@ class DecoderModel:
 
     # -- the forward pass of one step -------------------------------------------------
 
-    def forward(self, batch, cache) -> torch.Tensor:
+    def forward(self, batch, cache, trace: dict | None = None) -> torch.Tensor:
         """Run the tokens of ``batch`` from ``cache`` and return 32-bit logits
-        [wanted rows, vocabulary].  Pages are written; no length is moved."""
+        [wanted rows, vocabulary].  Pages are written; no length is moved.
+
+        ``trace``: a dict that receives the output of every module under the module's checkpoint
+        name plus ``.out`` (reference: model/mod.rs:34-80), rows in the order of the batch's tokens;
+        the final norm, the head and ``logits`` hold the wanted rows only.  32-bit models only."""
+        top = None
+        if trace is not None:
+            if self.dtype != torch.float32:
+                raise UnsupportedError("named activations are recorded on the 32-bit path only: in bfloat16 "
+                                       "most of them are stages inside kernels and never written")
+            top = ActivationTrace(trace)
         resid = kernels.embed(batch.token_ids, self.embed_tokens)
+        if top is not None:
+            top.record(self.spec.embed_name.rsplit(".", 1)[0] + ".out", resid)
         delta = None
         for entry in self.spec.schedule:
             own = entry.cache_from is None
             ctx = LayerContext(batch, cache, entry.layer, entry.layer if own else entry.cache_from, own)
+            if top is not None:
+                ctx.trace = top.child(self.spec.layers[entry.layer].weight_prefix)
             delta = self.blocks[entry.layer].forward(resid, delta, ctx)
+            if top is not None:
+                after = resid.clone()
+                if delta is not None:
+                    kernels.residual_add(after, delta)
+                ctx.trace.record("out", after)
         m = batch.num_logit_rows
         if m == 0:
             # A portion in the middle of a prompt runs only to fill the cache.
@@ -112,7 +134,15 @@ class DecoderModel:
             normed = PendingNorm(self.norm, resid, self.dtype, rows=batch.logit_rows)
         else:
             normed = self.norm.apply(resid, delta, self.dtype, rows=batch.logit_rows)
-        return self.lm_head.forward(normed, out_dtype=torch.float32)
+        if top is not None:
+            if isinstance(normed, PendingNorm):
+                normed = normed.materialize()
+            top.record(self.spec.final_norm_name.rsplit(".", 1)[0] + ".out", normed)
+        logits = self.lm_head.forward(normed, out_dtype=torch.float32)
+        if top is not None:
+            top.record(self.spec.head_name.rsplit(".", 1)[0] + ".out", logits)
+            top.record("logits", logits)
+        return logits
 
 
 def build_model(config, params: dict, dtype, device) -> DecoderModel:

@@ -16,7 +16,9 @@ if str(ROOT) not in sys.path:
 if str(ROOT / "tests") not in sys.path:
     sys.path.insert(0, str(ROOT / "tests"))
 
-REFERENCE_FIXTURE = Path("/root/reference/crates/pagedllm/tests/fixtures/tiny")
+# The reference's own tiny checkpoint with the activations it holds for it, read in place; where the
+# reference lies elsewhere (a machine that has only a copy of that folder), the variable names the folder.
+REFERENCE_FIXTURE = Path(os.environ.get("PAGEDLLM_REFERENCE_FIXTURE", "/root/reference/crates/pagedllm/tests/fixtures/tiny"))
 
 
 def pytest_configure(config):

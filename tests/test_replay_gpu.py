@@ -232,3 +232,120 @@ def test_drawn_configurations_mixed_and_decoded(tmp_path, case):
             got = replay(folder, dtype, prompts, steps, max_live=live, block_size=block_size)
             worst, where = ru.worst_error(got, want)
             assert worst <= TOLERANCE[dtype], f"{config} pages of {block_size}, {dtype}: {worst:.3e} at {where}"
+
+
+# --- the reference's own checkpoint -------------------------------------------------------------------
+
+from conftest import REFERENCE_FIXTURE  # noqa: E402
+
+needs_fixture = pytest.mark.skipif(not (REFERENCE_FIXTURE / "activations.safetensors").exists(),
+                                   reason="the reference's fixture is not readable here")
+
+
+def fixture_metric(got, want) -> float:
+    """The reference's own measure (tests/common/mod.rs:20-43): the largest difference over the
+    largest wanted magnitude, which counts as one at least."""
+    got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
+    assert got.size == want.size, f"{got.shape} against {want.shape}"
+    return float(np.abs(got.reshape(want.shape) - want).max() / max(1.0, np.abs(want).max()))
+
+
+@needs_fixture
+@pytest.mark.parametrize("cut", ["whole", "one by one", "1, 3, 4"])
+def test_the_engine_on_the_references_own_checkpoint(cut):
+    """The reference's tiny checkpoint, written by another program (extra keys in config.json, the rotary
+    base under rope_parameters, an untied head, a width of 24), read in place through the engine's own
+    loader and run in 32-bit: logits and the chosen token at every position against the outputs the
+    reference holds, at its own tolerance (tests/forward.rs:53-79); the prompt whole, token by token, and in
+    portions of 1, 3 and 4 tokens over pages of 4 (tests/batching.rs:308-312)."""
+    from safetensors.torch import load_file
+
+    from paged_llm_rs_amd.engine.replay import Replayer
+
+    manifest = json.loads((REFERENCE_FIXTURE / "manifest.json").read_text())
+    held = load_file(str(REFERENCE_FIXTURE / "activations.safetensors"))
+    prompt = manifest["prompt"]
+    sizes = {"whole": [len(prompt)], "one by one": [1] * len(prompt), "1, 3, 4": [1, 3, 4]}[cut]
+    assert sum(sizes) == len(prompt)
+    r = Replayer(REFERENCE_FIXTURE, "float32", max_tokens=64, block_size=4)
+    rows, at = [], 0
+    for n in sizes:
+        rows.append(r.step([{"id": "p", "tokens": prompt[at:at + n], "want": list(range(n))}], []))
+        at += n
+    got = np.concatenate(rows)
+    want = held["logits"][0].numpy()
+    assert fixture_metric(got, want) <= manifest["relative_tolerance"]
+    assert got.argmax(-1).tolist() == want.argmax(-1).tolist()
+
+
+@needs_fixture
+@pytest.mark.parametrize("cut", ["whole", "1, 3, 4"])
+def test_every_module_of_the_engine_on_the_references_own_checkpoint(cut):
+    """All 36 named activations that the reference holds for its checkpoint (tests/forward.rs:23-51,
+    manifest.json), from the engine's 32-bit path with its recorder of named activations on."""
+    from safetensors.torch import load_file
+
+    from paged_llm_rs_amd.engine.replay import Replayer
+
+    manifest = json.loads((REFERENCE_FIXTURE / "manifest.json").read_text())
+    held = load_file(str(REFERENCE_FIXTURE / "activations.safetensors"))
+    prompt = manifest["prompt"]
+    sizes = {"whole": [len(prompt)], "1, 3, 4": [1, 3, 4]}[cut]
+    r = Replayer(REFERENCE_FIXTURE, "float32", max_tokens=64, block_size=4)
+    parts, at = [], 0
+    for n in sizes:
+        trace: dict = {}
+        r.step([{"id": "p", "tokens": prompt[at:at + n], "want": list(range(n))}], [], trace=trace)
+        parts.append(trace)
+        at += n
+    assert len(manifest["tensors"]) == 36 and set(manifest["tensors"]) <= set(parts[0]), sorted(set(manifest["tensors"]) - set(parts[0]))
+    for name in manifest["tensors"]:
+        got = torch.cat([p[name] for p in parts]).cpu().numpy()
+        worst = fixture_metric(got, held[name].numpy())
+        assert worst <= manifest["relative_tolerance"], f"{name}: {worst:.3e}"
+
+
+def test_named_activations_are_refused_in_bfloat16(setups):
+    from paged_llm_rs_amd.engine.replay import Replayer
+    from paged_llm_rs_amd.errors import UnsupportedError
+
+    d, prompts, _ = setups("A", "bfloat16")
+    r = Replayer(d, "bfloat16", max_tokens=64)
+    with pytest.raises(UnsupportedError, match="32-bit"):
+        r.step([{"id": "p", "tokens": [1, 2, 3], "want": [2]}], [], trace={})
+
+
+@pytest.mark.parametrize("name,block_size", [("A", 16), ("B", 8), ("C", 4)])
+def test_every_module_against_the_plain_implementation(setups, name, block_size):
+    """The engine's named activations beside the plain implementation's, module by module (the plain
+    implementation is itself held to the reference's 36 recorded tensors): a difference in the logits is
+    then found at the module where it begins.  A prompt whole, and a second one in portions beside it."""
+    from paged_llm_rs_amd.engine.replay import Replayer
+
+    d, prompts, _ = setups(name, "float32")
+    cfg, weights = ru.load_plain(d)
+    a, b = prompts["r3"], prompts["r4"]
+    want = {}
+    for key, tokens in (("a", a), ("b", b)):
+        trace: dict = {}
+        ru.plain.forward(weights, cfg, tokens, trace=trace)
+        want[key] = trace
+    r = Replayer(d, "float32", max_tokens=ru.pool_tokens({"a": a, "b": b}, 2), block_size=block_size)
+    # step 1: a whole, beside the first 7 tokens of b; step 2: the rest of b
+    steps = [[("a", a), ("b", b[:7])], [("b", b[7:])]]
+    got = {"a": [], "b": []}
+    for step in steps:
+        trace = {}
+        r.step([{"id": k, "tokens": t, "want": list(range(len(t)))} for k, t in step], [], trace=trace)
+        row = 0
+        for k, t in step:
+            got[k].append({n: v[row:row + len(t)] for n, v in trace.items()})
+            row += len(t)
+    names = [n for n in want["a"] if n in got["a"][0]]
+    assert len(names) == 4 + 16 * cfg["num_hidden_layers"], sorted(set(want["a"]) ^ set(got["a"][0]))
+    for key in ("a", "b"):
+        for n in names:
+            mine = torch.cat([part[n] for part in got[key]]).double().cpu()
+            ref = want[key][n].double()
+            worst = float((mine.reshape(ref.shape) - ref).abs().max() / max(1.0, float(ref.abs().max())))
+            assert worst <= 1e-5, f"request {key}, {n}: {worst:.3e}"
