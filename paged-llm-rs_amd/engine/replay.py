@@ -19,7 +19,8 @@ class Replayer:
     LIVE_AT_MOST = 4        # requests that a trace holds at a time
 
     def __init__(self, model_dir, dtype: str, max_tokens: int, block_size: int = 16, device="cuda:0",
-                 max_live: int = 64, graphs: bool = True):
+                 max_live: int = 64, graphs: bool = True, pages: int | None = None):
+        """``pages`` sets the pool's size by hand instead of deriving it from ``max_tokens``."""
         device = require_gpu(device)
         self.config, self.model = load_model(model_dir, dtype, device)
         if max_tokens < 1:
@@ -28,9 +29,11 @@ class Replayer:
         # holds them when the page size divides 64.  With any other page size a request's last page may
         # reach past its multiple of 64: one page more for each of the requests that a trace may hold.
         tokens = (max_tokens + 63) // 64 * 64
-        pages = -(-tokens // block_size)
+        pages_given, pages = pages, -(-tokens // block_size)
         if 64 % block_size:
             pages += self.LIVE_AT_MOST
+        if pages_given is not None:
+            pages = pages_given
         self.cache = PagedCache(self.model.cache_layout, block_size, max(pages, 1), DTYPES[dtype], device,
                                 max_seqs=max_live)
         self.runner = StepRunner(self.model, self.cache, graphs=graphs)

@@ -52,6 +52,27 @@ def test_greedy_generation_matches_the_plain_implementation(model_dirs, name, dt
     assert m["available"] == m["total"] and m["tokens"] == 64
 
 
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_greedy_generation_that_does_not_repeat_the_prompts_last_token(tmp_path, dtype):
+    """With small weights and a tied head a random model's most likely next token is the one it was just
+    given, and a model with every layer left out would pass a comparison of tokens.  Here the head is its
+    own matrix and the weights are large: the tokens wander, and every one is the plain implementation's."""
+    from paged_llm_rs_amd import Engine
+    from paged_llm_rs_amd.weights import write_random_model
+
+    config = TINY_INIT["B"]["config"]
+    long_name = "float32" if dtype == "f32" else "bfloat16"
+    d = write_random_model(tmp_path / "m", config, seed=21, std=0.3, gain_std=0.2, dtype=long_name)
+    prompts = list(ru.make_prompts(config["vocab_size"], [5, 17, 33, 2], seed=4).values())
+    engine = Engine(d, dtype=dtype, block_size=8, num_blocks=64, max_batch=4, chunk=9)
+    out = engine.generate(prompts, max_tokens=16, temperature=0.0, stop_tokens=[])
+    for prompt, result in zip(prompts, out):
+        tokens = result["tokens"]
+        assert len(tokens) == 16
+        assert tokens[0] != prompt[-1] and len(set(tokens)) >= 4, f"{prompt[-1]} then {tokens}"
+        plain_greedy_check(d, prompt, tokens, 1e-5 if dtype == "f32" else 2e-2)
+
+
 def test_running_out_of_pages_changes_no_token(model_dirs):
     """Eviction recomputes a request from its history; the tokens it had already
     returned stay returned and the rest come out the same."""

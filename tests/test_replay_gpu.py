@@ -78,10 +78,10 @@ class LeftoversInFreePages:
         return out
 
 
-def replay(model_dir, dtype, prompts, steps, max_live, block_size=16, leftovers=False):
+def replay(model_dir, dtype, prompts, steps, max_live, block_size=16, leftovers=False, pages=None):
     from paged_llm_rs_amd.engine.replay import Replayer
 
-    r = Replayer(model_dir, dtype, max_tokens=ru.pool_tokens(prompts, max_live), block_size=block_size)
+    r = Replayer(model_dir, dtype, max_tokens=ru.pool_tokens(prompts, max_live), block_size=block_size, pages=pages)
     got = ru.collect(LeftoversInFreePages(r) if leftovers else r, steps)
     assert r.cache.manager.live_sequences == 0
     assert r.cache.manager.available() == r.cache.manager.total(), "every page came back"
@@ -151,6 +151,37 @@ def test_what_free_pages_hold_changes_no_logit(setups, name, dtype, block_size, 
         assert np.array_equal(row, spoiled[key]), f"{key}: differs by {np.abs(row - spoiled[key]).max():.3e}"
     worst, where = ru.worst_error(spoiled, want)
     assert worst <= TOLERANCE[dtype], f"{worst:.3e} at {where}"
+
+
+def pages_at_the_peak(steps, block_size: int) -> int:
+    """The most pages that the live requests of a trace hold at once."""
+    held, peak = {}, 0
+    for step in steps:
+        for e in step["entries"]:
+            held[e["id"]] = held.get(e["id"], 0) + len(e["tokens"])
+        peak = max(peak, sum(-(-n // block_size) for n in held.values()))
+        for name in step["end"]:
+            held.pop(name)
+    return peak
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,block_size,seed", [("A", 16, 1), ("B", 8, 2), ("C", 4, 3), ("D", 16, 5)])
+def test_a_pool_of_exactly_the_pages_a_trace_needs(setups, name, dtype, block_size, seed):
+    """The mixed trace in a pool with not one page to spare: every page that comes back is handed out again
+    (the trace allocates more pages than the pool has), and with one page fewer the trace does not fit."""
+    from paged_llm_rs_amd.errors import ConfigError
+
+    d, prompts, want = setups(name, dtype)
+    steps = ru.mixed(prompts, seed=seed, max_live=4)
+    peak = pages_at_the_peak(steps, block_size)
+    handed_out = sum(-(-len(t) // block_size) for t in prompts.values())
+    assert handed_out > peak, "pages have to be used again"
+    got = replay(d, dtype, prompts, steps, max_live=4, block_size=block_size, pages=peak)
+    worst, where = ru.worst_error(got, want)
+    assert worst <= TOLERANCE[dtype], f"{worst:.3e} at {where}"
+    with pytest.raises(ConfigError, match="--max-tokens is too small"):
+        replay(d, dtype, prompts, steps, max_live=4, block_size=block_size, pages=peak - 1)
 
 
 def test_schedules_agree_with_each_other_in_32_bit(setups):
