@@ -11,8 +11,8 @@ choice of the next token, which is what the next step is fed.  Weights are rando
 (the random-weights mode writes the model folder, the loader reads it back),
 prompts are seeded uniform token ids.  One JSON line is printed.
 
-The default sizes are those of BASELINE.json's third configuration.  Peaks are the
-published ones of the MI355X: 8 TB/s of HBM, 2.5 PFLOP/s dense bf16.
+The default sizes are the Qwen3-0.6B shape's.  Peaks are the published ones of the
+MI355X: 8 TB/s of HBM, 2.5 PFLOP/s dense bf16.
 """
 
 from __future__ import annotations
@@ -37,7 +37,7 @@ COMMON = {
     "attention_bias": False, "sliding_window": None, "head_dim": 128, "num_key_value_heads": 8,
     "rms_norm_eps": 1e-6, "rope_theta": 1000000.0, "vocab_size": 151936,
 }
-# The default is the Qwen3-0.6B shape (BASELINE.json, configs[2]); --shape 8b and 32b are configs[3] and [4]:
+# The default is the Qwen3-0.6B shape; --shape 8b and 32b are the Qwen3-8B and Qwen3-32B shapes:
 # (config.json keys, the context a decode step starts from, layers that the default run of that shape loads).
 SHAPES = {
     "0.6b": ("Qwen3-0.6B", dict(COMMON, hidden_size=1024, intermediate_size=3072, num_hidden_layers=28,
@@ -138,7 +138,7 @@ def main() -> int:
     parser.add_argument("--warmup", type=int, default=10)
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--shape", choices=sorted(SHAPES), default="0.6b",
-                        help="layer sizes: the headline 0.6b, or the 8b and 32b shapes of BASELINE.json")
+                        help="layer sizes: the headline 0.6b, or the 8b and 32b shapes")
     parser.add_argument("--layers", type=int, default=None,
                         help="fewer layers than the model has, where memory or time needs it; both numbers are reported")
     parser.add_argument("--no-graphs", action="store_true", help="run decode steps eagerly instead of as HIP graphs")

@@ -292,9 +292,9 @@ __global__ void qk_norm_rope_kv_write_kernel(
     }
     if (gain) {
         ss = wave_sum(ss);
-        const float denom = sqrtf(ss / static_cast<float>(d) + eps);
+        const float rinv = 1.f / sqrtf(ss / static_cast<float>(d) + eps);   // one division a head (the decode attention kernel does the same)
         __syncthreads();
-        for (int i = lane; i < d; i += PL_WAVE) head[i] = head[i] / denom * load_as_float(gain, gain_dtype, i);
+        for (int i = lane; i < d; i += PL_WAVE) head[i] = head[i] * rinv * load_as_float(gain, gain_dtype, i);
     }
     __syncthreads();
     const int half = rot / 2;
@@ -439,9 +439,9 @@ qk_norm_rope_kv_write_wide_kernel(
             const int base = hw * lph;
             for (int j = 0; j < lph; ++j) total += __shfl(ss, min(base + j, PL_WAVE - 1), PL_WAVE);
             if (normed[u]) {
-                const float denom = sqrtf(total / static_cast<float>(d) + eps);
+                const float rinv = 1.f / sqrtf(total / static_cast<float>(d) + eps);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) x[u][e] = x[u][e] / denom * (is_q[u] ? qg[e] : kg[e]);
+                for (int e = 0; e < 8; ++e) x[u][e] = x[u][e] * rinv * (is_q[u] ? qg[e] : kg[e]);
             }
             float px[8];
 #pragma unroll
@@ -519,9 +519,9 @@ qk_norm_rope_kv_write_128_kernel(
     ss += qk_dpp_mirror(ss);
     const bool is_v = !is_q && !is_k;
     if (gain && !is_v) {
-        const float denom = sqrtf(ss / static_cast<float>(D) + eps);
+        const float rinv = 1.f / sqrtf(ss / static_cast<float>(D) + eps);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) x[e] = x[e] / denom * g[e];
+        for (int e = 0; e < 8; ++e) x[e] = x[e] * rinv * g[e];
     }
     if (cos_table) {
         float px[8];

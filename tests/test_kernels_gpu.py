@@ -608,13 +608,16 @@ def test_decode_attention_that_prepares_its_own_queries_and_keys(nq, nkv, d, bs,
     kernels.paged_attention_decode(raw, stride, got, positions, seq_of, bt, bs, k_b, v_b, nq, nkv, d, scale, window, splits,
                                    fuse=kernels.QkFusion(q_gain, k_gain, 1e-5, cos, sin, rot, True))
     assert same_bits(k_a, k_b) and same_bits(v_a, v_b), "the same keys and values in the same places"
-    assert rel(got[:-1], want[:-1]) < 4e-3
+    # The outputs are bfloat16 and the probabilities are rounded to bfloat16 before they meet the values; the
+    # token's own key enters first and unrounded here, last and rounded there.  One unit in the last place of
+    # the largest element (2^-7 of it) is what two such sums may differ by.
+    assert rel(got[:-1], want[:-1]) < 8e-3
     assert bool((got[-1] == 7.0).all()), "a padding row is not written"
     # queries only: a layer that reads pages another layer wrote
     again = torch.full((n, nq * d), 7.0, dtype=dtype, device=DEV)
     kernels.paged_attention_decode(raw, stride, again, positions, seq_of, bt, bs, k_a, v_a, nq, nkv, d, scale, window, splits,
                                    fuse=kernels.QkFusion(q_gain, k_gain, 1e-5, cos, sin, rot, False))
-    assert rel(again[:-1], want[:-1]) < 4e-3
+    assert rel(again[:-1], want[:-1]) < 8e-3
 
 
 PORTION_CASES = [
