@@ -41,247 +41,199 @@ std::optional<size_t> Scheduler::prompt_in_flight() const {
     return std::nullopt;
 }
 
-PlanEntry Scheduler::entry_for(Sequence& s, size_t start, std::vector<uint32_t> tokens, bool wants) {
-    PlanEntry e{s.id, start, std::move(tokens), wants, s.state_slot, s.state_fresh};
-    s.state_fresh = false;
-    return e;
-}
-
-// Refuse first, then (with a budget) a mixed step or else a plain decode, or
-// (without one) a whole prompt or else a plain decode (scheduler.rs:368-381).
+// ---------------------------------------------------------------------------
+// Assembling a step.
+//
+// Three kinds of step come out of the same four moves.  With a token allowance
+// (chunk > 0): seat the residents, giving the step up if one of them finds no
+// page; feed prompts with what the residents left; if any prompt token went in,
+// that is the step.  Without an allowance: bring the front prompt in whole and
+// run it alone.  Whenever neither made a step: seat the residents again, this
+// time evicting for pages, and decode.  (scheduler.rs:368-381 has the same order
+// of preference as three separate planners.)
+// ---------------------------------------------------------------------------
 const Plan& Scheduler::plan() {
-    if (auto refused = refuse_unservable()) {
-        plan_ = std::move(*refused);
-        return plan_;
-    }
+    if (turn_away_front()) return plan_;
     if (chunk_ > 0) {
-        if (auto step = mixed()) {
-            plan_ = std::move(*step);
-            return plan_;
-        }
-        plan_ = decode();
-        return plan_;
+        // every row carries at least one token, so the allowance bounds the rows as well
+        Assembly step(chunk_, std::min(max_batch_, chunk_));
+        if (seat_residents(step, WhenDry::GiveUp) && feed_prompts(step, Entry::PortionWise))
+            return publish(step, PlanKind::Mixed);
+    } else {
+        Assembly step(SIZE_MAX, 1);
+        if (feed_prompts(step, Entry::Whole)) return publish(step, PlanKind::Prefill);
     }
-    if (auto step = admit()) {
-        plan_ = std::move(*step);
-        return plan_;
-    }
-    plan_ = decode();
-    return plan_;
+    Assembly step(max_batch_, max_batch_);
+    seat_residents(step, WhenDry::EvictNewest);
+    return publish(step, step.plan.entries.empty() ? PlanKind::Idle : PlanKind::Decode);
 }
 
-// One step carrying a portion of a prompt and every running request's next
-// token (scheduler.rs:388-499).
-std::optional<Plan> Scheduler::mixed() {
-    const size_t budget = chunk_;
-    // A prompt part-way through finishes before a new one starts.
-    std::optional<size_t> index = prompt_in_flight();
-
-    Plan step;
-    step.kind = PlanKind::Mixed;
-    // Decodes are taken first: they are what a client is watching.
-    const size_t cap = std::min(max_batch_, budget);
-    for (size_t row = 0; row < running_.size(); ++row) {
-        if (step.entries.size() >= cap) break;
-        Sequence& s = running_[row];
-        if ((index && row == *index) || s.finish != Finish::None || s.pending.size() != 1) continue;
-        if (!cache_->reserve(s.id, 1)) {
-            // A resident that needs a page from a dry pool is a preemption, and
-            // choosing the victim is the plain decode's job.  Give the step up
-            // rather than run without this request.
-            return std::nullopt;
-        }
-        step.ids.push_back(s.id);
-        step.advanced.emplace_back(s.id, 1);
-        step.entries.push_back(entry_for(s, cache_->tokens(s.id), {s.pending[0]}, true));
-    }
-    const size_t decodes = step.entries.size();
-
-    // Whatever the decodes left goes to the prompt in flight; and where that prompt ends within the budget,
-    // to the next waiting ones, as long as tokens and rows are left.  (The reference's step carries a slice
-    // of one prompt; short prompts then enter one a step however large the budget, and a batch takes as many
-    // steps to fill as it has requests.)  At most one prompt is left part-way by a step, so the next step
-    // finds one prompt in flight, as the reference's does.
-    size_t room = budget > decodes ? budget - decodes : 0;
-    if (room == 0) return std::nullopt;
-    bool any = false;
-    while (room > 0 && (!any || step.entries.size() < cap)) {
-        // A new prompt joins only now, after the residents have taken their pages.
-        if (!index) {
-            const size_t before = running_.size();
-            start_next_prompt();
-            if (running_.size() == before) break;
-            index = before;
-        }
-        Sequence& s = running_[*index];
-        const size_t done = s.history.size() - s.prompt_left;
-        const size_t want = std::min(room, s.prompt_left);
-        const size_t take = cache_->reserve_up_to(s.id, want);
-        if (take == 0) break;
-        const bool last = take == s.prompt_left;
-        if (last) step.ids.push_back(s.id);  // only the last portion asks for logits
-        step.advanced.emplace_back(s.id, take);
-        step.entries.push_back(entry_for(
-            s, done, std::vector<uint32_t>(s.history.begin() + done, s.history.begin() + done + take), last));
-        any = true;
-        room -= take;
-        if (!last) break;
-        index.reset();
-    }
-    if (!any) return std::nullopt;
-
-    metrics_.steps += 1;
-    metrics_.mixed_steps += 1;
-    metrics_.decode_rows += decodes;
-    if (decodes > 0) metrics_.decode_steps += 1;
-    return step;
+// One row of the step: `count` tokens of `s` from position `first` of its history.
+void Scheduler::row_of_tokens(Assembly& step, Sequence& s, size_t first, size_t count, bool wants_logits) {
+    if (wants_logits) step.plan.ids.push_back(s.id);
+    step.plan.advanced.emplace_back(s.id, count);
+    step.plan.entries.push_back(PlanEntry{
+        s.id, first, std::vector<uint32_t>(s.history.begin() + static_cast<long>(first),
+                                           s.history.begin() + static_cast<long>(first + count)),
+        wants_logits, s.state_slot, s.state_fresh});
+    s.state_fresh = false;
+    step.rows_left -= std::min<size_t>(step.rows_left, 1);
+    step.tokens_left -= std::min(step.tokens_left, count);
 }
 
-// Move the first waiting request into the running set without running it, so
-// that its prompt can be fed a portion at a time (scheduler.rs:503-539).
-void Scheduler::start_next_prompt() {
-    if (waiting_.empty()) return;
-    const size_t prompt_len = waiting_.front().pending.size();
-    if (cache_->min_available() == 0 || !cache_->state_slot_available()) {
-        metrics_.admission_stalls += 1;
-        return;
-    }
-    Sequence s = std::move(waiting_.front());
-    waiting_.pop_front();
-    s.state_slot = cache_->add_sequence(s.id);
-    s.state_fresh = s.state_slot >= 0;
-    const size_t shared = cache_->claim_prefix(s.id, s.pending.data(), s.pending.size());
-    // Claiming takes pages of its own, and a request whose whole prefix was
-    // resident still needs somewhere to write the token it is about to produce.
-    if (!cache_->reserve(s.id, 1)) {
-        cache_->free_sequence(s.id);
-        s.state_slot = -1;
-        s.pending = s.history;
-        waiting_.push_front(std::move(s));
-        metrics_.admission_stalls += 1;
-        return;
-    }
-    metrics_.cached_tokens += shared;
-    metrics_.prefilled_tokens += prompt_len - shared;
-    s.prompt_left = std::max<size_t>(prompt_len - shared, 1);
-    s.pending.clear();
-    metrics_.prefills += 1;
-    running_.push_back(std::move(s));
-}
-
-// Give a waiting request its pages and run its whole prompt (scheduler.rs:548-589).
-std::optional<Plan> Scheduler::admit() {
-    if (waiting_.empty()) return std::nullopt;
-    const size_t prompt_len = waiting_.front().pending.size();
-    if (!cache_->fits_from_scratch(prompt_len) || !cache_->state_slot_available()) {
-        metrics_.admission_stalls += 1;
-        return std::nullopt;
-    }
-    Sequence s = std::move(waiting_.front());
-    waiting_.pop_front();
-    s.state_slot = cache_->add_sequence(s.id);
-    s.state_fresh = s.state_slot >= 0;
-    const size_t shared = cache_->claim_prefix(s.id, s.pending.data(), s.pending.size());
-    if (!cache_->reserve(s.id, prompt_len - shared)) {
-        // The cache gave way and there is still nothing: put it back rather
-        // than admit it half served.
-        cache_->free_sequence(s.id);
-        s.state_slot = -1;
-        s.pending = s.history;
-        waiting_.push_front(std::move(s));
-        metrics_.admission_stalls += 1;
-        return std::nullopt;
-    }
-    metrics_.cached_tokens += shared;
-    metrics_.prefilled_tokens += prompt_len - shared;
-
-    Plan step;
-    step.kind = PlanKind::Prefill;
-    step.ids.push_back(s.id);
-    step.advanced.emplace_back(s.id, prompt_len - shared);
-    step.entries.push_back(
-        entry_for(s, shared, std::vector<uint32_t>(s.pending.begin() + shared, s.pending.end()), true));
-    s.pending.clear();
-    running_.push_back(std::move(s));
-    metrics_.steps += 1;
-    metrics_.prefills += 1;
-    return step;
-}
-
-// Advance every resident request by one token, evicting where the pools
-// cannot supply the page one of them needs (scheduler.rs:625-676).
-Plan Scheduler::decode() {
-    std::vector<size_t> chosen;
+// A row for the next token of every resident that has one to feed, in the order
+// of arrival, as far as the rows last.  Each needs room for one more token in
+// its pages.  Where the pools cannot give that: under GiveUp nothing is seated
+// and false comes back (the caller then decodes instead, which may evict; a
+// step that carried a prompt beside an incomplete set of residents would starve
+// the one left out); under EvictNewest the newest resident other than the asker
+// loses its pages and goes back to the front of the queue, and the asker tries
+// again (scheduler.rs:625-676).  A request that is alone and still finds no page
+// can never be served further and ends with what it has.
+bool Scheduler::seat_residents(Assembly& step, WhenDry policy) {
+    std::vector<uint64_t> seated;
     size_t index = 0;
-    while (index < running_.size() && chosen.size() < max_batch_) {
+    while (index < running_.size() && seated.size() < step.rows_left) {
         Sequence& s = running_[index];
-        if (s.finish != Finish::None || s.pending.size() != 1) {
+        if (s.finish != Finish::None || s.pending.size() != 1) {   // done, or still taking its prompt in
             ++index;
             continue;
         }
         if (cache_->reserve(s.id, 1)) {
-            chosen.push_back(index);
+            seated.push_back(s.id);
             ++index;
             continue;
         }
-        // Nothing left.  Evict the newest resident that is not this one and
-        // come back to this request with the pages it freed.
-        const auto victim = newest_evictable(index);
+        if (policy == WhenDry::GiveUp) return false;
+        const auto victim = newest_other_than(index);
         if (!victim) {
-            // Alone, and the pools cannot hold its next token: it ends here,
-            // or nothing would ever free anything.  (The reference would idle
-            // forever at this point.)
             s.finish = Finish::Length;
             ++index;
             continue;
         }
-        preempt(*victim);
-        chosen.erase(std::remove(chosen.begin(), chosen.end(), *victim), chosen.end());
-        for (size_t& taken : chosen)
-            if (taken > *victim) --taken;
-        if (*victim < index) --index;
+        seated.erase(std::remove(seated.begin(), seated.end(), running_[*victim].id), seated.end());
+        evict(*victim);
+        if (*victim < index) --index;      // the asker has moved down by one
     }
-    Plan step;
-    if (chosen.empty()) return step;  // Idle
-    step.kind = PlanKind::Decode;
-    for (size_t i : chosen) {
-        Sequence& s = running_[i];
-        step.ids.push_back(s.id);
-        step.advanced.emplace_back(s.id, 1);
-        step.entries.push_back(entry_for(s, cache_->tokens(s.id), {s.pending[0]}, true));
+    for (uint64_t id : seated) {
+        Sequence* s = sequence(id);
+        // the token to feed is the last of the history: what the step before produced
+        row_of_tokens(step, *s, cache_->tokens(id), 1, true);
     }
-    metrics_.steps += 1;
-    metrics_.decode_steps += 1;
-    metrics_.decode_rows += step.ids.size();
-    return step;
+    step.decode_rows = seated.size();
+    return true;
 }
 
-// Reject a waiting prompt the pools could never hold, or one past the longest
-// position the model knows (scheduler.rs:681-690).
-std::optional<Plan> Scheduler::refuse_unservable() {
+// Prompt tokens into what is left of the step: first the prompt that an earlier
+// step left part-way, then newcomers from the front of the queue, each from
+// where its cached or already fed tokens end.  A prompt that does not fit
+// whole gets what fits (what the pools can back, at most) and stays in flight;
+// since only one prompt may be in flight, nothing follows it.  Only the row
+// that holds a prompt's last token asks for logits.  True when at least one
+// prompt token went in.  (The reference feeds a slice of one prompt a step,
+// scheduler.rs:388-499; here short prompts share a step, so a batch of short
+// requests fills in a few steps instead of one step a request.)
+bool Scheduler::feed_prompts(Assembly& step, Entry entry) {
+    std::optional<size_t> index = entry == Entry::PortionWise ? prompt_in_flight() : std::nullopt;
+    // (The first prompt row goes in even when the residents have taken every row: a prompt in flight
+    // must not wait for a resident to finish.)
+    while (step.tokens_left > 0 && (step.prompt_tokens == 0 || step.rows_left > 0)) {
+        if (!index) {
+            // a newcomer takes its first pages only now, after the residents have theirs
+            index = bring_in_front(entry);
+            if (!index) break;
+        }
+        Sequence& s = running_[*index];
+        const size_t fed = s.history.size() - s.prompt_left;
+        const size_t take = cache_->reserve_up_to(s.id, std::min(step.tokens_left, s.prompt_left));
+        if (take == 0) break;
+        const bool completes = take == s.prompt_left;
+        row_of_tokens(step, s, fed, take, completes);
+        step.prompt_tokens += take;
+        if (!completes) break;
+        index.reset();
+    }
+    return step.prompt_tokens > 0;
+}
+
+// The front of the queue becomes a resident: a state slot, the pages of whatever
+// prefix of its prompt the cache already holds, and pages of its own for what
+// it needs at once (everything, when its prompt is to run whole; room for one
+// token otherwise, so that even a fully cached prompt has somewhere to write).
+// Where the pools or the slots cannot give that, everything is handed back, the
+// request keeps its place and the stall is counted (scheduler.rs:503-589).
+std::optional<size_t> Scheduler::bring_in_front(Entry entry) {
     if (waiting_.empty()) return std::nullopt;
     const size_t prompt_len = waiting_.front().pending.size();
-    const size_t budget = chunk_ > 0 ? chunk_ : prompt_len;
-    const bool too_long = max_positions_ > 0 && prompt_len > max_positions_;
-    if (!too_long && cache_->fits_in_total(prompt_len, budget)) return std::nullopt;
+    const bool room = entry == Entry::Whole ? cache_->fits_from_scratch(prompt_len) : cache_->min_available() > 0;
+    if (!room || !cache_->state_slot_available()) {
+        metrics_.admission_stalls += 1;
+        return std::nullopt;
+    }
     Sequence s = std::move(waiting_.front());
     waiting_.pop_front();
-    Plan step;
-    step.kind = PlanKind::Refused;
-    step.refused = s.id;
-    outcome_pending_refusal_ = FinishedInfo{s.id, Finish::Length, s.prompt_tokens, s.generated, s.preemptions};
-    return step;
+    s.state_slot = cache_->add_sequence(s.id);
+    s.state_fresh = s.state_slot >= 0;
+    const size_t shared = cache_->claim_prefix(s.id, s.pending.data(), s.pending.size());
+    const size_t at_once = entry == Entry::Whole ? prompt_len - shared : 1;
+    if (!cache_->reserve(s.id, at_once)) {
+        cache_->free_sequence(s.id);
+        s.state_slot = -1;
+        s.pending = s.history;
+        waiting_.push_front(std::move(s));
+        metrics_.admission_stalls += 1;
+        return std::nullopt;
+    }
+    metrics_.cached_tokens += shared;
+    metrics_.prefilled_tokens += prompt_len - shared;
+    metrics_.prefills += 1;
+    s.prompt_left = std::max<size_t>(prompt_len - shared, 1);   // the last token is always fed: its logits are wanted
+    s.pending.clear();                                          // nothing to decode until the prompt is in
+    running_.push_back(std::move(s));
+    return running_.size() - 1;
 }
 
-std::optional<size_t> Scheduler::newest_evictable(size_t protect) const {
+// The assembled step becomes the plan, and the counters learn of it.
+const Plan& Scheduler::publish(Assembly& step, PlanKind kind) {
+    plan_ = std::move(step.plan);
+    plan_.kind = kind;
+    if (kind == PlanKind::Idle) return plan_;
+    metrics_.steps += 1;
+    metrics_.decode_rows += step.decode_rows;
+    if (step.decode_rows > 0) metrics_.decode_steps += 1;
+    if (kind == PlanKind::Mixed) metrics_.mixed_steps += 1;
+    return plan_;
+}
+
+// A prompt at the front that no amount of waiting will serve (more pages than
+// the pools have in all, or more positions than the model knows) is answered at
+// once with an empty result, so that it does not block the queue behind it
+// (scheduler.rs:681-690).  The refusal is a step of its own: its commit reports it.
+bool Scheduler::turn_away_front() {
+    if (waiting_.empty()) return false;
+    const size_t prompt_len = waiting_.front().pending.size();
+    const size_t most_a_step = chunk_ > 0 ? chunk_ : prompt_len;
+    const bool too_long = max_positions_ > 0 && prompt_len > max_positions_;
+    if (!too_long && cache_->fits_in_total(prompt_len, most_a_step)) return false;
+    Sequence s = std::move(waiting_.front());
+    waiting_.pop_front();
+    plan_ = Plan{};
+    plan_.kind = PlanKind::Refused;
+    plan_.refused = s.id;
+    outcome_pending_refusal_ = FinishedInfo{s.id, Finish::Length, s.prompt_tokens, s.generated, s.preemptions};
+    return true;
+}
+
+std::optional<size_t> Scheduler::newest_other_than(size_t keep) const {
     for (size_t i = running_.size(); i-- > 0;)
-        if (i != protect && running_[i].finish == Finish::None) return i;
+        if (i != keep && running_[i].finish == Finish::None) return i;
     return std::nullopt;
 }
 
-// Take a request's pages back and put it at the front of the queue, to be
-// recomputed from everything the model has seen (scheduler.rs:700-712).
-void Scheduler::preempt(size_t index) {
+// A resident gives everything back and queues again at the front; when its turn
+// comes it is fed its whole history, prompt and output so far, as a prompt, so
+// the tokens it has already returned stay returned (scheduler.rs:700-712).
+void Scheduler::evict(size_t index) {
     Sequence s = std::move(running_[index]);
     running_.erase(running_.begin() + static_cast<long>(index));
     cache_->free_sequence(s.id);
@@ -294,7 +246,11 @@ void Scheduler::preempt(size_t index) {
     waiting_.push_front(std::move(s));
 }
 
-// Record that a step ran: keep its tokens, retire what it finished
+// The step ran.  Its rows' tokens are now in the pages (the lengths move, and
+// pages that filled up get their names for the prefix cache: only now is it
+// known that the tokens are really there); the sampled tokens join their
+// requests' histories and become what the next step feeds; requests that hit a
+// stop token, their budget or the model's last position are retired
 // (scheduler.rs:717-764).
 const Outcome& Scheduler::commit(const std::vector<uint32_t>& sampled) {
     outcome_ = Outcome{};
@@ -303,8 +259,6 @@ const Outcome& Scheduler::commit(const std::vector<uint32_t>& sampled) {
         if (!s) continue;
         cache_->advance(id, written);
         s->prompt_left = s->prompt_left > written ? s->prompt_left - written : 0;
-        // Name whatever this step filled.  Done here rather than in the step,
-        // because only now is it known that the tokens are really there.
         cache_->publish_full(id, s->history.data(), s->history.size());
     }
     const size_t count = std::min(plan_.ids.size(), sampled.size());
@@ -347,7 +301,7 @@ void Scheduler::cancel(uint64_t id) {
     retire(dropped);
 }
 
-// Hand every finished request's pages back to the pools (scheduler.rs:782-793).
+// Finished requests leave the running set and their pages return to the pools (scheduler.rs:782-793).
 void Scheduler::retire(Outcome& outcome) {
     size_t index = 0;
     while (index < running_.size()) {

@@ -1,9 +1,12 @@
 // What runs on the next step.  The scheduler decides and the engine executes:
-// nothing here touches a tensor.  It admits requests, cuts prompts into
-// portions under a token budget, puts one portion beside every running
-// request's next token, takes pages from the cache manager, evicts the newest
-// request when the pools run dry, and takes back the tokens that came out.
-// (Reference: crates/pagedllm/src/scheduler.rs.)
+// nothing here touches a tensor.  A step is assembled out of one allowance of
+// tokens and rows: first a row for every resident request's next token, then
+// the tokens of prompts (the one part-way through, then newcomers) until the
+// allowance is spent; pages come from the cache manager as rows are handed
+// out, the newest request gives its pages up when the pools run dry, and the
+// tokens that came out of a step are taken back in.  The policy (which request
+// goes first, who is evicted, what is refused) is the reference's,
+// crates/pagedllm/src/scheduler.rs, and its scenarios are the tests.
 #pragma once
 
 #include <cstdint>
@@ -105,16 +108,28 @@ public:
     Sequence* sequence(uint64_t id);
 
 private:
-    std::optional<Plan> mixed();
-    std::optional<Plan> admit();
-    Plan decode();
-    std::optional<Plan> refuse_unservable();
-    void start_next_prompt();
-    std::optional<size_t> newest_evictable(size_t protect) const;
-    void preempt(size_t index);
+    // A step under assembly: rows and tokens are handed out of one allowance, whoever asks.
+    struct Assembly {
+        Plan plan;
+        size_t tokens_left;
+        size_t rows_left;
+        size_t decode_rows = 0;
+        size_t prompt_tokens = 0;
+        Assembly(size_t tokens, size_t rows) : tokens_left(tokens), rows_left(rows) {}
+    };
+    enum class WhenDry { GiveUp, EvictNewest };   // what seating does when a resident's next token has no page
+    enum class Entry { PortionWise, Whole };      // how a newcomer's prompt will be fed
+
+    bool turn_away_front();
+    bool seat_residents(Assembly& step, WhenDry policy);
+    bool feed_prompts(Assembly& step, Entry entry);
+    std::optional<size_t> bring_in_front(Entry entry);
+    void row_of_tokens(Assembly& step, Sequence& s, size_t first, size_t count, bool wants_logits);
+    const Plan& publish(Assembly& step, PlanKind kind);
+    void evict(size_t index);
+    std::optional<size_t> newest_other_than(size_t keep) const;
     void retire(Outcome& outcome);
     std::optional<size_t> prompt_in_flight() const;
-    PlanEntry entry_for(Sequence& s, size_t start, std::vector<uint32_t> tokens, bool wants);
 
     CacheManager* cache_;
     std::deque<Sequence> waiting_;
