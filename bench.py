@@ -54,6 +54,8 @@ PREFILL_TOKENS = 2048
 BLOCK_SIZE = 16
 MIXED_SLICE = 512            # --only mixed: a slice of a prompt this long beside 63 decoded tokens
 MIXED_DECODES = 63
+# Layers of the two larger shapes in the default run's extra points (of 36 and 64).
+OTHER_SHAPE_LAYERS = {"8b": 6, "32b": 4}
 
 
 def say(message: str) -> None:
@@ -131,6 +133,123 @@ def timed(fn, steps: int, warmup: int) -> float:
     return (time.perf_counter() - start) / steps
 
 
+class Workbench:
+    """A random model of one of the shapes with some of its layers, its cache and a step runner, and the
+    measurements that are taken on it."""
+
+    def __init__(self, shape: str, layers: int, device, largest_batch: int, steps: int, graphs: bool = True,
+                 context: int | None = None, prefill_room: bool = True):
+        import torch
+
+        from paged_llm_rs_amd import write_random_model
+        from paged_llm_rs_amd.cache import PagedCache
+        from paged_llm_rs_amd.engine.step import StepRunner
+        from paged_llm_rs_amd.parts.model import load_model
+
+        self.model_name, config, self.context, _ = SHAPES[shape]
+        if context is not None:
+            self.context = context
+        self.full_layers = config["num_hidden_layers"]
+        self.layers = layers
+        self.cfg = dict(config)
+        self.cfg["num_hidden_layers"] = layers
+        self.tmp = tempfile.TemporaryDirectory()
+        say(f"writing a random {layers}-layer model folder of the {self.model_name} shape")
+        t0 = time.time()
+        self.folder = write_random_model(Path(self.tmp.name) / "model", self.cfg, seed=0, std=0.02, gain_std=0.1,
+                                         dtype="bfloat16")
+        say(f"written in {time.time() - t0:.0f} s; loading")
+        self.config, self.model = load_model(self.folder, "bfloat16", device)
+        say("loaded")
+        self.weight_bytes, self.layer_flops, self.head_flops = model_bytes_and_flops(self.cfg, 2)
+        self.kv_token = kv_bytes_per_token(self.cfg, 2)
+        pages = (largest_batch * (self.context + steps + 64) + (PREFILL_TOKENS + 64 if prefill_room else 0)) // BLOCK_SIZE + largest_batch
+        self.cache = PagedCache(self.model.cache_layout, BLOCK_SIZE, pages, torch.bfloat16, device, max_seqs=largest_batch + 1)
+        self.runner = StepRunner(self.model, self.cache, graphs=graphs)
+
+    def close(self) -> None:
+        import gc
+
+        import torch
+
+        self.runner = self.cache = self.model = None
+        self.tmp.cleanup()
+        gc.collect()
+        torch.cuda.empty_cache()
+
+    def decode_point(self, batch: int, steps: int, warmup: int):
+        """(seconds a step, tokens a second, bytes a step has to read) of decode steps at ``batch``."""
+        bench = DecodeBench(self.model, self.cache, self.runner, batch, self.context, seed=batch)
+        seconds = timed(bench.step, steps, warmup)
+        context_mid = self.context + warmup + steps / 2
+        bench.free()
+        return seconds, batch / seconds, self.weight_bytes + batch * context_mid * self.kv_token
+
+    def prefill_point(self, eager: bool = False):
+        from paged_llm_rs_amd.engine.batch import StepEntry
+        from paged_llm_rs_amd.engine.step import run_step
+
+        say(f"prefill, {PREFILL_TOKENS} tokens")
+        rng = random.Random(2048)
+        prompt = [rng.randrange(self.cfg["vocab_size"]) for _ in range(PREFILL_TOKENS)]
+        cache, model, runner = self.cache, self.model, self.runner
+
+        def prefill():
+            cache.manager.add_sequence(1000)
+            assert cache.manager.reserve(1000, PREFILL_TOKENS)
+            entry = [StepEntry(1000, prompt, 0, [PREFILL_TOKENS - 1])]
+            if eager:
+                run_step(model, cache, entry)
+            else:
+                runner.run(entry)        # as the engine runs it: a shape of step that comes again is replayed from a graph
+            cache.manager.free_sequence(1000)
+
+        seconds_prefill = timed(prefill, 5, 3)
+        d, nq = self.cfg["head_dim"], self.cfg["num_attention_heads"]
+        attention_flops = self.layers * 4 * nq * d * (PREFILL_TOKENS * (PREFILL_TOKENS + 1) // 2)
+        flops = self.layer_flops * PREFILL_TOKENS + self.head_flops + attention_flops
+        return {"value": round(PREFILL_TOKENS / seconds_prefill, 1), "tokens": PREFILL_TOKENS,
+                "ms": round(seconds_prefill * 1e3, 3),
+                "frac": round(flops / seconds_prefill / MFMA_PEAK["bf16"], 4)}
+
+    def mixed_point(self, steps: int, warmup: int):
+        """One step of the third slice of a prompt beside 63 requests that bring one token each.  The step is
+        not committed, so every run of it writes the same places of the cache again."""
+        from paged_llm_rs_amd.engine.batch import StepEntry
+        from paged_llm_rs_amd.engine.step import commit_step, run_step
+
+        cache, model, runner, cfg, context = self.cache, self.model, self.runner, self.cfg, self.context
+        say(f"mixed step: {MIXED_DECODES} decoded tokens at context {context} beside a slice of {MIXED_SLICE}")
+        bench = DecodeBench(model, cache, runner, MIXED_DECODES, context, seed=3)
+        rng = random.Random(512)
+        long_prompt = [rng.randrange(cfg["vocab_size"]) for _ in range(PREFILL_TOKENS)]
+        behind = 2 * MIXED_SLICE
+        cache.manager.add_sequence(1000)
+        assert cache.manager.reserve(1000, behind)
+        first = [StepEntry(1000, long_prompt[:behind], 0, [])]
+        run_step(model, cache, first)
+        commit_step(cache, first)
+        assert cache.manager.reserve(1000, MIXED_SLICE)
+        entries = [StepEntry(1000, long_prompt[behind:behind + MIXED_SLICE], behind, [])]
+        for i, tok in zip(bench.ids, bench.tokens):
+            assert cache.manager.reserve(i, 1)
+            entries.append(StepEntry(i, [tok], cache.manager.tokens(i), [0]))
+        seconds = timed(lambda: runner.run(entries).greedy_tokens(), steps, warmup)
+        cache.manager.free_sequence(1000)
+        bench.free()
+        rows = MIXED_SLICE + MIXED_DECODES
+        d, nq = cfg["head_dim"], cfg["num_attention_heads"]
+        attention_flops = self.layers * 4 * nq * d * (MIXED_SLICE * (behind + (MIXED_SLICE + 1) // 2) + MIXED_DECODES * context)
+        flops = self.layer_flops * rows + self.head_flops * MIXED_DECODES + attention_flops
+        step_bytes = self.weight_bytes + (MIXED_DECODES * context + behind + MIXED_SLICE) * self.kv_token
+        return {
+            "model": f"{self.model_name} shape", "layers": self.layers, "layers_full": self.full_layers, "rows": rows,
+            "decode_context": context, "ms": round(seconds * 1e3, 3), "tokens_per_s": round(rows / seconds, 1),
+            "hbm_floor_ms": round(step_bytes / HBM_PEAK * 1e3, 3), "mfma_floor_ms": round(flops / MFMA_PEAK["bf16"] * 1e3, 3),
+            "frac_hbm": round(step_bytes / seconds / HBM_PEAK, 4), "frac_mfma": round(flops / seconds / MFMA_PEAK["bf16"], 4),
+        }
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -143,6 +262,8 @@ def main() -> int:
                         help="fewer layers than the model has, where memory or time needs it; both numbers are reported")
     parser.add_argument("--no-graphs", action="store_true", help="run decode steps eagerly instead of as HIP graphs")
     parser.add_argument("--skip-points", action="store_true", help="leave out batch 1 and 64 and the prefill")
+    parser.add_argument("--no-other-shapes", action="store_true",
+                        help="leave out the points of the 8b shape (a mixed step) and the 32b shape (decode at batch 64)")
     parser.add_argument("--prefill-eager", action="store_true",
                         help="launch the prefill step kernel by kernel every time (a prompt length seen once)")
     parser.add_argument("--only", choices=["decode", "prefill", "engine", "mixed", "serving"], default=None,
@@ -159,100 +280,29 @@ def main() -> int:
 
     import torch
 
-    from paged_llm_rs_amd import write_random_model
-    from paged_llm_rs_amd.cache import PagedCache
     from paged_llm_rs_amd.engine.batch import StepEntry
-    from paged_llm_rs_amd.engine.step import StepRunner, commit_step, require_gpu, run_step
-    from paged_llm_rs_amd.parts.model import load_model
+    from paged_llm_rs_amd.engine.step import commit_step, require_gpu, run_step
 
     device = require_gpu("cuda:0")
     model_name, CONFIG, CONTEXT, default_layers = SHAPES[args.shape]
     FULL_LAYERS = CONFIG["num_hidden_layers"]
     if args.layers is None:
         args.layers = default_layers
-    cfg = dict(CONFIG)
-    cfg["num_hidden_layers"] = args.layers
-    tmp = tempfile.TemporaryDirectory()
-    say(f"writing a random {args.layers}-layer model folder")
-    t0 = time.time()
-    folder = write_random_model(Path(tmp.name) / "model", cfg, seed=0, std=0.02, gain_std=0.1, dtype="bfloat16")
-    say(f"written in {time.time() - t0:.0f} s; loading")
-    config, model = load_model(folder, "bfloat16", device)
-    say("loaded")
-
-    element = 2
-    weight_bytes, layer_flops, head_flops = model_bytes_and_flops(cfg, element)
-    kv_token = kv_bytes_per_token(cfg, element)
-    largest = max(64, args.batch)
-    pages = (largest * (CONTEXT + args.steps + args.warmup + 64) + PREFILL_TOKENS + 64) // BLOCK_SIZE + largest
-    cache = PagedCache(model.cache_layout, BLOCK_SIZE, pages, torch.bfloat16, device, max_seqs=largest + 1)
-
-    runner = StepRunner(model, cache, graphs=not args.no_graphs)
-
-    def decode_point(batch: int, steps: int, warmup: int):
-        bench = DecodeBench(model, cache, runner, batch, CONTEXT, seed=batch)
-        seconds = timed(bench.step, steps, warmup)
-        context_mid = CONTEXT + warmup + steps / 2
-        bench.free()
-        return seconds, batch / seconds, weight_bytes + batch * context_mid * kv_token
+    bench = Workbench(args.shape, args.layers, device, largest_batch=max(64, args.batch),
+                      steps=args.steps + args.warmup, graphs=not args.no_graphs)
+    cfg, model, cache, runner, folder, tmp = bench.cfg, bench.model, bench.cache, bench.runner, bench.folder, bench.tmp
+    weight_bytes, layer_flops, head_flops, kv_token = bench.weight_bytes, bench.layer_flops, bench.head_flops, bench.kv_token
+    decode_point = bench.decode_point
 
     def prefill_point():
-        say(f"prefill, {PREFILL_TOKENS} tokens")
-        rng = random.Random(2048)
-        prompt = [rng.randrange(cfg["vocab_size"]) for _ in range(PREFILL_TOKENS)]
-
-        def prefill():
-            cache.manager.add_sequence(1000)
-            assert cache.manager.reserve(1000, PREFILL_TOKENS)
-            entry = [StepEntry(1000, prompt, 0, [PREFILL_TOKENS - 1])]
-            if args.prefill_eager:
-                run_step(model, cache, entry)
-            else:
-                runner.run(entry)        # as the engine runs it: a shape of step that comes again is replayed from a graph
-            cache.manager.free_sequence(1000)
-
-        seconds_prefill = timed(prefill, 5, 3)
-        d, nq = cfg["head_dim"], cfg["num_attention_heads"]
-        attention_flops = args.layers * 4 * nq * d * (PREFILL_TOKENS * (PREFILL_TOKENS + 1) // 2)
-        flops = layer_flops * PREFILL_TOKENS + head_flops + attention_flops
-        return {"value": round(PREFILL_TOKENS / seconds_prefill, 1), "tokens": PREFILL_TOKENS,
-                "ms": round(seconds_prefill * 1e3, 3),
-                "frac": round(flops / seconds_prefill / MFMA_PEAK["bf16"], 4)}
+        return bench.prefill_point(eager=args.prefill_eager)
 
     if args.only == "prefill":
         print(json.dumps({"prefill": prefill_point()}), flush=True)
         tmp.cleanup()
         return 0
     if args.only == "mixed":
-        # 63 requests with CONTEXT tokens each bring one token; one more brings the third slice of a prompt.
-        # The step is not committed, so every run of it writes the same places of the cache again.
-        say(f"mixed step: {MIXED_DECODES} decoded tokens at context {CONTEXT} beside a slice of {MIXED_SLICE}")
-        bench = DecodeBench(model, cache, runner, MIXED_DECODES, CONTEXT, seed=3)
-        rng = random.Random(512)
-        long_prompt = [rng.randrange(cfg["vocab_size"]) for _ in range(PREFILL_TOKENS)]
-        behind = 2 * MIXED_SLICE
-        cache.manager.add_sequence(1000)
-        assert cache.manager.reserve(1000, behind)
-        first = [StepEntry(1000, long_prompt[:behind], 0, [])]
-        run_step(model, cache, first)
-        commit_step(cache, first)
-        assert cache.manager.reserve(1000, MIXED_SLICE)
-        entries = [StepEntry(1000, long_prompt[behind:behind + MIXED_SLICE], behind, [])]
-        for i, tok in zip(bench.ids, bench.tokens):
-            assert cache.manager.reserve(i, 1)
-            entries.append(StepEntry(i, [tok], cache.manager.tokens(i), [0]))
-        seconds = timed(lambda: runner.run(entries).greedy_tokens(), args.steps, args.warmup)
-        rows = MIXED_SLICE + MIXED_DECODES
-        d, nq = cfg["head_dim"], cfg["num_attention_heads"]
-        attention_flops = args.layers * 4 * nq * d * (MIXED_SLICE * (behind + (MIXED_SLICE + 1) // 2) + MIXED_DECODES * CONTEXT)
-        flops = layer_flops * rows + head_flops * MIXED_DECODES + attention_flops
-        step_bytes = weight_bytes + (MIXED_DECODES * CONTEXT + behind + MIXED_SLICE) * kv_token
-        print(json.dumps({"mixed": {
-            "model": f"{model_name} shape", "layers": args.layers, "layers_full": FULL_LAYERS, "rows": rows,
-            "decode_context": CONTEXT, "ms": round(seconds * 1e3, 3), "tokens_per_s": round(rows / seconds, 1),
-            "hbm_floor_ms": round(step_bytes / HBM_PEAK * 1e3, 3), "mfma_floor_ms": round(flops / MFMA_PEAK["bf16"] * 1e3, 3),
-            "frac_hbm": round(step_bytes / seconds / HBM_PEAK, 4), "frac_mfma": round(flops / seconds / MFMA_PEAK["bf16"], 4),
-        }}), flush=True)
+        print(json.dumps({"mixed": bench.mixed_point(args.steps, args.warmup)}), flush=True)
         tmp.cleanup()
         return 0
     if args.only == "serving":
@@ -374,6 +424,25 @@ def main() -> int:
             points[f"decode_b{batch}"] = round(v, 1)
         line["points"] = points
         line["prefill"] = prefill_point()
+        if args.shape == "0.6b" and not args.no_other_shapes:
+            # The two larger shapes, with fewer layers than they have (both numbers are in ``config``): the time
+            # of a layer is what their fractions of the peaks need, and the whole run stays a few minutes.
+            bench.close()
+            other = Workbench("8b", OTHER_SHAPE_LAYERS["8b"], device, largest_batch=MIXED_DECODES + 1, steps=8)
+            mixed = other.mixed_point(10, 3)
+            other.close()
+            points["mixed_8b_tok_s"] = mixed["tokens_per_s"]
+            points["mixed_8b_ms"] = mixed["ms"]
+            points["mixed_8b_frac_mfma"] = mixed["frac_mfma"]
+            other = Workbench("32b", OTHER_SHAPE_LAYERS["32b"], device, largest_batch=64, steps=20, prefill_room=False)
+            say("decode, batch 64, of the 32B shape")
+            s32, v32, bytes32 = other.decode_point(64, 10, 3)
+            other.close()
+            points["decode_32b_b64_tok_s"] = round(v32, 1)
+            points["decode_32b_b64_ms"] = round(s32 * 1e3, 3)
+            points["decode_32b_b64_frac_hbm"] = round(bytes32 / s32 / HBM_PEAK, 4)
+            line["config"].update({"layers_8b": OTHER_SHAPE_LAYERS["8b"], "layers_8b_full": SHAPES["8b"][1]["num_hidden_layers"],
+                                   "layers_32b": OTHER_SHAPE_LAYERS["32b"], "layers_32b_full": SHAPES["32b"][1]["num_hidden_layers"]})
 
     print(json.dumps(line), flush=True)
     tmp.cleanup()
