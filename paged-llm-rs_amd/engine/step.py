@@ -82,6 +82,21 @@ def _bucket(n: int, least: int = 1) -> int:
     return b
 
 
+def _all_idle(host: torch.Tensor, layout: dict) -> torch.Tensor:
+    """A copy of a step's descriptor in which every row is padding: position -1, no context, no state slot, no
+    pages.  The rows, the requests they belong to and the wanted places stay, so the step has the same shape;
+    a step of such rows reads and writes nothing that belongs to a request."""
+    idle = host.clone()
+    for name, (begin, count) in layout.items():
+        if name == "token_ids":
+            idle[begin:begin + count] = 0
+        elif name == "ctx_len":
+            idle[begin:begin + count] = 0
+        elif name in ("positions", "state_slots") or name.startswith("block_table_"):
+            idle[begin:begin + count] = -1
+    return idle
+
+
 class _DescriptorRing:
     """Pinned buffers for a graph's step descriptor, used in turn.  A descriptor travels to the device without
     the host waiting, so the copy of one step has to have left its buffer before that buffer is written again.
@@ -173,11 +188,15 @@ class DecodeGraph:
         return logits, kernels.argmax(logits)
 
     def capture(self) -> None:
-        self.device_buf.copy_(self.ring.host)
+        # The run before the capture (everything that initialises lazily does so there, outside the capture)
+        # and the capture itself see a step of idle rows only: they write no page and touch no request's
+        # state, so the one replay that follows is the only time the real step runs.  (A mixer that keeps
+        # state of its own would otherwise advance it twice on the step that brings a capture about.)
+        self.device_buf.copy_(_all_idle(self.ring.host, self.layout))
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
-            self._forward()        # everything that initialises lazily does so outside the capture
+            self._forward()
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         self.graph = torch.cuda.CUDAGraph()
@@ -250,7 +269,8 @@ class ShapeGraph:
                            pad_to=self.rows, short_bound=self.short_bound)
 
     def capture(self) -> None:
-        self.device_buf.copy_(self.ring.host)
+        # (over a step of idle rows, as in DecodeGraph.capture: the real step runs once, in the replay)
+        self.device_buf.copy_(_all_idle(self.ring.host, self.layout))
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):

@@ -276,6 +276,103 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path, dtype)
             tokens.append(produced)
 
 
+class RunningSumMixer:
+    """out[t] = W . sum(x[0..t]): the sum so far is the request's state.  Written with device operations only and
+    tolerant of padding rows (position -1, state slot -1), so its steps may be captured as graphs."""
+    graph_safe = True
+
+    @staticmethod
+    def declare(spec, hidden):
+        from paged_llm_rs_amd.weights.loader import ParamDecl
+        return [ParamDecl("proj.weight", (hidden, hidden))]
+
+    def __init__(self, spec, hidden, params, dtype, device, shared):
+        self.w, self.hidden = params["proj.weight"], hidden
+
+    def cache_spec(self):
+        return None
+
+    def state_spec(self):
+        from paged_llm_rs_amd.cache import StateSpec
+        return StateSpec((self.hidden,), torch.float32)
+
+    def forward(self, x, ctx):
+        b, state = ctx.batch, ctx.state()
+        seq, starts, counts, slots = b.seq_of.long(), b.q_start.long(), b.q_len.long(), b.state_slots.long()
+        live = slots >= 0
+        rows = torch.where((b.positions >= 0)[:, None], x.float(), torch.zeros((), device=x.device))
+        through = rows.cumsum(0)
+        before = torch.where((starts > 0)[:, None], through[(starts - 1).clamp_min(0)], torch.zeros((), device=x.device))
+        held = torch.where(live[:, None], state[slots.clamp_min(0)], torch.zeros((), device=x.device))
+        out = ((held[seq] + through - before[seq]) @ self.w.float().t()).to(x.dtype)
+        brought = through[(starts + counts - 1).clamp_min(0)] - before
+        state.index_add_(0, slots.clamp_min(0), torch.where((live & (counts > 0))[:, None], brought, torch.zeros((), device=x.device)))
+        return out
+
+
+@dataclass(frozen=True)
+class RunningSumSpec:
+    kind: str = "running_sum"
+
+
+class SumToyConfig(ToyConfig):
+    def model_spec(self):
+        import dataclasses
+
+        spec = super().model_spec()
+        first = dataclasses.replace(spec.layers[0], mixer=RunningSumSpec())
+        return dataclasses.replace(spec, layers=(first, spec.layers[1]))
+
+
+def sum_toy_plain(weights, tokens):
+    w = {k: v.double() for k, v in weights.items()}
+    n = len(tokens)
+    x = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+    eps = TOY["rms_norm_eps"]
+    normed = plain.rms_norm(x, w["model.layers.0.input_layernorm.weight"], eps)
+    x = x + normed.cumsum(0) @ w["model.layers.0.self_attn.proj.weight"].T
+    x = x + plain.swiglu_mlp(plain.rms_norm(x, w["model.layers.0.post_attention_layernorm.weight"], eps), w, "model.layers.0.mlp")
+    x = plain.decoder_block(x, w, "model.layers.1", TOY, torch.arange(n))
+    return plain.rms_norm(x, w["model.norm.weight"], eps) @ w["model.embed_tokens.weight"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_mixer_with_state_in_captured_steps(tmp_path, dtype):
+    """A mixer that adds every token it sees into its request's state slot, in steps that are captured as graphs:
+    the step that brings a capture about must advance the state once, like every other.  (The run before a
+    capture and the capture itself go over idle rows.)  Steps of one token a request are captured at their first
+    coming, steps of other shapes at their second; both happen here, and graphs on and off agree."""
+    from safetensors.torch import load_file
+
+    from paged_llm_rs_amd import register_architecture, write_random_model
+    from paged_llm_rs_amd.engine.replay import Replayer
+    from paged_llm_rs_amd.parts import register_mixer
+
+    register_mixer("running_sum", RunningSumMixer)
+    register_architecture("SumToyForCausalLM", SumToyConfig, model_type="sum_toy")
+    config = dict(TOY, architectures=["SumToyForCausalLM"], model_type="sum_toy")
+    folder = write_random_model(tmp_path / "toy", config, seed=6, std=0.05, gain_std=0.2, dtype=dtype)
+    weights = load_file(str(folder / "model.safetensors"))
+    prompts = ru.make_prompts(TOY["vocab_size"], [30, 9, 41, 17, 25, 12], seed=4)
+    want = {name: sum_toy_plain(weights, toks) for name, toks in prompts.items()}
+    tolerance = 1e-5 if dtype == "float32" else 2e-2
+    # the same portion sizes for every request, so that shapes of step come again and are captured
+    schedules = [(ru.tail_decoded(prompts, 8), 1), (ru.portions(prompts, sizes=(4, 4, 4, 4, 4, 4, 4, 4, 4, 4, 4)), 1),
+                 (ru.mixed(prompts, seed=7, max_live=3), 3)]
+    for steps, live in schedules:
+        outcomes = []
+        for graphs in (True, False):
+            r = Replayer(folder, dtype, max_tokens=ru.pool_tokens(prompts, live), block_size=8, max_live=4, graphs=graphs)
+            assert r.runner.use_graphs == graphs
+            got = ru.collect(r, steps)
+            worst, where = ru.worst_error(got, want)
+            assert worst <= tolerance, f"graphs {graphs}: {worst:.3e} at {where}"
+            if graphs:
+                assert r.runner.graph_steps > 0, "some steps were replayed from graphs"
+            outcomes.append(got)
+        assert outcomes[0].keys() == outcomes[1].keys()
+
+
 # --- a toy feed-forward with routing and a toy position encoding, defined here ----------------------------------------------
 
 @dataclass(frozen=True)
