@@ -85,8 +85,7 @@ extern "C" int pl_paged_attention_plain(const void* q, int q_stride, void* out, 
                                         int block_size, const void* k_pool, const void* v_pool, int n,
                                         int nq, int nkv, int d, float scale, int window, int dtype,
                                         hipStream_t stream) {
-    PL_REQUIRE(d > 0 && d <= PL_MAX_HEAD_DIM && d % 16 == 0,
-               "attention: head size %d, which has to be a multiple of 16 up to %d", d, PL_MAX_HEAD_DIM);
+    PL_REQUIRE(d > 0 && d <= PL_MAX_HEAD_DIM, "attention: head size %d, which has to be between 1 and %d", d, PL_MAX_HEAD_DIM);
     PL_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "attention: %d query heads over %d key heads", nq, nkv);
     PL_REQUIRE(block_size > 0 && max_blocks > 0 && q_stride >= nq * d && window >= 0,
                "attention: block size %d, %d blocks a row, query stride %d, window %d", block_size, max_blocks, q_stride, window);

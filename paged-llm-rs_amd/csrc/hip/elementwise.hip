@@ -546,8 +546,8 @@ extern "C" int pl_qk_norm_rope_kv_write(
     const float* cos_table, const float* sin_table, int rot, const int* positions,
     const int* seq_of, const int* block_table, int max_blocks, int block_size, void* k_pool,
     void* v_pool, int n, int nq, int nkv, int d, int write_kv, int dtype, hipStream_t stream) {
-    PL_REQUIRE(d > 0 && d <= PL_MAX_HEAD_DIM && d % 16 == 0,
-               "qk_norm_rope: head size %d, which has to be a multiple of 16 up to %d", d, PL_MAX_HEAD_DIM);
+    // (any head size: the kernels that work on eight elements a lane take multiples of 16, one wave a head takes the rest)
+    PL_REQUIRE(d > 0 && d <= PL_MAX_HEAD_DIM, "qk_norm_rope: head size %d, which has to be between 1 and %d", d, PL_MAX_HEAD_DIM);
     PL_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0, "qk_norm_rope: rotated width %d of a head of %d", rot, d);
     PL_REQUIRE(nq > 0 && nkv > 0 && block_size > 0 && max_blocks > 0,
                "qk_norm_rope: %d query heads, %d key heads, block size %d, %d blocks a row", nq, nkv, block_size, max_blocks);
@@ -570,7 +570,7 @@ extern "C" int pl_qk_norm_rope_kv_write(
         PL_CHECK_LAUNCH("qk_norm_rope_kv_write");
         return 0;
     }
-    if (rot % 16 == 0) {
+    if (rot % 16 == 0 && d % 16 == 0) {
         // a workgroup takes two groups of 4 * (64 / (d/8)) heads of a token at a time
         const int per_group = 4 * (PL_WAVE / (d / 8));
         dim3 wide(n, pl_ceil_div(heads, 2 * per_group));

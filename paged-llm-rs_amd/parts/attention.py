@@ -39,8 +39,11 @@ class PagedAttention:
         if spec.num_heads % spec.num_kv_heads:
             raise UnsupportedError(f"{spec.num_heads} query heads over {spec.num_kv_heads} key heads, "
                                    "which do not group evenly")
-        if spec.head_dim % 16 or not 16 <= spec.head_dim <= 256:
-            raise UnsupportedError(f"head size {spec.head_dim}: the kernels take multiples of 16 up to 256")
+        if not 1 <= spec.head_dim <= 256:
+            raise UnsupportedError(f"head size {spec.head_dim}: the kernels take head sizes up to 256")
+        if spec.head_dim % 16 and dtype != torch.float32:
+            raise UnsupportedError(f"head size {spec.head_dim}: the bfloat16 kernels take multiples of 16 "
+                                   "(the 32-bit path takes any size up to 256)")
         if spec.qk_norm is not None and spec.qk_norm.kind != "rms_norm":
             raise UnsupportedError(f"q/k norm {spec.qk_norm.kind!r}, only rms_norm is implemented")
         self.spec = spec

@@ -101,7 +101,7 @@ def tables(max_pos, rot, theta):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("nq,nkv,d,bs,norm", [(4, 2, 16, 4, True), (6, 1, 48, 16, True), (3, 3, 128, 8, False),
                                               (8, 2, 256, 2, True), (5, 5, 80, 16, True), (16, 8, 128, 16, True),
-                                              (7, 1, 128, 4, True)])
+                                              (7, 1, 128, 4, True), (3, 1, 24, 4, True), (2, 2, 10, 8, False)])
 def test_qk_norm_rope_kv_write(dtype, nq, nkv, d, bs, norm):
     from paged_llm_rs_amd import kernels
 
@@ -168,10 +168,10 @@ def test_rotation_of_part_of_a_head_and_refused_sizes():
     want = rope_ref(before.double().reshape(n, 4, d)[:, :nq], positions, 1e4, rot)
     assert rel(qkv.reshape(n, 4, d)[:, :nq], want) < 2e-6
     assert torch.equal(qkv.reshape(n, 4, d)[:, :nq, rot:], before.reshape(n, 4, d)[:, :nq, rot:])
-    with pytest.raises(TensorError, match="multiple of 16"):
-        kernels.qk_norm_rope_kv_write(torch.zeros(1, 4 * 24, device=DEV), None, None, 0.0, None, None, 0,
-                                      positions[:1], seq_of[:1], bt, bs, torch.zeros(16, 24, device=DEV),
-                                      torch.zeros(16, 24, device=DEV), 2, 1, 24)
+    with pytest.raises(TensorError, match="between 1 and 256"):
+        kernels.qk_norm_rope_kv_write(torch.zeros(1, 4 * 264, device=DEV), None, None, 0.0, None, None, 0,
+                                      positions[:1], seq_of[:1], bt, bs, torch.zeros(16, 264, device=DEV),
+                                      torch.zeros(16, 264, device=DEV), 2, 1, 264)
 
 
 # --- feed-forward ------------------------------------------------------------------------------------------
@@ -537,6 +537,28 @@ def test_paged_attention_of_single_tokens(kernel, nq, nkv, d, bs, ctx_lens, wind
         err = rel(out[i].reshape(nq, d), want)
         assert err < (2e-6 if dtype == torch.float32 else 1e-2), f"token {i} (request {s}, position {p}): {err:.3e}"
     assert bool((out[-1] == 7.0).all()), "a padding row is not written"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nq,nkv,d,bs,ctx_lens,window", [(3, 1, 24, 4, [37, 5], 0), (4, 2, 10, 8, [70], 0),
+                                                          (2, 2, 100, 16, [130, 20], 33), (5, 5, 1, 2, [9], 0)])
+def test_the_plain_attention_kernel_takes_any_head_size(dtype, nq, nkv, d, bs, ctx_lens, window):
+    """The plain kernel (the 32-bit path's, and the others' check) has no width it works in units of."""
+    from paged_llm_rs_amd import kernels
+
+    bt, k_pool, v_pool, keys, values = build_paged(nkv, d, bs, ctx_lens, dtype, seed=d)
+    toks = [(s, p) for s, c in enumerate(ctx_lens) for p in sorted({c - 1, c // 2, 0})]
+    n = len(toks)
+    stride = (nq + 2 * nkv) * d
+    q = torch.randn(n, stride, device=DEV).to(dtype)
+    positions = torch.tensor([p for _, p in toks], dtype=torch.int32, device=DEV)
+    seq_of = torch.tensor([s for s, _ in toks], dtype=torch.int32, device=DEV)
+    scale = 1 / math.sqrt(d)
+    out = torch.full((n, nq * d), 7.0, dtype=dtype, device=DEV)
+    kernels.paged_attention_plain(q, stride, out, positions, seq_of, bt, bs, k_pool, v_pool, nq, nkv, d, scale, window)
+    for i, (s, p) in enumerate(toks):
+        want = attention_ref(q[i, :nq * d].double().cpu().reshape(nq, d), keys[s], values[s], p, nq // nkv, scale, window)
+        assert rel(out[i].reshape(nq, d), want) < (2e-6 if dtype == torch.float32 else 1e-2), f"token {i}"
 
 
 @pytest.mark.parametrize("kernel", ["plain", "decode", "grouped-1", "grouped-4"])

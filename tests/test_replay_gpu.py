@@ -380,3 +380,24 @@ def test_every_module_against_the_plain_implementation(setups, name, block_size)
             ref = want[key][n].double()
             worst = float((mine.reshape(ref.shape) - ref).abs().max() / max(1.0, float(ref.abs().max())))
             assert worst <= 1e-5, f"request {key}, {n}: {worst:.3e}"
+
+
+def test_head_sizes_that_are_no_multiple_of_16_run_in_32_bit(tmp_path):
+    """config.json may give any head size; the 32-bit path takes every one up to 256, the bfloat16 kernels
+    work in units of 16 and say so."""
+    from paged_llm_rs_amd.engine.replay import Replayer
+    from paged_llm_rs_amd.errors import UnsupportedError
+    from paged_llm_rs_amd.weights import write_random_model
+
+    config = dict(TINY_INIT["A"]["config"], hidden_size=60, num_attention_heads=3, num_key_value_heads=1, head_dim=20,
+                  intermediate_size=100, vocab_size=131, tie_word_embeddings=False)
+    prompts = ru.make_prompts(config["vocab_size"], [40, 7, 23, 61], seed=2)
+    folder = write_random_model(tmp_path / "f32", config, seed=8, std=0.05, gain_std=0.2, dtype="float32")
+    want = ru.plain_logits(folder, prompts)
+    for steps, live in ((ru.whole(prompts), 1), (ru.mixed(prompts, seed=3, max_live=4), 4), (ru.tail_decoded(prompts, 16), 1)):
+        got = replay(folder, "float32", prompts, steps, max_live=live, block_size=4)
+        worst, where = ru.worst_error(got, want)
+        assert worst <= TOLERANCE["float32"], f"{worst:.3e} at {where}"
+    half = write_random_model(tmp_path / "bf16", config, seed=8, std=0.05, gain_std=0.2, dtype="bfloat16")
+    with pytest.raises(UnsupportedError, match="multiples of 16"):
+        Replayer(half, "bfloat16", max_tokens=64)
