@@ -72,6 +72,20 @@ __device__ __forceinline__ float block_sum(float v, float* scratch /* >= 16 floa
     return total;
 }
 
+// ---- the activation of a gated feed-forward's gate branch ------------------------
+#define PL_ACT_SILU 0
+#define PL_ACT_GELU_TANH 1
+#define PL_ACT_GELU 2
+
+// EXACT: the library's exponential (what the 32-bit path needs); otherwise the hardware's.  `act` is the
+// same for a whole launch.
+template <bool EXACT>
+__device__ __forceinline__ float pl_activate(float g, int act) {
+    if (act == PL_ACT_SILU) return g / (1.f + (EXACT ? expf(-g) : __expf(-g)));
+    if (act == PL_ACT_GELU_TANH) return 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    return 0.5f * g * (1.f + erff(g * 0.7071067811865476f));
+}
+
 // ---- the error channel -------------------------------------------------------
 // Launchers return 0 or a negative code and leave a message for pl_last_error().
 void pl_set_error(const char* fmt, ...);

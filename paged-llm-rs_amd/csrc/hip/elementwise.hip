@@ -603,24 +603,24 @@ extern "C" int pl_qk_norm_rope_kv_write(
 }
 
 // ---------------------------------------------------------------------------
-// SwiGLU on the fused projection row [gate | up]: out = silu(gate) * up.
+// The gated activation on the fused projection row [gate | up]: out = act(gate) * up (SiLU, or a GELU).
 // ---------------------------------------------------------------------------
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t count) {
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t count, int act) {
     const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (idx >= count) return;
     const size_t row = idx / I;
     const int c = static_cast<int>(idx % I);
     const float g = to_float(gu[row * 2 * I + c]);
     const float u = to_float(gu[row * 2 * I + I + c]);
-    out[idx] = from_float<T>(g / (1.f + expf(-g)) * u);
+    out[idx] = from_float<T>(pl_activate<true>(g, act) * u);
 }
 
 // The same, eight consecutive elements a thread (one 16-byte load of each half in bfloat16), for
 // widths that are a multiple of eight.
 template <typename T>
 __global__ void __launch_bounds__(256)
-swiglu_wide_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t chunks) {
+swiglu_wide_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t chunks, int act) {
     const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (idx >= chunks) return;
     const int per_row = I / 8;
@@ -630,29 +630,30 @@ swiglu_wide_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t 
     qk_vec<T>::load(gu + row * 2 * I + c, g);
     qk_vec<T>::load(gu + row * 2 * I + I + c, u);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) r[e] = g[e] / (1.f + expf(-g[e])) * u[e];
+    for (int e = 0; e < 8; ++e) r[e] = pl_activate<true>(g[e], act) * u[e];
     qk_vec<T>::store(out + row * I + c, r);
 }
 
-extern "C" int pl_swiglu(const void* gu, void* out, int n, int I, int dtype, hipStream_t stream) {
+extern "C" int pl_swiglu(const void* gu, void* out, int n, int I, int dtype, int act, hipStream_t stream) {
     PL_REQUIRE(n >= 0 && I > 0, "swiglu: rows %d, width %d", n, I);
+    PL_REQUIRE(act >= PL_ACT_SILU && act <= PL_ACT_GELU, "swiglu: activation code %d", act);
     const size_t count = static_cast<size_t>(n) * I;
     if (count == 0) return 0;
     if (I % 8 == 0 && (dtype == PL_DTYPE_F32 || dtype == PL_DTYPE_BF16)) {
         const size_t chunks = count / 8;
         const int wide_blocks = static_cast<int>((chunks + 255) / 256);
         if (dtype == PL_DTYPE_F32)
-            swiglu_wide_kernel<float><<<wide_blocks, 256, 0, stream>>>(static_cast<const float*>(gu), static_cast<float*>(out), I, chunks);
+            swiglu_wide_kernel<float><<<wide_blocks, 256, 0, stream>>>(static_cast<const float*>(gu), static_cast<float*>(out), I, chunks, act);
         else
-            swiglu_wide_kernel<bf16_t><<<wide_blocks, 256, 0, stream>>>(static_cast<const bf16_t*>(gu), static_cast<bf16_t*>(out), I, chunks);
+            swiglu_wide_kernel<bf16_t><<<wide_blocks, 256, 0, stream>>>(static_cast<const bf16_t*>(gu), static_cast<bf16_t*>(out), I, chunks, act);
         PL_CHECK_LAUNCH("swiglu");
         return 0;
     }
     const int blocks = static_cast<int>((count + 255) / 256);
     if (dtype == PL_DTYPE_F32)
-        swiglu_kernel<float><<<blocks, 256, 0, stream>>>(static_cast<const float*>(gu), static_cast<float*>(out), I, count);
+        swiglu_kernel<float><<<blocks, 256, 0, stream>>>(static_cast<const float*>(gu), static_cast<float*>(out), I, count, act);
     else if (dtype == PL_DTYPE_BF16)
-        swiglu_kernel<bf16_t><<<blocks, 256, 0, stream>>>(static_cast<const bf16_t*>(gu), static_cast<bf16_t*>(out), I, count);
+        swiglu_kernel<bf16_t><<<blocks, 256, 0, stream>>>(static_cast<const bf16_t*>(gu), static_cast<bf16_t*>(out), I, count, act);
     else
         PL_REQUIRE(false, "swiglu: dtype code %d", dtype);
     PL_CHECK_LAUNCH("swiglu");

@@ -89,7 +89,7 @@ template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT, bool PANEL = 
 __global__ void __launch_bounds__(64 * WV)
 gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OUT* __restrict__ y,
                    const float* __restrict__ gain, float eps, const int* __restrict__ rows, int n, int N_out,
-                   int K) {
+                   int K, int act) {
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
     const int nwaves = blockDim.x / PL_WAVE;
     extern __shared__ float sk_lds[];
@@ -337,7 +337,7 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
             }
             if (threadIdx.x < 256 && row < n && col < N_out) {
                 float r = v[0];
-                if (EPI == EPI_SWIGLU) r = v[0] / (1.f + __expf(-v[0])) * v[BT - 1];
+                if (EPI == EPI_SWIGLU) r = pl_activate<false>(v[0], act) * v[BT - 1];
                 const size_t at = static_cast<size_t>(row) * N_out + col;
                 if (EPI == EPI_ADD)
                     y[at] = from_float<OUT>(to_float(y[at]) + r);
@@ -357,7 +357,7 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
 
 template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT>
 static int launch_one(int waves, const void* x, const void* w, void* y, const float* gain, float eps,
-                      const int* rows, int n, int N_out, int K, hipStream_t stream) {
+                      const int* rows, int n, int N_out, int K, int act, hipStream_t stream) {
     const int row_tiles = pl_ceil_div(n, 16 * MT);   // more than one where launch_mt deals the rows out
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
     constexpr int UA = (WV == 16 && UNR >= 2) ? UNR / 2 : UNR;   // K steps a round when rounds overlap
@@ -376,10 +376,10 @@ static int launch_one(int waves, const void* x, const void* w, void* y, const fl
     const bool several = pl_ceil_div(pl_ceil_div(K, SK_KSTEP), waves) > UNR;
     if (several)
         gemm_skinny_kernel<MT, UA, WV, PRO, EPI, OUT, false, true><<<dim3(grid, row_tiles), 64 * waves, lds_bytes, stream>>>(
-            x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps, rows, n, N_out, K);
+            x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps, rows, n, N_out, K, act);
     else
         gemm_skinny_kernel<MT, UNR, WV, PRO, EPI, OUT><<<dim3(grid, row_tiles), 64 * waves, lds_bytes, stream>>>(
-            x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps, rows, n, N_out, K);
+            x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps, rows, n, N_out, K, act);
     PL_CHECK_LAUNCH("gemm_skinny");
     return 0;
 }
@@ -396,7 +396,7 @@ template <int MT, int WV, int STEPS, int PRO, int EPI, typename OUT>
 __global__ void __launch_bounds__(64 * WV)
 gemm_skinny_rows_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OUT* __restrict__ y,
                         const float* __restrict__ gain, float eps, const int* __restrict__ rows, int n, int N_out,
-                        int K) {
+                        int K, int act) {
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
     constexpr int NKS = WV / MT;                                // stretches of K
     extern __shared__ float sk_lds[];
@@ -542,7 +542,7 @@ gemm_skinny_rows_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ 
             }
             if (out_row < n && col < N_out) {
                 float r = v[0];
-                if (EPI == EPI_SWIGLU) r = v[0] / (1.f + __expf(-v[0])) * v[BT - 1];
+                if (EPI == EPI_SWIGLU) r = pl_activate<false>(v[0], act) * v[BT - 1];
                 const size_t at = static_cast<size_t>(out_row) * N_out + col;
                 if (EPI == EPI_ADD)
                     y[at] = from_float<OUT>(to_float(y[at]) + r);
@@ -557,7 +557,7 @@ gemm_skinny_rows_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ 
 // The rows variant's launch: WV waves, MT tiles of rows, WV / MT stretches of K of at most STEPS steps.
 template <int MT, int WV, int STEPS, int PRO, int EPI, typename OUT>
 static int launch_rows(const void* x, const void* w, void* y, const float* gain, float eps,
-                       const int* rows, int n, int N_out, int K, hipStream_t stream) {
+                       const int* rows, int n, int N_out, int K, int act, hipStream_t stream) {
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
     constexpr int NKS = WV / MT;
     const int grid = min(pl_ceil_div(N_out, SK_TILE_N), SK_MAX_GRID);
@@ -573,7 +573,7 @@ static int launch_rows(const void* x, const void* w, void* y, const float* gain,
         PL_REQUIRE(e == hipSuccess, "skinny product: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
     }
     kernel<<<grid, 64 * WV, lds_bytes, stream>>>(x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps,
-                                                rows, n, N_out, K);
+                                                rows, n, N_out, K, act);
     PL_CHECK_LAUNCH("gemm_skinny");
     return 0;
 }
@@ -581,7 +581,7 @@ static int launch_rows(const void* x, const void* w, void* y, const float* gain,
 // The panel variant: 8 waves (256 registers a lane); a wave holds 16 * MT rows of x for UNR K steps.
 template <int MT, int UNR, int PRO, int EPI, typename OUT>
 static int launch_panel(const void* x, const void* w, void* y, const float* gain, float eps,
-                        const int* rows, int n, int N_out, int K, hipStream_t stream) {
+                        const int* rows, int n, int N_out, int K, int act, hipStream_t stream) {
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
     constexpr int waves = 8;
     const int grid = min(pl_ceil_div(N_out, SK_TILE_N), SK_MAX_GRID);
@@ -595,7 +595,7 @@ static int launch_panel(const void* x, const void* w, void* y, const float* gain
         PL_REQUIRE(e == hipSuccess, "skinny product: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
     }
     kernel<<<grid, 64 * waves, lds_bytes, stream>>>(x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps,
-                                                   rows, n, N_out, K);
+                                                   rows, n, N_out, K, act);
     PL_CHECK_LAUNCH("gemm_skinny");
     return 0;
 }
@@ -615,7 +615,7 @@ struct SkShape {
 
 template <int MT, int PRO, int EPI, typename OUT>
 static int launch_unr(const void* x, const void* w, void* y, const float* gain, float eps,
-                      const int* rows, int n, int N_out, int K, hipStream_t stream) {
+                      const int* rows, int n, int N_out, int K, int act, hipStream_t stream) {
     using S = SkShape<MT, PRO, EPI>;
     if constexpr (MT == 2 || MT == 4) {
         // 16 waves: 16 / MT stretches of K, each a whole number of K steps that a wave can hold at once
@@ -624,10 +624,10 @@ static int launch_unr(const void* x, const void* w, void* y, const float* gain, 
         const size_t panel = static_cast<size_t>(BT) * 16 * K * 2 + (PRO == PRO_NORM ? static_cast<size_t>(K) * 4 : 0);
         const int need = K / SK_KSTEP / NKS;             // K steps a wave holds at once
         if (K % 512 == 0 && K / SK_KSTEP % NKS == 0 && panel <= 144 * 1024) {
-            if (need <= 8) return launch_rows<MT, 16, 8, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, stream);
+            if (need <= 8) return launch_rows<MT, 16, 8, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, stream);
             if constexpr (PRO == PRO_BF16) {             // the 32-bit stream takes twice the registers a step
                 // (24 steps would fit the registers of 16 waves only with spills: such a K goes the way below)
-                if (need <= 16) return launch_rows<MT, 16, 16, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, stream);
+                if (need <= 16) return launch_rows<MT, 16, 16, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, stream);
             }
         }
     }
@@ -635,52 +635,52 @@ static int launch_unr(const void* x, const void* w, void* y, const float* gain, 
         constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
         if (K % 512 == 0 && static_cast<size_t>(BT) * 16 * K * 2 <= 128 * 1024)
             return launch_panel<MT, (PRO == PRO_NORM ? (MT == 4 ? 1 : 2) : (MT == 4 ? 4 : 8)), PRO, EPI, OUT>(
-                x, w, y, gain, eps, rows, n, N_out, K, stream);
+                x, w, y, gain, eps, rows, n, N_out, K, act, stream);
     }
     const int steps = pl_ceil_div(K, SK_KSTEP);
     const int most = max(4 * S::U4, max(8 * S::U8, 16 * S::U16));
     const int need = min(steps, most);     // beyond that, several rounds
     if (need <= 4 * S::U4)
-        return launch_one<MT, S::U4, 4, PRO, EPI, OUT>(4, x, w, y, gain, eps, rows, n, N_out, K, stream);
+        return launch_one<MT, S::U4, 4, PRO, EPI, OUT>(4, x, w, y, gain, eps, rows, n, N_out, K, act, stream);
     if constexpr (S::U8 > 0) {
         if (need <= 8 * S::U8 || S::U16 == 0)
-            return launch_one<MT, S::U8, 8, PRO, EPI, OUT>(max(5, min(8, pl_ceil_div(steps, S::U8))), x, w, y, gain, eps, rows, n, N_out, K, stream);
+            return launch_one<MT, S::U8, 8, PRO, EPI, OUT>(max(5, min(8, pl_ceil_div(steps, S::U8))), x, w, y, gain, eps, rows, n, N_out, K, act, stream);
     }
     if constexpr (S::U16 > 0) {
-        return launch_one<MT, S::U16, 16, PRO, EPI, OUT>(max(9, min(16, pl_ceil_div(steps, S::U16))), x, w, y, gain, eps, rows, n, N_out, K, stream);
+        return launch_one<MT, S::U16, 16, PRO, EPI, OUT>(max(9, min(16, pl_ceil_div(steps, S::U16))), x, w, y, gain, eps, rows, n, N_out, K, act, stream);
     }
-    return launch_one<MT, S::U4, 4, PRO, EPI, OUT>(4, x, w, y, gain, eps, rows, n, N_out, K, stream);
+    return launch_one<MT, S::U4, 4, PRO, EPI, OUT>(4, x, w, y, gain, eps, rows, n, N_out, K, act, stream);
 }
 
 template <int PRO, int EPI, typename OUT>
 static int launch_mt(const void* x, const void* w, void* y, const float* gain, float eps,
-                     const int* rows, int n, int N_out, int K, hipStream_t stream) {
+                     const int* rows, int n, int N_out, int K, int act, hipStream_t stream) {
     // Few tiles of columns (a narrow output, as of the projections back into the stream): the tiles of 16 rows
     // go to workgroups of their own, the kernel for up to 16 rows on a grid of (column tiles, row tiles), so that
     // the launch has workgroups for every compute unit; each reads its rows of x only, and w comes from L2
     // from the second row tile on.
     if (n > 16 && pl_ceil_div(N_out, SK_TILE_N) * pl_ceil_div(n, 16) <= SK_ROW_TILES_GRID)
-        return launch_unr<1, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, stream);
+        return launch_unr<1, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, stream);
     switch (pl_ceil_div(n, 16)) {
-        case 1: return launch_unr<1, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, stream);
-        case 2: return launch_unr<2, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, stream);
-        case 3: return launch_unr<3, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, stream);
-        default: return launch_unr<4, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, stream);
+        case 1: return launch_unr<1, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, stream);
+        case 2: return launch_unr<2, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, stream);
+        case 3: return launch_unr<3, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, stream);
+        default: return launch_unr<4, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, stream);
     }
 }
 
 template <int PRO>
 static int sk_launch(int epilogue, int out_f32, const void* x, const void* w, void* y, const float* gain,
-                      float eps, const int* rows, int n, int N_out, int K, hipStream_t stream) {
+                      float eps, const int* rows, int n, int N_out, int K, int act, hipStream_t stream) {
     if (epilogue == EPI_STORE)
-        return out_f32 ? launch_mt<PRO, EPI_STORE, float>(x, w, y, gain, eps, rows, n, N_out, K, stream)
-                       : launch_mt<PRO, EPI_STORE, bf16_t>(x, w, y, gain, eps, rows, n, N_out, K, stream);
-    if (epilogue == EPI_SWIGLU) return launch_mt<PRO, EPI_SWIGLU, bf16_t>(x, w, y, gain, eps, rows, n, N_out, K, stream);
+        return out_f32 ? launch_mt<PRO, EPI_STORE, float>(x, w, y, gain, eps, rows, n, N_out, K, act, stream)
+                       : launch_mt<PRO, EPI_STORE, bf16_t>(x, w, y, gain, eps, rows, n, N_out, K, act, stream);
+    if (epilogue == EPI_SWIGLU) return launch_mt<PRO, EPI_SWIGLU, bf16_t>(x, w, y, gain, eps, rows, n, N_out, K, act, stream);
     if constexpr (PRO == PRO_NORM) {
         pl_set_error("skinny product: a product that reads the residual stream cannot add into it");
         return -1;
     } else {
-        return launch_mt<PRO, EPI_ADD, float>(x, w, y, gain, eps, rows, n, N_out, K, stream);
+        return launch_mt<PRO, EPI_ADD, float>(x, w, y, gain, eps, rows, n, N_out, K, act, stream);
     }
 }
 

@@ -49,7 +49,7 @@ __device__ __forceinline__ uint32_t gt_pack2(float lo, float hi) {
 template <int EPI>
 __global__ void __launch_bounds__(256, 2)
 gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ y_, int M, int N, int K,
-                  int row_tiles, int total) {
+                  int row_tiles, int total, int act) {
     extern __shared__ __attribute__((aligned(16))) uint16_t gt_lds[];   // [stage][x rows 0..127 | w rows 0..127][32]
 
     // Workgroups are dealt round-robin to the eight XCDs; consecutive tiles (the row tiles of one column
@@ -181,7 +181,7 @@ gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, vo
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const float g = acc[0][mb][4 * j + i];
-                    v[i] = g / (1.f + __expf(-g)) * acc[1][mb][4 * j + i];
+                    v[i] = pl_activate<false>(g, act) * acc[1][mb][4 * j + i];
                 }
                 uint2 packed;
                 packed.x = gt_pack2(v[0], v[1]);
@@ -213,7 +213,7 @@ gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, vo
 }
 
 template <int EPI>
-static int gt_launch(const void* x, const void* w, void* y, int M, int N, int K, hipStream_t stream) {
+static int gt_launch(const void* x, const void* w, void* y, int M, int N, int K, int act, hipStream_t stream) {
     constexpr int COLS = EPI == GT_SWIGLU ? GT_BN / 2 : GT_BN;
     const int row_tiles = pl_ceil_div(M, GT_BM);
     const long long total = static_cast<long long>(row_tiles) * (N / COLS);
@@ -227,7 +227,7 @@ static int gt_launch(const void* x, const void* w, void* y, int M, int N, int K,
         raised = true;
     }
     gemm_tiled_kernel<EPI><<<static_cast<int>(total), 256, lds_bytes, stream>>>(
-        static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), y, M, N, K, row_tiles, static_cast<int>(total));
+        static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), y, M, N, K, row_tiles, static_cast<int>(total), act);
     PL_CHECK_LAUNCH("gemm_tiled");
     return 0;
 }
@@ -240,11 +240,12 @@ extern "C" int pl_gemm_tiled_applies(int M, int N, int K, int epilogue) {
 }
 
 // x: bfloat16 [M, K].  w: bfloat16 [N, K], or [2 N, K] with the gate rows first for epilogue 1.
-// epilogue 0: y (bfloat16 [M, N]) = result.  1: y = silu(gate) * up.  2: y (32-bit [M, N]) += result.
-extern "C" int pl_gemm_tiled(const void* x, const void* w, void* y, int M, int N, int K, int epilogue, hipStream_t stream) {
+// epilogue 0: y (bfloat16 [M, N]) = result.  1: y = act(gate) * up (act: PL_ACT_*).  2: y (32-bit [M, N]) += result.
+extern "C" int pl_gemm_tiled(const void* x, const void* w, void* y, int M, int N, int K, int epilogue, int act, hipStream_t stream) {
+    PL_REQUIRE(act >= PL_ACT_SILU && act <= PL_ACT_GELU, "tiled product: activation code %d", act);
     PL_REQUIRE(pl_gemm_tiled_applies(M, N, K, epilogue), "tiled product: %d rows, %d columns, inner width %d, epilogue %d", M, N,
                K, epilogue);
-    if (epilogue == GT_SWIGLU) return gt_launch<GT_SWIGLU>(x, w, y, M, N, K, stream);
-    if (epilogue == GT_ADD) return gt_launch<GT_ADD>(x, w, y, M, N, K, stream);
-    return gt_launch<GT_STORE>(x, w, y, M, N, K, stream);
+    if (epilogue == GT_SWIGLU) return gt_launch<GT_SWIGLU>(x, w, y, M, N, K, act, stream);
+    if (epilogue == GT_ADD) return gt_launch<GT_ADD>(x, w, y, M, N, K, act, stream);
+    return gt_launch<GT_STORE>(x, w, y, M, N, K, act, stream);
 }

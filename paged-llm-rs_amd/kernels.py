@@ -31,14 +31,14 @@ def _signatures(lib) -> None:
         "pl_add_rmsnorm": [p, p, p, i, f, p, i, p, i, i, i, p],
         "pl_residual_add": [p, p, i, i, i, p],
         "pl_qk_norm_rope_kv_write": [p, p, p, i, f, p, p, i, p, p, p, i, i, p, p, i, i, i, i, i, i, p],
-        "pl_swiglu": [p, p, i, i, i, p],
+        "pl_swiglu": [p, p, i, i, i, i, p],
         "pl_gemm_plain": [p, p, p, i, i, i, i, i, i, i, p],
         "pl_paged_attention_plain": [p, i, p, p, p, p, i, i, p, p, i, i, i, i, f, i, i, p],
         "pl_paged_attention_prefill_tile": [i, i],
         "pl_argmax": [p, p, p, p, i, i, p],
         "pl_sample": [p, p, p, p, p, p, i, i, p],
-        "pl_gemm_skinny": [p, p, p, p, f, p, i, i, i, i, i, p],
-        "pl_gemm_tiled": [p, p, p, i, i, i, i, p],
+        "pl_gemm_skinny": [p, p, p, p, f, p, i, i, i, i, i, i, p],
+        "pl_gemm_tiled": [p, p, p, i, i, i, i, i, p],
         "pl_gemm_tiled_applies": [i, i, i, i],
         "pl_paged_attention_decode": [p, i, p, p, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, i, f, i, i,
                                       i, p, p, i, f, p, p, i, p],
@@ -181,8 +181,18 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_gain, k_gain, eps: float, cos, si
         _code(qkv, "fused q/k/v projection"), _stream()))
 
 
-def swiglu(gate_up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
-    """silu(gate) * up on rows laid out [gate | up]."""
+# The activations of a gated feed-forward's gate branch, by the names config.json gives them.
+ACTIVATIONS = {"silu": 0, "swish": 0, "gelu_pytorch_tanh": 1, "gelu_tanh": 1, "gelu_new": 1, "gelu": 2}
+
+
+def activation_code(name: str) -> int:
+    if name not in ACTIVATIONS:
+        raise TensorError(f"activation {name!r}, the kernels know {', '.join(sorted(ACTIVATIONS))}")
+    return ACTIVATIONS[name]
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor | None = None, activation: str = "silu") -> torch.Tensor:
+    """act(gate) * up on rows laid out [gate | up]; ``act`` is SiLU or a GELU."""
     n, two_i = gate_up.shape
     _need(gate_up, "fused gate/up projection")
     if two_i % 2:
@@ -191,7 +201,8 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tens
     if out is None:
         out = torch.empty((n, inter), dtype=gate_up.dtype, device=gate_up.device)
     _need(out, "feed-forward activation", (n, inter), gate_up.dtype)
-    _check(library().pl_swiglu(gate_up.data_ptr(), out.data_ptr(), n, inter, _code(gate_up, "gate/up"), _stream()))
+    _check(library().pl_swiglu(gate_up.data_ptr(), out.data_ptr(), n, inter, _code(gate_up, "gate/up"),
+                               activation_code(activation), _stream()))
     return out
 
 
@@ -584,12 +595,13 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nk
 
 def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, swiglu: bool = False,
                 norm_gain: torch.Tensor | None = None, eps: float = 0.0, rows: torch.Tensor | None = None,
-                add_into: torch.Tensor | None = None) -> torch.Tensor:
+                add_into: torch.Tensor | None = None, activation: str = "silu") -> torch.Tensor:
     """y = x . w^T for up to 64 rows on the matrix cores, the bfloat16 weights streamed once.
 
     ``x`` is bfloat16 [n, K]; or, with ``norm_gain``, the 32-bit residual stream, whose rows
     (``rows[i]`` for output row i when a row list is given) are RMS-normalised on the way in.
-    With ``swiglu`` the rows of ``w`` are [gate | up] and y = silu(x . gate^T) * (x . up^T), in bfloat16.
+    With ``swiglu`` the rows of ``w`` are [gate | up] and y = act(x . gate^T) * (x . up^T), in bfloat16
+    (``activation``: silu or a gelu).
     With ``add_into`` (the 32-bit residual stream, [n, N]) the result is added there and that
     tensor is returned."""
     K = x.shape[1]
@@ -622,7 +634,7 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
         epilogue, out_f32 = (1 if swiglu else 0), (1 if out_dtype == torch.float32 else 0)
     _check(library().pl_gemm_skinny(
         x.data_ptr(), w.data_ptr(), out.data_ptr(), _ptr(norm_gain), float(eps), _ptr(rows), n, N_out, K,
-        epilogue, out_f32, _stream()))
+        epilogue, out_f32, activation_code(activation), _stream()))
     return out
 
 
@@ -665,7 +677,8 @@ def tiled_swiglu_wins(rows: int, columns: int, width: int) -> bool:
             and gemm_tiled_applies(rows, columns, width, swiglu=True))
 
 
-def gemm_tiled(x: torch.Tensor, w: torch.Tensor, swiglu: bool = False, add_into: torch.Tensor | None = None) -> torch.Tensor:
+def gemm_tiled(x: torch.Tensor, w: torch.Tensor, swiglu: bool = False, add_into: torch.Tensor | None = None,
+               activation: str = "silu") -> torch.Tensor:
     """y = x . w^T for many rows of bfloat16 on the matrix cores, 32-bit sums, with SwiGLU (``w`` is
     [gate | up] stacked, silu(gate) * up comes back) or the sum into the 32-bit residual stream
     (``add_into``, which is returned) as the product's last stage."""
@@ -682,7 +695,8 @@ def gemm_tiled(x: torch.Tensor, w: torch.Tensor, swiglu: bool = False, add_into:
         out, epilogue = add_into, 2
     else:
         out, epilogue = torch.empty((M, N), dtype=torch.bfloat16, device=x.device), (1 if swiglu else 0)
-    _check(library().pl_gemm_tiled(x.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, epilogue, _stream()))
+    _check(library().pl_gemm_tiled(x.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, epilogue,
+                                   activation_code(activation), _stream()))
     return out
 
 

@@ -26,10 +26,10 @@ class Linear:
         return cls(torch.cat(list(weights), dim=0))
 
     def forward(self, x, out_dtype: torch.dtype | None = None, add_into: torch.Tensor | None = None,
-                swiglu: bool = False):
+                swiglu: bool = False, activation: str = "silu"):
         """The product of ``x`` (rows, or a norm still to run) with the weight.
 
-        ``swiglu``: the weight is [gate | up] stacked and silu(gate) * up comes back.
+        ``swiglu``: the weight is [gate | up] stacked and act(gate) * up comes back (``activation``: silu or a gelu).
         ``add_into``: the 32-bit residual stream; where the product kernel can add its result
         there itself it does and None comes back, otherwise the result comes back unadded."""
         if isinstance(x, PendingNorm):
@@ -39,7 +39,7 @@ class Linear:
                     and kernels.fused_norm_applies(x.num_rows, self.in_features, self.weight)
                     and self.out_features <= kernels.FUSED_NORM_MAX_COLUMNS):
                 return kernels.gemm_skinny(x.resid, self.weight, out_dtype or x.out_dtype, swiglu=swiglu,
-                                           norm_gain=x.norm.gain32, eps=x.norm.eps, rows=x.rows)
+                                           norm_gain=x.norm.gain32, eps=x.norm.eps, rows=x.rows, activation=activation)
             x = x.materialize()
         if x.dim() != 2 or x.shape[1] != self.in_features:
             raise TensorError(f"a linear of {self.in_features} inputs given {tuple(x.shape)}")
@@ -49,14 +49,14 @@ class Linear:
         if x.dtype == torch.float32:
             # the true 32-bit path: vector-unit multiply-add only
             y = kernels.gemm_plain(x, self.weight, out_dtype=torch.float32)
-            return kernels.swiglu(y) if swiglu else y
+            return kernels.swiglu(y, activation=activation) if swiglu else y
         if kernels.skinny_applies(x, self.weight):
             if add_into is not None and not swiglu:
                 kernels.gemm_skinny(x, self.weight, add_into=add_into)
                 return None
-            return kernels.gemm_skinny(x, self.weight, out_dtype, swiglu=swiglu)
+            return kernels.gemm_skinny(x, self.weight, out_dtype, swiglu=swiglu, activation=activation)
         if swiglu:
             if kernels.tiled_swiglu_wins(x.shape[0], self.out_features // 2, self.in_features):
-                return kernels.gemm_tiled(x, self.weight, swiglu=True)
-            return kernels.swiglu(kernels.linear_bf16(x, self.weight, x.dtype))
+                return kernels.gemm_tiled(x, self.weight, swiglu=True, activation=activation)
+            return kernels.swiglu(kernels.linear_bf16(x, self.weight, x.dtype), activation=activation)
         return kernels.linear_bf16(x, self.weight, out_dtype)

@@ -1,5 +1,5 @@
-"""The gated feed-forward: down(silu(gate(x)) * up(x)), the activation on the
-gate branch (reference: model/layers.rs:72-107)."""
+"""The gated feed-forward: down(act(gate(x)) * up(x)), the activation on the
+gate branch (reference: model/layers.rs:72-107, where it is SiLU; the spec names it)."""
 
 from __future__ import annotations
 
@@ -20,8 +20,9 @@ class GatedMlp:
                 ParamDecl("down_proj.weight", (hidden, i))]
 
     def __init__(self, spec, hidden: int, params: dict, dtype, device, shared: dict):
-        if spec.activation != "silu":
-            raise UnsupportedError(f"activation {spec.activation!r}, only silu is implemented")
+        if spec.activation not in kernels.ACTIVATIONS:
+            raise UnsupportedError(f"activation {spec.activation!r}, the kernels know {', '.join(sorted(kernels.ACTIVATIONS))}")
+        self.activation = spec.activation
         # one product for gate and up: the output row is [gate | up]
         self.gate_up_proj = Linear.fused([params["gate_proj.weight"], params["up_proj.weight"]])
         self.down_proj = Linear(params["down_proj.weight"])
@@ -39,12 +40,13 @@ class GatedMlp:
             inter = both.shape[1] // 2
             trace.record("gate_proj.out", both[:, :inter])
             trace.record("up_proj.out", both[:, inter:])
-            act = kernels.swiglu(both)
+            act = kernels.swiglu(both, activation=self.activation)
             trace.record("down_proj.in", act)
             out = self.down_proj.forward(act)
             trace.record("down_proj.out", out)
             return out
-        act = self.gate_up_proj.forward(x, swiglu=True)      # few rows: the activation is the product's epilogue
+        # (few rows: the activation is the product's epilogue)
+        act = self.gate_up_proj.forward(x, swiglu=True, activation=self.activation)
         return self.down_proj.forward(act, add_into=residual)
 
 

@@ -82,6 +82,41 @@ def test_feed_forward_part(dtype, rows):
     assert rel_err(part.forward(x.to(DEV)), want) < TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("activation", ["gelu_pytorch_tanh", "gelu", "silu"])
+@pytest.mark.parametrize("rows,hidden,inter", [(3, 96, 200), (70, 96, 200), (300, 128, 256), (1500, 64, 192)])
+def test_gated_feed_forward_with_other_activations(dtype, activation, rows, hidden, inter):
+    """The activation on the gate branch is the spec's: SiLU for this architecture, the two GELUs for others.  Few
+    rows take it as the last stage of the product kernel, some hundred as the tiled product's, many as a kernel of
+    its own behind the library's product."""
+    from paged_llm_rs_amd.config import GatedMlpSpec
+    from paged_llm_rs_amd.parts import FEED_FORWARDS
+
+    w = {"gate_proj.weight": randn(inter, hidden, std=0.1, seed=1).to(dtype),
+         "up_proj.weight": randn(inter, hidden, std=0.1, seed=2).to(dtype),
+         "down_proj.weight": randn(hidden, inter, std=0.1, seed=3).to(dtype)}
+    part = FEED_FORWARDS["gated_mlp"](GatedMlpSpec("gated_mlp", inter, activation), hidden,
+                                      {k: v.to(DEV) for k, v in w.items()}, dtype, DEV, {})
+    x = (randn(rows, hidden, seed=4) * 2).to(dtype)
+    d = {k: v.double() for k, v in w.items()}
+    gate, up = x.double() @ d["gate_proj.weight"].T, x.double() @ d["up_proj.weight"].T
+    act = {"silu": torch.nn.functional.silu, "gelu": torch.nn.functional.gelu,
+           "gelu_pytorch_tanh": lambda t: torch.nn.functional.gelu(t, approximate="tanh")}[activation]
+    want = (act(gate) * up) @ d["down_proj.weight"].T
+    assert rel_err(part.forward(x.to(DEV)), want) < TOL[dtype]
+
+
+def test_an_activation_nobody_knows_is_refused():
+    from paged_llm_rs_amd.config import GatedMlpSpec
+    from paged_llm_rs_amd.errors import UnsupportedError
+    from paged_llm_rs_amd.parts import FEED_FORWARDS
+
+    w = {"gate_proj.weight": torch.zeros(8, 8, device=DEV), "up_proj.weight": torch.zeros(8, 8, device=DEV),
+         "down_proj.weight": torch.zeros(8, 8, device=DEV)}
+    with pytest.raises(UnsupportedError, match="relu"):
+        FEED_FORWARDS["gated_mlp"](GatedMlpSpec("gated_mlp", 8, "relu"), 8, w, torch.float32, DEV, {})
+
+
 # --- mixer ---------------------------------------------------------------------------------------------------
 
 def one_layer_cache(mixer, block_size, pages, dtype):
