@@ -40,6 +40,8 @@ class AttentionSpec:
     position: Optional[PositionSpec] = None
     window: Optional[int] = None            # keys j with pos - window < j <= pos; None = all keys
     scale: Optional[float] = None           # None = 1/sqrt(head_dim)
+    qkv_bias: bool = False                  # q, k and v projections carry a bias each
+    out_bias: bool = False                  # the output projection carries one
 
 
 @dataclass(frozen=True)

@@ -215,6 +215,32 @@ extern "C" int pl_add_rmsnorm(float* resid, const void* delta, const void* gain,
     return 0;
 }
 
+// A projection's bias: y[r, c] += bias[c], in y's own type (the sum in 32-bit).
+template <typename T, typename B>
+__global__ void add_bias_kernel(T* __restrict__ y, const B* __restrict__ bias, int N, size_t count) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < count) y[i] = from_float<T>(to_float(y[i]) + to_float(bias[i % N]));
+}
+
+extern "C" int pl_add_bias(void* y, const void* bias, int dtype, int bias_dtype, int n, int N, hipStream_t stream) {
+    PL_REQUIRE(n >= 0 && N > 0, "add_bias: rows %d, width %d", n, N);
+    const size_t count = static_cast<size_t>(n) * N;
+    if (count == 0) return 0;
+    const int blocks = static_cast<int>((count + 255) / 256);
+    if (dtype == PL_DTYPE_F32 && bias_dtype == PL_DTYPE_F32)
+        add_bias_kernel<float, float><<<blocks, 256, 0, stream>>>(static_cast<float*>(y), static_cast<const float*>(bias), N, count);
+    else if (dtype == PL_DTYPE_BF16 && bias_dtype == PL_DTYPE_BF16)
+        add_bias_kernel<bf16_t, bf16_t><<<blocks, 256, 0, stream>>>(static_cast<bf16_t*>(y), static_cast<const bf16_t*>(bias), N, count);
+    else if (dtype == PL_DTYPE_BF16 && bias_dtype == PL_DTYPE_F32)
+        add_bias_kernel<bf16_t, float><<<blocks, 256, 0, stream>>>(static_cast<bf16_t*>(y), static_cast<const float*>(bias), N, count);
+    else if (dtype == PL_DTYPE_F32 && bias_dtype == PL_DTYPE_BF16)
+        add_bias_kernel<float, bf16_t><<<blocks, 256, 0, stream>>>(static_cast<float*>(y), static_cast<const bf16_t*>(bias), N, count);
+    else
+        PL_REQUIRE(false, "add_bias: dtype codes %d and %d", dtype, bias_dtype);
+    PL_CHECK_LAUNCH("add_bias");
+    return 0;
+}
+
 // A plain residual add for blocks whose next step is not a norm: resid += delta.
 template <typename T>
 __global__ void residual_add_kernel(float* __restrict__ resid, const T* __restrict__ delta, size_t count) {

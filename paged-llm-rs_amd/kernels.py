@@ -30,6 +30,7 @@ def _signatures(lib) -> None:
         "pl_embed": [p, p, i, p, i, i, i, p],
         "pl_add_rmsnorm": [p, p, p, i, f, p, i, p, i, i, i, p],
         "pl_residual_add": [p, p, i, i, i, p],
+        "pl_add_bias": [p, p, i, i, i, i, p],
         "pl_qk_norm_rope_kv_write": [p, p, p, i, f, p, p, i, p, p, p, i, i, p, p, i, i, i, i, i, i, p],
         "pl_swiglu": [p, p, i, i, i, i, p],
         "pl_gemm_plain": [p, p, p, i, i, i, i, i, i, i, p],
@@ -141,6 +142,16 @@ def residual_add(resid: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
     _need(delta, "residual delta", (n, H))
     _check(library().pl_residual_add(resid.data_ptr(), delta.data_ptr(), _code(delta, "residual delta"), n, H, _stream()))
     return resid
+
+
+def add_bias(y: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """y[r, c] += bias[c], in place."""
+    n, N = y.shape
+    _need(y, "projection output")
+    _need(bias, "bias", (N,))
+    _check(library().pl_add_bias(y.data_ptr(), bias.data_ptr(), _code(y, "projection output"), _code(bias, "bias"),
+                                 n, N, _stream()))
+    return y
 
 
 def qk_norm_rope_kv_write(qkv: torch.Tensor, q_gain, k_gain, eps: float, cos, sin, rot: int,

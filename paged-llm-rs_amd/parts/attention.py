@@ -33,6 +33,11 @@ class PagedAttention:
         if spec.qk_norm is not None:
             decls += [ParamDecl("q_norm.weight", (spec.head_dim,), "gain"),
                       ParamDecl("k_norm.weight", (spec.head_dim,), "gain")]
+        if spec.qkv_bias:
+            decls += [ParamDecl("q_proj.bias", (q,), "bias"), ParamDecl("k_proj.bias", (kv,), "bias"),
+                      ParamDecl("v_proj.bias", (kv,), "bias")]
+        if spec.out_bias:
+            decls.append(ParamDecl("o_proj.bias", (hidden,), "bias"))
         return decls
 
     def __init__(self, spec, hidden: int, params: dict, dtype, device, shared: dict):
@@ -51,8 +56,9 @@ class PagedAttention:
         self.scale = spec.scale if spec.scale is not None else 1.0 / math.sqrt(spec.head_dim)
         self.window = int(spec.window or 0)
         # one product for q, k and v: the output row is [q | k | v]
-        self.qkv_proj = Linear.fused([params["q_proj.weight"], params["k_proj.weight"], params["v_proj.weight"]])
-        self.o_proj = Linear(params["o_proj.weight"])
+        self.qkv_proj = Linear.fused([params["q_proj.weight"], params["k_proj.weight"], params["v_proj.weight"]],
+                                     [params.get("q_proj.bias"), params.get("k_proj.bias"), params.get("v_proj.bias")])
+        self.o_proj = Linear(params["o_proj.weight"], params.get("o_proj.bias"))
         self.q_gain = params.get("q_norm.weight")
         self.k_gain = params.get("k_norm.weight")
         self.eps = float(spec.qk_norm.eps) if spec.qk_norm is not None else 0.0

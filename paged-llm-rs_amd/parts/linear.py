@@ -1,6 +1,7 @@
-"""y = x . W^T, no bias; W is kept as stored, [out, in] (reference:
-model/layers.rs:9-36, which transposes at load; here both operands are read
-along their contiguous axis instead)."""
+"""y = x . W^T (+ b); W is kept as stored, [out, in] (reference:
+model/layers.rs:9-36, which transposes at load and has no bias; here both
+operands are read along their contiguous axis instead, and a bias is a vector
+added behind the product)."""
 
 from __future__ import annotations
 
@@ -12,18 +13,22 @@ from .norm import PendingNorm
 
 
 class Linear:
-    def __init__(self, weight: torch.Tensor):
+    def __init__(self, weight: torch.Tensor, bias: torch.Tensor | None = None):
         if weight.dim() != 2:
             raise TensorError(f"a linear weight of shape {tuple(weight.shape)}")
         self.weight = weight.contiguous()
         self.out_features, self.in_features = weight.shape
+        if bias is not None and tuple(bias.shape) != (self.out_features,):
+            raise TensorError(f"a bias of shape {tuple(bias.shape)} for {self.out_features} outputs")
+        self.bias = None if bias is None else bias.contiguous()
 
     @classmethod
-    def fused(cls, weights) -> "Linear":
+    def fused(cls, weights, biases=None) -> "Linear":
         """One product for several projections of the same input: the weights
-        are stacked along the output axis, so the output row is their
-        concatenation."""
-        return cls(torch.cat(list(weights), dim=0))
+        (and the biases, if they have any) are stacked along the output axis,
+        so the output row is their concatenation."""
+        biases = [b for b in (biases or []) if b is not None]
+        return cls(torch.cat(list(weights), dim=0), torch.cat(biases, dim=0) if biases else None)
 
     def forward(self, x, out_dtype: torch.dtype | None = None, add_into: torch.Tensor | None = None,
                 swiglu: bool = False, activation: str = "silu"):
@@ -32,6 +37,18 @@ class Linear:
         ``swiglu``: the weight is [gate | up] stacked and act(gate) * up comes back (``activation``: silu or a gelu).
         ``add_into``: the 32-bit residual stream; where the product kernel can add its result
         there itself it does and None comes back, otherwise the result comes back unadded."""
+        if self.bias is not None:
+            # The bias is added behind the product by a kernel of its own; what the product would have fused
+            # behind itself (the activation, the sum into the stream) then runs unfused as well.
+            if isinstance(x, PendingNorm):
+                x = x.materialize()
+            y = self._product(x, out_dtype if not swiglu else None)
+            kernels.add_bias(y, self.bias)
+            return kernels.swiglu(y, activation=activation) if swiglu else y
+        return self._product(x, out_dtype, add_into, swiglu, activation)
+
+    def _product(self, x, out_dtype: torch.dtype | None = None, add_into: torch.Tensor | None = None,
+                 swiglu: bool = False, activation: str = "silu"):
         if isinstance(x, PendingNorm):
             if x.width != self.in_features:
                 raise TensorError(f"a linear of {self.in_features} inputs given a stream of width {x.width}")

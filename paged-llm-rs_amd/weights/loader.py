@@ -26,8 +26,8 @@ from .safetensors_io import SafetensorsFile
 
 @dataclass(frozen=True)
 class ParamDecl:
-    """One tensor a part needs.  ``role`` is ``matrix``, ``embedding`` or
-    ``gain``; it picks the random initialisation and nothing else."""
+    """One tensor a part needs.  ``role`` is ``matrix``, ``embedding``, ``gain`` or
+    ``bias``; it picks the random initialisation and nothing else."""
     name: str
     shape: tuple
     role: str = "matrix"

@@ -162,6 +162,50 @@ def test_attention_part_in_portions(dtype, nq, nkv, d, block_size):
     assert rel_err(torch.cat(got), want) < TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_part_with_biases(dtype):
+    """Projections with a bias each (another family's attention): the plain attention on the input with a column
+    of ones appended and the biases as one more column of the weights gives the same q, k and v; the output
+    projection's bias is added to its result.  Decoded tokens and portions, so that the fused and the unfused
+    ways of a step are both taken."""
+    from paged_llm_rs_amd.config import AttentionSpec, NormSpec, PositionSpec
+    from paged_llm_rs_amd.engine.batch import StepEntry, build_batch
+    from paged_llm_rs_amd.parts import MIXERS, LayerContext
+
+    nq, nkv, d, block_size = 4, 2, 32, 8
+    hidden, eps, theta, n = 40, 1e-5, 5e5, 45
+    cfg = {"num_attention_heads": nq, "num_key_value_heads": nkv, "head_dim": d, "rms_norm_eps": eps, "rope_theta": theta}
+    w = {"q_proj.weight": randn(nq * d, hidden, std=0.2, seed=1), "k_proj.weight": randn(nkv * d, hidden, std=0.2, seed=2),
+         "v_proj.weight": randn(nkv * d, hidden, std=0.2, seed=3), "o_proj.weight": randn(hidden, nq * d, std=0.2, seed=4),
+         "q_norm.weight": 1 + randn(d, std=0.2, seed=5), "k_norm.weight": 1 + randn(d, std=0.2, seed=6),
+         "q_proj.bias": randn(nq * d, std=0.5, seed=7), "k_proj.bias": randn(nkv * d, std=0.5, seed=8),
+         "v_proj.bias": randn(nkv * d, std=0.5, seed=9), "o_proj.bias": randn(hidden, std=0.5, seed=10)}
+    w = {k: v.to(dtype) for k, v in w.items()}
+    spec = AttentionSpec("paged_attention", nq, nkv, d, NormSpec("rms_norm", eps), PositionSpec("rotary_half", d, theta, 128),
+                         None, None, qkv_bias=True, out_bias=True)
+    cls = MIXERS["paged_attention"]
+    assert {decl.name for decl in cls.declare(spec, hidden)} == set(w)
+    mixer = cls(spec, hidden, {k: v.to(DEV) for k, v in w.items()}, dtype, DEV, {})
+    cache = one_layer_cache(mixer, block_size, 24, dtype)
+    x = randn(n, hidden, seed=11).to(dtype)
+    ones = torch.ones(n, 1, dtype=torch.float64)
+    wide = {f"a.{p}_proj.weight": torch.cat([w[f"{p}_proj.weight"].double(), w[f"{p}_proj.bias"].double()[:, None]], dim=1)
+            for p in "qkv"}
+    wide.update({"a.o_proj.weight": w["o_proj.weight"].double(), "a.q_norm.weight": w["q_norm.weight"].double(),
+                 "a.k_norm.weight": w["k_norm.weight"].double()})
+    want = plain.attention(torch.cat([x.double(), ones], dim=1), wide, "a", cfg, torch.arange(n)) + w["o_proj.bias"].double()
+    cache.manager.add_sequence(1)
+    got, at = [], 0
+    for count in (20, 1, 1, 17, 1, 3, 2):
+        assert cache.manager.reserve(1, count)
+        batch = build_batch([StepEntry(1, [0] * count, at, [])], cache.manager, 1, 10, 128, DEV)
+        got.append(mixer.forward(x[at:at + count].to(DEV).contiguous(), LayerContext(batch, cache, 0, 0, True)))
+        cache.manager.advance(1, count)
+        at += count
+    assert at == n
+    assert rel_err(torch.cat(got), want) < TOL[dtype]
+
+
 # --- block ---------------------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
