@@ -271,8 +271,8 @@ extern "C" int pl_residual_add(float* resid, const void* delta, int dtype, int n
 //   slot(t) = block_table[seq_of[t], pos / bs] * bs + pos % bs
 //
 // A token with a negative position is padding and is skipped.  The rotation
-// pairs element i with i + rot/2 (the two halves of the head) and uses 32-bit
-// cos/sin tables of [max_pos, rot/2].
+// pairs element i with i + rot/2 (the two halves of the head) or, told so,
+// element 2 i with 2 i + 1, and uses 32-bit cos/sin tables of [max_pos, rot/2].
 // ---------------------------------------------------------------------------
 #define PL_MAX_HEAD_DIM 256
 
@@ -282,7 +282,7 @@ __global__ void qk_norm_rope_kv_write_kernel(
     int gain_dtype, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, int rot, const int* __restrict__ positions,
     const int* __restrict__ seq_of, const int* __restrict__ block_table, int max_blocks,
-    int block_size, T* __restrict__ k_pool, T* __restrict__ v_pool, int nq, int nkv, int d) {
+    int block_size, T* __restrict__ k_pool, T* __restrict__ v_pool, int nq, int nkv, int d, int neighbours) {
     __shared__ float head[PL_MAX_HEAD_DIM];
     const int t = blockIdx.x;
     const int h = blockIdx.y;
@@ -328,9 +328,11 @@ __global__ void qk_norm_rope_kv_write_kernel(
         const float* c = cos_table + static_cast<size_t>(pos) * half;
         const float* s = sin_table + static_cast<size_t>(pos) * half;
         for (int i = lane; i < half; i += PL_WAVE) {
-            const float x1 = head[i], x2 = head[i + half];
-            dst[i] = from_float<T>(x1 * c[i] - x2 * s[i]);
-            dst[i + half] = from_float<T>(x2 * c[i] + x1 * s[i]);
+            // the pair that angle i turns: the two halves' elements i, or the neighbours 2 i and 2 i + 1
+            const int a = neighbours ? 2 * i : i, b = neighbours ? 2 * i + 1 : i + half;
+            const float x1 = head[a], x2 = head[b];
+            dst[a] = from_float<T>(x1 * c[i] - x2 * s[i]);
+            dst[b] = from_float<T>(x2 * c[i] + x1 * s[i]);
         }
         for (int i = rot + lane; i < d; i += PL_WAVE) dst[i] = from_float<T>(head[i]);
     } else {
@@ -571,7 +573,7 @@ extern "C" int pl_qk_norm_rope_kv_write(
     void* qkv, const void* q_gain, const void* k_gain, int gain_dtype, float eps,
     const float* cos_table, const float* sin_table, int rot, const int* positions,
     const int* seq_of, const int* block_table, int max_blocks, int block_size, void* k_pool,
-    void* v_pool, int n, int nq, int nkv, int d, int write_kv, int dtype, hipStream_t stream) {
+    void* v_pool, int n, int nq, int nkv, int d, int write_kv, int dtype, int neighbours, hipStream_t stream) {
     // (any head size: the kernels that work on eight elements a lane take multiples of 16, one wave a head takes the rest)
     PL_REQUIRE(d > 0 && d <= PL_MAX_HEAD_DIM, "qk_norm_rope: head size %d, which has to be between 1 and %d", d, PL_MAX_HEAD_DIM);
     PL_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0, "qk_norm_rope: rotated width %d of a head of %d", rot, d);
@@ -581,7 +583,11 @@ extern "C" int pl_qk_norm_rope_kv_write(
     if (n <= 0) return 0;
     // Without the cache write (a layer that reads another layer's pages) only the query heads run.
     const int heads = write_kv ? nq + 2 * nkv : nq;
-    if (d == 128 && (rot == 128 || !cos_table)) {
+    // (neighbours: the rotation pairs elements 2 i and 2 i + 1 instead of i and i + rot/2; the kernel of one wave a
+    // head takes that, the others are written for the halves)
+    if (neighbours && cos_table) {
+        // falls through to the last kernel
+    } else if (d == 128 && (rot == 128 || !cos_table)) {
         dim3 rows(n, pl_ceil_div(heads, 16));
         if (dtype == PL_DTYPE_F32)
             qk_norm_rope_kv_write_128_kernel<float><<<rows, 256, 0, stream>>>(
@@ -596,7 +602,7 @@ extern "C" int pl_qk_norm_rope_kv_write(
         PL_CHECK_LAUNCH("qk_norm_rope_kv_write");
         return 0;
     }
-    if (rot % 16 == 0 && d % 16 == 0) {
+    if (rot % 16 == 0 && d % 16 == 0 && !(neighbours && cos_table)) {
         // a workgroup takes two groups of 4 * (64 / (d/8)) heads of a token at a time
         const int per_group = 4 * (PL_WAVE / (d / 8));
         dim3 wide(n, pl_ceil_div(heads, 2 * per_group));
@@ -617,11 +623,11 @@ extern "C" int pl_qk_norm_rope_kv_write(
     if (dtype == PL_DTYPE_F32)
         qk_norm_rope_kv_write_kernel<float><<<grid, PL_WAVE, 0, stream>>>(
             static_cast<float*>(qkv), q_gain, k_gain, gain_dtype, eps, cos_table, sin_table, rot, positions, seq_of,
-            block_table, max_blocks, block_size, static_cast<float*>(k_pool), static_cast<float*>(v_pool), nq, nkv, d);
+            block_table, max_blocks, block_size, static_cast<float*>(k_pool), static_cast<float*>(v_pool), nq, nkv, d, neighbours);
     else if (dtype == PL_DTYPE_BF16)
         qk_norm_rope_kv_write_kernel<bf16_t><<<grid, PL_WAVE, 0, stream>>>(
             static_cast<bf16_t*>(qkv), q_gain, k_gain, gain_dtype, eps, cos_table, sin_table, rot, positions, seq_of,
-            block_table, max_blocks, block_size, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), nq, nkv, d);
+            block_table, max_blocks, block_size, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), nq, nkv, d, neighbours);
     else
         PL_REQUIRE(false, "qk_norm_rope: dtype code %d", dtype);
     PL_CHECK_LAUNCH("qk_norm_rope_kv_write");

@@ -31,7 +31,7 @@ def _signatures(lib) -> None:
         "pl_add_rmsnorm": [p, p, p, i, f, p, i, p, i, i, i, p],
         "pl_residual_add": [p, p, i, i, i, p],
         "pl_add_bias": [p, p, i, i, i, i, p],
-        "pl_qk_norm_rope_kv_write": [p, p, p, i, f, p, p, i, p, p, p, i, i, p, p, i, i, i, i, i, i, p],
+        "pl_qk_norm_rope_kv_write": [p, p, p, i, f, p, p, i, p, p, p, i, i, p, p, i, i, i, i, i, i, i, p],
         "pl_swiglu": [p, p, i, i, i, i, p],
         "pl_gemm_plain": [p, p, p, i, i, i, i, i, i, i, p],
         "pl_paged_attention_plain": [p, i, p, p, p, p, i, i, p, p, i, i, i, i, f, i, i, p],
@@ -157,9 +157,10 @@ def add_bias(y: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
 def qk_norm_rope_kv_write(qkv: torch.Tensor, q_gain, k_gain, eps: float, cos, sin, rot: int,
                           positions: torch.Tensor, seq_of: torch.Tensor, block_table: torch.Tensor,
                           block_size: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
-                          nq: int, nkv: int, d: int, write_kv: bool = True) -> None:
+                          nq: int, nkv: int, d: int, write_kv: bool = True, neighbours: bool = False) -> None:
     """Per-head norm of q and k, rotation of q and k at each token's position, and
-    the write of k and v into their pages.  q is rewritten in place inside ``qkv``."""
+    the write of k and v into their pages.  q is rewritten in place inside ``qkv``.
+    The rotation turns the pairs (i, i + rot/2), or with ``neighbours`` the pairs (2 i, 2 i + 1)."""
     n = qkv.shape[0]
     _need(qkv, "fused q/k/v projection", (n, (nq + 2 * nkv) * d))
     _need(positions, "positions", (n,), torch.int32)
@@ -189,7 +190,7 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, q_gain, k_gain, eps: float, cos, si
         qkv.data_ptr(), _ptr(q_gain), _ptr(k_gain), gain_code, float(eps), _ptr(cos), _ptr(sin), rot,
         positions.data_ptr(), seq_of.data_ptr(), block_table.data_ptr(), block_table.shape[1], block_size,
         k_pool.data_ptr(), v_pool.data_ptr(), n, nq, nkv, d, 1 if write_kv else 0,
-        _code(qkv, "fused q/k/v projection"), _stream()))
+        _code(qkv, "fused q/k/v projection"), 1 if neighbours else 0, _stream()))
 
 
 # The activations of a gated feed-forward's gate branch, by the names config.json gives them.
@@ -390,11 +391,12 @@ class QkFusion:
     """What turns a raw projection row into queries and keys: the per-head norm's gains and eps, the
     rotation's tables and width, and whether key and value go into the pages."""
 
-    __slots__ = ("q_gain", "k_gain", "eps", "cos", "sin", "rot", "write_kv")
+    __slots__ = ("q_gain", "k_gain", "eps", "cos", "sin", "rot", "write_kv", "neighbours")
 
-    def __init__(self, q_gain, k_gain, eps: float, cos, sin, rot: int, write_kv: bool):
+    def __init__(self, q_gain, k_gain, eps: float, cos, sin, rot: int, write_kv: bool, neighbours: bool = False):
         self.q_gain, self.k_gain, self.eps, self.cos, self.sin = q_gain, k_gain, eps, cos, sin
         self.rot, self.write_kv = rot, write_kv
+        self.neighbours = neighbours        # the rotation pairs (2 i, 2 i + 1) instead of (i, i + rot/2)
 
 
 def paged_attention_prefill(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, q_start: torch.Tensor,
@@ -552,14 +554,14 @@ def attention_step(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nkv
     which every request brings one token (in bfloat16) does all of it in the attention kernel;
     any other step runs the stand-alone kernel for the first three and then attention."""
     if (qkv.dtype == torch.bfloat16 and _attention_mode == "kernel" and batch.max_q_len == 1
-            and prepare.rot % 16 == 0 and not grouped_applies(nq, nkv, d, kv.block_size)):
+            and prepare.rot % 16 == 0 and not prepare.neighbours and not grouped_applies(nq, nkv, d, kv.block_size)):
         splits = decode_splits(batch.num_tokens, nq, nkv, batch.max_ctx_len)
         return paged_attention_decode(qkv, qkv.shape[1], out, batch.positions, batch.seq_of, kv.block_table,
                                       kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window, splits,
                                       fuse=prepare)
     qk_norm_rope_kv_write(qkv, prepare.q_gain, prepare.k_gain, prepare.eps, prepare.cos, prepare.sin, prepare.rot,
                           batch.positions, batch.seq_of, kv.block_table, kv.block_size, kv.k_pool, kv.v_pool,
-                          nq, nkv, d, write_kv=prepare.write_kv)
+                          nq, nkv, d, write_kv=prepare.write_kv, neighbours=prepare.neighbours)
     return paged_attention(qkv, out, batch, kv, nq, nkv, d, scale, window)
 
 

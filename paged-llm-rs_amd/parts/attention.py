@@ -86,7 +86,8 @@ class PagedAttention:
         cos = self.rotary.cos if self.rotary is not None else None
         sin = self.rotary.sin if self.rotary is not None else None
         rot = self.rotary.dim if self.rotary is not None else 0
-        prepare = kernels.QkFusion(self.q_gain, self.k_gain, self.eps, cos, sin, rot, ctx.writes_cache)
+        prepare = kernels.QkFusion(self.q_gain, self.k_gain, self.eps, cos, sin, rot, ctx.writes_cache,
+                                   neighbours=bool(getattr(self.rotary, "neighbours", False)))
         out = torch.empty((qkv.shape[0], self.nq * self.d), dtype=qkv.dtype, device=qkv.device)
         if ctx.trace is not None:
             self._record_projections(qkv, batch, kv, ctx.trace)

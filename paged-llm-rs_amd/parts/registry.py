@@ -17,8 +17,8 @@ norm          ``declare(spec, width)``; ``__init__(spec, width, params, dtype, d
               ``delta`` into the 32-bit residual stream and returns the normalised rows.
 position      ``__init__(spec, device)`` giving ``dim`` (how many elements of a head are rotated),
               ``cos`` and ``sin`` ([max_positions, dim/2], 32-bit, on the device) and
-              ``max_positions``: the rotation by pairs (i, i + dim/2) that the attention kernels
-              apply is fixed, the angles are the encoding's own.
+              ``max_positions``; optionally ``neighbours = True`` when an angle turns the elements
+              2 i and 2 i + 1 rather than i and i + dim/2.  The angles are the encoding's own.
 block         ``declare(layer_spec, hidden)``; ``__init__(layer_spec, hidden, params, dtype,
               device, shared)``; ``forward(resid, delta, ctx) -> delta`` where the returned
               delta is the output not yet added to the residual stream.

@@ -14,9 +14,10 @@ from .registry import POSITIONS, lookup, register_position
 
 
 class RotaryTables:
+    # which elements of a head an angle turns: i and i + dim/2 (False), or 2 i and 2 i + 1 (True)
+    neighbours = False
+
     def __init__(self, spec, device):
-        if spec.kind != "rotary_half":
-            raise UnsupportedError(f"position encoding {spec.kind!r}, only rotary_half is implemented")
         if spec.dim % 2 or spec.dim <= 0:
             raise UnsupportedError(f"a rotation over {spec.dim} values, which do not pair")
         self.dim = spec.dim
@@ -28,7 +29,14 @@ class RotaryTables:
         self.max_positions = spec.max_positions
 
 
+class RotaryNeighbourTables(RotaryTables):
+    """The same angles, turning neighbouring elements: the layout of checkpoints that were not permuted for
+    the half-split form."""
+    neighbours = True
+
+
 register_position("rotary_half", RotaryTables)
+register_position("rotary_neighbours", RotaryNeighbourTables)
 
 
 def rotary_tables(spec, device, shared: dict):

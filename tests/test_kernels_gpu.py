@@ -151,6 +151,36 @@ def test_qk_norm_rope_kv_write(dtype, nq, nkv, d, bs, norm):
     assert torch.equal(again.reshape(n, -1, d)[:, :nq], got_q)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nq,nkv,d,rot", [(4, 2, 128, 128), (3, 1, 48, 32), (2, 2, 20, 20)])
+def test_rotation_of_neighbouring_elements(dtype, nq, nkv, d, rot):
+    """The other layout of rotary checkpoints: angle i turns the elements 2 i and 2 i + 1.  Rotating halves after
+    gathering the even elements before the odd ones is the same thing, which is how it is checked."""
+    from paged_llm_rs_amd import kernels
+
+    n, bs = 5, 4
+    qkv = torch.randn(n, (nq + 2 * nkv) * d, device=DEV).to(dtype)
+    positions = torch.tensor([0, 3, 9, 14, 15], dtype=torch.int32, device=DEV)
+    seq_of = torch.zeros(n, dtype=torch.int32, device=DEV)
+    bt = torch.arange(4, dtype=torch.int32, device=DEV).reshape(1, 4)
+    kp = torch.zeros(16, nkv * d, dtype=dtype, device=DEV)
+    vp = torch.zeros_like(kp)
+    gain = (1 + 0.2 * torch.randn(d, device=DEV)).to(dtype)
+    cos, sin = tables(16, rot, 1e4)
+    before = qkv.clone()
+    kernels.qk_norm_rope_kv_write(qkv, gain, gain, 1e-5, cos, sin, rot, positions, seq_of, bt, bs, kp, vp, nq, nkv, d,
+                                  neighbours=True)
+    x = before.double().reshape(n, nq + 2 * nkv, d)[:, :nq + nkv]
+    x = x / torch.sqrt((x * x).mean(-1, keepdim=True) + 1e-5) * gain.double()
+    order = torch.cat([torch.arange(0, rot, 2), torch.arange(1, rot, 2), torch.arange(rot, d)]).to(DEV)
+    turned = rope_ref(x[..., order], positions, 1e4, rot)
+    want = torch.empty_like(turned)
+    want[..., order] = turned
+    assert rel(qkv.reshape(n, -1, d)[:, :nq], want[:, :nq]) < tol(dtype)
+    for t in range(n):
+        assert rel(kp[int(positions[t])].reshape(nkv, d), want[t, nq:]) < tol(dtype)
+
+
 def test_rotation_of_part_of_a_head_and_refused_sizes():
     from paged_llm_rs_amd import kernels
     from paged_llm_rs_amd.errors import TensorError

@@ -206,6 +206,44 @@ def test_attention_part_with_biases(dtype):
     assert rel_err(torch.cat(got), want) < TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_part_with_the_rotation_of_neighbours(dtype):
+    """A position encoding whose angles turn neighbouring elements, chosen by its kind in the spec.  Scores do not
+    change when the elements of q and k are reordered alike, so the plain attention over weights whose q and k
+    rows are gathered even-before-odd within each head (and gains alike) is the reference."""
+    from paged_llm_rs_amd.config import AttentionSpec, NormSpec, PositionSpec
+    from paged_llm_rs_amd.engine.batch import StepEntry, build_batch
+    from paged_llm_rs_amd.parts import MIXERS, LayerContext
+
+    nq, nkv, d, block_size = 4, 2, 32, 8
+    hidden, eps, theta, n = 40, 1e-5, 1e4, 37
+    cfg = {"num_attention_heads": nq, "num_key_value_heads": nkv, "head_dim": d, "rms_norm_eps": eps, "rope_theta": theta}
+    w = {"q_proj.weight": randn(nq * d, hidden, std=0.2, seed=1), "k_proj.weight": randn(nkv * d, hidden, std=0.2, seed=2),
+         "v_proj.weight": randn(nkv * d, hidden, std=0.2, seed=3), "o_proj.weight": randn(hidden, nq * d, std=0.2, seed=4),
+         "q_norm.weight": 1 + randn(d, std=0.2, seed=5), "k_norm.weight": 1 + randn(d, std=0.2, seed=6)}
+    w = {k: v.to(dtype) for k, v in w.items()}
+    spec = AttentionSpec("paged_attention", nq, nkv, d, NormSpec("rms_norm", eps),
+                         PositionSpec("rotary_neighbours", d, theta, 128), None, None)
+    mixer = MIXERS["paged_attention"](spec, hidden, {k: v.to(DEV) for k, v in w.items()}, dtype, DEV, {})
+    cache = one_layer_cache(mixer, block_size, 16, dtype)
+    x = randn(n, hidden, seed=11).to(dtype)
+    order = torch.cat([torch.arange(0, d, 2), torch.arange(1, d, 2)])
+    gathered = {"a.q_proj.weight": w["q_proj.weight"].double().reshape(nq, d, hidden)[:, order].reshape(nq * d, hidden),
+                "a.k_proj.weight": w["k_proj.weight"].double().reshape(nkv, d, hidden)[:, order].reshape(nkv * d, hidden),
+                "a.v_proj.weight": w["v_proj.weight"].double(), "a.o_proj.weight": w["o_proj.weight"].double(),
+                "a.q_norm.weight": w["q_norm.weight"].double()[order], "a.k_norm.weight": w["k_norm.weight"].double()[order]}
+    want = plain.attention(x.double(), gathered, "a", cfg, torch.arange(n))
+    cache.manager.add_sequence(1)
+    got, at = [], 0
+    for count in (20, 1, 1, 15):
+        assert cache.manager.reserve(1, count)
+        batch = build_batch([StepEntry(1, [0] * count, at, [])], cache.manager, 1, 10, 128, DEV)
+        got.append(mixer.forward(x[at:at + count].to(DEV).contiguous(), LayerContext(batch, cache, 0, 0, True)))
+        cache.manager.advance(1, count)
+        at += count
+    assert rel_err(torch.cat(got), want) < TOL[dtype]
+
+
 # --- block ---------------------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
