@@ -41,6 +41,8 @@ def _signatures(lib) -> None:
         "pl_gemm_skinny": [p, p, p, p, f, p, i, i, i, i, i, i, p],
         "pl_gemm_tiled": [p, p, p, i, i, i, i, i, p],
         "pl_gemm_tiled_applies": [i, i, i, i],
+        "pl_gemm_stream": [p, p, p, p, i, i, i, i, i, i, i, p],
+        "pl_gemm_stream_splits": [i, i, i, i],
         "pl_paged_attention_decode": [p, i, p, p, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, i, f, i, i,
                                       i, p, p, i, f, p, p, i, p],
         "pl_paged_attention_prefill": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, i, p],
@@ -664,7 +666,7 @@ SKINNY_F32_FEW_K = 4096     # the widest stream whose projection onto a large vo
 
 
 def skinny_wins(rows: int, weight_rows: int, width: int) -> bool:
-    if not 0 < rows <= SKINNY_ROWS or width % 8:
+    if not 0 < rows <= SKINNY_ROWS or width % 8 or stream_wins(rows, weight_rows, width):
         return False
     if rows <= 16:
         return weight_rows * width * 2 <= SKINNY_WEIGHT_BYTES or width >= SKINNY_DEEP * weight_rows
@@ -713,6 +715,61 @@ def gemm_tiled(x: torch.Tensor, w: torch.Tensor, swiglu: bool = False, add_into:
     return out
 
 
+STREAM_ROWS = 64
+# Where the streamed product beats both the library and the skinny kernel (each timed over weights from
+# memory, at 8 to 64 rows).  The library cuts a deep product over few columns badly (5,120 x 25,600 at 64
+# rows: 158 us against 67 here), and from 17 rows on it slows down where this kernel does not (151,936 x
+# 4,096 at 32 rows: 272 us against 244).  A wide product of moderate depth (51,200 x 5,120) stays the
+# library's: its columns give too few workgroups for an even share a compute unit, and cutting K there
+# costs more in partial results than it gains.
+STREAM_DEEP = 1.5            # K / N from which the product counts as deep, with more than 16 rows
+STREAM_VERY_DEEP = 4.0       # the same for up to 16 rows (below it the library is the fastest of the three)
+STREAM_WEIGHT_BYTES = 48 << 20
+STREAM_MANY_COLUMNS = 131072
+
+
+def stream_wins(rows: int, weight_rows: int, width: int) -> bool:
+    if not 0 < rows <= STREAM_ROWS or width % 8 or weight_rows * width * 2 < STREAM_WEIGHT_BYTES:
+        return False
+    if rows <= 16:
+        return width >= STREAM_VERY_DEEP * weight_rows
+    return width >= STREAM_DEEP * weight_rows or weight_rows >= STREAM_MANY_COLUMNS
+
+
+def gemm_stream(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, swiglu: bool = False,
+                add_into: torch.Tensor | None = None, activation: str = "silu",
+                splits: int | None = None) -> torch.Tensor:
+    """y = x . w^T for up to 64 rows of bfloat16 over a large weight matrix: a workgroup owns 128 rows
+    of ``w`` and a stretch of K, its waves take their weights from memory straight into registers, a chunk
+    ahead, and share the rows of ``x`` through LDS.  ``swiglu``: ``w`` is [gate | up] stacked and
+    act(gate) * up comes back.  ``add_into``: the 32-bit residual stream takes the sum and is returned.
+    ``splits``: into how many stretches K is cut between workgroups (chosen here when not given); with
+    more than one, a second kernel adds the partial results in a fixed order."""
+    _need(x, "matrix product input", None, torch.bfloat16)
+    _need(w, "weight", None, torch.bfloat16)
+    if x.dim() != 2 or w.dim() != 2 or w.shape[1] != x.shape[1]:
+        raise TensorError(f"weight has shape {tuple(w.shape)} for an input of shape {tuple(x.shape)}")
+    n, K = x.shape
+    if swiglu and (w.shape[0] % 2 or add_into is not None):
+        raise TensorError("the activation needs an even number of weight rows and is not added into the stream")
+    N_out = w.shape[0] // 2 if swiglu else w.shape[0]
+    if add_into is not None:
+        _need(add_into, "residual stream", (n, N_out), torch.float32)
+        out, epilogue, out_f32 = add_into, 2, 1
+    else:
+        if out_dtype not in (torch.bfloat16, torch.float32) or (swiglu and out_dtype != torch.bfloat16):
+            raise TensorError(f"matrix product output {out_dtype}" + (" after the activation" if swiglu else ""))
+        out = torch.empty((n, N_out), dtype=out_dtype, device=x.device)
+        epilogue, out_f32 = (1 if swiglu else 0), (1 if out_dtype == torch.float32 else 0)
+    lib = library()
+    if splits is None:
+        splits = lib.pl_gemm_stream_splits(n, N_out, K, 1 if swiglu else 0)
+    workspace = torch.empty((splits * n * w.shape[0],), dtype=torch.float32, device=x.device) if splits > 1 else None
+    _check(lib.pl_gemm_stream(x.data_ptr(), w.data_ptr(), out.data_ptr(), _ptr(workspace), n, N_out, K, epilogue,
+                              out_f32, activation_code(activation), int(splits), _stream()))
+    return out
+
+
 def skinny_applies(x: torch.Tensor, w: torch.Tensor | None = None) -> bool:
     """Whether the product of ``x`` goes to the hand-written kernel: whether it can, and, given the
     weight, whether it is the faster of the two."""
@@ -748,6 +805,8 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> tor
     _need(w, "weight", None, torch.bfloat16)
     if out_dtype == torch.float32:
         # the projection onto the vocabulary: 32-bit out of the 32-bit sums, from either product
+        if stream_wins(x.shape[0], w.shape[0], x.shape[1]):
+            return gemm_stream(x, w, torch.float32)
         if skinny_applies(x) and x.shape[1] <= (SKINNY_F32_FEW_K if x.shape[0] <= 16 else SKINNY_SHALLOW_K):
             return gemm_skinny(x, w, torch.float32)
         if x.shape[1] % 8 == 0:
@@ -755,4 +814,6 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> tor
         return gemm_plain(x, w, out_dtype=torch.float32)
     if skinny_applies(x, w):
         return gemm_skinny(x, w, out_dtype)
+    if stream_wins(x.shape[0], w.shape[0], x.shape[1]):
+        return gemm_stream(x, w, out_dtype)
     return torch.mm(x, w.t())

@@ -72,6 +72,11 @@ class Linear:
                 kernels.gemm_skinny(x, self.weight, add_into=add_into)
                 return None
             return kernels.gemm_skinny(x, self.weight, out_dtype, swiglu=swiglu, activation=activation)
+        if kernels.stream_wins(x.shape[0], self.out_features, self.in_features):
+            if add_into is not None and not swiglu:
+                kernels.gemm_stream(x, self.weight, add_into=add_into)
+                return None
+            return kernels.gemm_stream(x, self.weight, out_dtype, swiglu=swiglu, activation=activation)
         if swiglu:
             if kernels.tiled_swiglu_wins(x.shape[0], self.out_features // 2, self.in_features):
                 return kernels.gemm_tiled(x, self.weight, swiglu=True, activation=activation)

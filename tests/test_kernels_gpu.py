@@ -367,6 +367,89 @@ def test_the_librarys_projection_onto_a_real_vocabulary(M, K):
     assert torch.equal(kernels.linear_bf16(eye, w, torch.float32), w[:, idx].T.float().contiguous())
 
 
+@pytest.mark.parametrize("n", [1, 8, 16, 17, 33, 48, 64])
+@pytest.mark.parametrize("N,K", [(48, 136), (130, 256), (1000, 384), (129, 4096), (514, 2056), (2048, 128), (16, 8)])
+@pytest.mark.parametrize("splits", [1, 3, 16])
+def test_gemm_stream(n, N, K, splits):
+    """The product that streams a large weight matrix, at small and odd sizes (columns that are no multiple
+    of a workgroup's 128, a K that is no multiple of a chunk's 128), whole and with K cut between workgroups,
+    with each of its last stages, against 64-bit products of the same bfloat16 numbers."""
+    from paged_llm_rs_amd import kernels
+
+    x = torch.randn(n, K, device=DEV).bfloat16()
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).bfloat16()
+    want = x.double() @ w.double().T
+    assert rel(kernels.gemm_stream(x, w, torch.float32, splits=splits), want) < 1e-5, "products of bfloat16 summed in 32-bit"
+    assert rel(kernels.gemm_stream(x, w, splits=splits), want) < 6e-3
+    stream = torch.randn(n, N, device=DEV)
+    before = stream.clone()
+    assert kernels.gemm_stream(x, w, add_into=stream, splits=splits) is stream
+    assert rel(stream.double() - before.double(), want) < 1e-5
+    if N % 2 == 0:
+        act = torch.nn.functional.silu(want[:, :N // 2]) * want[:, N // 2:]
+        got = kernels.gemm_stream(x, w, swiglu=True, splits=splits)
+        assert got.shape == (n, N // 2) and rel(got, act) < 6e-3
+        gelu = torch.nn.functional.gelu(want[:, :N // 2], approximate="tanh") * want[:, N // 2:]
+        assert rel(kernels.gemm_stream(x, w, swiglu=True, activation="gelu_tanh", splits=splits), gelu) < 6e-3
+    # one-hot rows pick single weights: a wrong operand layout cannot pass this
+    eye, idx = one_hot_rows(min(n, K), K)
+    assert torch.equal(kernels.gemm_stream(eye, w, splits=splits), w[:, idx].T.contiguous())
+    # a row's result does not depend on what else is in the batch, nor a call's on the call before: bitwise
+    alone = kernels.gemm_stream(x[:1].contiguous(), w, torch.float32, splits=splits)
+    assert torch.equal(alone, kernels.gemm_stream(x, w, torch.float32, splits=splits)[:1])
+
+
+@pytest.mark.parametrize("n,N,K", [(24, 2048, 8192), (64, 1024, 25600), (40, 151936, 1024), (8, 1024, 8192)])
+def test_gemm_stream_at_sizes_where_it_is_chosen(n, N, K):
+    """Deep products and the projection onto a large vocabulary, the shapes this kernel is there for: its own
+    choice of stretches, against the 32-bit product of the same numbers, eager and replayed from a graph."""
+    from paged_llm_rs_amd import kernels
+
+    x = torch.randn(n, K, device=DEV).bfloat16()
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).bfloat16()
+    want = x.float() @ w.float().T
+    got = kernels.gemm_stream(x, w, torch.float32)
+    assert rel(got, want) < 1e-5
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        kernels.gemm_stream(x, w, torch.float32)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = kernels.gemm_stream(x, w, torch.float32)
+    for replay in range(3):
+        x.copy_(torch.randn(n, K, device=DEV).bfloat16())
+        eager = kernels.gemm_stream(x, w, torch.float32).clone()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager), f"replay {replay} differs from the eager product"
+
+
+def test_gemm_stream_refusals_and_where_it_is_chosen():
+    from paged_llm_rs_amd import kernels
+    from paged_llm_rs_amd.errors import TensorError
+
+    with pytest.raises(TensorError, match="multiple of 8"):
+        kernels.gemm_stream(torch.zeros(2, 100, device=DEV, dtype=torch.bfloat16),
+                            torch.zeros(5, 100, device=DEV, dtype=torch.bfloat16))
+    with pytest.raises(TensorError, match="64 at most"):
+        kernels.gemm_stream(torch.zeros(65, 64, device=DEV, dtype=torch.bfloat16),
+                            torch.zeros(5, 64, device=DEV, dtype=torch.bfloat16))
+    with pytest.raises(TensorError, match="stretches"):
+        kernels.gemm_stream(torch.zeros(4, 64, device=DEV, dtype=torch.bfloat16),
+                            torch.zeros(5, 64, device=DEV, dtype=torch.bfloat16), splits=17)
+    # a deep product over a large matrix and the vocabulary from 17 rows on are this kernel's; small
+    # matrices, wide products of moderate depth and anything beyond 64 rows are not
+    assert kernels.stream_wins(64, 5120, 25600) and kernels.stream_wins(8, 5120, 25600)
+    assert kernels.stream_wins(32, 151936, 1024) and not kernels.stream_wins(16, 151936, 1024)
+    assert not kernels.stream_wins(64, 1024, 3072) and not kernels.stream_wins(64, 51200, 5120)
+    assert not kernels.stream_wins(65, 5120, 25600) and not kernels.stream_wins(8, 4096, 12288)
+    assert not kernels.skinny_wins(8, 5120, 25600), "one product, one kernel"
+
+
 @pytest.mark.parametrize("M", [1, 127, 128, 300, 2048])
 @pytest.mark.parametrize("N,K", [(128, 32), (256, 96), (1024, 1024), (384, 2080)])
 @pytest.mark.parametrize("kind", ["store", "swiglu", "add"])
