@@ -98,6 +98,7 @@ __device__ __forceinline__ uint32_t ap_pack2(float lo, float hi) {
 // before, and the four rows of 64 bytes that 32 lanes read transposed fall on every bank twice.
 __host__ __device__ constexpr int ap_vpad(int dt) { return dt % 2 == 0 ? 32 : 0; }
 __host__ __device__ constexpr int ap_value_buffers(int ks) { return ks == 2 ? 3 : 2; }
+__host__ __device__ constexpr int ap_direct_ahead(bool grouped) { return grouped ? 1 : 2; }
 
 // The direct feed's permutation of the 16-byte pieces of an unpadded row in LDS (64 banks of 4 bytes: a row
 // of 128 elements covers them all once, of 64 elements half).  Piece c of the key with row number r (mod 16)
@@ -189,9 +190,13 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     // Two tiles of keys [AP_BN][KROW], then NVB tiles of values [AP_BN][VROW].  The values of a tile
     // are read one round after its keys, and with two groups of waves half a round apart they live
     // for three rounds.
-    // (The direct feed asks for a tile two rounds before its keys are read: a buffer more of each.)
-    constexpr int NKB = DIRECT ? 3 : 2;
-    constexpr int NVB = DIRECT ? 4 : ap_value_buffers(KS);
+    // (The direct feed asks for a tile AHEAD rounds before its keys are read: AHEAD - 1 buffers more of each.
+    // Grouped, a workgroup is two waves with a round of some 2 us, far more than a trip to memory; what it
+    // lacks is company on its compute unit, and with one round ahead instead of two its tiles take 80 KB
+    // instead of 112, so that two workgroups share a compute unit.)
+    constexpr int AHEAD = ap_direct_ahead(GR);
+    constexpr int NKB = DIRECT ? AHEAD + 1 : 2;
+    constexpr int NVB = DIRECT ? AHEAD + 2 : ap_value_buffers(KS);
     constexpr int KTILE = AP_BN * KROW, VTILE = AP_BN * VROW;
     uint16_t* const Kbase = lds;
     uint16_t* const Vbase = lds + NKB * KTILE;
@@ -460,10 +465,12 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     if constexpr (DIRECT) {
         lookup(k_first);
         ask();
-        lookup(k_first + AP_BN);
-        ask();
-        lookup(k_first + 2 * AP_BN);             // for the first round's asking
-        __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): the first two tiles have landed
+        if constexpr (AHEAD == 2) {
+            lookup(k_first + AP_BN);
+            ask();
+        }
+        lookup(k_first + AHEAD * AP_BN);         // for the first round's asking
+        __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0): the first tiles have landed
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
     } else {
@@ -656,27 +663,45 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         __builtin_amdgcn_sched_barrier(0);
     };
     const bool behind_group = KS == 2 && kt0 != 0;
-    if (behind_group) {              // half a round in which the later group only moves a tile
-        look_ahead(k_first + (staged + 2) * AP_BN);
-        advance();
-        half_done();
-    }
-    // The direct feed in the multiplying half of round t: ask for tile t + 2 (pages looked up a round
-    // before), look up the pages of tile t + 3, and at the end wait until this wave's loads of tile
-    // t + 1 have landed: two rounds of flight, and after the barrier every wave's have.
-    constexpr int LOADS_A_TILE = 2 * KI;
+    // One round ahead, both groups ask for a tile in the same half (the earlier group's multiplying half, the
+    // later group's half before) and wait for it a round later, each before the barrier that ends the half
+    // before the earlier group reads it.
+    const bool ask_late = DIRECT && AHEAD == 1 && behind_group;
     auto feed_before = [&]() {
         if constexpr (DIRECT) {
             ask();
             look_ahead(k_first + asked * AP_BN);
         }
     };
+    if (behind_group) {              // half a round in which the later group only moves a tile
+        look_ahead(k_first + (staged + 2) * AP_BN);
+        advance();
+        if (ask_late) feed_before();
+        half_done();
+    }
+    // The direct feed in the multiplying half of round t: ask for tile t + AHEAD (pages looked up a round
+    // before), look up the pages of the tile after it, and wait until this wave's loads of tile t + 1 have
+    // landed, after the barrier every wave's have: two rounds ahead at the end of the multiplying half (all
+    // but the newest tile), one round ahead at the end of the round (everything), a whole round of flight.
+    constexpr int LOADS_A_TILE = 2 * KI;
     auto feed_after = [&]() {
         if constexpr (DIRECT) {
             take_pages();
             __builtin_amdgcn_sched_barrier(0);
-            // vmcnt(LOADS_A_TILE): all but the newest tile (the count's bits 4 and 5 stand at bits 14 and 15)
-            __builtin_amdgcn_s_waitcnt(0x0F70 | (LOADS_A_TILE & 15) | ((LOADS_A_TILE >> 4) << 14));
+            if constexpr (AHEAD == 2) {
+                // vmcnt(LOADS_A_TILE): all but the newest tile (the count's bits 4 and 5 stand at bits 14 and 15)
+                __builtin_amdgcn_s_waitcnt(0x0F70 | (LOADS_A_TILE & 15) | ((LOADS_A_TILE >> 4) << 14));
+            } else if (ask_late) {
+                __builtin_amdgcn_s_waitcnt(0x0F70);
+            }
+        }
+    };
+    auto feed_landed = [&]() {       // before the barrier that ends a round
+        if constexpr (DIRECT && AHEAD == 1) {
+            if (!ask_late) {
+                __builtin_amdgcn_sched_barrier(0);
+                __builtin_amdgcn_s_waitcnt(0x0F70);
+            }
         }
     };
     // First the tiles that every query of the workgroup sees whole: no masks, no wave stands idle
@@ -702,27 +727,31 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     };
     const int open_stop = min(open_end, k_end);
     for (; k0 < open_stop; next_tile()) {
-        feed_before();
+        if (!ask_late) feed_before();
         multiply(kbuf, vbuf_before, true);
         feed_after();
         half_done();
         if constexpr (!DIRECT) look_ahead(k_first + (staged + 2) * AP_BN);
+        if (ask_late) feed_before();
         soften(k0, false);
         advance();
+        feed_landed();
         half_done();
     }
     for (; k0 < k_end; next_tile()) {
         // a wave whose queries all stand before this tile, or that has no queries, has nothing to add
         const bool idle = !wave_active || k0 + 32 * kt0 > wave_last ||
                           (window > 0 && k0 + 32 * (kt0 + KT) - 1 <= wave_first - window);
-        feed_before();
+        if (!ask_late) feed_before();
         multiply(kbuf, vbuf_before, !idle);
         feed_after();
         half_done();
         if constexpr (!DIRECT) look_ahead(k_first + (staged + 2) * AP_BN);
+        if (ask_late) feed_before();
         if (!idle) soften(k0, true);
         else no_weights();
         advance();
+        feed_landed();
         half_done();
     }
     multiply(kbuf, vbuf_before, false);
@@ -870,7 +899,7 @@ static int launch_prefill(const void* q, int q_stride, void* out, const int* q_s
                           int total_rows, int short_rows, hipStream_t stream) {
     constexpr int DP = 32 * DT;
     constexpr int BM = 32 * NW;
-    const size_t tile_bytes = FEED == 2 ? (3 + 4) * static_cast<size_t>(AP_BN) * DP * 2
+    const size_t tile_bytes = FEED == 2 ? (2 * ap_direct_ahead(GR) + 3) * static_cast<size_t>(AP_BN) * DP * 2
                                         : (2 * static_cast<size_t>(AP_BN) * (DP + AP_KPAD) +
                                            ap_value_buffers(KS) * static_cast<size_t>(AP_BN) * (DP + ap_vpad(DT))) * 2;
     const size_t hand_bytes = KS == 2 ? static_cast<size_t>(NW) * (16 * DT + 2) * PL_WAVE * sizeof(float) : 0;

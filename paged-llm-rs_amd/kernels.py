@@ -466,11 +466,13 @@ def grouped_applies(nq: int, nkv: int, d: int, block_size: int) -> bool:
 
 
 def grouped_splits(tokens: int, nkv: int, max_ctx: int) -> int:
-    """Into how many shares the keys of a token are cut for the grouped kernel: a workgroup a compute
-    unit if the tokens and key heads alone do not give that many, every share two tiles of keys at least."""
+    """Into how many shares the keys of a token are cut for the grouped kernel: two workgroups a compute
+    unit (as many as its LDS holds) if the tokens and key heads alone do not give that many, every share
+    two tiles of keys at least.  (Context 4,096 over 8 key heads: 16 tokens take 65 us in four shares and
+    67 in two, 8 tokens 39 us in eight shares and 41 in four.)"""
     base = max(tokens * nkv, 1)
     key_tiles = -(-max(max_ctx, 1) // 64)
-    return max(1, min(16, key_tiles // 2, -(-compute_units() // base)))
+    return max(1, min(16, key_tiles // 2, -(-2 * compute_units() // base)))
 
 
 def paged_attention_grouped(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, q_start: torch.Tensor,
@@ -718,14 +720,17 @@ def gemm_tiled(x: torch.Tensor, w: torch.Tensor, swiglu: bool = False, add_into:
 STREAM_ROWS = 64
 # Where the streamed product beats both the library and the skinny kernel (each timed over weights from
 # memory, at 8 to 64 rows).  The library cuts a deep product over few columns badly (5,120 x 25,600 at 64
-# rows: 158 us against 67 here), and from 17 rows on it slows down where this kernel does not (151,936 x
-# 4,096 at 32 rows: 272 us against 244).  A wide product of moderate depth (51,200 x 5,120) stays the
+# rows: 158 us against 67 here), and from 17 rows on it is slower over very many columns of a narrow stream
+# (the vocabulary of 151,936 over a width of 1,024, 32-bit out, 17 to 64 rows: 74 to 84 us against 62 to
+# 77; over widths of 4,096 and 5,120 the two are within a tenth of each other, either way, and the
+# library keeps them).  A wide product of moderate depth (51,200 x 5,120) stays the
 # library's: its columns give too few workgroups for an even share a compute unit, and cutting K there
 # costs more in partial results than it gains.
 STREAM_DEEP = 1.5            # K / N from which the product counts as deep, with more than 16 rows
 STREAM_VERY_DEEP = 4.0       # the same for up to 16 rows (below it the library is the fastest of the three)
 STREAM_WEIGHT_BYTES = 48 << 20
 STREAM_MANY_COLUMNS = 131072
+STREAM_NARROW_WIDTH = 2048
 
 
 def stream_wins(rows: int, weight_rows: int, width: int) -> bool:
@@ -733,7 +738,7 @@ def stream_wins(rows: int, weight_rows: int, width: int) -> bool:
         return False
     if rows <= 16:
         return width >= STREAM_VERY_DEEP * weight_rows
-    return width >= STREAM_DEEP * weight_rows or weight_rows >= STREAM_MANY_COLUMNS
+    return width >= STREAM_DEEP * weight_rows or (weight_rows >= STREAM_MANY_COLUMNS and width <= STREAM_NARROW_WIDTH)
 
 
 def gemm_stream(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, swiglu: bool = False,

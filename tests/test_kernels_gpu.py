@@ -446,6 +446,7 @@ def test_gemm_stream_refusals_and_where_it_is_chosen():
     assert kernels.stream_wins(64, 5120, 25600) and kernels.stream_wins(8, 5120, 25600)
     assert kernels.stream_wins(32, 151936, 1024) and not kernels.stream_wins(16, 151936, 1024)
     assert not kernels.stream_wins(64, 1024, 3072) and not kernels.stream_wins(64, 51200, 5120)
+    assert not kernels.stream_wins(64, 151936, 5120)
     assert not kernels.stream_wins(65, 5120, 25600) and not kernels.stream_wins(8, 4096, 12288)
     assert not kernels.skinny_wins(8, 5120, 25600), "one product, one kernel"
 
