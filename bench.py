@@ -19,6 +19,7 @@ from __future__ import annotations
 
 import argparse
 import json
+import math
 import os
 import random
 import sys
@@ -250,6 +251,55 @@ class Workbench:
         }
 
 
+def products_table(torch) -> int:
+    """Microseconds of y = x . w^T over large weight matrices that come from memory (several copies of each
+    matrix in turn, inside one captured graph), by the library, the skinny and the streamed product, and
+    which of them `Linear` takes.  One JSON line."""
+    from paged_llm_rs_amd import kernels
+    from paged_llm_rs_amd.engine.step import require_gpu
+
+    device = require_gpu("cuda:0")
+
+    def microseconds(calls):
+        for call in calls[:2]:
+            call()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for call in calls:
+                call()
+        graph.replay()
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        graph.replay()
+        graph.replay()
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) / len(calls) / 2 * 1e3
+
+    shapes = [("32b_qkv", 10240, 5120), ("32b_o", 5120, 8192), ("32b_gate_up", 51200, 5120), ("32b_down", 5120, 25600),
+              ("8b_qkv", 6144, 4096), ("8b_o", 4096, 4096), ("8b_gate_up", 24576, 4096), ("8b_down", 4096, 12288)]
+    table = {}
+    for name, columns, width in shapes:
+        copies = max(2, min(24, int(1.5e9 // (columns * width * 2))))
+        weights = [(torch.randn(columns, width, device=device) / math.sqrt(width)).bfloat16() for _ in range(copies)]
+        for rows in (8, 16, 32, 64):
+            x = torch.randn(rows, width, device=device).bfloat16()
+            entry = {"MB": round(columns * width * 2 / 1e6),
+                     "library_us": round(microseconds([lambda w=w: torch.mm(x, w.t()) for w in weights]), 1),
+                     "stream_us": round(microseconds([lambda w=w: kernels.gemm_stream(x, w) for w in weights]), 1),
+                     "skinny_us": round(microseconds([lambda w=w: kernels.gemm_skinny(x, w) for w in weights]), 1),
+                     "taken": "stream" if kernels.stream_wins(rows, columns, width) else
+                              ("skinny" if kernels.skinny_wins(rows, columns, width) else "library")}
+            table[f"{name}_rows{rows}"] = entry
+            print(f"[bench] {name} {rows} rows: {entry}", file=sys.stderr, flush=True)
+        del weights
+    print(json.dumps({"metric": "products of few rows over large weights, microseconds", "unit": "us", "dtype": "bf16",
+                      "data": "synthetic: random weights from memory", "products": table}))
+    return 0
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -266,19 +316,24 @@ def main() -> int:
                         help="leave out the points of the 8b shape (a mixed step) and the 32b shape (decode at batch 64)")
     parser.add_argument("--prefill-eager", action="store_true",
                         help="launch the prefill step kernel by kernel every time (a prompt length seen once)")
-    parser.add_argument("--only", choices=["decode", "prefill", "engine", "mixed", "serving"], default=None,
+    parser.add_argument("--only", choices=["decode", "prefill", "engine", "mixed", "serving", "products"], default=None,
                         help="run one part alone: the decode steps at --batch, the prefill, or (not part of the "
                              "default line) the whole engine on 1/4/16/32/64 requests at once, 16 prompt tokens and "
                              "128 generated each, as the reference's own table of clients does; mixed: one step of a "
                              "512-token slice of a prompt beside 63 decoded tokens; serving: the reference's two other "
                              "tables, first tokens behind a shared preamble with the prefix cache off and on, and the "
-                             "gaps between the tokens of four running requests when a long prompt arrives, by --chunk")
+                             "gaps between the tokens of four running requests when a long prompt arrives, by --chunk; "
+                             "products: the layer products of the 8B and 32B shapes at 8 to 64 rows, weights from memory, "
+                             "by the library and by the two hand-written products of few rows")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU; this engine has no multi-GPU path (N must be 1)")
         return 2
 
     import torch
+
+    if args.only == "products":
+        return products_table(torch)
 
     from paged_llm_rs_amd.engine.batch import StepEntry
     from paged_llm_rs_amd.engine.step import commit_step, require_gpu, run_step

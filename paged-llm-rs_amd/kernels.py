@@ -663,7 +663,8 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
 SKINNY_WEIGHT_BYTES = 48 << 20
 SKINNY_DEEP = 4
 SKINNY_SHALLOW_K = 2048
-SKINNY_ROW_TILES_GRID = 512  # column tiles times row tiles up to which the rows are dealt to workgroups too
+SKINNY_ROW_TILES_GRID = 512  # column tiles times row tiles up to which the rows are dealt to workgroups too ...
+SKINNY_ROW_TILES_BYTES = 16 << 20   # ... for weights up to this size (4,096 x 4,096 at 32 rows: 19.8 us against the library's 14.0)
 SKINNY_F32_FEW_K = 4096     # the widest stream whose projection onto a large vocabulary it wins, up to 16 rows
 
 
@@ -673,7 +674,8 @@ def skinny_wins(rows: int, weight_rows: int, width: int) -> bool:
     if rows <= 16:
         return weight_rows * width * 2 <= SKINNY_WEIGHT_BYTES or width >= SKINNY_DEEP * weight_rows
     # ... or a narrow output, whose tiles of 16 rows go to workgroups of their own (the kernel for up to 16 rows)
-    return width <= SKINNY_SHALLOW_K or (weight_rows // 16) * -(-rows // 16) <= SKINNY_ROW_TILES_GRID
+    return width <= SKINNY_SHALLOW_K or ((weight_rows // 16) * -(-rows // 16) <= SKINNY_ROW_TILES_GRID
+                                         and weight_rows * width * 2 <= SKINNY_ROW_TILES_BYTES)
 
 
 def gemm_tiled_applies(rows: int, columns: int, width: int, swiglu: bool = False, add: bool = False) -> bool:
