@@ -82,6 +82,38 @@ def test_feed_forward_part(dtype, rows):
     assert rel_err(part.forward(x.to(DEV)), want) < TOL[dtype]
 
 
+@pytest.mark.parametrize("rows,columns,width,route", [
+    (8, 1024, 2048, "skinny"), (40, 1024, 2048, "skinny"), (300, 1024, 2048, "library"),
+    (8, 2048, 16384, "stream"), (40, 4096, 8192, "stream"), (64, 4096, 8192, "stream"), (65, 4096, 8192, "library"),
+    (40, 8192, 4096, "library")])
+def test_a_linear_by_each_of_its_products(rows, columns, width, route):
+    """Which kernel runs a projection is decided by its shape alone, in one place; whichever it is, the plain
+    product, the one that adds into the 32-bit stream and the gated one agree with 64-bit products of the same
+    bfloat16 numbers."""
+    from paged_llm_rs_amd import kernels
+    from paged_llm_rs_amd.parts.linear import Linear
+
+    took = ("stream" if kernels.stream_wins(rows, columns, width) else
+            "skinny" if kernels.skinny_wins(rows, columns, width) else "library")
+    assert took == route
+    w = (torch.randn(columns, width, device=DEV) / math.sqrt(width)).bfloat16()
+    x = torch.randn(rows, width, device=DEV).bfloat16()
+    want = x.double() @ w.double().T
+    linear = Linear(w)
+    assert rel_err(linear.forward(x), want) < TOL[torch.bfloat16]
+    stream = torch.randn(rows, columns, device=DEV)
+    before = stream.clone()
+    back = linear.forward(x, add_into=stream)
+    total = stream if back is None else before + back.float()
+    assert rel_err(total.double() - before.double(), want) < TOL[torch.bfloat16]
+    if back is None:
+        assert rel_err(stream.double() - before.double(), want) < 1e-5, "added in 32-bit, not through bfloat16"
+    gated = linear.forward(x, swiglu=True)
+    half = columns // 2
+    assert gated.shape == (rows, half)
+    assert rel_err(gated, torch.nn.functional.silu(want[:, :half]) * want[:, half:]) < TOL[torch.bfloat16]
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("activation", ["gelu_pytorch_tanh", "gelu", "silu"])
 @pytest.mark.parametrize("rows,hidden,inter", [(3, 96, 200), (70, 96, 200), (300, 128, 256), (1500, 64, 192)])
