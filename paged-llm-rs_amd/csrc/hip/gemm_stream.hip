@@ -339,3 +339,26 @@ extern "C" int pl_gemm_stream(const void* x, const void* w, void* y, float* ws, 
     if (n <= 48) return gs_launch<3, GS_WAVES>(xb, wb, y, ws, n, N_out, K, mode, act, splits, stream);
     return gs_launch<4, GS_WAVES>(xb, wb, y, ws, n, N_out, K, mode, act, splits, stream);
 }
+
+// The second kernel alone, for partial products that came from elsewhere (a deep product of some hundred
+// rows that the library ran as a batch of stretches of K): ws is 32-bit [splits, n, N_out] (for epilogue 1
+// [splits, n, 2 N_out], gate columns then up columns); the partial results are added in their order and
+// stored (epilogue 0: bfloat16 or, out_f32, 32-bit; 1: act(gate) * up, bfloat16) or added into the 32-bit
+// residual stream y (epilogue 2).  Any number of rows.
+extern "C" int pl_gemm_finish(const float* ws, void* y, long long n, int N_out, int splits, int epilogue, int out_f32,
+                              int act, hipStream_t stream) {
+    PL_REQUIRE(n > 0 && N_out > 0 && splits >= 1 && splits <= 64 && ws != nullptr && y != nullptr,
+               "sum of partial products: %lld rows, %d columns, %d parts", n, N_out, splits);
+    PL_REQUIRE(epilogue >= 0 && epilogue <= 2, "sum of partial products: epilogue %d", epilogue);
+    PL_REQUIRE(act == PL_ACT_SILU || act == PL_ACT_GELU_TANH || act == PL_ACT_GELU, "sum of partial products: activation code %d", act);
+    PL_REQUIRE(n * N_out < (1ll << 31) * 256 && n <= 0x7fffffff, "sum of partial products: %lld x %d results", n, N_out);
+    const int Nw = epilogue == 1 ? 2 * N_out : N_out;
+    const int blocks = static_cast<int>((static_cast<size_t>(n) * N_out + 255) / 256);
+    const int rows = static_cast<int>(n);
+    if (epilogue == 1) gemm_stream_finish_kernel<GS_SWIGLU><<<blocks, 256, 0, stream>>>(ws, y, rows, N_out, Nw, splits, act);
+    else if (epilogue == 2) gemm_stream_finish_kernel<GS_ADD><<<blocks, 256, 0, stream>>>(ws, y, rows, N_out, Nw, splits, act);
+    else if (out_f32) gemm_stream_finish_kernel<GS_STORE_F32><<<blocks, 256, 0, stream>>>(ws, y, rows, N_out, Nw, splits, act);
+    else gemm_stream_finish_kernel<GS_STORE_BF16><<<blocks, 256, 0, stream>>>(ws, y, rows, N_out, Nw, splits, act);
+    PL_CHECK_LAUNCH("gemm_stream_finish");
+    return 0;
+}

@@ -43,6 +43,7 @@ def _signatures(lib) -> None:
         "pl_gemm_tiled_applies": [i, i, i, i],
         "pl_gemm_stream": [p, p, p, p, i, i, i, i, i, i, i, p],
         "pl_gemm_stream_splits": [i, i, i, i],
+        "pl_gemm_finish": [p, p, ctypes.c_longlong, i, i, i, i, i, p],
         "pl_paged_attention_decode": [p, i, p, p, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, i, f, i, i,
                                       i, p, p, i, f, p, p, i, p],
         "pl_paged_attention_prefill": [p, i, p, p, p, p, i, i, i, p, i, i, p, p, i, i, i, f, i, i, p, p, i, p],
@@ -777,6 +778,58 @@ def gemm_stream(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
     return out
 
 
+# A deep product of some hundred rows the library runs as one workgroup a tile of the output, each walking
+# all of K: with few tiles (a projection back to the width of the model) most of the chip idles.  The same
+# product as a batch of stretches of K (strided views of x and w, no copies; 32-bit partial results) fills
+# it, and the kernel that ends the streamed product adds the parts in their order and stores them or adds
+# them into the stream.  Measured over weights from memory: 4,096 x 12,288 at 576 rows 102 us whole, 62 in
+# four stretches (and 6 for the sum); 5,120 x 25,600 at 576 rows 270 against 150 in two, at 1,088 rows 428
+# against 237; at 2,048 rows nothing is gained, and neither for small matrices (1,024 x 3,072), where the
+# second kernel costs what the stretches save.
+SPLIT_DEEP = 2.5             # K / N from which it pays
+SPLIT_MAX_ROWS = 1280
+SPLIT_WEIGHT_BYTES = 48 << 20
+
+
+def library_splits(rows: int, weight_rows: int, width: int) -> int:
+    """Into how many stretches of K the library's product of this shape is cut (1: not at all)."""
+    if (rows <= STREAM_ROWS or rows > SPLIT_MAX_ROWS or width < SPLIT_DEEP * weight_rows
+            or weight_rows * width * 2 < SPLIT_WEIGHT_BYTES):
+        return 1
+    for splits in ((4, 2) if rows <= 640 else (2,)):
+        if width % (8 * splits) == 0:
+            return splits
+    return 1
+
+
+def gemm_split_library(x: torch.Tensor, w: torch.Tensor, splits: int, out_dtype: torch.dtype = torch.bfloat16,
+                       add_into: torch.Tensor | None = None) -> torch.Tensor:
+    """y = x . w^T as ``splits`` products over stretches of K, run by the library as one batch, and their sum in
+    a fixed order: stored, or added into the 32-bit residual stream ``add_into`` (which is returned)."""
+    _need(x, "matrix product input", None, torch.bfloat16)
+    _need(w, "weight", None, torch.bfloat16)
+    if x.dim() != 2 or w.dim() != 2 or w.shape[1] != x.shape[1]:
+        raise TensorError(f"weight has shape {tuple(w.shape)} for an input of shape {tuple(x.shape)}")
+    M, K = x.shape
+    N = w.shape[0]
+    if splits < 2 or K % (8 * splits):
+        raise TensorError(f"a width of {K} in {splits} stretches")
+    part = K // splits
+    partial = torch.bmm(x.view(M, splits, part).transpose(0, 1), w.view(N, splits, part).permute(1, 2, 0),
+                        out_dtype=torch.float32)
+    if add_into is not None:
+        _need(add_into, "residual stream", (M, N), torch.float32)
+        out, epilogue, out_f32 = add_into, 2, 1
+    else:
+        if out_dtype not in (torch.bfloat16, torch.float32):
+            raise TensorError(f"matrix product output {out_dtype}")
+        out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+        epilogue, out_f32 = 0, (1 if out_dtype == torch.float32 else 0)
+    _check(library().pl_gemm_finish(partial.data_ptr(), out.data_ptr(), M, N, splits, epilogue, out_f32,
+                                    activation_code("silu"), _stream()))
+    return out
+
+
 def skinny_applies(x: torch.Tensor, w: torch.Tensor | None = None) -> bool:
     """Whether the product of ``x`` goes to the hand-written kernel: whether it can, and, given the
     weight, whether it is the faster of the two."""
@@ -823,4 +876,7 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> tor
         return gemm_skinny(x, w, out_dtype)
     if stream_wins(x.shape[0], w.shape[0], x.shape[1]):
         return gemm_stream(x, w, out_dtype)
+    splits = library_splits(x.shape[0], w.shape[0], x.shape[1])
+    if splits > 1:
+        return gemm_split_library(x, w, splits, out_dtype)
     return torch.mm(x, w.t())

@@ -77,6 +77,11 @@ class Linear:
                 kernels.gemm_stream(x, self.weight, add_into=add_into)
                 return None
             return kernels.gemm_stream(x, self.weight, out_dtype, swiglu=swiglu, activation=activation)
+        if add_into is not None and not swiglu:
+            splits = kernels.library_splits(x.shape[0], self.out_features, self.in_features)
+            if splits > 1:
+                kernels.gemm_split_library(x, self.weight, splits, add_into=add_into)
+                return None
         if swiglu:
             if kernels.tiled_swiglu_wins(x.shape[0], self.out_features // 2, self.in_features):
                 return kernels.gemm_tiled(x, self.weight, swiglu=True, activation=activation)

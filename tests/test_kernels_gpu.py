@@ -428,6 +428,44 @@ def test_gemm_stream_at_sizes_where_it_is_chosen(n, N, K):
         assert torch.equal(y, eager), f"replay {replay} differs from the eager product"
 
 
+@pytest.mark.parametrize("M,N,K,splits", [(70, 96, 256, 2), (576, 512, 3072, 4), (1000, 130, 1032, 3), (300, 1024, 12288, 4)])
+def test_a_deep_product_as_a_batch_of_stretches(M, N, K, splits):
+    """The library's product over stretches of K as one batch, and the sum of the 32-bit partial results by the
+    kernel that ends the streamed product: stored and added into the stream, eager and replayed from a graph."""
+    from paged_llm_rs_amd import kernels
+
+    x = torch.randn(M, K, device=DEV).bfloat16()
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).bfloat16()
+    want = x.double() @ w.double().T
+    assert rel(kernels.gemm_split_library(x, w, splits, torch.float32), want) < 1e-5
+    assert rel(kernels.gemm_split_library(x, w, splits), want) < 6e-3
+    stream = torch.randn(M, N, device=DEV)
+    before = stream.clone()
+    assert kernels.gemm_split_library(x, w, splits, add_into=stream) is stream
+    assert rel(stream.double() - before.double(), want) < 1e-5
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        kernels.gemm_split_library(x, w, splits, torch.float32)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = kernels.gemm_split_library(x, w, splits, torch.float32)
+    other = torch.randn(256, 256, device=DEV)
+    for replay in range(3):
+        x.copy_(torch.randn(M, K, device=DEV).bfloat16())
+        float((other @ other).sum())
+        eager = kernels.gemm_split_library(x, w, splits, torch.float32).clone()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager), f"replay {replay} differs from the eager product"
+    assert kernels.library_splits(576, 4096, 12288) == 4 and kernels.library_splits(1088, 5120, 25600) == 2
+    assert kernels.library_splits(2048, 4096, 12288) == 1 and kernels.library_splits(576, 1024, 3072) == 1
+    assert kernels.library_splits(64, 4096, 12288) == 1 and kernels.library_splits(576, 6144, 4096) == 1
+
+
 def test_gemm_stream_refusals_and_where_it_is_chosen():
     from paged_llm_rs_amd import kernels
     from paged_llm_rs_amd.errors import TensorError

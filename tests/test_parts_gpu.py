@@ -85,7 +85,7 @@ def test_feed_forward_part(dtype, rows):
 @pytest.mark.parametrize("rows,columns,width,route", [
     (8, 1024, 2048, "skinny"), (40, 1024, 2048, "skinny"), (300, 1024, 2048, "library"),
     (8, 2048, 16384, "stream"), (40, 4096, 8192, "stream"), (64, 4096, 8192, "stream"), (65, 4096, 8192, "library"),
-    (40, 8192, 4096, "library")])
+    (40, 8192, 4096, "library"), (300, 4096, 12288, "split"), (1100, 4096, 12288, "split"), (1500, 4096, 12288, "library")])
 def test_a_linear_by_each_of_its_products(rows, columns, width, route):
     """Which kernel runs a projection is decided by its shape alone, in one place; whichever it is, the plain
     product, the one that adds into the 32-bit stream and the gated one agree with 64-bit products of the same
@@ -94,7 +94,8 @@ def test_a_linear_by_each_of_its_products(rows, columns, width, route):
     from paged_llm_rs_amd.parts.linear import Linear
 
     took = ("stream" if kernels.stream_wins(rows, columns, width) else
-            "skinny" if kernels.skinny_wins(rows, columns, width) else "library")
+            "skinny" if kernels.skinny_wins(rows, columns, width) else
+            "split" if kernels.library_splits(rows, columns, width) > 1 else "library")
     assert took == route
     w = (torch.randn(columns, width, device=DEV) / math.sqrt(width)).bfloat16()
     x = torch.randn(rows, width, device=DEV).bfloat16()
