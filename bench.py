@@ -53,6 +53,7 @@ SHAPES = {
 }
 PREFILL_TOKENS = 2048
 BLOCK_SIZE = 16
+LONG_CONTEXT = 3968          # a point of the default line: decode from contexts near the 0.6B shape's 4,096 positions
 MIXED_SLICE = 512            # --only mixed: a slice of a prompt this long beside 63 decoded tokens
 MIXED_DECODES = 63
 # Layers of the two larger shapes in the default run's extra points (of 36 and 64).
@@ -178,11 +179,13 @@ class Workbench:
         gc.collect()
         torch.cuda.empty_cache()
 
-    def decode_point(self, batch: int, steps: int, warmup: int):
-        """(seconds a step, tokens a second, bytes a step has to read) of decode steps at ``batch``."""
-        bench = DecodeBench(self.model, self.cache, self.runner, batch, self.context, seed=batch)
+    def decode_point(self, batch: int, steps: int, warmup: int, context: int | None = None):
+        """(seconds a step, tokens a second, bytes a step has to read) of decode steps at ``batch``, from
+        contexts of ``context`` tokens (the shape's own where not given)."""
+        context = self.context if context is None else context
+        bench = DecodeBench(self.model, self.cache, self.runner, batch, context, seed=batch)
         seconds = timed(bench.step, steps, warmup)
-        context_mid = self.context + warmup + steps / 2
+        context_mid = context + warmup + steps / 2
         bench.free()
         return seconds, batch / seconds, self.weight_bytes + batch * context_mid * self.kv_token
 
@@ -477,6 +480,12 @@ def main() -> int:
             say(f"decode, batch {batch}")
             s, v, _ = decode_point(batch, max(args.steps // 2, 5), max(args.warmup // 2, 2))
             points[f"decode_b{batch}"] = round(v, 1)
+        if args.shape == "0.6b":
+            # the same batch as the headline from contexts eight times as long: the step is the attention's then
+            say(f"decode, batch {args.batch}, context {LONG_CONTEXT}")
+            s_long, v_long, bytes_long = decode_point(args.batch, 20, 5, context=LONG_CONTEXT)
+            points[f"decode_b{args.batch}_ctx{LONG_CONTEXT}"] = round(v_long, 1)
+            points[f"decode_b{args.batch}_ctx{LONG_CONTEXT}_frac_hbm"] = round(bytes_long / s_long / HBM_PEAK, 4)
         line["points"] = points
         line["prefill"] = prefill_point()
         if args.shape == "0.6b" and not args.no_other_shapes:
