@@ -72,7 +72,7 @@ gemm_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, v
     const int count = min(c_hi, K / GS_BK) - c_lo;     // whole chunks
     const bool ragged = c_hi > K / GS_BK;
 
-    // a thread's share of a chunk of x: rows p*16 + tid/16, 16 bytes at element 8 (tid%16) of the chunk
+    // a thread's share of a chunk of x: rows p*XR + tid/16, 16 bytes at element 8 (tid%16) of the chunk
     constexpr int XR = 4 * WV;                          // rows of x the workgroup's threads cover at once
     constexpr int XP = (MT * 16 + XR - 1) / XR;         // turns a thread takes
     const int xpiece = tid % 16, xr = tid / 16;
@@ -123,26 +123,25 @@ gemm_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, v
     // way into (stage, wb), and chunk i+2 is asked for as soon as wa is free.
     // (The loop can only be reached with both chunks asked for: where paths with fewer loads in flight join
     // it, the compiler places its waits for the fewest, and the queue of loads runs dry once a round.)
-    auto chunk_at = [&](int j) { return c_lo + j; };
     gs_u32x4 wa[8], wb[8], stage[XP];
     if (count >= 2) {
-        ask_x(chunk_at(0), stage);
-        ask_w(chunk_at(0), wa);
+        ask_x(c_lo, stage);
+        ask_w(c_lo, wa);
         put_x(0, stage);
-        ask_x(chunk_at(1), stage);
-        ask_w(chunk_at(1), wb);
+        ask_x(c_lo + 1, stage);
+        ask_w(c_lo + 1, wb);
         __syncthreads();
         int i = 0;
         for (; i + 3 < count; i += 2) {
             multiply(0, wa);
             put_x(1, stage);
-            ask_x(chunk_at(i + 2), stage);
-            ask_w(chunk_at(i + 2), wa);
+            ask_x(c_lo + i + 2, stage);
+            ask_w(c_lo + i + 2, wa);
             __syncthreads();
             multiply(1, wb);
             put_x(0, stage);
-            ask_x(chunk_at(i + 3), stage);
-            ask_w(chunk_at(i + 3), wb);
+            ask_x(c_lo + i + 3, stage);
+            ask_w(c_lo + i + 3, wb);
             __syncthreads();
         }
         // two or three chunks are left: chunk i is ready, chunk i+1 on its way
@@ -150,8 +149,8 @@ gemm_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, v
         multiply(0, wa);
         put_x(1, stage);
         if (third) {
-            ask_x(chunk_at(i + 2), stage);
-            ask_w(chunk_at(i + 2), wa);
+            ask_x(c_lo + i + 2, stage);
+            ask_w(c_lo + i + 2, wa);
         }
         __syncthreads();
         multiply(1, wb);
@@ -161,8 +160,8 @@ gemm_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, v
             multiply(0, wa);
         }
     } else if (count == 1) {
-        ask_x(chunk_at(0), stage);
-        ask_w(chunk_at(0), wa);
+        ask_x(c_lo, stage);
+        ask_w(c_lo, wa);
         put_x(0, stage);
         __syncthreads();
         multiply(0, wa);
