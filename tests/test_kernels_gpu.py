@@ -873,6 +873,8 @@ GROUPED_CASES = [
     (10, 2, 128, 4, [(97, 1), (130, 2)], 0),
     (32, 4, 128, 64, [(513, 1), (300, 2)], 0),
     (16, 2, 64, 256, [(700, 3)], 100),
+    # contexts around the edges of the 64-key tiles, through more tiles than the rings of LDS buffers hold
+    (64, 8, 128, 16, [(63, 1), (127, 1), (128, 1), (191, 1), (192, 1), (193, 1), (384, 1), (385, 1), (449, 2)], 0),
 ]
 
 
