@@ -3,7 +3,7 @@
 from __future__ import annotations
 
 import ctypes
-from ctypes import POINTER, c_char_p, c_float, c_int, c_long, c_size_t, c_uint32, c_uint64, c_void_p
+from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_long, c_size_t, c_uint32, c_uint64, c_void_p
 
 from . import build
 from .errors import ConfigError
@@ -54,6 +54,12 @@ def _signatures(lib) -> None:
         "plh_sched_metrics": ([vp, P(u64)], None),
         "plh_sched_sample": ([vp, u64, vp, sz], lg),
         "plh_sched_sampling_of": ([vp, u64, P(f32), P(i32), P(f32), P(f32)], lg),
+        "plh_oracle_rms_norm": ([vp, vp, c_double, lg, lg, vp], None),
+        "plh_oracle_rotate": ([vp, vp, lg, lg, lg, lg, c_double, i32], None),
+        "plh_oracle_product": ([vp, vp, lg, lg, lg, vp], None),
+        "plh_oracle_swiglu": ([vp, lg, lg, vp], None),
+        "plh_oracle_paged_attention": ([vp, vp, vp, vp, vp, vp, lg, lg, lg, lg, lg, lg, c_double, lg, vp], None),
+        "plh_oracle_argmax": ([vp, lg, lg, vp], None),
     }
     for name, (argtypes, restype) in table.items():
         fn = getattr(lib, name)

@@ -1204,3 +1204,94 @@ def test_sampling_kernel_on_rows_made_by_hand():
     got = kernels.sample(logits, col(1, torch.float32), col(2, torch.int32), col(3, torch.float32),
                          col(4, torch.float32)).cpu().tolist()
     assert got == [c[5] for c in cases]
+
+
+# --- every kernel beside its plain C++ oracle ----------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_the_kernels_beside_their_plain_cpp_oracles(dtype):
+    """The oracles are the sequential C++ functions of csrc/host/oracle.cpp (pinned on the CPU by
+    tests/test_oracle.py); each kernel is run on the same numbers, at sizes that are no powers of two."""
+    from paged_llm_rs_amd import kernels, oracle
+
+    tol = 2e-5 if dtype == torch.float32 else 1.2e-2
+    g = torch.Generator().manual_seed(11)
+    rnd = lambda *shape: torch.randn(*shape, generator=g).to(dtype)
+
+    # norm (with the residual sum before it)
+    resid, delta, gain = torch.randn(7, 200, generator=g), rnd(7, 200), rnd(200)
+    out = torch.empty(7, 200, dtype=dtype, device=DEV)
+    stream = resid.to(DEV)
+    kernels.add_rmsnorm(stream, delta.to(DEV), gain.to(DEV), 1e-5, out)
+    assert rel(out, oracle.rms_norm(resid + delta.float(), gain, 1e-5)) < tol
+    assert rel(stream, resid + delta.float()) < 1e-6
+
+    # activation and argmax
+    gu = rnd(9, 2 * 77)
+    assert rel(kernels.swiglu(gu.to(DEV)), oracle.swiglu(gu)) < tol
+    logits = torch.randn(5, 1003, generator=g)
+    logits[2, 17] = logits[2, 900] = 50.0
+    assert kernels.argmax(logits.to(DEV)).cpu().tolist() == oracle.argmax(logits).tolist()
+
+    # products: the plain one in either dtype, the matrix-core ones in bfloat16
+    x, w = rnd(19, 264), (torch.randn(130, 264, generator=g) / 16).to(dtype)
+    want = oracle.product(x, w)
+    assert rel(kernels.gemm_plain(x.to(DEV), w.to(DEV), out_dtype=torch.float32), want) < 2e-5
+    if dtype == torch.bfloat16:
+        assert rel(kernels.gemm_skinny(x.to(DEV), w.to(DEV), torch.float32), want) < 2e-5
+        assert rel(kernels.gemm_stream(x.to(DEV), w.to(DEV), torch.float32), want) < 2e-5
+        xm, wm = rnd(200, 96), (torch.randn(256, 96, generator=g) / 10).to(dtype)
+        assert rel(kernels.gemm_tiled(xm.to(DEV), wm.to(DEV)), oracle.product(xm, wm)) < tol
+
+    # q/k norm, rotation (either layout) and the write into the pages
+    nq, nkv, d, bs, rot, theta = 6, 2, 48, 4, 32, 10000.0
+    ctx = [13, 6]
+    bt, k_pool, v_pool, _, _ = build_paged(nkv, d, bs, ctx, dtype, seed=5)
+    positions = [12, 5, 4]
+    seq_of = [0, 1, 1]
+    qkv = rnd(3, (nq + 2 * nkv) * d)
+    q_gain, k_gain = 1 + 0.2 * torch.randn(d, generator=g), 1 + 0.2 * torch.randn(d, generator=g)
+    as_i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    for neighbours in (False, True):
+        angle = torch.arange(64, dtype=torch.float64)[:, None] * theta ** (-torch.arange(rot // 2, dtype=torch.float64) * 2 / rot)
+        cos, sin = angle.cos().float().to(DEV), angle.sin().float().to(DEV)
+        buf, kp, vp = qkv.to(DEV).clone(), k_pool.clone(), v_pool.clone()
+        kernels.qk_norm_rope_kv_write(buf, q_gain.to(DEV), k_gain.to(DEV), 1e-6, cos, sin, rot, as_i32(positions), as_i32(seq_of),
+                                      bt, bs, kp, vp, nq, nkv, d, neighbours=neighbours)
+        heads = qkv.float().view(3, nq + 2 * nkv, d)
+        q_want = oracle.rotate(oracle.rms_norm(heads[:, :nq].reshape(-1, d), q_gain, 1e-6).view(3, nq, d), positions, rot, theta, neighbours)
+        k_want = oracle.rotate(oracle.rms_norm(heads[:, nq:nq + nkv].reshape(-1, d), k_gain, 1e-6).view(3, nkv, d), positions, rot, theta, neighbours)
+        assert rel(buf[:, :nq * d].view(3, nq, d), q_want) < tol
+        for t in range(3):
+            slot = int(bt[seq_of[t], positions[t] // bs]) * bs + positions[t] % bs
+            assert rel(kp[slot].view(nkv, d), k_want[t]) < tol
+            assert rel(vp[slot].view(nkv, d), heads[t, nq + nkv:]) < 1e-6
+
+    # attention over the pages: every kernel that serves single tokens and portions
+    nq, nkv, d, bs = 8, 2, 64, 16
+    ctx = [150, 37, 64]
+    bt, k_pool, v_pool, _, _ = build_paged(nkv, d, bs, ctx, dtype, seed=9)
+    positions = [149, 36, 63, 20, -1]
+    seq_of = [0, 1, 2, 0, 0]
+    stride = (nq + 2 * nkv) * d
+    q = rnd(5, stride).to(DEV)
+    scale = 1 / math.sqrt(d)
+    for window in (0, 40):
+        want = oracle.paged_attention(q, k_pool, v_pool, bt, positions, seq_of, nq, nkv, d, bs, scale, window)
+        out = torch.zeros(5, nq * d, dtype=dtype, device=DEV)
+        kernels.paged_attention_plain(q, stride, out, as_i32(positions), as_i32(seq_of), bt, bs, k_pool, v_pool, nq, nkv, d, scale, window)
+        assert rel(out[:4], want[:4]) < tol
+        if dtype == torch.bfloat16:
+            for splits in (1, 3):
+                out = torch.zeros(5, nq * d, dtype=dtype, device=DEV)
+                kernels.paged_attention_decode(q, stride, out, as_i32(positions), as_i32(seq_of), bt, bs, k_pool, v_pool, nq, nkv, d,
+                                               scale, window, splits=splits)
+                assert rel(out[:4], want[:4]) < tol, f"single-token kernel, {splits} shares, window {window}"
+            # the tiled kernel and its grouped mode take requests, not rows: the last token of each request
+            last = [149, 36, 63]
+            q3 = q[:3].contiguous()
+            want3 = oracle.paged_attention(q3, k_pool, v_pool, bt, last, [0, 1, 2], nq, nkv, d, bs, scale, window)
+            one, start, lens = as_i32([1, 1, 1]), as_i32([0, 1, 2]), as_i32(ctx)
+            out = torch.zeros(3, nq * d, dtype=dtype, device=DEV)
+            kernels.paged_attention_prefill(q3, stride, out, start, one, lens, 1, bt, bs, k_pool, v_pool, nq, nkv, d, scale, window)
+            assert rel(out, want3) < tol, f"tiled kernel, window {window}"
