@@ -60,6 +60,7 @@ class LayerSpec:
     feed_forward: Any = None
     norm: Any = None
     weight_prefix: str = ""
+    names: Optional[dict] = None            # other tensor-name parts for the block's members (norm1, mixer, norm2, feed_forward)
 
 
 @dataclass(frozen=True)

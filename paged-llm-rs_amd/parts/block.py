@@ -11,6 +11,7 @@ product kernel and the norm becomes the first stage of the next product.
 
 from __future__ import annotations
 
+from ..errors import ConfigError
 from .norm import PendingNorm
 from .registry import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, lookup, prefixed, register_block, scoped)
 
@@ -20,18 +21,27 @@ class PreNormBlock:
              "feed_forward": "mlp"}
 
     @classmethod
+    def names_of(cls, layer) -> dict:
+        """The name parts of the members' tensors: this architecture's, or the layer spec's own."""
+        given = getattr(layer, "names", None) or {}
+        unknown = sorted(set(given) - set(cls.NAMES))
+        if unknown:
+            raise ConfigError(f"a layer names members that this arrangement does not have: {unknown}")
+        return {**cls.NAMES, **given}
+
+    @classmethod
     def declare(cls, layer, hidden: int) -> list:
         norm = lookup(NORMS, layer.norm.kind, "norm")
         mixer = lookup(MIXERS, layer.mixer.kind, "mixer")
         ffn = lookup(FEED_FORWARDS, layer.feed_forward.kind, "feed-forward")
-        n = cls.NAMES
+        n = cls.names_of(layer)
         return (prefixed(norm.declare(layer.norm, hidden), n["norm1"])
                 + prefixed(mixer.declare(layer.mixer, hidden), n["mixer"])
                 + prefixed(norm.declare(layer.norm, hidden), n["norm2"])
                 + prefixed(ffn.declare(layer.feed_forward, hidden), n["feed_forward"]))
 
     def __init__(self, layer, hidden: int, params: dict, dtype, device, shared: dict):
-        n = self.NAMES
+        n = self.names = self.names_of(layer)
         norm = lookup(NORMS, layer.norm.kind, "norm")
         self.dtype = dtype
         self.norm1 = norm(layer.norm, hidden, scoped(params, n["norm1"]), dtype, device)
@@ -74,7 +84,7 @@ class PreNormBlock:
         every norm runs as a kernel and no part adds into the stream itself.  A part whose class sets
         ``records = True`` takes the recorder (``ctx.trace`` for a mixer, ``trace=`` for a feed-forward)
         and records what happens inside it."""
-        n, trace = self.NAMES, ctx.trace
+        n, trace = self.names, ctx.trace
         x = self.norm1.apply(resid, delta, self.dtype)
         trace.record(f"{n['norm1']}.out", x)
         ctx.trace = trace.child(n["mixer"]) if getattr(self.mixer, "records", False) else None

@@ -975,6 +975,60 @@ def test_a_toy_norm_and_a_toy_arrangement_of_a_layer(tmp_path, dtype):
         assert worst <= tolerance, f"{worst:.3e} at {where}"
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_same_arrangement_under_other_tensor_names(tmp_path, model_dirs, dtype):
+    """The members of a layer carry this architecture's names unless the layer's spec gives others: the same
+    weights under another family's names, through the same block class, give the same bits."""
+    import dataclasses
+    import json
+
+    from safetensors.torch import load_file, save_file
+
+    from paged_llm_rs_amd.config import register_architecture
+    from paged_llm_rs_amd.config.qwen3 import Qwen3Config
+    from paged_llm_rs_amd.engine.replay import Replayer
+    from paged_llm_rs_amd.errors import ConfigError
+
+    renamed = {"norm1": "ln_1", "mixer": "attn", "norm2": "ln_2", "feed_forward": "ffn"}
+
+    class OtherNamesConfig(Qwen3Config):
+        @classmethod
+        def from_dict(cls, d):
+            return super().from_dict({**d, "model_type": "qwen3", "architectures": ["Qwen3ForCausalLM"]})
+
+        def model_spec(self):
+            spec = super().model_spec()
+            layers = tuple(dataclasses.replace(layer, names=renamed, weight_prefix=f"transformer.h.{i}")
+                           for i, layer in enumerate(spec.layers))
+            return dataclasses.replace(spec, layers=layers)
+
+    register_architecture("OtherNamesForCausalLM", OtherNamesConfig, model_type="other_names")
+    source = model_dirs("B", dtype)
+    config = json.loads((source / "config.json").read_text())
+    config.update(architectures=["OtherNamesForCausalLM"], model_type="other_names")
+    folder = tmp_path / "other_names"
+    folder.mkdir()
+    (folder / "config.json").write_text(json.dumps(config))
+    standard = {"input_layernorm": "ln_1", "self_attn": "attn", "post_attention_layernorm": "ln_2", "mlp": "ffn"}
+    tensors = {}
+    for name, tensor in load_file(str(source / "model.safetensors")).items():
+        parts = name.split(".")
+        if parts[:2] == ["model", "layers"]:
+            parts = ["transformer", "h", parts[2], standard[parts[3]]] + parts[4:]
+        tensors[".".join(parts)] = tensor
+    save_file(tensors, str(folder / "model.safetensors"))
+    prompts = ru.make_prompts(config["vocab_size"], [29, 7], seed=3)
+    got = [ru.collect(Replayer(d, dtype, max_tokens=ru.pool_tokens(prompts, 1), block_size=8), ru.tail_decoded(prompts, 5))
+           for d in (source, folder)]
+    assert got[0].keys() == got[1].keys() and len(got[0]) > 10
+    for place in got[0]:
+        assert np.array_equal(np.asarray(got[0][place]), np.asarray(got[1][place])), place
+    with pytest.raises(ConfigError, match="does not have"):
+        bad = dataclasses.replace(OtherNamesConfig.from_dict(config).model_spec().layers[0], names={"norm3": "x"})
+        from paged_llm_rs_amd.parts.block import PreNormBlock
+        PreNormBlock.declare(bad, config["hidden_size"])
+
+
 # --- long decoding, first tokens, long portions -----------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
