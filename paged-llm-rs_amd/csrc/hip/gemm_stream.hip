@@ -224,23 +224,68 @@ gemm_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, v
 }
 
 // Adds the partial tiles of the stretches of K, in their order, and does what follows the product.
-// One thread a column of a row (two weights' columns for GS_SWIGLU).
-template <int MODE>
+// A thread takes V neighbouring columns of a row (V = 4 where the width allows 16-byte loads, else 1), and
+// for GS_SWIGLU the gate's and the up's.
+template <int MODE, int V>
 __global__ void __launch_bounds__(256)
 gemm_stream_finish_kernel(const float* __restrict__ ws, void* __restrict__ y_, int n, int N_out, int Nw, int splits, int act) {
     const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (idx >= static_cast<size_t>(n) * N_out) return;
-    const int row = static_cast<int>(idx / N_out), col = static_cast<int>(idx - static_cast<size_t>(row) * N_out);
-    float first = 0.f, second = 0.f;
+    const int groups = N_out / V;                       // (V divides N_out)
+    if (idx >= static_cast<size_t>(n) * groups) return;
+    const int row = static_cast<int>(idx / groups), col = static_cast<int>(idx - static_cast<size_t>(row) * groups) * V;
+    float first[V], second[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) first[e] = second[e] = 0.f;
     for (int s = 0; s < splits; ++s) {
         const float* at = ws + (static_cast<size_t>(s) * n + row) * Nw;
-        first += at[col];
-        if constexpr (MODE == GS_SWIGLU) second += at[N_out + col];
+        if constexpr (V == 4) {
+            const gs_f32x4 a = *reinterpret_cast<const gs_f32x4*>(at + col);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) first[e] += a[e];
+            if constexpr (MODE == GS_SWIGLU) {
+                const gs_f32x4 b = *reinterpret_cast<const gs_f32x4*>(at + N_out + col);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) second[e] += b[e];
+            }
+        } else {
+            first[0] += at[col];
+            if constexpr (MODE == GS_SWIGLU) second[0] += at[N_out + col];
+        }
     }
-    if constexpr (MODE == GS_SWIGLU) static_cast<bf16_t*>(y_)[idx] = from_float<bf16_t>(pl_activate<false>(first, act) * second);
-    else if constexpr (MODE == GS_STORE_BF16) static_cast<bf16_t*>(y_)[idx] = from_float<bf16_t>(first);
-    else if constexpr (MODE == GS_STORE_F32) static_cast<float*>(y_)[idx] = first;
-    else static_cast<float*>(y_)[idx] += first;
+    const size_t out = static_cast<size_t>(row) * N_out + col;
+    if constexpr (V == 4 && (MODE == GS_ADD || MODE == GS_STORE_F32)) {
+        // (16-byte aligned: the launcher looked at y as it looked at ws)
+        gs_f32x4* to = reinterpret_cast<gs_f32x4*>(static_cast<float*>(y_) + out);
+        gs_f32x4 v = {first[0], first[1], first[2], first[3]};
+        if constexpr (MODE == GS_ADD) v += *to;
+        *to = v;
+        return;
+    }
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+        if constexpr (MODE == GS_SWIGLU) static_cast<bf16_t*>(y_)[out + e] = from_float<bf16_t>(pl_activate<false>(first[e], act) * second[e]);
+        else if constexpr (MODE == GS_STORE_BF16) static_cast<bf16_t*>(y_)[out + e] = from_float<bf16_t>(first[e]);
+        else if constexpr (MODE == GS_STORE_F32) static_cast<float*>(y_)[out + e] = first[e];
+        else static_cast<float*>(y_)[out + e] += first[e];
+    }
+}
+
+// mode: one of GS_STORE_BF16, GS_STORE_F32, GS_SWIGLU, GS_ADD.
+static void gs_finish(const float* ws, void* y, int n, int N_out, int Nw, int splits, int mode, int act, hipStream_t stream) {
+    const bool wide = N_out % 4 == 0 && Nw % 4 == 0 && reinterpret_cast<uintptr_t>(ws) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0;
+    const int blocks = static_cast<int>((static_cast<size_t>(n) * (N_out / (wide ? 4 : 1)) + 255) / 256);
+#define GS_FINISH(MODE)                                                                                              \
+    do {                                                                                                             \
+        if (wide) gemm_stream_finish_kernel<MODE, 4><<<blocks, 256, 0, stream>>>(ws, y, n, N_out, Nw, splits, act);  \
+        else gemm_stream_finish_kernel<MODE, 1><<<blocks, 256, 0, stream>>>(ws, y, n, N_out, Nw, splits, act);       \
+    } while (0)
+    switch (mode) {
+        case GS_STORE_BF16: GS_FINISH(GS_STORE_BF16); break;
+        case GS_STORE_F32: GS_FINISH(GS_STORE_F32); break;
+        case GS_SWIGLU: GS_FINISH(GS_SWIGLU); break;
+        default: GS_FINISH(GS_ADD); break;
+    }
+#undef GS_FINISH
 }
 
 static int gs_column_groups(int N_out, bool swiglu, int waves = GS_WAVES) { return swiglu ? pl_ceil_div(N_out, 16 * waves) : pl_ceil_div(N_out, 32 * waves); }
@@ -294,14 +339,7 @@ static int gs_launch(const bf16_t* x, const bf16_t* w, void* y, float* ws, int n
         gemm_stream_kernel<MT, GS_PARTIAL, WV><<<dim3(pl_ceil_div(Nw, 32 * WV), grid.y), 64 * WV, 0, stream>>>(
             x, w, y, ws, n, Nw, Nw, K, act, per_split);
         PL_CHECK_LAUNCH("gemm_stream");
-        const int blocks = static_cast<int>((static_cast<size_t>(n) * N_out + 255) / 256);
-        const int parts = static_cast<int>(grid.y);
-        switch (mode) {
-            case GS_STORE_BF16: gemm_stream_finish_kernel<GS_STORE_BF16><<<blocks, 256, 0, stream>>>(ws, y, n, N_out, Nw, parts, act); break;
-            case GS_STORE_F32: gemm_stream_finish_kernel<GS_STORE_F32><<<blocks, 256, 0, stream>>>(ws, y, n, N_out, Nw, parts, act); break;
-            case GS_SWIGLU: gemm_stream_finish_kernel<GS_SWIGLU><<<blocks, 256, 0, stream>>>(ws, y, n, N_out, Nw, parts, act); break;
-            default: gemm_stream_finish_kernel<GS_ADD><<<blocks, 256, 0, stream>>>(ws, y, n, N_out, Nw, parts, act); break;
-        }
+        gs_finish(ws, y, n, N_out, Nw, static_cast<int>(grid.y), mode, act, stream);
         PL_CHECK_LAUNCH("gemm_stream_finish");
         return 0;
     }
@@ -352,12 +390,8 @@ extern "C" int pl_gemm_finish(const float* ws, void* y, long long n, int N_out, 
     PL_REQUIRE(act == PL_ACT_SILU || act == PL_ACT_GELU_TANH || act == PL_ACT_GELU, "sum of partial products: activation code %d", act);
     PL_REQUIRE(n * N_out < (1ll << 31) * 256 && n <= 0x7fffffff, "sum of partial products: %lld x %d results", n, N_out);
     const int Nw = epilogue == 1 ? 2 * N_out : N_out;
-    const int blocks = static_cast<int>((static_cast<size_t>(n) * N_out + 255) / 256);
-    const int rows = static_cast<int>(n);
-    if (epilogue == 1) gemm_stream_finish_kernel<GS_SWIGLU><<<blocks, 256, 0, stream>>>(ws, y, rows, N_out, Nw, splits, act);
-    else if (epilogue == 2) gemm_stream_finish_kernel<GS_ADD><<<blocks, 256, 0, stream>>>(ws, y, rows, N_out, Nw, splits, act);
-    else if (out_f32) gemm_stream_finish_kernel<GS_STORE_F32><<<blocks, 256, 0, stream>>>(ws, y, rows, N_out, Nw, splits, act);
-    else gemm_stream_finish_kernel<GS_STORE_BF16><<<blocks, 256, 0, stream>>>(ws, y, rows, N_out, Nw, splits, act);
+    const int mode = epilogue == 1 ? GS_SWIGLU : (epilogue == 2 ? GS_ADD : (out_f32 ? GS_STORE_F32 : GS_STORE_BF16));
+    gs_finish(ws, y, static_cast<int>(n), N_out, Nw, splits, mode, act, stream);
     PL_CHECK_LAUNCH("gemm_stream_finish");
     return 0;
 }
