@@ -208,7 +208,7 @@ class Workbench:
                 runner.run(entry)        # as the engine runs it: a shape of step that comes again is replayed from a graph
             cache.manager.free_sequence(1000)
 
-        seconds_prefill = timed(prefill, 5, 3)
+        seconds_prefill = timed(prefill, 10, 5)
         d, nq = self.cfg["head_dim"], self.cfg["num_attention_heads"]
         attention_flops = self.layers * 4 * nq * d * (PREFILL_TOKENS * (PREFILL_TOKENS + 1) // 2)
         flops = self.layer_flops * PREFILL_TOKENS + self.head_flops + attention_flops
