@@ -318,19 +318,44 @@ def set_attention(mode: str) -> None:
     _attention_mode = mode
 
 
-def decode_splits(tokens: int, nq: int, nkv: int, max_ctx: int) -> int:
-    """How many stretches the context is cut into, so that a launch fills the chip: none when the
-    tokens and heads alone give a workgroup a compute unit (two, with more than two query heads a key
-    head: a workgroup then has more arithmetic a key), else up to about that many workgroups, each with at
-    least 128 keys (two rounds of loads).  (More shares were slower wherever they were measured, 1 to 64
-    tokens at contexts of 512 to 4,096: 8 tokens at context 4,096 take 39.7 us with 16 shares and 34.0 with 4.)"""
+# What a compute unit takes in from memory (bytes a microsecond), what the merge of the shares costs beside the
+# kernel (microseconds), and the compute units: the figures of the estimate below.
+DECODE_INTAKE = 22e3
+DECODE_MERGE_US = 4.0
+
+
+def decode_splits(tokens: int, nq: int, nkv: int, max_ctx: int, d: int = 128) -> int:
+    """Into how many stretches the context is cut for the single-token kernel, each with at least 128 keys
+    (two rounds of loads).
+
+    Up to two query heads a key head the kernel waits for memory, and a compute unit takes in only so much:
+    the launch is as long as the keys and values of its busiest compute unit take (workgroups are dealt to
+    the compute units in turn), plus the merge's kernel where there are shares; the count with the smallest
+    such estimate is taken.  (Measured, 16 query over 8 key heads of 128, one share against the estimate's
+    choice: 12 tokens at context 2,048, three shares 32.9 us, eight 28.0; 24 tokens, two 50.1, four 45.4; 48
+    tokens at 1,024, one 48.1, two 45.3; 24 tokens at 512, two 20.9, one 18.8.)
+    With more query heads a key head a workgroup has more arithmetic a key and the compute units are what
+    is short: none when the tokens and heads alone give about two workgroups a compute unit, else up to
+    that many (8 tokens at context 2,048 with four heads a key head: eight shares 24.6 us, four 25.9; 32
+    tokens, two 61.9, one 68.3; 63 tokens, one 105.7, two 111.2)."""
     g = nq // nkv
     gt = 8 if g >= 8 else (4 if g > 2 else g)
     base = max(tokens * nkv * ((g + gt - 1) // gt), 1)
-    target = 256 if g <= 2 else 512
-    if base >= target:
-        return 1
-    return max(1, min((target + base - 1) // base, (max_ctx + 127) // 128, 64))
+    most = max(1, min((max_ctx + 127) // 128, 64))
+    if g > 2:
+        target = 2 * compute_units()
+        if base >= target - target // 16:
+            return 1
+        return max(1, min((target + base - 1) // base, most))
+    units = compute_units()
+    best, best_us = 1, None
+    for splits in range(1, most + 1):
+        busiest = -(-base * splits // units)                      # workgroups on one compute unit
+        keys = -(-max_ctx // splits)
+        us = busiest * keys * (4 * d) / DECODE_INTAKE + (DECODE_MERGE_US if splits > 1 else 0.0)
+        if best_us is None or us < best_us - 1e-9:
+            best, best_us = splits, us
+    return best
 
 
 def paged_attention_decode(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, positions: torch.Tensor,
@@ -560,7 +585,7 @@ def attention_step(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nkv
     any other step runs the stand-alone kernel for the first three and then attention."""
     if (qkv.dtype == torch.bfloat16 and _attention_mode == "kernel" and batch.max_q_len == 1
             and prepare.rot % 16 == 0 and not prepare.neighbours and not grouped_applies(nq, nkv, d, kv.block_size)):
-        splits = decode_splits(batch.num_tokens, nq, nkv, batch.max_ctx_len)
+        splits = decode_splits(batch.num_tokens, nq, nkv, batch.max_ctx_len, d)
         return paged_attention_decode(qkv, qkv.shape[1], out, batch.positions, batch.seq_of, kv.block_table,
                                       kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window, splits,
                                       fuse=prepare)
@@ -604,7 +629,7 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nk
                                        kv.k_pool, kv.v_pool, nq, nkv, d, scale, window,
                                        short_limit=SHORT_PORTION if mixed else 0, max_ctx=batch.max_ctx_len,
                                        live_seqs=getattr(batch, "live_seqs", None), tokens=batch.short_tokens)
-    splits = decode_splits(batch.short_tokens, nq, nkv, batch.max_ctx_len)
+    splits = decode_splits(batch.short_tokens, nq, nkv, batch.max_ctx_len, d)
     return paged_attention_decode(qkv, stride, out, batch.positions, batch.seq_of, kv.block_table,
                                   kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window, splits,
                                   q_len=batch.q_len if mixed else None, short_limit=SHORT_PORTION if mixed else 0,
