@@ -85,4 +85,12 @@ class ModelSpec:
     embed_name: str = "model.embed_tokens.weight"
     final_norm_name: str = "model.norm.weight"
     head_name: str = "lm_head.weight"
+    # Tensors a checkpoint of this family carries and the model does not use (buffers, tables that are
+    # computed here): shell patterns over tensor names, e.g. "*.rotary_emb.inv_freq".  They are neither
+    # loaded nor reported as unexpected.
+    ignored_tensors: tuple = ()
+    # What the decoder does beside the layers, by the names of registered transforms:
+    # ``extra["embed_transform"]`` is applied to the 32-bit stream right after the embedding gather (a scale,
+    # a learned position added to it), ``extra["logit_transform"]`` to the 32-bit logits (a soft cap, a
+    # scale).  Each transform reads its own constants from ``extra`` too.  None of the two by default.
     extra: dict = field(default_factory=dict)

@@ -616,7 +616,6 @@ static int launch_decode_keys(const void* q, int q_stride, void* out, float* par
 // where a workgroup serves many query heads), so that several workgroups fit a compute unit.  The choice
 // goes by the step's rows, not by the rows that get workgroups, so that a step computes the same bits
 // however its launch is sized.
-#define AD_FEW_WORKGROUPS 256
 
 template <int LPK, int GT>
 static int launch_decode(const void* q, int q_stride, void* out, float* part_acc, float* part_ml,
@@ -630,7 +629,7 @@ static int launch_decode(const void* q, int q_stride, void* out, float* part_acc
                                           short_limit, num_seqs, short_rows, block_table, max_blocks, block_size,  \
                                           k_pool, v_pool, n, nq, nkv, d, scale, window, splits, fuse, stream)
     if constexpr (GT <= 2) {
-        if (workgroups <= AD_FEW_WORKGROUPS) AD_KEYS_CALL(8);
+        if (workgroups <= pl_compute_units()) AD_KEYS_CALL(8);
         AD_KEYS_CALL(4);
     } else {
         AD_KEYS_CALL(2);

@@ -90,6 +90,9 @@ __device__ __forceinline__ float pl_activate(float g, int act) {
 // Launchers return 0 or a negative code and leave a message for pl_last_error().
 void pl_set_error(const char* fmt, ...);
 
+// The compute units of the current device (launch-size choices go by it).
+int pl_compute_units();
+
 #define PL_REQUIRE(cond, ...)            \
     do {                                 \
         if (!(cond)) {                   \

@@ -172,7 +172,8 @@ gemm_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, v
         const bool x_in = k0 + xpiece * 8 < K;
 #pragma unroll
         for (int p = 0; p < XP; ++p) {
-            const gs_u32x4 got = *reinterpret_cast<const gs_u32x4*>(xp[p] + (x_in ? k0 : 0));
+            // (a lane whose piece lies past K reads the start of its row instead: K is 8 at least)
+            const gs_u32x4 got = *reinterpret_cast<const gs_u32x4*>(xp[p] + (x_in ? k0 : -xpiece * 8));
 #pragma unroll
             for (int e = 0; e < 4; ++e) stage[p].v[e] = x_in ? got.v[e] : 0u;
         }
@@ -181,7 +182,7 @@ gemm_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, v
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
                 const bool in = k0 + s * 32 + g * 8 < K;
-                const gs_u32x4 got = *reinterpret_cast<const gs_u32x4*>(wp[t] + (in ? k0 + s * 32 : 0));
+                const gs_u32x4 got = *reinterpret_cast<const gs_u32x4*>(wp[t] + (in ? k0 + s * 32 : -g * 8));
 #pragma unroll
                 for (int e = 0; e < 4; ++e) wa[t * 4 + s].v[e] = in ? got.v[e] : 0u;
             }
@@ -297,9 +298,9 @@ static int gs_column_groups(int N_out, bool swiglu, int waves = GS_WAVES) { retu
 // 5,120: 400 workgroups, 4.2 TB/s; 65,536 rows: 512 workgroups, 5.0 TB/s).  More stretches make the shares
 // more even, but every stretch beyond the first writes and reads its partial tiles, n x (rows of w) floats.
 // The count with the smallest estimate of (bytes moved) / (evenness) is taken.
-#define GS_UNITS 256
 extern "C" int pl_gemm_stream_splits(int n, int N_out, int K, int swiglu) {
     if (n <= 0 || N_out <= 0 || K <= 0) return 1;
+    const long long units = pl_compute_units();
     const long long Nw = static_cast<long long>(N_out) * (swiglu ? 2 : 1);
     const int nchunks = pl_ceil_div(K, GS_BK);
     const double weights = static_cast<double>(Nw) * K * 2;
@@ -312,8 +313,8 @@ extern "C" int pl_gemm_stream_splits(int n, int N_out, int K, int swiglu) {
         if (parts != splits) continue;                       // the same launch as a smaller count
         const long long groups = splits > 1 ? (Nw + 32 * GS_WAVES - 1) / (32 * GS_WAVES) : gs_column_groups(N_out, swiglu != 0);
         const long long workgroups = groups * parts;
-        const long long rounds = (workgroups + GS_UNITS - 1) / GS_UNITS;
-        const double even = static_cast<double>(workgroups) / (static_cast<double>(rounds) * GS_UNITS);
+        const long long rounds = (workgroups + units - 1) / units;
+        const double even = static_cast<double>(workgroups) / (static_cast<double>(rounds) * units);
         // (the second kernel's launch counts as the bytes that three microseconds move)
         const double moved = weights + (splits > 1 ? 2.0 * splits * n * static_cast<double>(Nw) * 4 + 1.5e7 : 0.0);
         const double cost = moved / even;

@@ -35,7 +35,7 @@ class StepBatch:
 
     def __init__(self, packed: torch.Tensor, layout: dict, num_tokens: int, num_seqs: int, max_blocks: list,
                  num_logit_rows: int, max_q_len: int, max_ctx_len: int, seq_ids: list,
-                 short_tokens: int | None = None):
+                 tokens_each=None, padded: bool = False, short_bounds: dict | None = None):
         self.packed = packed
         self.layout = layout
         self.num_tokens = num_tokens
@@ -45,8 +45,13 @@ class StepBatch:
         self.max_q_len = max_q_len
         self.max_ctx_len = max_ctx_len
         self.seq_ids = seq_ids
-        # tokens of requests that bring fewer than SHORT_PORTION tokens: the single-token kernel's share
-        self.short_tokens = num_tokens if short_tokens is None else short_tokens
+        # On the host: the tokens every live request brings; whether the step reports bounds instead of
+        # counts (a padded step does); and, for such a step, {limit: the most tokens that requests of fewer
+        # than ``limit`` tokens bring together}.
+        self.tokens_each = (np.ones(num_seqs, np.int64) if tokens_each is None
+                            else np.asarray(tokens_each, dtype=np.int64))
+        self.padded = padded
+        self.short_bounds = dict(short_bounds or {})
 
         def view(name, *shape):
             begin, count = layout[name]
@@ -61,6 +66,16 @@ class StepBatch:
         self.state_slots = view("state_slots", num_seqs)
         self.logit_rows = view("logit_rows", num_logit_rows)
         self.block_tables = [view(f"block_table_{g}", num_seqs, mb) for g, mb in enumerate(max_blocks)]
+
+    def tokens_of_short_requests(self, limit: int) -> int:
+        """How many tokens the requests that bring fewer than ``limit`` tokens bring together: what a
+        mixer that runs such requests through a kernel of their own sizes that launch by.  A padded step
+        gives a bound (the one it was laid out with for this limit, else all its rows), or 0 when there
+        is no such request."""
+        short = int(self.tokens_each[self.tokens_each < limit].sum())
+        if not self.padded or short == 0:
+            return short
+        return min(self.num_tokens, self.short_bounds.get(limit, self.num_tokens))
 
 
 def context_bound(longest: int) -> int:
@@ -109,7 +124,7 @@ def token_bucket(tokens: int) -> int:
 
 def build_batch(entries, manager, num_groups: int, vocab_size: int, max_positions: int, device,
                 check_start: bool = True, widths: list | None = None, ctx_bound: int | None = None,
-                pad_to: int | None = None, short_bound: int | None = None) -> StepBatch:
+                pad_to: int | None = None, short_bounds: dict | None = None) -> StepBatch:
     """Validate the entries against the cache manager and lay the step out for the device.
 
     ``widths`` fixes the pages a row of each group's block table has (TableTooWide if a request
@@ -121,9 +136,9 @@ def build_batch(entries, manager, num_groups: int, vocab_size: int, max_position
     (token 0, position -1, no pages, no context, state slot -1; it has no rows when none are
     missing).  The batch then reports bounds instead of counts (every row might belong to one
     request, or to short ones), so that steps with the same rows, requests and wanted places give
-    the kernels the same launch sizes.  ``short_bound`` says how many tokens the requests with fewer
-    than SHORT_PORTION tokens bring at most (ShortTokensOutgrown if they bring more); without it every
-    row might be one of theirs.
+    the kernels the same launch sizes.  ``short_bounds`` maps a limit to how many tokens the requests
+    with fewer than ``limit`` tokens bring together at most (ShortTokensOutgrown if they bring more);
+    for a limit it does not name every row might be one of theirs.
 
     Refused with ConfigError: an empty step, an entry without tokens, a token id
     outside the vocabulary, a position with no page or past the longest position
@@ -206,22 +221,23 @@ def build_batch(entries, manager, num_groups: int, vocab_size: int, max_position
         begin, count = layout[name]
         host[begin:begin + count] = arr
     packed = torch.from_numpy(host).to(device)
-    from ..kernels import SHORT_PORTION
     longest = int(ctx_len.max())
     if ctx_bound is None:
         ctx_bound = context_bound(longest)
     if longest > ctx_bound:
         raise ContextTooLong(f"a context of {longest} tokens in a step laid out for {ctx_bound}")
     longest = ctx_bound
+    each = q_len[:len(entries)]
     if pad_to is not None:
-        # every row might belong to one request; if any request is short, every row might
-        short = int(q_len[:S - 1][q_len[:S - 1] < SHORT_PORTION].sum())
-        if short_bound is not None and short > short_bound:
-            raise ShortTokensOutgrown(f"{short} tokens of short requests in a step laid out for {short_bound}")
-        bound = n if short_bound is None else min(n, short_bound)
+        # every row might belong to one request
+        for limit, bound in (short_bounds or {}).items():
+            short = int(each[each < limit].sum())
+            if short > bound:
+                raise ShortTokensOutgrown(f"{short} tokens of requests that bring fewer than {limit} "
+                                          f"in a step laid out for {bound}")
         batch = StepBatch(packed, layout, n, S, max_blocks, len(logit_rows), n, longest,
-                          [e.seq_id for e in entries], short_tokens=bound if short > 0 else 0)
+                          [e.seq_id for e in entries], tokens_each=each, padded=True, short_bounds=short_bounds)
         batch.live_seqs = S - 1
         return batch
     return StepBatch(packed, layout, n, S, max_blocks, len(logit_rows), int(q_len.max()), longest,
-                     [e.seq_id for e in entries], short_tokens=int(q_len[q_len < SHORT_PORTION].sum()))
+                     [e.seq_id for e in entries], tokens_each=each)

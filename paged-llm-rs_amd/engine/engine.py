@@ -22,7 +22,7 @@ from ..config import GenerationConfig
 from ..errors import ConfigError, PagedLLMError
 from ..parts.model import DTYPES, load_model
 from ..sampling.sampler import Sampling
-from ..weights.safetensors_io import SafetensorsFile
+from ..weights.loader import CheckpointFiles
 from . import scheduler as sched
 from .step import StepRunner, require_gpu
 
@@ -38,7 +38,7 @@ def default_seed() -> int:
 
 def checkpoint_dtype(model_dir) -> str:
     """``auto``: whatever the checkpoint stores its embedding in (reference: model/mod.rs:175)."""
-    f = SafetensorsFile(Path(model_dir) / "model.safetensors")
+    f = CheckpointFiles(model_dir)
     try:
         for name in f.names():
             if name.endswith("embed_tokens.weight"):

@@ -44,12 +44,12 @@ def require_gpu(device) -> torch.device:
 
 
 def run_step(model, cache, entries, check_start: bool = True, pad_to: int | None = None,
-             short_bound: int | None = None, trace: dict | None = None) -> torch.Tensor:
+             short_bounds: dict | None = None, trace: dict | None = None) -> torch.Tensor:
     """32-bit logits [wanted places, vocabulary], in the order of the entries and of their ``want``.
     ``trace`` receives the named activations of the step (32-bit models; see ``DecoderModel.forward``)."""
     batch = build_batch(entries, cache.manager, len(cache.layout.groups), model.spec.vocab_size,
                         model.spec.max_positions, model.device, check_start=check_start, pad_to=pad_to,
-                        short_bound=short_bound)
+                        short_bounds=short_bounds)
     for e in entries:
         if e.fresh_state and e.state_slot >= 0:
             cache.clear_state_slot(e.state_slot)
@@ -247,9 +247,9 @@ class ShapeGraph:
     """A step of one shape (rows after padding, requests, wanted places), with block tables of
     ``widths`` pages a row and contexts up to ``ctx_bound``, captured."""
 
-    def __init__(self, model, cache, entries, widths: list, ctx_bound: int, rows: int, short_bound: int):
+    def __init__(self, model, cache, entries, widths: list, ctx_bound: int, rows: int, short_bounds: dict):
         self.model, self.cache, self.widths, self.ctx_bound, self.rows = model, cache, list(widths), ctx_bound, rows
-        self.short_bound = short_bound
+        self.short_bounds = dict(short_bounds)
         first = self._lay_out(entries)
         self.size = first.packed.numel()
         self.ring = _DescriptorRing(self.size)
@@ -258,7 +258,7 @@ class ShapeGraph:
         self.layout = first.layout
         self.batch = StepBatch(self.device_buf, first.layout, first.num_tokens, first.num_seqs, list(widths),
                                first.num_logit_rows, first.max_q_len, ctx_bound, [],
-                               short_tokens=first.short_tokens)
+                               tokens_each=first.tokens_each, padded=True, short_bounds=first.short_bounds)
         self.batch.live_seqs = first.live_seqs
         self.graph = None
         self.logits = None
@@ -266,7 +266,7 @@ class ShapeGraph:
     def _lay_out(self, entries):
         return build_batch(entries, self.cache.manager, len(self.cache.layout.groups), self.model.spec.vocab_size,
                            self.model.spec.max_positions, "cpu", widths=self.widths, ctx_bound=self.ctx_bound,
-                           pad_to=self.rows, short_bound=self.short_bound)
+                           pad_to=self.rows, short_bounds=self.short_bounds)
 
     def capture(self) -> None:
         # (over a step of idle rows, as in DecodeGraph.capture: the real step runs once, in the replay)
@@ -320,15 +320,18 @@ class StepRunner:
         graph from the second time on (while the requests' tables and contexts fit the capture)."""
         tokens = sum(len(e.tokens) for e in entries)
         rows = token_bucket(tokens) if self.pads and tokens <= SHAPE_GRAPH_MAX_TOKENS else None
-        # the tokens of requests that bring few, rounded up: the kernel for single tokens gets so many workgroups
-        short = sum(len(e.tokens) for e in entries if len(e.tokens) < kernels.SHORT_PORTION)
-        short_bound = None
+        # For every limit below which a mixer of the model runs a request through a kernel of its own: the
+        # tokens of such requests, rounded up (that kernel gets so many workgroups).  Part of the shape.
+        short_bounds = None
         if rows is not None:
-            short_bound = min(rows, _bucket(short, 16)) if short else 0
+            short_bounds = {}
+            for limit in getattr(self.model, "portion_limits", ()):
+                short = sum(len(e.tokens) for e in entries if len(e.tokens) < limit)
+                short_bounds[limit] = min(rows, _bucket(short, 16)) if short else 0
         if not self.use_graphs or rows is None or len(entries) > GRAPH_MAX_REQUESTS:
             self.eager_steps += 1
-            return StepOutput(run_step(self.model, self.cache, entries, pad_to=rows, short_bound=short_bound))
-        shape = (rows, len(entries), sum(len(e.want) for e in entries), short_bound)
+            return StepOutput(run_step(self.model, self.cache, entries, pad_to=rows, short_bounds=short_bounds))
+        shape = (rows, len(entries), sum(len(e.want) for e in entries), tuple(sorted(short_bounds.items())))
         known = shape in self._shapes
         graph = self._shapes.pop(shape, None)
         if not known:
@@ -336,7 +339,7 @@ class StepRunner:
             while len(self._shapes) > 256:
                 self._shapes.pop(next(iter(self._shapes)))
             self.eager_steps += 1
-            return StepOutput(run_step(self.model, self.cache, entries, pad_to=rows, short_bound=short_bound))
+            return StepOutput(run_step(self.model, self.cache, entries, pad_to=rows, short_bounds=short_bounds))
         for e in entries:
             if e.fresh_state and e.state_slot >= 0:
                 self.cache.clear_state_slot(e.state_slot)
@@ -350,7 +353,7 @@ class StepRunner:
                 pass                            # a request has outgrown the capture: a new one below
         widths = [_bucket(w + 1, 32) for w in self._widths_needed(entries)]
         longest = max(e.start + len(e.tokens) for e in entries)
-        graph = ShapeGraph(self.model, self.cache, entries, widths, context_bound(longest), rows, short_bound)
+        graph = ShapeGraph(self.model, self.cache, entries, widths, context_bound(longest), rows, short_bounds)
         out = graph.run(entries)
         self._shapes[shape] = graph
         live = [k for k, g in self._shapes.items() if g is not None]

@@ -609,17 +609,18 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nk
         return paged_attention_plain(qkv, qkv.shape[1], out, batch.positions, batch.seq_of, kv.block_table,
                                      kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window)
     stride = qkv.shape[1]
+    short_tokens = batch.tokens_of_short_requests(SHORT_PORTION)
     if batch.max_q_len >= SHORT_PORTION:
         # A few short requests beside a long portion ride along in the tiled kernel, a token tile each: their
         # workgroups run beside the portion's and finish sooner, which saves the other kernel's launch and
         # its merge.  (Counted by requests, which a step's shape fixes; the tokens of short ones it does not.)
-        all_tiled = (batch.short_tokens > 0 and batch.num_seqs * nq <= TILED_TAKES_SHORT_WORKGROUPS
+        all_tiled = (short_tokens > 0 and batch.num_seqs * nq <= TILED_TAKES_SHORT_WORKGROUPS
                      and not grouped_applies(nq, nkv, d, kv.block_size))   # (grouped, a token reads its keys once for all its heads)
         paged_attention_prefill(qkv, stride, out, batch.q_start, batch.q_len, batch.ctx_len, batch.max_q_len,
                                 kv.block_table, kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window,
                                 short_limit=0 if all_tiled else SHORT_PORTION, max_ctx=batch.max_ctx_len,
                                 live_seqs=getattr(batch, "live_seqs", None))
-        if batch.short_tokens == 0 or all_tiled:
+        if short_tokens == 0 or all_tiled:
             return out
     mixed = batch.max_q_len >= SHORT_PORTION
     if grouped_applies(nq, nkv, d, kv.block_size):
@@ -628,12 +629,12 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nk
                                        min(batch.max_q_len, SHORT_PORTION - 1), kv.block_table, kv.block_size,
                                        kv.k_pool, kv.v_pool, nq, nkv, d, scale, window,
                                        short_limit=SHORT_PORTION if mixed else 0, max_ctx=batch.max_ctx_len,
-                                       live_seqs=getattr(batch, "live_seqs", None), tokens=batch.short_tokens)
-    splits = decode_splits(batch.short_tokens, nq, nkv, batch.max_ctx_len, d)
+                                       live_seqs=getattr(batch, "live_seqs", None), tokens=short_tokens)
+    splits = decode_splits(short_tokens, nq, nkv, batch.max_ctx_len, d)
     return paged_attention_decode(qkv, stride, out, batch.positions, batch.seq_of, kv.block_table,
                                   kv.block_size, kv.k_pool, kv.v_pool, nq, nkv, d, scale, window, splits,
                                   q_len=batch.q_len if mixed else None, short_limit=SHORT_PORTION if mixed else 0,
-                                  live_seqs=getattr(batch, "live_seqs", None), short_rows=batch.short_tokens)
+                                  live_seqs=getattr(batch, "live_seqs", None), short_rows=short_tokens)
 
 
 def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, swiglu: bool = False,

@@ -72,6 +72,9 @@ class PagedAttention:
     def state_spec(self):
         return None
 
+    # requests that bring fewer tokens than this go to a kernel of their own, which a step sizes by their tokens
+    short_portion = kernels.SHORT_PORTION
+
     # forward takes a norm still to run in place of rows, and may add its result into ctx.residual
     fuses = True
     # ... and records named activations into ctx.trace

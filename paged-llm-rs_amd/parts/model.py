@@ -19,11 +19,22 @@ from ..weights.loader import ParamDecl, load_weights
 from . import attention, block, mlp, norm  # noqa: F401  (register the built-in parts)
 from .linear import Linear
 from .norm import PendingNorm
-from .registry import BLOCKS, NORMS, lookup, prefixed, scoped
+from .registry import BLOCKS, EMBED_TRANSFORMS, LOGIT_TRANSFORMS, NORMS, lookup, prefixed, scoped
 from .trace import ActivationTrace
 
 DTYPES = {"float32": torch.float32, "f32": torch.float32, "bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
           torch.float32: torch.float32, torch.bfloat16: torch.bfloat16}
+
+
+def _transforms(spec) -> list:
+    """(attribute, class) of the transforms the spec names: of the stream behind the embedding and of the logits."""
+    found = []
+    for key, registry, what in (("embed_transform", EMBED_TRANSFORMS, "embedding transform"),
+                                ("logit_transform", LOGIT_TRANSFORMS, "logit transform")):
+        kind = (spec.extra or {}).get(key)
+        if kind is not None:
+            found.append((key, lookup(registry, kind, what)))
+    return found
 
 
 def declare_parameters(spec) -> list:
@@ -37,6 +48,9 @@ def declare_parameters(spec) -> list:
     decls += prefixed(final.declare(spec.final_norm, spec.hidden_size), stem)
     # A tied checkpoint may still store the output projection; the stored tensor wins.
     decls.append(ParamDecl(spec.head_name, (spec.vocab_size, spec.hidden_size), "matrix", optional=True))
+    for _, cls in _transforms(spec):
+        if hasattr(cls, "declare"):
+            decls += list(cls.declare(spec))
     return decls
 
 
@@ -87,13 +101,23 @@ class DecoderModel:
         else:
             raise WeightError(f"no {spec.head_name}, and the config does not tie the embeddings")
         self.lm_head = Linear(head)
+        self.embed_transform = self.logit_transform = None
+        for key, cls in _transforms(spec):
+            setattr(self, key, cls(spec, params, dtype, self.device))
         for entry in spec.schedule:
             if not 0 <= entry.layer < len(self.blocks):
                 raise ConfigError(f"the schedule names layer {entry.layer} of {len(self.blocks)}")
             if entry.cache_from is not None and not 0 <= entry.cache_from < len(self.blocks):
                 raise ConfigError(f"the schedule reads the cache of layer {entry.cache_from} of {len(self.blocks)}")
         self.cache_layout = CacheLayout.from_blocks(self.blocks, spec.schedule)
-        self.graph_safe = all(getattr(b, "graph_safe", True) for b in self.blocks)
+        self.graph_safe = (all(getattr(b, "graph_safe", True) for b in self.blocks)
+                           and getattr(self.embed_transform, "graph_safe", True)
+                           and getattr(self.logit_transform, "graph_safe", True))
+        # Mixers that hand requests of few tokens to a kernel of their own say from how many tokens on a
+        # request counts as a long portion; a step reports the tokens of the shorter ones for each such limit.
+        self.portion_limits = tuple(sorted({int(limit) for b in self.blocks
+                                            for limit in [getattr(getattr(b, "mixer", None), "short_portion", None)]
+                                            if limit}))
 
     # -- the forward pass of one step -------------------------------------------------
 
@@ -111,6 +135,8 @@ class DecoderModel:
                                        "most of them are stages inside kernels and never written")
             top = ActivationTrace(trace)
         resid = kernels.embed(batch.token_ids, self.embed_tokens)
+        if self.embed_transform is not None:
+            resid = self.embed_transform(resid, batch)
         if top is not None:
             top.record(self.spec.embed_name.rsplit(".", 1)[0] + ".out", resid)
         delta = None
@@ -139,6 +165,8 @@ class DecoderModel:
                 normed = normed.materialize()
             top.record(self.spec.final_norm_name.rsplit(".", 1)[0] + ".out", normed)
         logits = self.lm_head.forward(normed, out_dtype=torch.float32)
+        if self.logit_transform is not None:
+            logits = self.logit_transform(logits, batch)
         if top is not None:
             top.record(self.spec.head_name.rsplit(".", 1)[0] + ".out", logits)
             top.record("logits", logits)
@@ -157,5 +185,5 @@ def load_model(model_dir, dtype="bfloat16", device="cuda:0"):
     model_dir = Path(model_dir)
     config = load_config(model_dir)
     spec = config.model_spec()
-    params = load_weights(model_dir, declare_parameters(spec), DTYPES[dtype], device)
+    params = load_weights(model_dir, declare_parameters(spec), DTYPES[dtype], device, ignored=spec.ignored_tensors)
     return config, DecoderModel(spec, params, DTYPES[dtype], device)

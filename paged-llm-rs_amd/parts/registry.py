@@ -22,6 +22,12 @@ position      ``__init__(spec, device)`` giving ``dim`` (how many elements of a 
 block         ``declare(layer_spec, hidden)``; ``__init__(layer_spec, hidden, params, dtype,
               device, shared)``; ``forward(resid, delta, ctx) -> delta`` where the returned
               delta is the output not yet added to the residual stream.
+transform     of the stream behind the embedding (``register_embed_transform``) or of the logits
+              (``register_logit_transform``), named by ``ModelSpec.extra["embed_transform"]`` /
+              ``["logit_transform"]``: optional ``declare(spec) -> [ParamDecl]`` (checkpoint names);
+              ``__init__(spec, params, dtype, device)`` (``params``: all tensors by checkpoint name);
+              ``__call__(x, batch) -> x``: the 32-bit stream [rows, hidden] (padding rows have
+              position -1), or the 32-bit logits [wanted rows, vocabulary]; it may work in place.
 """
 
 from __future__ import annotations
@@ -33,6 +39,8 @@ FEED_FORWARDS: dict = {}
 NORMS: dict = {}
 BLOCKS: dict = {}
 POSITIONS: dict = {}
+EMBED_TRANSFORMS: dict = {}
+LOGIT_TRANSFORMS: dict = {}
 
 
 def register_mixer(kind: str, cls) -> None:
@@ -53,6 +61,14 @@ def register_block(kind: str, cls) -> None:
 
 def register_position(kind: str, cls) -> None:
     POSITIONS[kind] = cls
+
+
+def register_embed_transform(kind: str, cls) -> None:
+    EMBED_TRANSFORMS[kind] = cls
+
+
+def register_logit_transform(kind: str, cls) -> None:
+    LOGIT_TRANSFORMS[kind] = cls
 
 
 def lookup(registry: dict, kind: str, what: str):

@@ -148,6 +148,9 @@ LAYERS_WIDE = {
 # tiles in a loop (few rows) or goes to the library (many), which no smaller vocabulary shows.
 LAYERS_0P6B_REAL_VOCAB = dict(LAYERS_0P6B, vocab_size=151936)
 
+# ... and with room for contexts beyond four thousand tokens.
+LAYERS_0P6B_LONG = dict(LAYERS_0P6B, max_position_embeddings=8192)
+
 TINY_INIT = {
     "A": dict(config=TINY_A, seed=0, std=0.02, gain_std=0.1),
     "B": dict(config=TINY_B, seed=1, std=0.05, gain_std=0.2),
@@ -155,6 +158,7 @@ TINY_INIT = {
     "D": dict(config=LAYERS_0P6B, seed=3, std=0.02, gain_std=0.1),
     "E": dict(config=LAYERS_WIDE, seed=4, std=0.02, gain_std=0.1),
     "V": dict(config=LAYERS_0P6B_REAL_VOCAB, seed=5, std=0.02, gain_std=0.1),
+    "L": dict(config=LAYERS_0P6B_LONG, seed=6, std=0.02, gain_std=0.1),
 }
 
 

@@ -53,8 +53,8 @@ def apply_rope(x: torch.Tensor, positions: torch.Tensor, theta: float) -> torch.
     """out = x*cos + rotate_half(x)*sin at each token's own position
     (model/rope.rs:95-99).  ``x`` is [seq, heads, head_dim]."""
     cos, sin = rope_tables(x.shape[-1], positions, theta)
-    cos = cos[:, None, :].to(x.dtype)
-    sin = sin[:, None, :].to(x.dtype)
+    cos = cos[:, None, :].to(x)
+    sin = sin[:, None, :].to(x)
     return x * cos + rotate_half(x) * sin
 
 
@@ -95,7 +95,7 @@ def attention_core(q, k, v, scale: float, window: int | None = None) -> torch.Te
     """softmax(q k^T * scale + mask) v per head (model/attention.rs:99-104).
     q [sq, heads, d]; k, v [sk, heads, d]; the queries are the last sq positions."""
     scores = torch.einsum("qhd,khd->hqk", q, k) * scale
-    scores = scores + causal_mask(q.shape[0], k.shape[0], window).to(scores.dtype)[None]
+    scores = scores + causal_mask(q.shape[0], k.shape[0], window).to(scores)[None]
     weights = softmax_last(scores)
     return torch.einsum("hqk,khd->qhd", weights, v)
 
@@ -196,12 +196,14 @@ def lm_head_weight(w: dict, cfg: dict) -> torch.Tensor:
 
 
 def forward(weights: dict, cfg: dict, tokens, *, offset: int = 0, trace: dict | None = None,
-            dtype=torch.float64, window: int | None = None) -> torch.Tensor:
+            dtype=torch.float64, window: int | None = None, device="cpu") -> torch.Tensor:
     """Logits [seq, vocab] for one whole sequence, no cache
     (model/mod.rs:271-303): embedding gather without scaling, every block,
-    final norm on all positions, output projection."""
-    w = {k: v.to(dtype) for k, v in weights.items()}
-    ids = torch.as_tensor(list(tokens), dtype=torch.long)
+    final norm on all positions, output projection.  ``device``: where torch does the
+    arithmetic (a sequence of thousands of tokens takes a minute on the CPU); the result
+    comes back to the CPU."""
+    w = {k: v.to(device=device, dtype=dtype) for k, v in weights.items()}
+    ids = torch.as_tensor(list(tokens), dtype=torch.long, device=device)
     if ids.numel() == 0:
         raise ValueError("cannot run a forward pass on no tokens")
     positions = torch.arange(ids.numel()) + offset
@@ -214,7 +216,7 @@ def forward(weights: dict, cfg: dict, tokens, *, offset: int = 0, trace: dict | 
     logits = x @ lm_head_weight(w, cfg).T
     _record(trace, "lm_head.out", logits)
     _record(trace, "logits", logits)
-    return logits
+    return logits.cpu()
 
 
 def greedy_generate(weights: dict, cfg: dict, prompt, steps: int) -> list[int]:

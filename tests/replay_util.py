@@ -17,10 +17,10 @@ def make_prompts(vocab: int, lengths, seed: int) -> dict:
     return {f"r{i}": [rng.randrange(vocab) for _ in range(n)] for i, n in enumerate(lengths)}
 
 
-def plain_logits(model_dir, prompts: dict) -> dict:
+def plain_logits(model_dir, prompts: dict, device="cpu") -> dict:
     """name -> float64 logits [len, vocab] of the whole sequence, no cache."""
     cfg, weights = load_plain(model_dir)
-    return {name: plain.forward(weights, cfg, toks) for name, toks in prompts.items()}
+    return {name: plain.forward(weights, cfg, toks, device=device) for name, toks in prompts.items()}
 
 
 # --- schedules: lists of steps {"step", "entries", "end"} ------------------------------------

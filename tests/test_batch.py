@@ -41,7 +41,7 @@ def test_a_step_without_padding_reports_what_it_holds():
     m = manager()
     batch = build_batch(requests(m, [5, 1, 20], written=[0, 9, 3]), m, 1, 100, 0, "cpu")
     assert (batch.num_tokens, batch.num_seqs, batch.live_seqs, batch.num_logit_rows) == (26, 3, 3, 3)
-    assert batch.max_q_len == 20 and batch.max_ctx_len == 1024 and batch.short_tokens == 6
+    assert batch.max_q_len == 20 and batch.max_ctx_len == 1024 and batch.tokens_of_short_requests(16) == 6
     assert piece(batch, "positions").tolist() == list(range(5)) + [9] + list(range(3, 23))
     assert piece(batch, "q_start").tolist() == [0, 5, 6] and piece(batch, "ctx_len").tolist() == [5, 10, 23]
     assert piece(batch, "logit_rows").tolist() == [4, 5, 25]
@@ -52,21 +52,21 @@ def test_padding_adds_a_request_that_holds_nothing_and_bounds_instead_of_counts(
     entries = requests(m, [5, 20], written=[0, 3])
     batch = build_batch(entries, m, 1, 100, 0, "cpu", pad_to=32)
     assert (batch.num_tokens, batch.num_seqs, batch.live_seqs) == (32, 3, 2)
-    assert batch.max_q_len == 32 and batch.short_tokens == 32          # a short request is there: every row might be short
+    assert batch.max_q_len == 32 and batch.tokens_of_short_requests(16) == 32          # a short request is there: every row might be short
     assert piece(batch, "positions")[25:].tolist() == [-1] * 7 and piece(batch, "seq_of")[25:].tolist() == [2] * 7
     assert piece(batch, "q_start").tolist() == [0, 5, 25] and piece(batch, "q_len").tolist() == [5, 20, 7]
     assert piece(batch, "ctx_len").tolist() == [5, 23, 0] and piece(batch, "state_slots")[2] == -1
     table = piece(batch, "block_table_0").reshape(3, -1)
     assert (table[2] == -1).all() and table[1, 0] >= 0
     # told how many tokens the short requests bring at most, the batch reports that bound; more of them are refused
-    bounded = build_batch(entries, m, 1, 100, 0, "cpu", pad_to=32, short_bound=16)
-    assert bounded.short_tokens == 16 and bounded.max_q_len == 32
+    bounded = build_batch(entries, m, 1, 100, 0, "cpu", pad_to=32, short_bounds={16: 16})
+    assert bounded.tokens_of_short_requests(16) == 16 and bounded.max_q_len == 32
     with pytest.raises(ShortTokensOutgrown):
-        build_batch(entries, m, 1, 100, 0, "cpu", pad_to=32, short_bound=4)
+        build_batch(entries, m, 1, 100, 0, "cpu", pad_to=32, short_bounds={16: 4})
     # the same step without short requests reports no short rows; a full bucket has a request of no rows
     m2 = manager()
     full = build_batch(requests(m2, [16, 16]), m2, 1, 100, 0, "cpu", pad_to=32)
-    assert full.short_tokens == 0 and piece(full, "q_len").tolist() == [16, 16, 0]
+    assert full.tokens_of_short_requests(16) == 0 and piece(full, "q_len").tolist() == [16, 16, 0]
     with pytest.raises(ConfigError):
         build_batch(requests(manager(), [40]), manager(), 1, 100, 0, "cpu", pad_to=32)
 
@@ -87,4 +87,4 @@ def test_steps_of_one_shape_have_one_layout():
     one = build_batch(requests(a, [40, 1], written=[0, 7]), a, 1, 100, 0, "cpu", widths=[32], ctx_bound=1024, pad_to=64)
     two = build_batch(requests(b, [13, 30], written=[50, 0]), b, 1, 100, 0, "cpu", widths=[32], ctx_bound=1024, pad_to=64)
     assert one.layout == two.layout and one.packed.numel() == two.packed.numel()
-    assert (one.max_q_len, one.short_tokens, one.num_seqs) == (two.max_q_len, two.short_tokens, two.num_seqs)
+    assert (one.max_q_len, one.tokens_of_short_requests(16), one.num_seqs) == (two.max_q_len, two.tokens_of_short_requests(16), two.num_seqs)

@@ -216,3 +216,177 @@ def test_check_declared_passes_optional():
     check_declared(decls, {"a": (2, 3), "b": (4,)}, "x")
     with pytest.raises(WeightError):
         check_declared(decls, {"b": (4,)}, "x")
+
+
+# ---- sharded checkpoints -------------------------------------------------------------------------------
+
+def shard_folder(tmp_path, config, seed, pieces=2, dtype="float32"):
+    """A model folder whose tensors lie in ``pieces`` files behind model.safetensors.index.json,
+    beside the same model in one file; returns (sharded folder, whole folder, shard names)."""
+    whole = write_random_model(tmp_path / "whole", config, seed=seed, dtype=dtype)
+    f = SafetensorsFile(whole / "model.safetensors")
+    names = f.names()
+    sharded = tmp_path / "sharded"
+    sharded.mkdir()
+    (sharded / "config.json").write_text((whole / "config.json").read_text())
+    weight_map, shards = {}, []
+    for i in range(pieces):
+        shard = f"model-{i + 1:05d}-of-{pieces:05d}.safetensors"
+        mine = names[i::pieces]                   # interleaved, so neighbouring tensors lie in different files
+        write_safetensors(sharded / shard, {n: f.tensor(n).clone() for n in mine})
+        weight_map.update({n: shard for n in mine})
+        shards.append(shard)
+    (sharded / "model.safetensors.index.json").write_text(json.dumps({"metadata": {}, "weight_map": weight_map}))
+    return sharded, whole, shards
+
+
+def test_a_checkpoint_in_shards_loads_like_the_same_checkpoint_in_one_file(tmp_path):
+    """The reference opens one file (weights.rs:24-32); folders of the larger models of the family
+    carry an index and shards."""
+    sharded, whole, shards = shard_folder(tmp_path, TINY_B, seed=3, pieces=3)
+    spec = load_config(sharded).model_spec()
+    a = load_weights(sharded, declare_parameters(spec), torch.float32, "cpu")
+    b = load_weights(whole, declare_parameters(spec), torch.float32, "cpu")
+    assert a.keys() == b.keys() and len(a) > 30
+    for name in a:
+        assert torch.equal(a[name], b[name]), name
+    from paged_llm_rs_amd.engine.engine import checkpoint_dtype
+
+    assert checkpoint_dtype(sharded) == "float32"
+
+
+def test_a_missing_shard_is_an_io_error_that_names_it(tmp_path):
+    from paged_llm_rs_amd.errors import IoError
+
+    sharded, _, shards = shard_folder(tmp_path, TINY_A, seed=0)
+    (sharded / shards[1]).unlink()
+    spec = load_config(sharded).model_spec()
+    with pytest.raises(IoError, match=shards[1]):
+        load_weights(sharded, declare_parameters(spec), torch.float32, "cpu")
+    with pytest.raises(IoError, match="model.safetensors"):         # neither one file nor an index
+        load_weights(tmp_path, declare_parameters(spec), torch.float32, "cpu")
+
+
+def test_the_one_report_covers_all_shards(tmp_path):
+    sharded, _, shards = shard_folder(tmp_path, TINY_B, seed=1)
+    index = json.loads((sharded / "model.safetensors.index.json").read_text())
+    # a tensor of the wrong shape in one shard, an unknown one in the other, a missing one in the index
+    first = SafetensorsFile(sharded / shards[0])
+    tensors = {n: first.tensor(n).clone() for n in first.names()}
+    victim = next(n for n in tensors if n.endswith("k_norm.weight"))
+    tensors[victim] = torch.zeros(96)
+    write_safetensors(sharded / shards[0], tensors)
+    second = SafetensorsFile(sharded / shards[1])
+    tensors = {n: second.tensor(n).clone() for n in second.names()}
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(16)
+    gone = next(n for n in tensors if n.endswith("down_proj.weight"))
+    del tensors[gone]
+    write_safetensors(sharded / shards[1], tensors)
+    index["weight_map"]["model.layers.0.self_attn.rotary_emb.inv_freq"] = shards[1]
+    del index["weight_map"][gone]
+    (sharded / "model.safetensors.index.json").write_text(json.dumps(index))
+    spec = load_config(sharded).model_spec()
+    with pytest.raises(WeightError) as e:
+        load_weights(sharded, declare_parameters(spec), torch.float32, "cpu")
+    text = str(e.value)
+    assert "index.json" in text and f"missing (1): {gone}" in text
+    assert "unexpected (1)" in text and "inv_freq" in text
+    assert f"wrong shape (1): {victim} has shape [96], expected [32]" in text
+    # an index that names a tensor its shard does not hold is refused as such
+    index["weight_map"][gone] = shards[1]
+    (sharded / "model.safetensors.index.json").write_text(json.dumps(index))
+    with pytest.raises(WeightError, match="do not hold"):
+        load_weights(sharded, declare_parameters(spec), torch.float32, "cpu")
+
+
+# ---- tensors a family's checkpoints carry and the model does not use ------------------------------------
+
+def test_tensors_that_a_spec_says_to_ignore_are_not_unexpected(tmp_path):
+    import dataclasses
+
+    d = write_random_model(tmp_path / "m", TINY_A, seed=0, dtype="float32")
+    f = SafetensorsFile(d / "model.safetensors")
+    tensors = {n: f.tensor(n).clone() for n in f.names()}
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    tensors["model.layers.1.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    tensors["model.stray.weight"] = torch.zeros(3)
+    write_safetensors(d / "model.safetensors", tensors)
+    spec = load_config(d).model_spec()
+    with pytest.raises(WeightError, match=r"unexpected \(3\)"):
+        load_weights(d, declare_parameters(spec), torch.float32, "cpu", ignored=spec.ignored_tensors)
+    lenient = dataclasses.replace(spec, ignored_tensors=("*.rotary_emb.inv_freq",))
+    with pytest.raises(WeightError, match=r"unexpected \(1\): model.stray.weight"):
+        load_weights(d, declare_parameters(lenient), torch.float32, "cpu", ignored=lenient.ignored_tensors)
+    lenient = dataclasses.replace(spec, ignored_tensors=("*.rotary_emb.inv_freq", "model.stray.*"))
+    w = load_weights(d, declare_parameters(lenient), torch.float32, "cpu", ignored=lenient.ignored_tensors)
+    assert "model.stray.weight" not in w and not any("inv_freq" in n for n in w)
+
+
+# ---- the reference's own checkpoint through the loader ----------------------------------------------------
+
+def test_the_references_own_checkpoint_through_config_declaration_and_shape_check():
+    """The part of "the engine on the reference's checkpoint" that needs no GPU: its config.json (rotary base
+    nested under rope_parameters, keys the engine does not read, a width of 24 with heads of 16:
+    tests/fixtures/tiny/config.json:1-37) through the registry, the declaration of every tensor, the one
+    check against the file and the model's construction."""
+    from conftest import REFERENCE_FIXTURE
+    from paged_llm_rs_amd.parts.model import load_model
+
+    if not (REFERENCE_FIXTURE / "model.safetensors").exists():
+        pytest.skip("the reference's fixture is not on this machine")
+    config, model = load_model(REFERENCE_FIXTURE, "float32", "cpu")
+    assert isinstance(config, Qwen3Config) and config.rope_theta == 1e6
+    assert (config.hidden_size, config.num_attention_heads, config.num_key_value_heads, config.head_dim) == (24, 4, 2, 16)
+    assert not config.tie_word_embeddings and model.lm_head.weight.shape == (128, 24)
+    assert len(model.blocks) == 2 and model.embed_tokens.dtype == torch.float32
+    f = SafetensorsFile(REFERENCE_FIXTURE / "model.safetensors")
+    declared = {d.name for d in declare_parameters(config.model_spec())}
+    assert set(f.names()) == declared                      # 2 + 2 * 11 tensors, none optional left out
+    attention = model.blocks[1].mixer
+    assert torch.equal(attention.q_gain, f.tensor("model.layers.1.self_attn.q_norm.weight"))
+    assert torch.equal(attention.qkv_proj.weight[64:96], f.tensor("model.layers.1.self_attn.k_proj.weight"))
+
+
+# ---- what a spec names beside the layers ------------------------------------------------------------------
+
+def test_transforms_named_by_a_spec_are_declared_and_built(tmp_path):
+    import dataclasses
+
+    from paged_llm_rs_amd.parts import register_embed_transform, register_logit_transform
+    from paged_llm_rs_amd.parts.model import DecoderModel
+
+    class Shift:
+        @staticmethod
+        def declare(spec):
+            return [ParamDecl("model.shift.weight", (spec.hidden_size,), "matrix")]
+
+        def __init__(self, spec, params, dtype, device):
+            self.by = params["model.shift.weight"]
+
+        def __call__(self, x, batch):
+            return x + self.by
+
+    class Halve:
+        graph_safe = False
+
+        def __init__(self, spec, params, dtype, device):
+            self.factor = spec.extra["factor"]
+
+        def __call__(self, logits, batch):
+            return logits * self.factor
+
+    register_embed_transform("toy_shift", Shift)
+    register_logit_transform("toy_halve", Halve)
+    spec = load_config(TINY_A).model_spec()
+    assert not any(d.name == "model.shift.weight" for d in declare_parameters(spec))
+    plain = DecoderModel(spec, {d.name: torch.zeros(d.shape) for d in declare_parameters(spec)}, torch.float32, "cpu")
+    assert plain.embed_transform is None and plain.logit_transform is None and plain.graph_safe
+    named = dataclasses.replace(spec, extra={"embed_transform": "toy_shift", "logit_transform": "toy_halve", "factor": 0.5})
+    decls = declare_parameters(named)
+    assert any(d.name == "model.shift.weight" and d.shape == (64,) for d in decls)
+    model = DecoderModel(named, {d.name: torch.ones(d.shape) for d in decls}, torch.float32, "cpu")
+    assert isinstance(model.embed_transform, Shift) and model.logit_transform.factor == 0.5
+    assert not model.graph_safe                      # a transform that cannot be captured keeps the model's steps eager
+    assert model.portion_limits == (16,)             # what the attention mixers report, not a constant of the engine
+    with pytest.raises(UnsupportedError, match="toy_nothing"):
+        declare_parameters(dataclasses.replace(spec, extra={"logit_transform": "toy_nothing"}))

@@ -147,6 +147,30 @@ def test_sampling_with_a_seed_repeats_and_stop_tokens_end_a_request(model_dirs, 
     assert [x["tokens"] for x in g] == [x["tokens"] for x in k]
 
 
+@pytest.mark.parametrize("sampler", ["device", "host"])
+def test_sampling_with_cuts_over_a_vocabulary_of_thousands(model_dirs, sampler):
+    """Several requests at once, each with its own generator, temperature, top-k and top-p over 4,099 logits:
+    the plain sampler on the plain model's logits picks the tokens the engine picked (sampler.rs:113-183)."""
+    from paged_llm_rs_amd import Engine
+
+    d = model_dirs("D", "float32")
+    vocab = TINY_INIT["D"]["config"]["vocab_size"]
+    prompts = list(ru.make_prompts(vocab, [5, 23, 12], seed=8).values())
+    cfg, weights = load_plain(d)
+    engine = Engine(d, dtype="f32", block_size=16, num_blocks=32, max_batch=4, chunk=16, sampler=sampler)
+    for temperature, top_k, top_p in ((0.9, 40, 0.9), (1.3, None, 0.7), (0.7, 300, None)):
+        out = engine.generate(prompts, max_tokens=8, temperature=temperature, top_k=top_k, top_p=top_p, seed=77,
+                              stop_tokens=[])
+        assert len({tuple(o["tokens"]) for o in out}) == 3
+        for i, (prompt, result) in enumerate(zip(prompts, out)):
+            rng = plain.SplitMix64(77 + i)
+            tokens = list(prompt)
+            for produced in result["tokens"]:
+                logits = plain.forward(weights, cfg, tokens)[-1].float().numpy()
+                assert plain.sample(logits, temperature, top_k, top_p, rng) == produced, (temperature, top_k, top_p, i)
+                tokens.append(produced)
+
+
 def test_the_command_line(model_dirs, tmp_path):
     d = model_dirs("A", "float32")
     proc = subprocess.run(

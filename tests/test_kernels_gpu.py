@@ -1295,3 +1295,60 @@ def test_the_kernels_beside_their_plain_cpp_oracles(dtype):
             out = torch.zeros(3, nq * d, dtype=dtype, device=DEV)
             kernels.paged_attention_prefill(q3, stride, out, start, one, lens, 1, bt, bs, k_pool, v_pool, nq, nkv, d, scale, window)
             assert rel(out, want3) < tol, f"tiled kernel, window {window}"
+
+
+@pytest.mark.parametrize("requests,splits,window", [(70, 2, 0), (70, 8, 48), (5, 8, 48), (5, 1, 0), (40, 16, 20)])
+def test_the_single_token_kernel_that_prepares_its_keys_beside_the_oracles(requests, splits, window):
+    """One token a request through the kernel that also normalises and rotates q and the new k and writes k and v
+    into the pages, against the plain C++ oracles of each of those stages: with few workgroups (eight keys a lane
+    group in flight) and with many (four), with a window whose newest key is the token's own, with more shares
+    than the window has rounds of keys (the trailing ones are empty), and with one key at the window's far edge
+    (or the context's first) that carries nearly all the weight, so that a dropped edge cannot hide."""
+    from paged_llm_rs_amd import kernels, oracle
+
+    nq, nkv, d, bs, rot, theta, eps = 4, 2, 64, 16, 64, 10000.0, 1e-6
+    g = nq // nkv
+    gen = torch.Generator().manual_seed(requests * 100 + splits)
+    ctx = [200] + [int(c) for c in torch.randint(1, 230, (requests - 1,), generator=gen)]
+    bt, k_pool, v_pool, _, _ = build_paged(nkv, d, bs, ctx, torch.bfloat16, seed=requests + splits)
+    n = requests + 1                                    # and a padding row
+    positions = [c - 1 for c in ctx] + [-1]
+    seq_of = list(range(requests)) + [0]
+    stride = (nq + 2 * nkv) * d
+    qkv = torch.randn(n, stride, generator=gen).to(torch.bfloat16)
+    q_gain, k_gain = 1 + 0.2 * torch.randn(d, generator=gen), 1 + 0.2 * torch.randn(d, generator=gen)
+    angle = torch.arange(256, dtype=torch.float64)[:, None] * theta ** (-torch.arange(rot // 2, dtype=torch.float64) * 2 / rot)
+    cos, sin = angle.cos().float().to(DEV), angle.sin().float().to(DEV)
+    # what the stages before attention make of the rows, by their oracles, rounded as the kernel keeps them
+    live = list(range(requests))
+    heads = qkv[live].float().view(requests, nq + 2 * nkv, d)
+    pos_live = positions[:requests]
+    q_want = oracle.rotate(oracle.rms_norm(heads[:, :nq].reshape(-1, d), q_gain, eps).view(requests, nq, d), pos_live, rot, theta)
+    k_want = oracle.rotate(oracle.rms_norm(heads[:, nq:nq + nkv].reshape(-1, d), k_gain, eps).view(requests, nkv, d), pos_live, rot, theta)
+    q_want, k_want = q_want.to(torch.bfloat16), k_want.to(torch.bfloat16)
+    # the far key of request 0: the oldest key its token sees answers the first head of every group
+    far = max(0, 199 - window + 1) if window else 0
+    far_slot = int(bt[0, far // bs]) * bs + far % bs
+    for kvh in range(nkv):
+        k_pool[far_slot, kvh * d:(kvh + 1) * d] = (q_want[0, kvh * g].float() * 4).to(torch.bfloat16).to(DEV)
+    kp, vp = k_pool.cpu().clone(), v_pool.cpu().clone()
+    for t in range(requests):
+        slot = int(bt[t, pos_live[t] // bs]) * bs + pos_live[t] % bs
+        kp[slot] = k_want[t].reshape(-1)
+        vp[slot] = heads[t, nq + nkv:].reshape(-1).to(torch.bfloat16)
+    scale = 1 / math.sqrt(d)
+    want = oracle.paged_attention(q_want.reshape(requests, nq * d), kp, vp, bt, pos_live, live, nq, nkv, d, bs, scale, window)
+    as_i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    out = torch.full((n, nq * d), 7.0, dtype=torch.bfloat16, device=DEV)
+    fuse = kernels.QkFusion(q_gain.to(DEV), k_gain.to(DEV), eps, cos, sin, rot, True)
+    kernels.paged_attention_decode(qkv.to(DEV), stride, out, as_i32(positions), as_i32(seq_of), bt, bs, k_pool, v_pool,
+                                   nq, nkv, d, scale, window, splits=splits, fuse=fuse)
+    for t in range(requests):
+        err = rel(out[t], want[t])
+        assert err < 1.2e-2, f"request {t} (context {ctx[t]}), {splits} shares, window {window}: {err:.3e}"
+        slot = int(bt[t, pos_live[t] // bs]) * bs + pos_live[t] % bs
+        assert rel(k_pool[slot], kp[slot]) < 1e-2 and torch.equal(v_pool[slot].cpu(), vp[slot])
+    for kvh in range(nkv):
+        found = rel(out[0].view(nq, d)[kvh * g], v_pool[far_slot].view(nkv, d)[kvh])
+        assert found < 0.05, f"the key at {far}, the oldest that position 199 sees with window {window}: {found:.3e}"
+    assert bool((out[-1] == 7.0).all()), "a padding row is not written"
