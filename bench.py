@@ -140,7 +140,7 @@ class Workbench:
     measurements that are taken on it."""
 
     def __init__(self, shape: str, layers: int, device, largest_batch: int, steps: int, graphs: bool = True,
-                 context: int | None = None, prefill_room: bool = True):
+                 context: int | None = None, prefill_room: bool = True, most_tokens: int = 0):
         import torch
 
         from paged_llm_rs_amd import write_random_model
@@ -165,7 +165,9 @@ class Workbench:
         say("loaded")
         self.weight_bytes, self.layer_flops, self.head_flops = model_bytes_and_flops(self.cfg, 2)
         self.kv_token = kv_bytes_per_token(self.cfg, 2)
-        pages = (largest_batch * (self.context + steps + 64) + (PREFILL_TOKENS + 64 if prefill_room else 0)) // BLOCK_SIZE + largest_batch
+        # (most_tokens: what the largest of the points keeps in the cache at once, where that is more)
+        tokens = max(largest_batch * (self.context + steps + 64), most_tokens)
+        pages = (tokens + (PREFILL_TOKENS + 64 if prefill_room else 0)) // BLOCK_SIZE + largest_batch
         self.cache = PagedCache(self.model.cache_layout, BLOCK_SIZE, pages, torch.bfloat16, device, max_seqs=largest_batch + 1)
         self.runner = StepRunner(self.model, self.cache, graphs=graphs)
 
@@ -346,8 +348,10 @@ def main() -> int:
     FULL_LAYERS = CONFIG["num_hidden_layers"]
     if args.layers is None:
         args.layers = default_layers
+    long_points = args.shape == "0.6b" and not args.skip_points and args.only is None
     bench = Workbench(args.shape, args.layers, device, largest_batch=max(64, args.batch),
-                      steps=args.steps + args.warmup, graphs=not args.no_graphs)
+                      steps=args.steps + args.warmup, graphs=not args.no_graphs,
+                      most_tokens=max(64, args.batch) * (LONG_CONTEXT + 128) if long_points else 0)
     cfg, model, cache, runner, folder, tmp = bench.cfg, bench.model, bench.cache, bench.runner, bench.folder, bench.tmp
     weight_bytes, layer_flops, head_flops, kv_token = bench.weight_bytes, bench.layer_flops, bench.head_flops, bench.kv_token
     decode_point = bench.decode_point
@@ -486,6 +490,10 @@ def main() -> int:
             s_long, v_long, bytes_long = decode_point(args.batch, 20, 5, context=LONG_CONTEXT)
             points[f"decode_b{args.batch}_ctx{LONG_CONTEXT}"] = round(v_long, 1)
             points[f"decode_b{args.batch}_ctx{LONG_CONTEXT}_frac_hbm"] = round(bytes_long / s_long / HBM_PEAK, 4)
+            say(f"decode, batch 64, context {LONG_CONTEXT}")
+            s_long, v_long, bytes_long = decode_point(64, 12, 4, context=LONG_CONTEXT)
+            points[f"decode_b64_ctx{LONG_CONTEXT}"] = round(v_long, 1)
+            points[f"decode_b64_ctx{LONG_CONTEXT}_frac_hbm"] = round(bytes_long / s_long / HBM_PEAK, 4)
         line["points"] = points
         line["prefill"] = prefill_point()
         if args.shape == "0.6b" and not args.no_other_shapes:
@@ -494,15 +502,23 @@ def main() -> int:
             bench.close()
             other = Workbench("8b", OTHER_SHAPE_LAYERS["8b"], device, largest_batch=MIXED_DECODES + 1, steps=8)
             mixed = other.mixed_point(30, 10)       # (ten untimed steps: the chip has idled while the model was made)
-            other.close()
-            points["mixed_8b_tok_s"] = mixed["tokens_per_s"]
+            # The times of these points are of steps over a few layers (and the whole projection onto the
+            # vocabulary); they are no model's rate.  What carries over to the whole model is the share of
+            # the peak that binds: for this step the memory (63 contexts of keys and values beside the
+            # weights outweigh the 575 rows of arithmetic), for the decode steps the memory as well.
             points["mixed_8b_ms"] = mixed["ms"]
+            points["mixed_8b_frac_hbm"] = mixed["frac_hbm"]
             points["mixed_8b_frac_mfma"] = mixed["frac_mfma"]
+            points["mixed_8b_bound"] = "hbm" if mixed["hbm_floor_ms"] >= mixed["mfma_floor_ms"] else "mfma"
+            say("decode, batch 8, of the 8B shape")
+            s8, _, bytes8 = other.decode_point(8, 20, 6)
+            other.close()
+            points["decode_8b_b8_ms"] = round(s8 * 1e3, 3)
+            points["decode_8b_b8_frac_hbm"] = round(bytes8 / s8 / HBM_PEAK, 4)
             other = Workbench("32b", OTHER_SHAPE_LAYERS["32b"], device, largest_batch=64, steps=20, prefill_room=False)
             say("decode, batch 64, of the 32B shape")
             s32, v32, bytes32 = other.decode_point(64, 12, 6)
             other.close()
-            points["decode_32b_b64_tok_s"] = round(v32, 1)
             points["decode_32b_b64_ms"] = round(s32 * 1e3, 3)
             points["decode_32b_b64_frac_hbm"] = round(bytes32 / s32 / HBM_PEAK, 4)
             line["config"].update({"layers_8b": OTHER_SHAPE_LAYERS["8b"], "layers_8b_full": SHAPES["8b"][1]["num_hidden_layers"],
