@@ -23,6 +23,12 @@
 //   EPI_ADD     the 32-bit residual stream takes the result: resid[r, c] += result.  Every
 //               element has one owner, so the sum does not depend on timing.
 //
+// The norm handed forward.  A product that adds into the stream (EPI_ADD) owns whole 16-column stripes of
+// the updated stream, so it can leave the next norm's work behind: bf16(stream * gain) for its stripe, and
+// for every row the sum of squares over the stripe.  The product behind that norm then loads bfloat16 rows
+// (half the bytes of the stream, nothing to convert or square), adds the stripes' sums in a fixed order and
+// scales its result by 1 / sqrt(sum / K + eps), which is where PRO_NORM applies the statistic as well.
+//
 // With more than 16 rows a wave's registers fill with x (every 16 rows are another operand a K step), and
 // little of w is on its way at a time.  PANEL then brings the workgroup's 16 (or 32) rows of w into LDS
 // first: every wave asks for its share with loads that write LDS themselves (global_load_lds_dwordx4), so
@@ -51,6 +57,19 @@ struct __attribute__((aligned(16))) sk_f32x4 {
 struct __attribute__((aligned(16))) sk_u32x4 {
     uint32_t v[4];
 };
+
+// What is handed forward (see above).  All null: nothing is.
+struct sk_hand_t {
+    // from a product that adds into the stream: the next norm's gains [N_out]; x [n, N_out] takes
+    // bf16(stream * gain) and ssq [n, column tiles] the stripes' sums of squares
+    const float* gain;
+    bf16_t* x;
+    float* ssq;
+    // to a product of bfloat16 rows that such a product left: their stripes' sums of squares [n, count]
+    const float* parts;
+    int count;
+};
+#define SK_HAND_CHUNK 8      // sums a lane adds up: sixteen lanes a row, so count <= 128 (a stream of 2,048)
 
 __device__ __forceinline__ bf16x8 sk_load8(const bf16_t* p) {
     return *reinterpret_cast<const bf16x8*>(p);
@@ -85,12 +104,17 @@ __device__ __forceinline__ void sk_load_to_lds(const void* from, const void* lds
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(at), "v"(from) : "memory", "m0");
 }
 
-template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT, bool PANEL = false, bool AHEAD = false>
+// HANDS (an adding product): the kernel leaves the next norm's work behind.  It is a kernel of its own because
+// what that adds to the last stage costs the product registers that the 16-wave shapes do not have.
+template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT, bool PANEL = false, bool AHEAD = false, bool HANDS = false>
 __global__ void __launch_bounds__(64 * WV)
 gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OUT* __restrict__ y,
                    const float* __restrict__ gain, float eps, const int* __restrict__ rows, int n, int N_out,
-                   int K, int act) {
+                   int K, int act, sk_hand_t hand) {
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
+    // may be handed the sums of squares of its rows (a product that adds into the stream reads a part's output,
+    // never a norm's)
+    constexpr bool TAKES = PRO == PRO_BF16 && MT == 1 && EPI != EPI_ADD;
     const int nwaves = blockDim.x / PL_WAVE;
     extern __shared__ float sk_lds[];
     // PANEL: [BT * 16][K] bfloat16, in the same place as the partial tiles (which are written when it is done with)
@@ -179,9 +203,46 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
     bool x_asked = one_round && kbeg < kend;
     if (x_asked) ask_x(kbeg);
 
+    // Handed sums of squares: the sixteen threads that will finish a row's sixteen columns each ask for a
+    // run of the row's sums now, with x, and add them up behind the products (inside the loop over K the
+    // sum cost the kernel sixty registers).  Asked for from a place that exists in any case, like x.
+    float hp[TAKES ? SK_HAND_CHUNK : 1];
+    bool hand_pending = false;
+    float hand_rinv = 1.f;
+    if constexpr (TAKES) {
+        hand_pending = hand.parts != nullptr;
+        const float* from = hand_pending ? hand.parts : static_cast<const float*>(x_);
+        const int ft = threadIdx.x % 256;
+        const int frow = row0 + (ft / 64) * 4 + ft % 4, fc = (ft / 4) % 16;
+        const int run = pl_ceil_div(hand.count, 16);
+#pragma unroll
+        for (int j = 0; j < SK_HAND_CHUNK; ++j) {
+            const int idx = fc * run + j;
+            const bool ok = hand_pending && frow < n && j < run && idx < hand.count;
+            const float got = from[ok ? static_cast<size_t>(frow) * hand.count + idx : 0];
+            hp[j] = ok ? got : 0.f;
+        }
+    }
+    auto take_hand = [&]() {
+        if constexpr (TAKES) {
+            if (hand_pending) {
+                float s = 0.f;
+#pragma unroll
+                for (int j = 0; j < SK_HAND_CHUNK; ++j) s += hp[j];
+                s += __shfl_xor(s, 4, PL_WAVE);
+                s += __shfl_xor(s, 8, PL_WAVE);
+                s += __shfl_xor(s, 16, PL_WAVE);
+                s += __shfl_xor(s, 32, PL_WAVE);
+                hand_rinv = 1.f / sqrtf(s / static_cast<float>(K) + eps);
+                hand_pending = false;
+            }
+        }
+    };
+
     for (int tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
         const int n0 = tile * SK_TILE_N;
         const bool col_ok = n0 + c < N_out;
+
         const bf16_t* wrow[BT];
         wrow[0] = w + static_cast<size_t>(col_ok ? n0 + c : 0) * K;
         if (BT == 2) wrow[BT - 1] = w + static_cast<size_t>(N_out + (col_ok ? n0 + c : 0)) * K;
@@ -292,6 +353,14 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
             }
         }
 
+        take_hand();
+        // the next norm's gain of the column this thread will finish (a product that hands forward): asked for
+        // here, where the registers of the products are free, and used behind the sums through LDS
+        float hand_gain = 1.f;
+        if constexpr (HANDS) {
+            const int hc = n0 + (threadIdx.x % 256 / 4) % 16;
+            hand_gain = hand.gain[hc < N_out ? hc : 0];
+        }
         if constexpr (PANEL) __syncthreads();   // every wave has read its last of the panel
         // A lane holds rows (lane/16)*4 + i, i = 0..3, of column lane%16 of its 16x16 tile.
 #pragma unroll
@@ -335,14 +404,36 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
 #pragma unroll
                 for (int b = 0; b < BT; ++b) v[b] *= rinv;
             }
-            if (threadIdx.x < 256 && row < n && col < N_out) {
+            if constexpr (TAKES) {
+#pragma unroll
+                for (int b = 0; b < BT; ++b) v[b] *= hand_rinv;      // (1 where nothing was handed)
+            }
+            const bool mine = threadIdx.x < 256 && row < n && col < N_out;
+            float updated = 0.f;
+            if (mine) {
                 float r = v[0];
                 if (EPI == EPI_SWIGLU) r = pl_activate<false>(v[0], act) * v[BT - 1];
                 const size_t at = static_cast<size_t>(row) * N_out + col;
-                if (EPI == EPI_ADD)
-                    y[at] = from_float<OUT>(to_float(y[at]) + r);
-                else
+                if (EPI == EPI_ADD) {
+                    updated = to_float(y[at]) + r;
+                    y[at] = from_float<OUT>(updated);
+                } else {
                     y[at] = from_float<OUT>(r);
+                }
+            }
+            if constexpr (HANDS) {
+                {
+                    // the stripe of the updated stream, as the next norm's product will want it, and its sum of
+                    // squares a row: the sixteen columns of a row are sixteen lanes of one wave, four apart
+                    if (mine) hand.x[static_cast<size_t>(row) * N_out + col] = from_float<bf16_t>(updated * hand_gain);
+                    float sq = updated * updated;
+                    sq += __shfl_xor(sq, 4, PL_WAVE);
+                    sq += __shfl_xor(sq, 8, PL_WAVE);
+                    sq += __shfl_xor(sq, 16, PL_WAVE);
+                    sq += __shfl_xor(sq, 32, PL_WAVE);
+                    if (threadIdx.x < 256 && row < n && src_lane % 16 == 0)
+                        hand.ssq[static_cast<size_t>(row) * num_tiles + tile] = sq;
+                }
             }
         }
         __syncthreads();  // the next tile writes the same LDS
@@ -357,7 +448,8 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
 
 template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT>
 static int launch_one(int waves, const void* x, const void* w, void* y, const float* gain, float eps,
-                      const int* rows, int n, int N_out, int K, int act, hipStream_t stream) {
+                      const int* rows, int n, int N_out, int K, int act, const sk_hand_t& hand, hipStream_t stream) {
+    PL_REQUIRE(!hand.parts || (MT == 1 && PRO == PRO_BF16 && EPI != EPI_ADD), "skinny product: this shape of product takes no handed norm");
     const int row_tiles = pl_ceil_div(n, 16 * MT);   // more than one where launch_mt deals the rows out
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
     constexpr int UA = (WV == 16 && UNR >= 2) ? UNR / 2 : UNR;   // K steps a round when rounds overlap
@@ -374,12 +466,34 @@ static int launch_one(int waves, const void* x, const void* w, void* y, const fl
     // A wave's share of K in more rounds of loads than one: the rounds overlap, two of them on their way at
     // a time (of half the steps each where sixteen waves leave a lane 128 registers).
     const bool several = pl_ceil_div(pl_ceil_div(K, SK_KSTEP), waves) > UNR;
+    const dim3 grid3(grid, row_tiles);
+    const bf16_t* wb = static_cast<const bf16_t*>(w);
+    OUT* yo = static_cast<OUT*>(y);
+    PL_REQUIRE(!hand.x || (EPI == EPI_ADD && MT == 1), "skinny product: this shape of product hands nothing forward");
+    if constexpr (EPI == EPI_ADD && MT == 1) {
+        if (hand.x) {
+            // (with 16 waves the last stage's extra work would spill beside eight K steps of loads: six then)
+            constexpr int UH = WV == 16 ? (UNR * 3) / 4 : UNR;
+            constexpr int UHA = (WV == 16 && UH >= 2) ? UH / 2 : UH;
+            const int steps = pl_ceil_div(K, SK_KSTEP);
+            const int wh = WV == 16 ? max(9, min(16, pl_ceil_div(steps, UH))) : waves;    // as many waves as cover K in one round
+            const size_t lds_h = static_cast<size_t>(wh) * (BT * MT * 256 + MT * 16) * sizeof(float);
+            if (pl_ceil_div(steps, wh) > UH)
+                gemm_skinny_kernel<MT, UHA, WV, PRO, EPI, OUT, false, true, true><<<grid3, 64 * wh, lds_h, stream>>>(
+                    x, wb, yo, gain, eps, rows, n, N_out, K, act, hand);
+            else
+                gemm_skinny_kernel<MT, UH, WV, PRO, EPI, OUT, false, false, true><<<grid3, 64 * wh, lds_h, stream>>>(
+                    x, wb, yo, gain, eps, rows, n, N_out, K, act, hand);
+            PL_CHECK_LAUNCH("gemm_skinny");
+            return 0;
+        }
+    }
     if (several)
-        gemm_skinny_kernel<MT, UA, WV, PRO, EPI, OUT, false, true><<<dim3(grid, row_tiles), 64 * waves, lds_bytes, stream>>>(
-            x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps, rows, n, N_out, K, act);
+        gemm_skinny_kernel<MT, UA, WV, PRO, EPI, OUT, false, true><<<grid3, 64 * waves, lds_bytes, stream>>>(
+            x, wb, yo, gain, eps, rows, n, N_out, K, act, hand);
     else
-        gemm_skinny_kernel<MT, UNR, WV, PRO, EPI, OUT><<<dim3(grid, row_tiles), 64 * waves, lds_bytes, stream>>>(
-            x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps, rows, n, N_out, K, act);
+        gemm_skinny_kernel<MT, UNR, WV, PRO, EPI, OUT><<<grid3, 64 * waves, lds_bytes, stream>>>(
+            x, wb, yo, gain, eps, rows, n, N_out, K, act, hand);
     PL_CHECK_LAUNCH("gemm_skinny");
     return 0;
 }
@@ -396,8 +510,9 @@ template <int MT, int WV, int STEPS, int PRO, int EPI, typename OUT>
 __global__ void __launch_bounds__(64 * WV)
 gemm_skinny_rows_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OUT* __restrict__ y,
                         const float* __restrict__ gain, float eps, const int* __restrict__ rows, int n, int N_out,
-                        int K, int act) {
+                        int K, int act, sk_hand_t hand) {
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
+    constexpr bool TAKES = PRO == PRO_BF16 && EPI != EPI_ADD && WV * 64 >= MT * 256;   // may be handed the sums of squares of its rows
     constexpr int NKS = WV / MT;                                // stretches of K
     extern __shared__ float sk_lds[];
     bf16_t* panel = reinterpret_cast<bf16_t*>(sk_lds);          // [BT * 16][K], pieces permuted
@@ -440,6 +555,38 @@ gemm_skinny_rows_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ 
     if (PRO == PRO_NORM)
         for (int k = threadIdx.x * 4; k < K; k += blockDim.x * 4)
             *reinterpret_cast<sk_f32x4*>(gain_lds + k) = *reinterpret_cast<const sk_f32x4*>(gain + k);
+    // Handed sums of squares (see gemm_skinny_kernel): thread e finishes element e % 256 of tile e / 256, and
+    // the sixteen threads of a row each ask for a run of the row's sums, before the panel is asked for.
+    float hp[TAKES ? SK_HAND_CHUNK : 1];
+    bool hand_pending = false;
+    float hand_rinv = 1.f;
+    if constexpr (TAKES) {
+        hand_pending = hand.parts != nullptr;
+        const float* from = hand_pending ? hand.parts : static_cast<const float*>(x_);
+        const int ft = threadIdx.x % 256;
+        const int frow = (threadIdx.x / 256) * 16 + (ft / 64) * 4 + ft % 4, fc = (ft / 4) % 16;
+        const int run = pl_ceil_div(hand.count, 16);
+        if (hand.count % 64 == 0) {
+            // a lane's run is whole groups of four sums, 16 bytes aligned: one load a group
+            static_assert(SK_HAND_CHUNK == 8, "two groups of four");
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const bool ok = hand_pending && frow < n && q * 4 < run;
+                const sk_f32x4 got = *reinterpret_cast<const sk_f32x4*>(
+                    from + (ok ? static_cast<size_t>(frow) * hand.count + fc * run + q * 4 : 0));
+#pragma unroll
+                for (int e = 0; e < 4; ++e) hp[q * 4 + e] = ok ? got.v[e] : 0.f;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < SK_HAND_CHUNK; ++j) {
+                const int idx = fc * run + j;
+                const bool ok = hand_pending && frow < n && j < run && idx < hand.count;
+                const float got = from[ok ? static_cast<size_t>(frow) * hand.count + idx : 0];
+                hp[j] = ok ? got : 0.f;
+            }
+        }
+    }
 
     for (int tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
         const int n0 = tile * SK_TILE_N;
@@ -455,6 +602,19 @@ gemm_skinny_rows_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ 
         }
         __builtin_amdgcn_s_waitcnt(0x0F70);                     // vmcnt(0): x and this wave's share of the panel
         __syncthreads();
+        if constexpr (TAKES) {
+            if (hand_pending) {
+                float s = 0.f;
+#pragma unroll
+                for (int j = 0; j < SK_HAND_CHUNK; ++j) s += hp[j];
+                s += __shfl_xor(s, 4, PL_WAVE);
+                s += __shfl_xor(s, 8, PL_WAVE);
+                s += __shfl_xor(s, 16, PL_WAVE);
+                s += __shfl_xor(s, 32, PL_WAVE);
+                hand_rinv = 1.f / sqrtf(s / static_cast<float>(K) + eps);
+                hand_pending = false;
+            }
+        }
 
         f32x4 acc[BT];
 #pragma unroll
@@ -540,6 +700,12 @@ gemm_skinny_rows_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ 
 #pragma unroll
                 for (int b = 0; b < BT; ++b) v[b] *= rinv;
             }
+            if constexpr (TAKES) {
+                // (the launch has a thread for every element, so e is this thread's own index and the
+                // statistic it holds is its row's)
+#pragma unroll
+                for (int b = 0; b < BT; ++b) v[b] *= hand_rinv;
+            }
             if (out_row < n && col < N_out) {
                 float r = v[0];
                 if (EPI == EPI_SWIGLU) r = pl_activate<false>(v[0], act) * v[BT - 1];
@@ -557,7 +723,9 @@ gemm_skinny_rows_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ 
 // The rows variant's launch: WV waves, MT tiles of rows, WV / MT stretches of K of at most STEPS steps.
 template <int MT, int WV, int STEPS, int PRO, int EPI, typename OUT>
 static int launch_rows(const void* x, const void* w, void* y, const float* gain, float eps,
-                       const int* rows, int n, int N_out, int K, int act, hipStream_t stream) {
+                       const int* rows, int n, int N_out, int K, int act, const sk_hand_t& hand, hipStream_t stream) {
+    PL_REQUIRE(!hand.x, "skinny product: this shape of product hands nothing forward");
+    PL_REQUIRE(!hand.parts || (PRO == PRO_BF16 && EPI != EPI_ADD && WV * 64 >= MT * 256), "skinny product: this shape of product takes no handed norm");
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
     constexpr int NKS = WV / MT;
     const int grid = min(pl_ceil_div(N_out, SK_TILE_N), SK_MAX_GRID);
@@ -573,7 +741,7 @@ static int launch_rows(const void* x, const void* w, void* y, const float* gain,
         PL_REQUIRE(e == hipSuccess, "skinny product: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
     }
     kernel<<<grid, 64 * WV, lds_bytes, stream>>>(x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps,
-                                                rows, n, N_out, K, act);
+                                                rows, n, N_out, K, act, hand);
     PL_CHECK_LAUNCH("gemm_skinny");
     return 0;
 }
@@ -581,7 +749,9 @@ static int launch_rows(const void* x, const void* w, void* y, const float* gain,
 // The panel variant: 8 waves (256 registers a lane); a wave holds 16 * MT rows of x for UNR K steps.
 template <int MT, int UNR, int PRO, int EPI, typename OUT>
 static int launch_panel(const void* x, const void* w, void* y, const float* gain, float eps,
-                        const int* rows, int n, int N_out, int K, int act, hipStream_t stream) {
+                        const int* rows, int n, int N_out, int K, int act, const sk_hand_t& hand, hipStream_t stream) {
+    PL_REQUIRE(!hand.parts || (MT == 1 && EPI != EPI_ADD), "skinny product: this shape of product takes no handed norm");
+    PL_REQUIRE(!hand.x, "skinny product: this shape of product hands nothing forward");
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
     constexpr int waves = 8;
     const int grid = min(pl_ceil_div(N_out, SK_TILE_N), SK_MAX_GRID);
@@ -595,7 +765,7 @@ static int launch_panel(const void* x, const void* w, void* y, const float* gain
         PL_REQUIRE(e == hipSuccess, "skinny product: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
     }
     kernel<<<grid, 64 * waves, lds_bytes, stream>>>(x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps,
-                                                   rows, n, N_out, K, act);
+                                                   rows, n, N_out, K, act, hand);
     PL_CHECK_LAUNCH("gemm_skinny");
     return 0;
 }
@@ -615,7 +785,7 @@ struct SkShape {
 
 template <int MT, int PRO, int EPI, typename OUT>
 static int launch_unr(const void* x, const void* w, void* y, const float* gain, float eps,
-                      const int* rows, int n, int N_out, int K, int act, hipStream_t stream) {
+                      const int* rows, int n, int N_out, int K, int act, const sk_hand_t& hand, hipStream_t stream) {
     using S = SkShape<MT, PRO, EPI>;
     if constexpr (MT == 2 || MT == 4) {
         // 16 waves: 16 / MT stretches of K, each a whole number of K steps that a wave can hold at once
@@ -624,10 +794,10 @@ static int launch_unr(const void* x, const void* w, void* y, const float* gain, 
         const size_t panel = static_cast<size_t>(BT) * 16 * K * 2 + (PRO == PRO_NORM ? static_cast<size_t>(K) * 4 : 0);
         const int need = K / SK_KSTEP / NKS;             // K steps a wave holds at once
         if (K % 512 == 0 && K / SK_KSTEP % NKS == 0 && panel <= 144 * 1024) {
-            if (need <= 8) return launch_rows<MT, 16, 8, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, stream);
+            if (need <= 8) return launch_rows<MT, 16, 8, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
             if constexpr (PRO == PRO_BF16) {             // the 32-bit stream takes twice the registers a step
                 // (24 steps would fit the registers of 16 waves only with spills: such a K goes the way below)
-                if (need <= 16) return launch_rows<MT, 16, 16, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, stream);
+                if (need <= 16) return launch_rows<MT, 16, 16, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
             }
         }
     }
@@ -635,52 +805,75 @@ static int launch_unr(const void* x, const void* w, void* y, const float* gain, 
         constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
         if (K % 512 == 0 && static_cast<size_t>(BT) * 16 * K * 2 <= 128 * 1024)
             return launch_panel<MT, (PRO == PRO_NORM ? (MT == 4 ? 1 : 2) : (MT == 4 ? 4 : 8)), PRO, EPI, OUT>(
-                x, w, y, gain, eps, rows, n, N_out, K, act, stream);
+                x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
     }
     const int steps = pl_ceil_div(K, SK_KSTEP);
     const int most = max(4 * S::U4, max(8 * S::U8, 16 * S::U16));
     const int need = min(steps, most);     // beyond that, several rounds
     if (need <= 4 * S::U4)
-        return launch_one<MT, S::U4, 4, PRO, EPI, OUT>(4, x, w, y, gain, eps, rows, n, N_out, K, act, stream);
+        return launch_one<MT, S::U4, 4, PRO, EPI, OUT>(4, x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
     if constexpr (S::U8 > 0) {
         if (need <= 8 * S::U8 || S::U16 == 0)
-            return launch_one<MT, S::U8, 8, PRO, EPI, OUT>(max(5, min(8, pl_ceil_div(steps, S::U8))), x, w, y, gain, eps, rows, n, N_out, K, act, stream);
+            return launch_one<MT, S::U8, 8, PRO, EPI, OUT>(max(5, min(8, pl_ceil_div(steps, S::U8))), x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
     }
     if constexpr (S::U16 > 0) {
-        return launch_one<MT, S::U16, 16, PRO, EPI, OUT>(max(9, min(16, pl_ceil_div(steps, S::U16))), x, w, y, gain, eps, rows, n, N_out, K, act, stream);
+        return launch_one<MT, S::U16, 16, PRO, EPI, OUT>(max(9, min(16, pl_ceil_div(steps, S::U16))), x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
     }
-    return launch_one<MT, S::U4, 4, PRO, EPI, OUT>(4, x, w, y, gain, eps, rows, n, N_out, K, act, stream);
+    return launch_one<MT, S::U4, 4, PRO, EPI, OUT>(4, x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
 }
 
 template <int PRO, int EPI, typename OUT>
 static int launch_mt(const void* x, const void* w, void* y, const float* gain, float eps,
-                     const int* rows, int n, int N_out, int K, int act, hipStream_t stream) {
+                     const int* rows, int n, int N_out, int K, int act, const sk_hand_t& hand, hipStream_t stream) {
     // Few tiles of columns (a narrow output, as of the projections back into the stream): the tiles of 16 rows
     // go to workgroups of their own, the kernel for up to 16 rows on a grid of (column tiles, row tiles), so that
     // the launch has workgroups for every compute unit; each reads its rows of x only, and w comes from L2
     // from the second row tile on.
     if (n > 16 && pl_ceil_div(N_out, SK_TILE_N) * pl_ceil_div(n, 16) <= SK_ROW_TILES_GRID)
-        return launch_unr<1, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, stream);
+        return launch_unr<1, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
     switch (pl_ceil_div(n, 16)) {
-        case 1: return launch_unr<1, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, stream);
-        case 2: return launch_unr<2, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, stream);
-        case 3: return launch_unr<3, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, stream);
-        default: return launch_unr<4, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, stream);
+        case 1: return launch_unr<1, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
+        case 2: return launch_unr<2, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
+        case 3:
+            // (a handed norm is taken by the kernel of two or four tiles of rows: three go as four, one of them empty)
+            if (hand.parts) return launch_unr<4, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
+            return launch_unr<3, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
+        default: return launch_unr<4, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
     }
+}
+
+// Which kernel the launchers above take for a product of bfloat16 rows, as far as the handed norm goes:
+// whether the product can take the sums of squares of its rows (taking), or leave them and the normalised
+// stripe behind (an adding product, !taking).  The same conditions as in launch_mt and launch_unr.
+static inline bool sk_hand_applies(int n, int N_out, int K, int epilogue, bool taking) {
+    if (n <= 0 || n > 64 || K % 8 || N_out <= 0) return false;
+    if (taking && (epilogue == EPI_ADD || pl_ceil_div(K, SK_TILE_N) > 16 * SK_HAND_CHUNK)) return false;
+    if (!taking && epilogue != EPI_ADD) return false;
+    const int row_tiles = pl_ceil_div(n, 16);
+    if (n <= 16 || pl_ceil_div(N_out, SK_TILE_N) * row_tiles <= SK_ROW_TILES_GRID) return true;   // the kernel for one tile of rows
+    const int MT = (taking && row_tiles == 3) ? 4 : row_tiles;
+    const int BT = epilogue == EPI_SWIGLU ? 2 : 1;
+    bool rows_kernel = false;
+    if (MT == 2 || MT == 4) {
+        const int NKS = 16 / MT;
+        const size_t panel = static_cast<size_t>(BT) * 16 * K * 2;
+        rows_kernel = K % 512 == 0 && K / SK_KSTEP % NKS == 0 && panel <= 144 * 1024 && K / SK_KSTEP / NKS <= 16;
+    }
+    return taking && rows_kernel;        // (an adding product hands forward from the kernel for one tile of rows only)
 }
 
 template <int PRO>
 static int sk_launch(int epilogue, int out_f32, const void* x, const void* w, void* y, const float* gain,
-                      float eps, const int* rows, int n, int N_out, int K, int act, hipStream_t stream) {
+                      float eps, const int* rows, int n, int N_out, int K, int act, const sk_hand_t& hand, hipStream_t stream) {
     if (epilogue == EPI_STORE)
-        return out_f32 ? launch_mt<PRO, EPI_STORE, float>(x, w, y, gain, eps, rows, n, N_out, K, act, stream)
-                       : launch_mt<PRO, EPI_STORE, bf16_t>(x, w, y, gain, eps, rows, n, N_out, K, act, stream);
-    if (epilogue == EPI_SWIGLU) return launch_mt<PRO, EPI_SWIGLU, bf16_t>(x, w, y, gain, eps, rows, n, N_out, K, act, stream);
+        return out_f32 ? launch_mt<PRO, EPI_STORE, float>(x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream)
+                       : launch_mt<PRO, EPI_STORE, bf16_t>(x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
+    if (epilogue == EPI_SWIGLU) return launch_mt<PRO, EPI_SWIGLU, bf16_t>(x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
     if constexpr (PRO == PRO_NORM) {
         pl_set_error("skinny product: a product that reads the residual stream cannot add into it");
         return -1;
     } else {
-        return launch_mt<PRO, EPI_ADD, float>(x, w, y, gain, eps, rows, n, N_out, K, act, stream);
+        return launch_mt<PRO, EPI_ADD, float>(x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
     }
 }
 

@@ -39,6 +39,8 @@ def _signatures(lib) -> None:
         "pl_argmax": [p, p, p, p, i, i, p],
         "pl_sample": [p, p, p, p, p, p, i, i, p],
         "pl_gemm_skinny": [p, p, p, p, f, p, i, i, i, i, i, i, p],
+        "pl_gemm_skinny_hand": [p, p, p, i, i, i, i, i, i, p, i, f, p, p, p, p],
+        "pl_gemm_skinny_hand_applies": [i, i, i, i, i],
         "pl_gemm_tiled": [p, p, p, i, i, i, i, i, p],
         "pl_gemm_tiled_applies": [i, i, i, i],
         "pl_gemm_stream": [p, p, p, p, i, i, i, i, i, i, i, p],
@@ -637,9 +639,49 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nk
                                   live_seqs=getattr(batch, "live_seqs", None), short_rows=short_tokens)
 
 
+class HandedNorm:
+    """An RMSNorm handed forward by the product that last added into the stream: that product owns whole
+    16-column stripes of the updated stream, so it leaves ``x`` = bfloat16(stream * gain) [n, width] and, for
+    every row, the sum of squares over each stripe, ``ssq`` [n, stripes].  The product that stands behind the
+    norm then loads ``x`` (half the bytes of the 32-bit stream, nothing to convert or square), adds a row's
+    sums in a fixed order and scales its result by 1 / sqrt(sum / width + eps).  ``filled`` says that a
+    product has written both."""
+
+    __slots__ = ("gain", "eps", "x", "ssq", "filled")
+
+    def __init__(self, gain: torch.Tensor, eps: float, rows: int, width: int, device):
+        self.gain, self.eps = gain, float(eps)
+        self.x = torch.empty((rows, width), dtype=torch.bfloat16, device=device)
+        self.ssq = torch.empty((rows, (width + 15) // 16), dtype=torch.float32, device=device)
+        self.filled = False
+
+
+# From this many rows on a norm is handed forward.  With fewer the product behind the norm normalises the 32-bit
+# stream itself at no cost that shows, and what the adding product does more is not made up for (decode steps of
+# the 0.6B shape, handed against not, ms: 1 row 1.103 / 1.080, 4 rows 1.152 / 1.134, 8 rows 1.252 / 1.251, 16 rows
+# 1.422 / 1.438, 17 rows 1.547 / 1.721, 32 rows 1.692 / 1.872, 64 rows 2.161 / 2.314).
+HAND_FROM_ROWS = 16
+
+
+def hands_norm_forward(rows: int, columns: int, width: int) -> bool:
+    """Whether the product of ``rows`` bfloat16 rows that adds into a stream of ``columns`` hands the next
+    norm forward: rows enough that the norm would otherwise be a kernel of its own or a costly first stage,
+    against a stream that is not wide (every product behind the norm adds up all of a row's stripes)."""
+    return (rows >= HAND_FROM_ROWS and columns <= FUSED_NORM_MAX_WIDTH and skinny_wins(rows, columns, width)
+            and bool(library().pl_gemm_skinny_hand_applies(rows, columns, width, 2, 0)))
+
+
+def takes_handed_norm(rows: int, columns: int, width: int, swiglu: bool = False) -> bool:
+    """Whether the product of ``rows`` rows against ``columns`` (outputs) can take a norm handed forward."""
+    return (width <= FUSED_NORM_MAX_WIDTH and columns <= FUSED_NORM_MAX_COLUMNS
+            and skinny_wins(rows, columns * (2 if swiglu else 1), width)
+            and bool(library().pl_gemm_skinny_hand_applies(rows, columns, width, 1 if swiglu else 0, 1)))
+
+
 def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, swiglu: bool = False,
                 norm_gain: torch.Tensor | None = None, eps: float = 0.0, rows: torch.Tensor | None = None,
-                add_into: torch.Tensor | None = None, activation: str = "silu") -> torch.Tensor:
+                add_into: torch.Tensor | None = None, activation: str = "silu",
+                handed: "HandedNorm | None" = None, hand: "HandedNorm | None" = None) -> torch.Tensor:
     """y = x . w^T for up to 64 rows on the matrix cores, the bfloat16 weights streamed once.
 
     ``x`` is bfloat16 [n, K]; or, with ``norm_gain``, the 32-bit residual stream, whose rows
@@ -647,7 +689,14 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
     With ``swiglu`` the rows of ``w`` are [gate | up] and y = act(x . gate^T) * (x . up^T), in bfloat16
     (``activation``: silu or a gelu).
     With ``add_into`` (the 32-bit residual stream, [n, N]) the result is added there and that
-    tensor is returned."""
+    tensor is returned.
+    ``handed``: a norm that an earlier product left behind; its rows are the input (``x`` is not looked at)
+    and its sums of squares scale the result.  ``hand`` (with ``add_into``): the norm that follows the
+    stream is left behind in it."""
+    if handed is not None:
+        if norm_gain is not None or not handed.filled:
+            raise TensorError("a handed norm is the product's input by itself, once a product has written it")
+        x = handed.x
     K = x.shape[1]
     if norm_gain is None:
         _need(x, "matrix product input", None, torch.bfloat16)
@@ -676,6 +725,24 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
             raise TensorError(f"matrix product output {out_dtype}" + (" after the activation" if swiglu else ""))
         out = torch.empty((n, N_out), dtype=out_dtype, device=x.device)
         epilogue, out_f32 = (1 if swiglu else 0), (1 if out_dtype == torch.float32 else 0)
+    if handed is not None or hand is not None:
+        if hand is not None:
+            if add_into is None:
+                raise TensorError("a norm is handed forward by a product that adds into the stream")
+            _need(hand.gain, "gain of the norm handed forward", (N_out,), torch.float32)
+            _need(hand.x, "rows of the norm handed forward", (n, N_out), torch.bfloat16)
+            _need(hand.ssq, "sums of squares of the norm handed forward", (n, (N_out + 15) // 16), torch.float32)
+        if handed is not None:
+            _need(handed.ssq, "sums of squares of the handed norm", (n, (K + 15) // 16), torch.float32)
+        _check(library().pl_gemm_skinny_hand(
+            x.data_ptr(), w.data_ptr(), out.data_ptr(), n, N_out, K, epilogue, out_f32, activation_code(activation),
+            _ptr(handed.ssq if handed is not None else None), handed.ssq.shape[1] if handed is not None else 0,
+            float(handed.eps if handed is not None else 0.0),
+            _ptr(hand.gain if hand is not None else None), _ptr(hand.x if hand is not None else None),
+            _ptr(hand.ssq if hand is not None else None), _stream()))
+        if hand is not None:
+            hand.filled = True
+        return out
     _check(library().pl_gemm_skinny(
         x.data_ptr(), w.data_ptr(), out.data_ptr(), _ptr(norm_gain), float(eps), _ptr(rows), n, N_out, K,
         epilogue, out_f32, activation_code(activation), _stream()))

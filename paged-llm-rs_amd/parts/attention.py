@@ -100,7 +100,8 @@ class PagedAttention:
             out = self.o_proj.forward(out)
             ctx.trace.record("o_proj.out", out)
             return out
-        return self.o_proj.forward(out, add_into=ctx.residual)
+        return self.o_proj.forward(out, add_into=ctx.residual,
+                                   hand=getattr(ctx, "hand", None) if ctx.residual is not None else None)
 
     def _record_projections(self, qkv, batch, kv, trace) -> None:
         """q, k and v as projected, and q and k after their per-head norm (before the rotation).  The

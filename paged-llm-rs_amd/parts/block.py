@@ -11,6 +11,8 @@ product kernel and the norm becomes the first stage of the next product.
 
 from __future__ import annotations
 
+import torch
+
 from ..errors import ConfigError
 from .norm import PendingNorm
 from .registry import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, lookup, prefixed, register_block, scoped)
@@ -57,6 +59,17 @@ class PreNormBlock:
         reads device values on the host, or allocates by data, sets ``graph_safe = False``."""
         return getattr(self.mixer, "graph_safe", True) and getattr(self.feed_forward, "graph_safe", True)
 
+    @property
+    def first_norm(self):
+        """The norm this block applies to the stream first: the block before may leave its work behind."""
+        return self.norm1
+
+    @staticmethod
+    def _room(norm, resid):
+        """Room for ``norm`` handed forward over the rows of ``resid``, where the norm has such a thing."""
+        make = getattr(norm, "handoff", None)
+        return make(resid.shape[0], resid.device) if make is not None else None
+
     def forward(self, resid, delta, ctx):
         """``delta``: what the block before has not added to the stream yet, or None.  Returns this
         block's own unadded output, or None when the feed-forward added it itself."""
@@ -64,18 +77,29 @@ class PreNormBlock:
             return self._forward_recorded(resid, delta, ctx)
         mixer_fuses = getattr(self.mixer, "fuses", False)
         ffn_fuses = getattr(self.feed_forward, "fuses", False)
+        half = self.dtype == torch.bfloat16
         if delta is None and mixer_fuses:
-            x = PendingNorm(self.norm1, resid, self.dtype)       # every sum is in the stream already
+            # every sum is in the stream already (and the product that added the last may have left this norm's work)
+            x = PendingNorm(self.norm1, resid, self.dtype, handed=getattr(ctx, "handed", None))
         else:
             x = self.norm1.apply(resid, delta, self.dtype)
         ctx.residual = resid if mixer_fuses else None
+        # a mixer that adds into the stream may leave the second norm's work behind ...
+        ctx.hand = self._room(self.norm2, resid) if half and mixer_fuses and ffn_fuses else None
         mixed = self.mixer.forward(x, ctx)
-        ctx.residual = None
+        left, ctx.residual, ctx.hand = ctx.hand, None, None
         if mixed is None and ffn_fuses:
-            x = PendingNorm(self.norm2, resid, self.dtype)
+            x = PendingNorm(self.norm2, resid, self.dtype, handed=left)
         else:
             x = self.norm2.apply(resid, mixed, self.dtype)
         if ffn_fuses:
+            # ... and a feed-forward that does, the next layer's first norm's
+            after = getattr(ctx, "norm_after", None)
+            if half and after is not None and getattr(self.feed_forward, "hands_forward", False):
+                room = self._room(after, resid)
+                out = self.feed_forward.forward(x, residual=resid, hand=room)
+                ctx.handed_out = room if out is None and room is not None and room.filled else None
+                return out
             return self.feed_forward.forward(x, residual=resid)
         return self.feed_forward.forward(x)
 

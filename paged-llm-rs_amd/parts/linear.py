@@ -31,12 +31,14 @@ class Linear:
         return cls(torch.cat(list(weights), dim=0), torch.cat(biases, dim=0) if biases else None)
 
     def forward(self, x, out_dtype: torch.dtype | None = None, add_into: torch.Tensor | None = None,
-                swiglu: bool = False, activation: str = "silu"):
+                swiglu: bool = False, activation: str = "silu", hand=None):
         """The product of ``x`` (rows, or a norm still to run) with the weight.
 
         ``swiglu``: the weight is [gate | up] stacked and act(gate) * up comes back (``activation``: silu or a gelu).
         ``add_into``: the 32-bit residual stream; where the product kernel can add its result
-        there itself it does and None comes back, otherwise the result comes back unadded."""
+        there itself it does and None comes back, otherwise the result comes back unadded.
+        ``hand``: room for the norm that follows the stream (``kernels.HandedNorm``); a product kernel that adds
+        into the stream and can leave that norm's work behind fills it, any other way leaves it unfilled."""
         if self.bias is not None:
             # The bias is added behind the product by a kernel of its own; what the product would have fused
             # behind itself (the activation, the sum into the stream) then runs unfused as well.
@@ -45,13 +47,18 @@ class Linear:
             y = self._product(x, out_dtype if not swiglu else None)
             kernels.add_bias(y, self.bias)
             return kernels.swiglu(y, activation=activation) if swiglu else y
-        return self._product(x, out_dtype, add_into, swiglu, activation)
+        return self._product(x, out_dtype, add_into, swiglu, activation, hand)
 
     def _product(self, x, out_dtype: torch.dtype | None = None, add_into: torch.Tensor | None = None,
-                 swiglu: bool = False, activation: str = "silu"):
+                 swiglu: bool = False, activation: str = "silu", hand=None):
         if isinstance(x, PendingNorm):
             if x.width != self.in_features:
                 raise TensorError(f"a linear of {self.in_features} inputs given a stream of width {x.width}")
+            columns = self.out_features // 2 if swiglu else self.out_features
+            if (x.handed is not None and add_into is None and self.weight.dtype == torch.bfloat16
+                    and kernels.takes_handed_norm(x.num_rows, columns, self.in_features, swiglu)):
+                return kernels.gemm_skinny(None, self.weight, out_dtype or x.out_dtype, swiglu=swiglu,
+                                           activation=activation, handed=x.handed)
             if (getattr(x.norm, "fuses_into_product", False) and add_into is None
                     and kernels.fused_norm_applies(x.num_rows, self.in_features, self.weight)
                     and self.out_features <= kernels.FUSED_NORM_MAX_COLUMNS):
@@ -69,7 +76,9 @@ class Linear:
             return kernels.swiglu(y, activation=activation) if swiglu else y
         if kernels.skinny_applies(x, self.weight):
             if add_into is not None and not swiglu:
-                kernels.gemm_skinny(x, self.weight, add_into=add_into)
+                if hand is not None and not kernels.hands_norm_forward(x.shape[0], self.out_features, self.in_features):
+                    hand = None
+                kernels.gemm_skinny(x, self.weight, add_into=add_into, hand=hand)
                 return None
             return kernels.gemm_skinny(x, self.weight, out_dtype, swiglu=swiglu, activation=activation)
         if kernels.stream_wins(x.shape[0], self.out_features, self.in_features):

@@ -31,10 +31,13 @@ class GatedMlp:
     fuses = True
     # ... and a recorder of named activations
     records = True
+    # ... and room for the norm that follows the stream, which the product that adds into it may fill
+    hands_forward = True
 
-    def forward(self, x, residual: torch.Tensor | None = None, trace=None):
+    def forward(self, x, residual: torch.Tensor | None = None, trace=None, hand=None):
         """``x``: normalised rows, or a PendingNorm.  With ``residual`` (the 32-bit stream) the
-        result is added there where the product kernel can do it, and None comes back."""
+        result is added there where the product kernel can do it, and None comes back; ``hand``
+        (``kernels.HandedNorm``) is then filled where that kernel can leave the next norm's work behind."""
         if trace is not None:
             both = self.gate_up_proj.forward(x)
             inter = both.shape[1] // 2
@@ -47,7 +50,7 @@ class GatedMlp:
             return out
         # (few rows: the activation is the product's epilogue)
         act = self.gate_up_proj.forward(x, swiglu=True, activation=self.activation)
-        return self.down_proj.forward(act, add_into=residual)
+        return self.down_proj.forward(act, add_into=residual, hand=hand if residual is not None else None)
 
 
 register_feed_forward("gated_mlp", GatedMlp)

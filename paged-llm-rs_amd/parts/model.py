@@ -58,7 +58,8 @@ class LayerContext:
     """What one run of one layer sees of the step: the batch, its own pages (or
     the pages of the layer it reads from) and its state slots."""
 
-    __slots__ = ("batch", "cache", "layer", "cache_layer", "writes_cache", "residual", "trace")
+    __slots__ = ("batch", "cache", "layer", "cache_layer", "writes_cache", "residual", "trace", "hand", "handed",
+                 "norm_after", "handed_out")
 
     def __init__(self, batch, cache, layer: int, cache_layer: int, writes_cache: bool):
         self.batch = batch
@@ -70,6 +71,14 @@ class LayerContext:
         self.residual = None
         # an ActivationTrace for the part that runs, when named activations are recorded; None otherwise
         self.trace = None
+        # Norms handed forward (``kernels.HandedNorm``; all optional, a part that knows nothing of them loses
+        # nothing).  ``hand``: while a mixer that adds its own output runs, room for the norm that follows the
+        # stream then.  ``handed``: what the layer before left of this layer's first norm.  ``norm_after``: the
+        # norm that the next layer applies to the stream first; a block that can leaves its work in ``handed_out``.
+        self.hand = None
+        self.handed = None
+        self.norm_after = None
+        self.handed_out = None
 
     def kv(self):
         return self.cache.layer_view(self.cache_layer, self.batch)
@@ -140,12 +149,18 @@ class DecoderModel:
         if top is not None:
             top.record(self.spec.embed_name.rsplit(".", 1)[0] + ".out", resid)
         delta = None
-        for entry in self.spec.schedule:
+        handed = None
+        schedule = self.spec.schedule
+        for at, entry in enumerate(schedule):
             own = entry.cache_from is None
             ctx = LayerContext(batch, cache, entry.layer, entry.layer if own else entry.cache_from, own)
             if top is not None:
                 ctx.trace = top.child(self.spec.layers[entry.layer].weight_prefix)
+            ctx.handed = handed
+            if at + 1 < len(schedule):
+                ctx.norm_after = getattr(self.blocks[schedule[at + 1].layer], "first_norm", None)
             delta = self.blocks[entry.layer].forward(resid, delta, ctx)
+            handed = ctx.handed_out if delta is None else None
             if top is not None:
                 after = resid.clone()
                 if delta is not None:

@@ -16,10 +16,13 @@ class PendingNorm:
     A part that is handed one may pass it on to ``Linear.forward``, which runs norm and
     product as one kernel where that pays, or call ``materialize()`` for the normalised rows."""
 
-    __slots__ = ("norm", "resid", "out_dtype", "rows")
+    __slots__ = ("norm", "resid", "out_dtype", "rows", "handed")
 
-    def __init__(self, norm, resid: torch.Tensor, out_dtype: torch.dtype, rows=None):
+    def __init__(self, norm, resid: torch.Tensor, out_dtype: torch.dtype, rows=None, handed=None):
         self.norm, self.resid, self.out_dtype, self.rows = norm, resid, out_dtype, rows
+        # what the product that last added into the stream left of this norm's work (a filled
+        # ``kernels.HandedNorm`` of this very norm, all rows), or None
+        self.handed = handed if handed is not None and handed.filled and rows is None else None
 
     @property
     def num_rows(self) -> int:
@@ -49,6 +52,13 @@ class RmsNorm:
         self.gain = params["weight"]
         # the product kernels that take the norm as their first stage read the gain in 32-bit
         self.gain32 = self.gain if self.gain.dtype == torch.float32 else self.gain.float()
+
+    def handoff(self, rows: int, device):
+        """Room for this norm handed forward by a product that adds into the stream (``kernels.HandedNorm``),
+        or None where no product would take it: many rows, a wide stream."""
+        if rows > kernels.SKINNY_ROWS or self.width > kernels.FUSED_NORM_MAX_WIDTH or self.width % 8:
+            return None
+        return kernels.HandedNorm(self.gain32, self.eps, rows, self.width, device)
 
     def apply(self, resid: torch.Tensor, delta, out_dtype: torch.dtype, rows=None) -> torch.Tensor:
         n = resid.shape[0] if rows is None else rows.numel()

@@ -1352,3 +1352,50 @@ def test_the_single_token_kernel_that_prepares_its_keys_beside_the_oracles(reque
         found = rel(out[0].view(nq, d)[kvh * g], v_pool[far_slot].view(nkv, d)[kvh])
         assert found < 0.05, f"the key at {far}, the oldest that position 199 sees with window {window}: {found:.3e}"
     assert bool((out[-1] == 7.0).all()), "a padding row is not written"
+
+
+@pytest.mark.parametrize("n", [1, 8, 16, 17, 33, 40, 64])
+@pytest.mark.parametrize("H,deep,N2,swiglu", [(1024, 3072, 4096, False), (1024, 2048, 3072, True), (1000, 264, 130, False),
+                                              (2048, 512, 1000, True), (512, 1024, 20000, False), (1000, 264, 4096, False)])
+def test_a_norm_handed_forward_from_one_product_to_the_next(n, H, deep, N2, swiglu):
+    """The product that adds into the stream leaves the next norm's work behind (the normalised stripe in
+    bfloat16, the stripe's sum of squares a row); the product behind that norm takes both.  Each half against
+    64-bit arithmetic, and the pair against the product that normalises the 32-bit stream itself."""
+    from paged_llm_rs_amd import kernels
+
+    g = torch.Generator().manual_seed(n * 7 + H)
+    eps = 1e-6
+    stream = torch.randn(n, H, generator=g).to(DEV)
+    before = stream.clone()
+    part = torch.randn(n, deep, generator=g).bfloat16().to(DEV)
+    w_add = (torch.randn(H, deep, generator=g) / math.sqrt(deep)).bfloat16().to(DEV)
+    gain = (1 + 0.2 * torch.randn(H, generator=g)).to(DEV)
+    w_next = (torch.randn(N2 * (2 if swiglu else 1), H, generator=g) / math.sqrt(H)).bfloat16().to(DEV)
+    assert kernels.hands_norm_forward(n, H, deep) == (n >= kernels.HAND_FROM_ROWS)     # (the kernel takes any count)
+    hand = kernels.HandedNorm(gain, eps, n, H, DEV)
+    hand.x.fill_(7.0)
+    hand.ssq.fill_(float("nan"))
+    kernels.gemm_skinny(part, w_add, add_into=stream, hand=hand)
+    assert hand.filled
+    want_stream = before.double() + part.double() @ w_add.double().T
+    assert rel(stream, want_stream) < 1e-5
+    assert rel(hand.x, stream.double() * gain.double()) < 5e-3               # one rounding to bfloat16
+    stripes = torch.nn.functional.pad(stream.double() ** 2, (0, -H % 16)).reshape(n, -1, 16).sum(-1)
+    assert hand.ssq.shape == stripes.shape and rel(hand.ssq, stripes) < 1e-5
+    # the product behind the norm
+    takes = kernels.takes_handed_norm(n, N2, H, swiglu)
+    # (beyond 16 rows: the kernel for one tile of rows where the launch stays small, else the kernel whose waves
+    # take a tile of rows each, which wants a stream that is a multiple of 512 wide)
+    assert takes == (n <= 16 or -(-N2 // 16) * -(-n // 16) <= 512 or H % 512 == 0)
+    if not takes:
+        with pytest.raises(Exception, match="take no handed norm"):
+            kernels.gemm_skinny(None, w_next, swiglu=swiglu, handed=hand)
+        return
+    got = kernels.gemm_skinny(None, w_next, torch.bfloat16, swiglu=swiglu, handed=hand)
+    rinv = 1 / torch.sqrt((stream.double() ** 2).mean(-1, keepdim=True) + eps)
+    raw = (hand.x.double() @ w_next.double().T) * rinv
+    want = torch.nn.functional.silu(raw[:, :N2]) * raw[:, N2:] if swiglu else raw
+    assert rel(got, want) < 1e-2
+    if n <= 32 and N2 <= 32768:
+        own = kernels.gemm_skinny(stream, w_next, torch.bfloat16, swiglu=swiglu, norm_gain=gain, eps=eps)
+        assert rel(got, own.double()) < 1e-2
