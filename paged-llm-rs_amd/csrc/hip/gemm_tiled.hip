@@ -168,13 +168,21 @@ gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, vo
     if (step < steps) one_step(0, step);
     __builtin_amdgcn_s_waitcnt(0x0F70);              // nothing may still be on its way into LDS when the workgroup ends
 
+    // The last stage goes through LDS: a lane holds, for one row, groups of four neighbouring columns, and
+    // stored from there a wave's store would touch 32 rows with 8 or 16 bytes each (a product of 2,048 rows
+    // against 4,096 columns spent 8.7 us of its 29 storing 16 MB so).  The tile is laid down in LDS as rows
+    // (a pitch of the row plus 16 bytes, so that the rows a store of LDS touches fall on different banks)
+    // and leaves in whole rows, 16 bytes a lane.
     // acc[t][mb][4 j + i]: output column (of the wave's 32 of half t) 8 j + 4 h + i, row 64 wm + 32 mb + r32
+    __syncthreads();                                 // every wave has read its last operands
+    constexpr int OUT_COLS = EPI == GT_SWIGLU ? GT_BN / 2 : GT_BN;
+    constexpr int OUT_BYTES = EPI == GT_ADD ? 4 : 2;
+    constexpr int PITCH = OUT_COLS * OUT_BYTES + 16;      // bytes (a multiple of 16: rows are read 16 bytes a lane)
+    char* staged = reinterpret_cast<char*>(gt_lds);
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb) {
-        const int row = m0 + 64 * wm + 32 * mb + r32;
-        if (row >= M) continue;
+        char* at_row = staged + (64 * wm + 32 * mb + r32) * PITCH;
         if constexpr (EPI == GT_SWIGLU) {
-            bf16_t* out = static_cast<bf16_t*>(y_) + static_cast<size_t>(row) * N + n0 + 32 * wn + 4 * h;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 float v[4];
@@ -186,28 +194,45 @@ gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, vo
                 uint2 packed;
                 packed.x = gt_pack2(v[0], v[1]);
                 packed.y = gt_pack2(v[2], v[3]);
-                *reinterpret_cast<uint2*>(out + 8 * j) = packed;
+                *reinterpret_cast<uint2*>(at_row + (32 * wn + 4 * h + 8 * j) * 2) = packed;
             }
         } else {
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                const size_t at = static_cast<size_t>(row) * N + n0 + 64 * wn + 32 * t + 4 * h;
+            for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
+                    const int col = 64 * wn + 32 * t + 4 * h + 8 * j;
                     if constexpr (EPI == GT_ADD) {
-                        float* out = static_cast<float*>(y_) + at + 8 * j;
-                        gt_f32x4 old = *reinterpret_cast<const gt_f32x4*>(out);
+                        gt_f32x4 v;
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) old[i] += acc[t][mb][4 * j + i];
-                        *reinterpret_cast<gt_f32x4*>(out) = old;
+                        for (int i = 0; i < 4; ++i) v[i] = acc[t][mb][4 * j + i];
+                        *reinterpret_cast<gt_f32x4*>(at_row + col * 4) = v;
                     } else {
                         uint2 packed;
                         packed.x = gt_pack2(acc[t][mb][4 * j], acc[t][mb][4 * j + 1]);
                         packed.y = gt_pack2(acc[t][mb][4 * j + 2], acc[t][mb][4 * j + 3]);
-                        *reinterpret_cast<uint2*>(static_cast<bf16_t*>(y_) + at + 8 * j) = packed;
+                        *reinterpret_cast<uint2*>(at_row + col * 2) = packed;
                     }
                 }
-            }
+        }
+    }
+    __syncthreads();
+    constexpr int LANES_A_ROW = OUT_COLS * OUT_BYTES / 16;       // 8, 16 or 32
+    constexpr int ROWS_A_PASS = 256 / LANES_A_ROW;
+    const int piece = tid % LANES_A_ROW;
+#pragma unroll 4
+    for (int r = tid / LANES_A_ROW; r < GT_BM; r += ROWS_A_PASS) {
+        const int row = m0 + r;
+        if (row >= M) break;
+        const gt_f32x4 got = *reinterpret_cast<const gt_f32x4*>(staged + r * PITCH + piece * 16);
+        char* out = static_cast<char*>(y_) + (static_cast<size_t>(row) * N + n0) * OUT_BYTES + piece * 16;
+        if constexpr (EPI == GT_ADD) {
+            gt_f32x4 old = *reinterpret_cast<const gt_f32x4*>(out);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) old[i] += got[i];
+            *reinterpret_cast<gt_f32x4*>(out) = old;
+        } else {
+            *reinterpret_cast<gt_f32x4*>(out) = got;
         }
     }
 }
@@ -218,7 +243,10 @@ static int gt_launch(const void* x, const void* w, void* y, int M, int N, int K,
     const int row_tiles = pl_ceil_div(M, GT_BM);
     const long long total = static_cast<long long>(row_tiles) * (N / COLS);
     PL_REQUIRE(total > 0 && total < (1ll << 30), "tiled product: %lld workgroups", total);
-    const size_t lds_bytes = static_cast<size_t>(GT_STAGES) * GT_STAGE_ELEMS * 2;
+    // the stages of operands, or the tile on its way out (32-bit rows of 128 with their pitch), whichever is more
+    constexpr size_t out_bytes = static_cast<size_t>(GT_BM) * (EPI == GT_ADD ? GT_BN * 4 + 16 : (EPI == GT_SWIGLU ? GT_BN + 16 : GT_BN * 2 + 16));
+    constexpr size_t stage_bytes = static_cast<size_t>(GT_STAGES) * GT_STAGE_ELEMS * 2;
+    const size_t lds_bytes = out_bytes > stage_bytes ? out_bytes : stage_bytes;
     static bool raised = false;
     if (!raised) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiled_kernel<EPI>),
