@@ -101,6 +101,12 @@ class Engine:
                                          chunk=None if chunk is None else int(chunk),
                                          max_positions=self.model.spec.max_positions, prefix_cache=prefix_cache)
         self.runner = StepRunner(self.model, self.cache, graphs=graphs)
+        # Pages are shared between requests only where every layer keeps all its keys in pages of one size and
+        # no layer keeps state of its own beside them (a window's pages are given back, a state is not in pages):
+        # asked for and not possible is said, in the banner and in the metrics, not passed over.
+        self.prefix_cache = "on" if prefix_cache else "off"
+        if prefix_cache and not self.cache.manager.sharing_possible():
+            self.prefix_cache = "off (asked for; this model's layers keep a window of their keys or state of their own)"
         self.default_max_tokens = max_tokens
         self.sampler = sampler
         self._next_id = 1
@@ -240,6 +246,7 @@ class Engine:
         m.update({k: manager.counter(k) for k in
                   ("available", "total", "in_use", "cached_blocks", "handed_out", "hits", "misses", "evictions")})
         m["wasted_tokens"] = self.scheduler.wasted_tokens()
+        m["prefix_cache"] = self.prefix_cache
         return m
 
     def describe(self) -> str:
@@ -253,7 +260,7 @@ class Engine:
             f"  stop     {self.generation.eos_token_ids}\n"
             f"  cache    {self.num_blocks} blocks of {self.block_size} tokens, "
             f"{self.cache.bytes / 2 ** 30:.2f} GiB, {self.bytes_per_token} bytes a token, "
-            f"{self.num_blocks * self.block_size} tokens held at once")
+            f"{self.num_blocks * self.block_size} tokens held at once, prefix cache {self.prefix_cache}")
 
     @property
     def scheduler_chunk(self):

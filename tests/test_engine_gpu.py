@@ -114,6 +114,8 @@ def test_prefix_sharing_changes_no_token(model_dirs):
     want = off.generate(prompts, max_tokens=8, stop_tokens=[])
     assert [g["tokens"] for g in got] == [w["tokens"] for w in want]
     assert on.metrics()["cached_tokens"] >= 3 * 16 and off.metrics()["cached_tokens"] == 0
+    assert on.metrics()["prefix_cache"] == "on" and "prefix cache on" in on.describe()
+    assert off.metrics()["prefix_cache"] == "off" and "prefix cache off" in off.describe()
     assert got[0]["tokens"] == got[3]["tokens"], "the same prompt gives the same tokens"
 
 

@@ -759,6 +759,14 @@ def test_layers_with_a_window_beside_layers_without(tmp_path, dtype):
     assert r.cache.manager.in_use(1) <= -(-WINDOWED["window"] // 8) + 2
     r.step([], ["x"])
     assert r.cache.manager.in_use(0) == 0 and r.cache.manager.in_use(1) == 0
+    # pages that a window gives back cannot be shared between requests: an engine asked to share them says that it does not
+    from paged_llm_rs_amd import Engine
+
+    engine = Engine(folder, dtype="f32" if dtype == "float32" else "bf16", block_size=8, num_blocks=64, max_batch=2, chunk=16,
+                    prefix_cache=True)
+    assert engine.metrics()["prefix_cache"].startswith("off (asked for") and "prefix cache off (asked for" in engine.describe()
+    twice = engine.generate([prompts["r1"], prompts["r1"]], max_tokens=4, temperature=0.0, stop_tokens=[])
+    assert twice[0]["tokens"] == twice[1]["tokens"] and engine.metrics()["cached_tokens"] == 0
 
 
 # --- a layer that runs twice, and layers that read another layer's keys and values --------------------------------------

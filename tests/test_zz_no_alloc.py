@@ -79,3 +79,26 @@ def test_it_allocates_nothing():
     free_after, _ = torch.cuda.mem_get_info()
     assert free_after == free_before
     assert torch.equal(out.long().cpu(), torch.argmax(logits, dim=-1).cpu())
+
+
+def test_it_runs_where_allocating_is_an_error():
+    """Free memory need not move when a small allocation is made.  A stream that is being captured is a place
+    where hipMalloc and hipFree are errors that end the capture: the entry point is recorded there (as one of the
+    callers it is for would), and the graph, replayed over other logits, gives what the ordinary entry point gives."""
+    lib = _entry_points()
+    logits = torch.randn(11, 4099, device=DEV)
+    out = torch.full((11,), -3, dtype=torch.int32, device=DEV)
+    lib.pl_argmax_static(logits.data_ptr(), out.data_ptr(), 11, 4099, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    out.fill_(-3)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        status = lib.pl_argmax_static(logits.data_ptr(), out.data_ptr(), 11, 4099, torch.cuda.current_stream().cuda_stream)
+    assert status == 0, lib.pl_last_error().decode()
+    assert bool((out == -3).all()), "recorded, not run"
+    for seed in (1, 2, 3):
+        logits.copy_(torch.randn(11, 4099, generator=torch.Generator().manual_seed(seed)))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.long().cpu(), torch.argmax(logits, dim=-1).cpu())
