@@ -191,19 +191,19 @@ class Workbench:
         bench.free()
         return seconds, batch / seconds, self.weight_bytes + batch * context_mid * self.kv_token
 
-    def prefill_point(self, eager: bool = False):
+    def prefill_point(self, eager: bool = False, tokens: int = PREFILL_TOKENS):
         from paged_llm_rs_amd.engine.batch import StepEntry
         from paged_llm_rs_amd.engine.step import run_step
 
-        say(f"prefill, {PREFILL_TOKENS} tokens")
+        say(f"prefill, {tokens} tokens")
         rng = random.Random(2048)
-        prompt = [rng.randrange(self.cfg["vocab_size"]) for _ in range(PREFILL_TOKENS)]
+        prompt = [rng.randrange(self.cfg["vocab_size"]) for _ in range(tokens)]
         cache, model, runner = self.cache, self.model, self.runner
 
         def prefill():
             cache.manager.add_sequence(1000)
-            assert cache.manager.reserve(1000, PREFILL_TOKENS)
-            entry = [StepEntry(1000, prompt, 0, [PREFILL_TOKENS - 1])]
+            assert cache.manager.reserve(1000, tokens)
+            entry = [StepEntry(1000, prompt, 0, [tokens - 1])]
             if eager:
                 run_step(model, cache, entry)
             else:
@@ -212,9 +212,9 @@ class Workbench:
 
         seconds_prefill = timed(prefill, 10, 5)
         d, nq = self.cfg["head_dim"], self.cfg["num_attention_heads"]
-        attention_flops = self.layers * 4 * nq * d * (PREFILL_TOKENS * (PREFILL_TOKENS + 1) // 2)
-        flops = self.layer_flops * PREFILL_TOKENS + self.head_flops + attention_flops
-        return {"value": round(PREFILL_TOKENS / seconds_prefill, 1), "tokens": PREFILL_TOKENS,
+        attention_flops = self.layers * 4 * nq * d * (tokens * (tokens + 1) // 2)
+        flops = self.layer_flops * tokens + self.head_flops + attention_flops
+        return {"value": round(tokens / seconds_prefill, 1), "tokens": tokens,
                 "ms": round(seconds_prefill * 1e3, 3),
                 "frac": round(flops / seconds_prefill / MFMA_PEAK["bf16"], 4)}
 
@@ -512,6 +512,11 @@ def main() -> int:
             points["mixed_8b_bound"] = "hbm" if mixed["hbm_floor_ms"] >= mixed["mfma_floor_ms"] else "mfma"
             say("decode, batch 8, of the 8B shape")
             s8, _, bytes8 = other.decode_point(8, 20, 6)
+            # a whole prompt of the shape's own context: 8,192 tokens give every compute unit eight workgroups of
+            # attention and the library whole tiles, which 2,048 tokens of the small shape do not
+            long_prefill = other.prefill_point(tokens=SHAPES["8b"][1]["max_position_embeddings"])
+            points["prefill_8b_8192_ms"] = long_prefill["ms"]
+            points["prefill_8b_8192_frac_mfma"] = long_prefill["frac"]
             other.close()
             points["decode_8b_b8_ms"] = round(s8 * 1e3, 3)
             points["decode_8b_b8_frac_hbm"] = round(bytes8 / s8 / HBM_PEAK, 4)
