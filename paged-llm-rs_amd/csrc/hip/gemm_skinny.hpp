@@ -114,7 +114,8 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
     // may be handed the sums of squares of its rows (a product that adds into the stream reads a part's output,
     // never a norm's)
-    constexpr bool TAKES = PRO == PRO_BF16 && MT == 1 && EPI != EPI_ADD;
+    // (nor a product so deep that it takes sixteen waves: the norm of a stream that wide is not handed forward)
+    constexpr bool TAKES = PRO == PRO_BF16 && MT == 1 && EPI != EPI_ADD && WV <= 8;
     const int nwaves = blockDim.x / PL_WAVE;
     extern __shared__ float sk_lds[];
     // PANEL: [BT * 16][K] bfloat16, in the same place as the partial tiles (which are written when it is done with)
@@ -449,7 +450,7 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
 template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT>
 static int launch_one(int waves, const void* x, const void* w, void* y, const float* gain, float eps,
                       const int* rows, int n, int N_out, int K, int act, const sk_hand_t& hand, hipStream_t stream) {
-    PL_REQUIRE(!hand.parts || (MT == 1 && PRO == PRO_BF16 && EPI != EPI_ADD), "skinny product: this shape of product takes no handed norm");
+    PL_REQUIRE(!hand.parts || (MT == 1 && PRO == PRO_BF16 && EPI != EPI_ADD && WV <= 8), "skinny product: this shape of product takes no handed norm");
     const int row_tiles = pl_ceil_div(n, 16 * MT);   // more than one where launch_mt deals the rows out
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
     constexpr int UA = (WV == 16 && UNR >= 2) ? UNR / 2 : UNR;   // K steps a round when rounds overlap
@@ -512,7 +513,8 @@ gemm_skinny_rows_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ 
                         const float* __restrict__ gain, float eps, const int* __restrict__ rows, int n, int N_out,
                         int K, int act, sk_hand_t hand) {
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
-    constexpr bool TAKES = PRO == PRO_BF16 && EPI != EPI_ADD && WV * 64 >= MT * 256;   // may be handed the sums of squares of its rows
+    // may be handed the sums of squares of its rows (a stream of up to 2,048: eight steps a wave, or sixteen with four tiles of rows)
+    constexpr bool TAKES = PRO == PRO_BF16 && EPI != EPI_ADD && WV * 64 >= MT * 256 && (STEPS <= 8 || MT == 4);
     constexpr int NKS = WV / MT;                                // stretches of K
     extern __shared__ float sk_lds[];
     bf16_t* panel = reinterpret_cast<bf16_t*>(sk_lds);          // [BT * 16][K], pieces permuted
@@ -725,7 +727,8 @@ template <int MT, int WV, int STEPS, int PRO, int EPI, typename OUT>
 static int launch_rows(const void* x, const void* w, void* y, const float* gain, float eps,
                        const int* rows, int n, int N_out, int K, int act, const sk_hand_t& hand, hipStream_t stream) {
     PL_REQUIRE(!hand.x, "skinny product: this shape of product hands nothing forward");
-    PL_REQUIRE(!hand.parts || (PRO == PRO_BF16 && EPI != EPI_ADD && WV * 64 >= MT * 256), "skinny product: this shape of product takes no handed norm");
+    PL_REQUIRE(!hand.parts || (PRO == PRO_BF16 && EPI != EPI_ADD && WV * 64 >= MT * 256 && (STEPS <= 8 || MT == 4)),
+               "skinny product: this shape of product takes no handed norm");
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
     constexpr int NKS = WV / MT;
     const int grid = min(pl_ceil_div(N_out, SK_TILE_N), SK_MAX_GRID);
