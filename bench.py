@@ -83,11 +83,12 @@ def kv_bytes_per_token(cfg: dict, element: int) -> int:
 class DecodeBench:
     """B requests with ``context`` tokens each in the cache, then timed decode steps."""
 
-    def __init__(self, model, cache, runner, batch: int, context: int, seed: int):
-        from paged_llm_rs_amd.engine.batch import StepEntry
+    def __init__(self, model, cache, runner, batch: int, context: int, seed: int, ahead: bool = True):
+        from paged_llm_rs_amd.engine.batch import CannotFeed, StepEntry
 
         self.model, self.cache, self.batch = model, cache, batch
-        self.StepEntry = StepEntry
+        self.StepEntry, self.CannotFeed = StepEntry, CannotFeed
+        self.ahead, self.flight = ahead, None
         rng = random.Random(seed)
         vocab = model.spec.vocab_size
         self.ids = list(range(1, batch + 1))
@@ -108,16 +109,31 @@ class DecodeBench:
         self.tokens = firsts
 
     def step(self) -> None:
+        """Queue one decode step behind the one in flight, fed that step's tokens on the device, then read
+        the tokens of the step in flight: what the engine does while nothing but greedy decoding goes on
+        (``Engine._launch_ahead``).  Every step's tokens reach the host, one step late."""
         manager = self.cache.manager
-        entries = []
-        for i, tok in zip(self.ids, self.tokens):
+        for i in self.ids:
             assert manager.reserve(i, 1)
-            entries.append(self.StepEntry(i, [tok], manager.tokens(i), [0]))
-        out = self.runner.run(entries)
-        self.tokens = out.greedy_tokens().cpu().tolist()   # the tokens the next step is fed
-        self.commit_step(self.cache, entries)
+        out = None
+        if self.ahead and self.flight is not None:
+            entries = [self.StepEntry(i, [0], manager.tokens(i), [0], fed_row=row) for row, i in enumerate(self.ids)]
+            try:
+                out = self.runner.run(entries)
+            except self.CannotFeed:
+                pass
+        if self.flight is not None:
+            self.tokens = self.flight.greedy_on_host()
+            self.flight = None
+        if out is None:
+            entries = [self.StepEntry(i, [tok], manager.tokens(i), [0]) for i, tok in zip(self.ids, self.tokens)]
+            out = self.runner.run(entries)
+        self.commit_step(self.cache, entries)      # queued: written, for every step behind it
+        self.flight = out
 
     def free(self) -> None:
+        if self.flight is not None:
+            self.tokens, self.flight = self.flight.greedy_on_host(), None
         for i in self.ids:
             self.cache.manager.free_sequence(i)
 

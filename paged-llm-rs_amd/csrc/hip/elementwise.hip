@@ -5,13 +5,21 @@
 
 // ---------------------------------------------------------------------------
 // Embedding: out[t, :] = table[ids[t], :] as the 32-bit residual stream.
-// A negative id marks a padding row and gives zeros.
+// A negative id marks a padding row and gives zeros.  With `src` and `fed`, a
+// row t whose src[t] is not negative takes its id from fed[src[t]] instead: the
+// token that the step before chose on the device, which the host has not read
+// when it launches this step.
 // ---------------------------------------------------------------------------
 template <typename T>
-__global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+__global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict__ src,
+                             const int* __restrict__ fed, const T* __restrict__ table,
                              float* __restrict__ out, int H, int V) {
     const int t = blockIdx.x;
-    const int id = ids[t];
+    int id = ids[t];
+    if (src != nullptr) {
+        const int from = src[t];
+        if (from >= 0) id = fed[from];
+    }
     float* o = out + static_cast<size_t>(t) * H;
     if (id < 0 || id >= V) {
         for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = 0.f;
@@ -21,19 +29,27 @@ __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ 
     for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_float(row[i]);
 }
 
-extern "C" int pl_embed(const int* ids, const void* table, int dtype, float* out, int n, int H,
-                        int V, hipStream_t stream) {
+// `src` and `fed` come together or not at all (both null: every id is ids[t]).
+// The caller has checked that every src[t] is a row of `fed`.
+extern "C" int pl_embed_fed(const int* ids, const int* src, const int* fed, const void* table, int dtype,
+                            float* out, int n, int H, int V, hipStream_t stream) {
     PL_REQUIRE(n >= 0 && H > 0 && V > 0, "embed: n %d, width %d, vocabulary %d", n, H, V);
+    PL_REQUIRE((src == nullptr) == (fed == nullptr), "embed: rows fed from the step before need both the rows and the tokens");
     if (n == 0) return 0;
     const int threads = H >= 256 ? 256 : 64;
     if (dtype == PL_DTYPE_F32)
-        embed_kernel<float><<<n, threads, 0, stream>>>(ids, static_cast<const float*>(table), out, H, V);
+        embed_kernel<float><<<n, threads, 0, stream>>>(ids, src, fed, static_cast<const float*>(table), out, H, V);
     else if (dtype == PL_DTYPE_BF16)
-        embed_kernel<bf16_t><<<n, threads, 0, stream>>>(ids, static_cast<const bf16_t*>(table), out, H, V);
+        embed_kernel<bf16_t><<<n, threads, 0, stream>>>(ids, src, fed, static_cast<const bf16_t*>(table), out, H, V);
     else
         PL_REQUIRE(false, "embed: dtype code %d", dtype);
     PL_CHECK_LAUNCH("embed");
     return 0;
+}
+
+extern "C" int pl_embed(const int* ids, const void* table, int dtype, float* out, int n, int H,
+                        int V, hipStream_t stream) {
+    return pl_embed_fed(ids, nullptr, nullptr, table, dtype, out, n, H, V, stream);
 }
 
 // ---------------------------------------------------------------------------

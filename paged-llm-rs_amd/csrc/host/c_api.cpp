@@ -228,25 +228,18 @@ long plh_sched_submit(void* s, uint64_t id, const uint32_t* prompt, size_t lengt
     });
 }
 
-// Decides the next step and keeps it; returns its kind.  sizes: entries, tokens
-// (all entries together), ids, advanced.
-long plh_sched_plan(void* s, size_t* sizes) {
-    return guarded([&] {
-        const Plan& p = static_cast<Scheduler*>(s)->plan();
-        size_t tokens = 0;
-        for (const PlanEntry& e : p.entries) tokens += e.tokens.size();
-        sizes[0] = p.entries.size();
-        sizes[1] = tokens;
-        sizes[2] = p.ids.size();
-        sizes[3] = p.advanced.size();
-        return static_cast<long>(p.kind);
-    });
+static void plan_sizes(const Plan& p, size_t* sizes) {
+    size_t tokens = 0;
+    for (const PlanEntry& e : p.entries) tokens += e.tokens.size();
+    sizes[0] = p.entries.size();
+    sizes[1] = tokens;
+    sizes[2] = p.ids.size();
+    sizes[3] = p.advanced.size();
 }
 
-void plh_sched_plan_read(void* s, uint64_t* entry_id, int* entry_start, int* entry_len, int* entry_wants,
-                         int* entry_state_slot, int* entry_fresh, uint32_t* tokens, uint64_t* ids,
-                         uint64_t* advanced_id, int* advanced_count, uint64_t* refused) {
-    const Plan& p = static_cast<Scheduler*>(s)->last_plan();
+static void plan_read(const Plan& p, uint64_t* entry_id, int* entry_start, int* entry_len, int* entry_wants,
+                      int* entry_state_slot, int* entry_fresh, int* entry_fed_row, uint32_t* tokens, uint64_t* ids,
+                      uint64_t* advanced_id, int* advanced_count, uint64_t* refused) {
     size_t at = 0;
     for (size_t i = 0; i < p.entries.size(); ++i) {
         const PlanEntry& e = p.entries[i];
@@ -256,6 +249,7 @@ void plh_sched_plan_read(void* s, uint64_t* entry_id, int* entry_start, int* ent
         entry_wants[i] = e.wants_logits ? 1 : 0;
         entry_state_slot[i] = e.state_slot;
         entry_fresh[i] = e.state_fresh ? 1 : 0;
+        entry_fed_row[i] = i < p.fed_rows.size() ? p.fed_rows[i] : -1;
         std::memcpy(tokens + at, e.tokens.data(), e.tokens.size() * sizeof(uint32_t));
         at += e.tokens.size();
     }
@@ -267,6 +261,41 @@ void plh_sched_plan_read(void* s, uint64_t* entry_id, int* entry_start, int* ent
     *refused = p.refused;
 }
 
+// Decides the next step and keeps it; returns its kind.  sizes: entries, tokens
+// (all entries together), ids, advanced.
+long plh_sched_plan(void* s, size_t* sizes) {
+    return guarded([&] {
+        const Plan& p = static_cast<Scheduler*>(s)->plan();
+        plan_sizes(p, sizes);
+        return static_cast<long>(p.kind);
+    });
+}
+
+// Reads the planned step; `which` 1 reads the step planned ahead instead.
+void plh_sched_plan_read(void* s, int which, uint64_t* entry_id, int* entry_start, int* entry_len, int* entry_wants,
+                         int* entry_state_slot, int* entry_fresh, int* entry_fed_row, uint32_t* tokens,
+                         uint64_t* ids, uint64_t* advanced_id, int* advanced_count, uint64_t* refused) {
+    const Scheduler* q = static_cast<Scheduler*>(s);
+    const Plan* p = which == 1 ? q->ahead() : &q->last_plan();
+    if (!p) return;
+    plan_read(*p, entry_id, entry_start, entry_len, entry_wants, entry_state_slot, entry_fresh, entry_fed_row,
+              tokens, ids, advanced_id, advanced_count, refused);
+}
+
+// The planned step is queued on the device: the lengths in the cache move.
+long plh_sched_launched(void* s) {
+    return guarded([&] { static_cast<Scheduler*>(s)->launched(); return 0L; });
+}
+// Plans the step behind the launched one, if it can be known: 1 and its sizes, else 0.
+long plh_sched_plan_ahead(void* s, size_t* sizes) {
+    return guarded([&]() -> long {
+        const Plan* p = static_cast<Scheduler*>(s)->plan_ahead();
+        if (!p) return 0L;
+        plan_sizes(*p, sizes);
+        return 1L;
+    });
+}
+void plh_sched_drop_ahead(void* s) { static_cast<Scheduler*>(s)->drop_ahead(); }
 static void read_outcome_sizes(const Outcome& o, size_t* sizes) {
     sizes[0] = o.tokens.size();
     sizes[1] = o.finished.size();

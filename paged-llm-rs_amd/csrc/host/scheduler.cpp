@@ -53,6 +53,8 @@ std::optional<size_t> Scheduler::prompt_in_flight() const {
 // of preference as three separate planners.)
 // ---------------------------------------------------------------------------
 const Plan& Scheduler::plan() {
+    if (!plan_.fed_rows.empty() || ahead_)
+        throw Error("a step planned ahead is on the device: commit it before planning another");
     if (turn_away_front()) return plan_;
     if (chunk_ > 0) {
         // every row carries at least one token, so the allowance bounds the rows as well
@@ -246,21 +248,71 @@ void Scheduler::evict(size_t index) {
     waiting_.push_front(std::move(s));
 }
 
-// The step ran.  Its rows' tokens are now in the pages (the lengths move, and
-// pages that filled up get their names for the prefix cache: only now is it
-// known that the tokens are really there); the sampled tokens join their
-// requests' histories and become what the next step feeds; requests that hit a
-// stop token, their budget or the model's last position are retired
-// (scheduler.rs:717-764).
-const Outcome& Scheduler::commit(const std::vector<uint32_t>& sampled) {
-    outcome_ = Outcome{};
+// The planned step is queued on the device.  Its rows' tokens are in the pages for
+// everything that runs behind it: the lengths move, and pages that filled up get
+// their names for the prefix cache (as far as the history names their tokens: a
+// token that was fed on the device joins the history only at the commit of the
+// step that chose it, and its page is named at the commit after).
+void Scheduler::launched() {
+    if (plan_.launched) return;
+    plan_.launched = true;
     for (const auto& [id, written] : plan_.advanced) {
         Sequence* s = sequence(id);
-        if (!s) continue;
+        if (!s) continue;       // ended by a stop token of the step before, or cancelled
         cache_->advance(id, written);
         s->prompt_left = s->prompt_left > written ? s->prompt_left - written : 0;
         cache_->publish_full(id, s->history.data(), s->history.size());
     }
+}
+
+// The step behind a launched decoding step: a row for every request of that step
+// which it cannot end but by a stop token, fed the token of its row there.
+const Plan* Scheduler::plan_ahead() {
+    if (ahead_) throw Error("a step is planned ahead already");
+    if (plan_.kind != PlanKind::Decode || !plan_.launched || !waiting_.empty()) return nullptr;
+    size_t present = 0;      // (a step that was itself planned ahead may hold rows of requests that have ended since)
+    for (uint64_t id : plan_.ids) present += sequence(id) != nullptr;
+    if (present != running_.size()) return nullptr;              // someone has no row: the planner decides
+    Plan next;
+    next.kind = PlanKind::Decode;
+    for (size_t row = 0; row < plan_.ids.size(); ++row) {
+        Sequence* s = sequence(plan_.ids[row]);
+        if (!s) continue;
+        if (s->finish != Finish::None || s->pending.size() != 1) return nullptr;
+        if (s->generated + 1 >= s->max_tokens) continue;                                   // its last token
+        if (max_positions_ > 0 && s->history.size() + 1 > max_positions_) continue;        // its last position
+        if (!cache_->reserve(s->id, 1)) return nullptr;
+        next.ids.push_back(s->id);
+        next.advanced.emplace_back(s->id, 1);
+        next.entries.push_back(PlanEntry{s->id, cache_->tokens(s->id), std::vector<uint32_t>(1, 0), true,
+                                         s->state_slot, false});
+        next.fed_rows.push_back(static_cast<int>(row));
+    }
+    if (next.entries.empty()) return nullptr;
+    metrics_.steps += 1;
+    metrics_.decode_steps += 1;
+    metrics_.decode_rows += next.entries.size();
+    ahead_ = std::move(next);
+    return &*ahead_;
+}
+
+void Scheduler::drop_ahead() {
+    if (!ahead_) return;
+    metrics_.steps -= 1;
+    metrics_.decode_steps -= 1;
+    metrics_.decode_rows -= ahead_->entries.size();
+    ahead_.reset();           // (the pages reserved for its rows stay with their requests, whose next step needs them)
+}
+
+// The step ran.  The sampled tokens join their requests' histories and become
+// what the next step feeds; requests that hit a stop token, their budget or the
+// model's last position are retired (scheduler.rs:717-764).  A token for a
+// request that is no longer there (a row of a step planned ahead, whose request
+// the step before ended) is dropped.  The step planned ahead, if there is one,
+// becomes the planned step.
+const Outcome& Scheduler::commit(const std::vector<uint32_t>& sampled) {
+    outcome_ = Outcome{};
+    launched();
     const size_t count = std::min(plan_.ids.size(), sampled.size());
     for (size_t i = 0; i < count; ++i) {
         Sequence* s = sequence(plan_.ids[i]);
@@ -285,7 +337,12 @@ const Outcome& Scheduler::commit(const std::vector<uint32_t>& sampled) {
         outcome_pending_refusal_.reset();
     }
     retire(outcome_);
-    plan_ = Plan{};
+    if (ahead_) {
+        plan_ = std::move(*ahead_);
+        ahead_.reset();
+    } else {
+        plan_ = Plan{};
+    }
     return outcome_;
 }
 

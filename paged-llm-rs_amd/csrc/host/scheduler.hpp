@@ -57,6 +57,10 @@ struct Plan {
     std::vector<std::pair<uint64_t, size_t>> advanced;  // (id, tokens written)
     std::vector<PlanEntry> entries;
     uint64_t refused = 0;
+    // A step planned ahead (see plan_ahead): for every entry the row of the step before whose token it is
+    // fed; the entry's own token is a placeholder.  Empty for every other step.
+    std::vector<int> fed_rows;
+    bool launched = false;                              // the lengths in the cache have moved for it
 };
 
 struct FinishedInfo {
@@ -99,6 +103,25 @@ public:
 
     const Plan& plan();
     const Plan& last_plan() const { return plan_; }
+
+    // Decoding a step ahead.  The tokens of a decoding step decide nothing about the next step but which
+    // requests a stop token ends, so the next step can be on the device before they have been read:
+    //   plan(); [run]; launched(); plan_ahead(); [run, fed on the device]; commit(tokens of the first);
+    //   launched(); plan_ahead(); [run]; commit(tokens of the second); ...
+    // `launched` says that the planned step is queued on the device: its tokens are as good as written
+    // for everything queued behind it, so the lengths in the cache move now (commit does this itself
+    // where nobody has).  `plan_ahead` gives the step behind a launched decoding step, or nothing when
+    // that step is not known yet: a request waits or is part-way through its prompt, a resident was left
+    // without a row, or the pools have no page for a row (then the ordinary planner decides who gives
+    // way, after the commit).  Requests that the launched step ends by their budget or the model's last
+    // position have no row in it; one that a stop token ends has, and that row's token is dropped when
+    // it is committed.  After the commit of the step before, the step planned ahead is the planned
+    // step, and `plan` may not be asked until it is committed too.  `drop_ahead` forgets a step planned
+    // ahead that was not launched after all.
+    void launched();
+    const Plan* plan_ahead();
+    const Plan* ahead() const { return ahead_ ? &*ahead_ : nullptr; }
+    void drop_ahead();
     const Outcome& last_outcome() const { return outcome_; }
     // `sampled` is one token per id of the plan, in the same order.
     const Outcome& commit(const std::vector<uint32_t>& sampled);
@@ -139,6 +162,7 @@ private:
     size_t max_positions_;
     Metrics metrics_;
     Plan plan_;
+    std::optional<Plan> ahead_;
     Outcome outcome_;
     std::optional<FinishedInfo> outcome_pending_refusal_;
 };

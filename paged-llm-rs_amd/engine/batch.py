@@ -28,6 +28,9 @@ class StepEntry:
     want: list = field(default_factory=list)
     state_slot: int = -1
     fresh_state: bool = False
+    # For a single token that the host does not know yet: the row of the decoding step launched just before
+    # whose chosen token this is (``tokens`` then holds a placeholder).  -1: ``tokens`` is what is fed.
+    fed_row: int = -1
 
 
 class StepBatch:
@@ -58,6 +61,10 @@ class StepBatch:
             return packed[begin:begin + count].view(*shape)
 
         self.token_ids = view("token_ids", num_tokens)
+        # Rows whose id is a token that the step before left on the device: for each row the row of
+        # ``fed_tokens`` it takes, or -1 for its own ``token_ids``.  Both None where no step feeds another.
+        self.token_src = view("token_src", num_tokens) if "token_src" in layout else None
+        self.fed_tokens = None
         self.positions = view("positions", num_tokens)
         self.seq_of = view("seq_of", num_tokens)
         self.q_start = view("q_start", num_seqs)
@@ -90,6 +97,11 @@ def context_bound(longest: int) -> int:
             return bound + bound // 2
         bound *= 2
     return bound
+
+
+class CannotFeed(Exception):
+    """A step that was to take tokens from the step before on the device cannot: nothing was launched, and
+    the caller reads those tokens and runs the step with them instead."""
 
 
 class CaptureOutgrown(Exception):

@@ -3,7 +3,9 @@
 One iteration (reference: crates/pagedllm-server/src/engine.rs:180-250): ask the
 scheduler for a plan, run the step function, choose a token for every request a
 token comes back for, commit.  A failed step fails the requests in it and
-commits nothing; lengths only move after a step has succeeded.
+commits nothing; lengths only move once a step is on the device.  While only
+greedy decoding goes on, the step after is queued before this one's tokens are
+read (``Engine._launch_ahead``).
 """
 
 from __future__ import annotations
@@ -24,6 +26,7 @@ from ..parts.model import DTYPES, load_model
 from ..sampling.sampler import Sampling
 from ..weights.loader import CheckpointFiles
 from . import scheduler as sched
+from .batch import CannotFeed
 from .step import StepRunner, require_gpu
 
 _seed_counter = itertools.count()
@@ -66,11 +69,18 @@ class Engine:
     (on), ``chunk`` (128; None or "off" runs a prompt whole), ``max_tokens`` (512,
     the budget of a request that names none).  ``num_blocks`` sets the pool
     directly instead of ``cache_mib``.
+
+    ``ahead``: while nothing but greedy decoding is going on, the next step is queued on the device
+    before the tokens of the one before have been read (they are fed to it on the device), so the
+    device does not wait for the host between steps.  The tokens a request gets do not depend on it;
+    a request that arrives meanwhile is admitted one step later, and the row of a request that a
+    stop token has just ended runs once more for nothing.
     """
 
     def __init__(self, model, dtype: str = "auto", block_size: int = 16, cache_mib: int = 3584,
                  num_blocks: Optional[int] = None, max_batch: int = 16, chunk=128, prefix_cache: bool = True,
-                 max_tokens: int = 512, device="cuda:0", sampler: str = "device", graphs: bool = True):
+                 max_tokens: int = 512, device="cuda:0", sampler: str = "device", graphs: bool = True,
+                 ahead: bool = True):
         self.device = require_gpu(device)
         dtype = {"auto": None, "f32": "float32", "bf16": "bfloat16"}.get(dtype, dtype)
         if dtype is None:
@@ -109,6 +119,9 @@ class Engine:
             self.prefix_cache = "off (asked for; this model's layers keep a window of their keys or state of their own)"
         self.default_max_tokens = max_tokens
         self.sampler = sampler
+        self.ahead = bool(ahead)
+        self._flight = None      # (plan, output) of a step that is on the device and not yet committed
+        self.steps_ahead = 0     # steps that were launched before the tokens of the one before were read
         self._next_id = 1
         self._results: dict = {}
         self._open: dict = {}
@@ -164,7 +177,7 @@ class Engine:
         greedy = [self._greedy.get(i, True) for i in plan.ids]
         if self.sampler == "device":
             if all(greedy):
-                return output.greedy_tokens().cpu().tolist()
+                return output.greedy_on_host()
             how = [self.scheduler.sampling_of(i) for i in plan.ids]     # draws the number of a request that samples
             params = torch.tensor([[t, float(k), p, u] for t, k, p, u in how], dtype=torch.float32).pin_memory()
             params = params.to(logits.device, non_blocking=True)
@@ -176,18 +189,28 @@ class Engine:
 
     def step(self):
         """One iteration.  Returns the outcome, or None when there is nothing to run."""
-        plan = self.scheduler.plan()
-        if plan.kind == sched.IDLE:
-            outcome = self.scheduler.drain_finished()
-            self._record(outcome)
-            return outcome if outcome.finished else None
+        if self._flight is not None:
+            plan, output = self._flight       # launched during the step before; by now the planned step
+            self._flight = None
+        else:
+            plan = self.scheduler.plan()
+            if plan.kind == sched.IDLE:
+                outcome = self.scheduler.drain_finished()
+                self._record(outcome)
+                return outcome if outcome.finished else None
+            output = None
         sampled = []
         if plan.entries:
             try:
-                sampled = self._choose(plan, self.runner.run(plan.entries))
+                if output is None:
+                    output = self.runner.run(plan.entries)
+                self._launch_ahead(plan)
+                sampled = self._choose(plan, output)
             except PagedLLMError:
                 # A failed step fails every request in it; nothing was committed
                 # (reference: engine.rs:340-348).
+                self.scheduler.drop_ahead()
+                self._flight = None
                 for e in plan.entries:
                     self.scheduler.cancel(e.seq_id)
                     done = self._open.pop(e.seq_id, None)
@@ -198,6 +221,23 @@ class Engine:
         outcome = self.scheduler.commit(sampled)
         self._record(outcome)
         return outcome
+
+    def _launch_ahead(self, plan) -> None:
+        """With the step of ``plan`` queued on the device: queue the one behind it as well, if it is known
+        without this one's tokens (see ``Scheduler.plan_ahead``) and every request takes its largest logit
+        (a drawn token comes out of a kernel that runs outside the step)."""
+        if not (self.ahead and self.sampler == "device" and plan.kind == sched.DECODE
+                and all(self._greedy.get(i, True) for i in plan.ids)):
+            return
+        self.scheduler.launched()
+        following = self.scheduler.plan_ahead()
+        if following is None:
+            return
+        try:
+            self._flight = (following, self.runner.run(following.entries))
+            self.steps_ahead += 1
+        except CannotFeed:
+            self.scheduler.drop_ahead()      # (a graph has to be captured first: the step runs the ordinary way)
 
     def _record(self, outcome) -> None:
         for seq_id, token in outcome.tokens:
@@ -221,6 +261,8 @@ class Engine:
         while self._open:
             if self.step() is None and self._open:
                 raise PagedLLMError("the scheduler idles while requests are open")
+        if self._flight is not None:
+            self.step()        # a step queued ahead whose requests have all ended: its tokens are dropped
 
     def take_result(self, seq_id: int) -> Completion:
         return self._results.pop(seq_id)
@@ -247,6 +289,7 @@ class Engine:
                   ("available", "total", "in_use", "cached_blocks", "handed_out", "hits", "misses", "evictions")})
         m["wasted_tokens"] = self.scheduler.wasted_tokens()
         m["prefix_cache"] = self.prefix_cache
+        m["steps_ahead"] = self.steps_ahead
         return m
 
     def describe(self) -> str:

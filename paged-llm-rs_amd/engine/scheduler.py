@@ -85,24 +85,48 @@ class Scheduler:
     def plan(self) -> Plan:
         sizes = (ctypes.c_size_t * 4)()
         kind = native.check(self._lib.plh_sched_plan(self._h, sizes))
+        return self._read_plan(kind, sizes, 0)
+
+    def _read_plan(self, kind: int, sizes, which: int) -> Plan:
         n_entries, n_tokens, n_ids, n_adv = (int(x) for x in sizes)
         u64, i32, u32 = ctypes.c_uint64, ctypes.c_int, ctypes.c_uint32
         e_id, e_start, e_len = (u64 * max(n_entries, 1))(), (i32 * max(n_entries, 1))(), (i32 * max(n_entries, 1))()
         e_want, e_slot, e_fresh = (i32 * max(n_entries, 1))(), (i32 * max(n_entries, 1))(), (i32 * max(n_entries, 1))()
+        e_fed = (i32 * max(n_entries, 1))()
         tokens = (u32 * max(n_tokens, 1))()
         ids = (u64 * max(n_ids, 1))()
         a_id, a_n = (u64 * max(n_adv, 1))(), (i32 * max(n_adv, 1))()
         refused = u64(0)
-        self._lib.plh_sched_plan_read(self._h, e_id, e_start, e_len, e_want, e_slot, e_fresh, tokens, ids,
-                                      a_id, a_n, ctypes.byref(refused))
+        self._lib.plh_sched_plan_read(self._h, which, e_id, e_start, e_len, e_want, e_slot, e_fresh, e_fed, tokens,
+                                      ids, a_id, a_n, ctypes.byref(refused))
         entries, at = [], 0
         for i in range(n_entries):
             count = e_len[i]
             entries.append(StepEntry(int(e_id[i]), list(tokens[at:at + count]), e_start[i],
-                                     [count - 1] if e_want[i] else [], e_slot[i], bool(e_fresh[i])))
+                                     [count - 1] if e_want[i] else [], e_slot[i], bool(e_fresh[i]), e_fed[i]))
             at += count
         return Plan(kind, [int(x) for x in ids[:n_ids]], [(int(a_id[i]), a_n[i]) for i in range(n_adv)],
                     entries, int(refused.value))
+
+    def launched(self) -> None:
+        """The planned step is queued on the device: what it writes is there for everything queued behind
+        it, so the lengths in the cache move now.  (``commit`` does this itself where nobody has.)"""
+        native.check(self._lib.plh_sched_launched(self._h))
+
+    def plan_ahead(self):
+        """The step behind a launched decoding step, before that step's tokens are known: a row for every
+        request of it that it can only end by a stop token, each fed on the device the token of its row
+        there (``StepEntry.fed_row``).  None when the next step is not known yet (a request waits, pages
+        have run out, a resident has no row).  Once the step before is committed, the step planned ahead
+        is the planned step: it is committed next, and ``plan`` may not be asked before."""
+        sizes = (ctypes.c_size_t * 4)()
+        if not native.check(self._lib.plh_sched_plan_ahead(self._h, sizes)):
+            return None
+        return self._read_plan(DECODE, sizes, 1)
+
+    def drop_ahead(self) -> None:
+        """Forget the step planned ahead: it was not launched after all."""
+        self._lib.plh_sched_drop_ahead(self._h)
 
     def _read_outcome(self, sizes) -> Outcome:
         n_tok, n_fin = int(sizes[0]), int(sizes[1])

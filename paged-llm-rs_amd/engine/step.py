@@ -9,6 +9,13 @@ HIP graph over static buffers, per (requests, pages a request) bucket, and
 replayed; the descriptor of the step is written into a pinned host buffer by the
 native cache manager and copied in with one transfer.
 
+A plain decoding step may be launched before the host has read the tokens of
+the one before: an entry then names the row of that step whose chosen token it
+feeds (``StepEntry.fed_row``), and the embedding takes the id from the buffer
+that every decoding step's argmax writes.  The chosen tokens also travel to
+pinned memory behind every decoding step, so that reading those of one step does
+not wait for the next, which is already queued behind it.
+
 Any other step costs the host some five milliseconds to launch, which is more
 than the GPU needs for a portion of a few hundred tokens.  Such steps are
 padded with rows that belong to no request up to a bucket of tokens, so that
@@ -28,7 +35,7 @@ import torch
 
 from .. import kernels
 from ..errors import ConfigError, PagedLLMError, TensorError
-from .batch import CaptureOutgrown, StepBatch, TableTooWide, build_batch, context_bound, token_bucket
+from .batch import CannotFeed, CaptureOutgrown, StepBatch, TableTooWide, build_batch, context_bound, token_bucket
 
 GRAPH_MAX_REQUESTS = 256     # requests a captured step may have (steps of more run kernel by kernel)
 SHAPE_GRAPH_ROWS_KEPT = 32768    # rows over all captured shapes of steps other than plain decoding (the
@@ -66,13 +73,25 @@ def commit_step(cache, entries) -> None:
 
 @dataclass
 class StepOutput:
+    """What a step left on the device.  The tensors of a captured step are the graph's own: the next step
+    of the same kind overwrites them."""
     logits: torch.Tensor                      # [wanted, vocabulary], 32-bit, on the device
     greedy: Optional[torch.Tensor] = None     # [wanted] int32 on the device, when already computed
+    sent: Optional[torch.Tensor] = None       # the same in pinned memory, once ``arrived`` has passed
+    arrived: Optional[torch.cuda.Event] = None
 
     def greedy_tokens(self) -> torch.Tensor:
         if self.greedy is None:
             self.greedy = kernels.argmax(self.logits)
         return self.greedy
+
+    def greedy_on_host(self) -> list:
+        """The largest logit's index of every wanted row, as a list.  Waits for this step only, where
+        the step sent its tokens to the host itself."""
+        if self.sent is not None:
+            self.arrived.synchronize()
+            return self.sent.tolist()
+        return self.greedy_tokens().cpu().tolist()
 
 
 def _bucket(n: int, least: int = 1) -> int:
@@ -139,24 +158,35 @@ class _DescriptorRing:
 class DecodeGraph:
     """One decode step for up to ``cap`` requests with up to ``widths[g]`` pages each, captured; or, with
     ``captured=False``, launched kernel by kernel over the same buffers with the same idle rows, so that a
-    runner without graphs computes what one with graphs replays."""
+    runner without graphs computes what one with graphs replays.  The chosen tokens go into the first
+    ``cap`` places of ``chosen``, the runner's buffer, where the next decoding step (of this graph or of
+    another of the runner's) finds the tokens that are fed to it on the device."""
 
-    def __init__(self, model, cache, cap: int, widths: list, captured: bool = True):
+    def __init__(self, model, cache, cap: int, widths: list, chosen: torch.Tensor, captured: bool = True):
         self.model, self.cache, self.cap, self.widths = model, cache, cap, list(widths)
         self.captured = captured
+        self.feeds = bool(getattr(model, "takes_fed_tokens", False))
         pieces = [("token_ids", cap), ("positions", cap), ("seq_of", cap), ("q_start", cap), ("q_len", cap),
                   ("ctx_len", cap), ("state_slots", cap), ("logit_rows", cap)]
+        if self.feeds:
+            pieces.append(("token_src", cap))
         pieces += [(f"block_table_{g}", cap * w) for g, w in enumerate(widths)]
         self.layout, offset = {}, 0
         for name, count in pieces:
             self.layout[name] = (offset, count)
             offset += (count + 3) // 4 * 4
         self.ring = _DescriptorRing(offset)
+        self.sent = [torch.zeros(cap, dtype=torch.int32).pin_memory() for _ in range(self.ring.LAP)]
+        self.arrived = [torch.cuda.Event() for _ in range(self.ring.LAP)]
         self.ids = np.zeros(cap, dtype=np.uint64)
         self.device_buf = torch.zeros(offset, dtype=torch.int32, device=model.device)
         block_size = cache.block_size
         self.batch = StepBatch(self.device_buf, self.layout, cap, cap, list(widths), cap, 1,
                                context_bound(max(widths or [1]) * block_size), [])
+        self.all_chosen = chosen
+        self.tokens = chosen[:cap]
+        if self.feeds:
+            self.batch.fed_tokens = chosen
         for _ in range(self.ring.LAP):         # what no step changes, in every buffer
             h = self.ring.view
             for name in ("seq_of", "q_start", "logit_rows"):
@@ -168,7 +198,6 @@ class DecodeGraph:
             self.ring.advance()
         self.graph = None
         self.logits = None
-        self.tokens = None
 
     def _view(self, name):
         b, c = self.layout[name]
@@ -177,6 +206,8 @@ class DecodeGraph:
     def _idle_rows(self, live: int) -> None:
         """Rows past the live requests are padding: position -1, no pages."""
         self._view("token_ids")[live:] = 0
+        if self.feeds:
+            self._view("token_src")[live:] = -1
         self._view("positions")[live:] = -1
         self._view("ctx_len")[live:] = 0
         self._view("state_slots")[live:] = -1
@@ -185,13 +216,16 @@ class DecodeGraph:
 
     def _forward(self):
         logits = self.model.forward(self.batch, self.cache)
-        return logits, kernels.argmax(logits)
+        kernels.argmax(logits, out=self.tokens)
+        return logits
 
     def capture(self) -> None:
         # The run before the capture (everything that initialises lazily does so there, outside the capture)
         # and the capture itself see a step of idle rows only: they write no page and touch no request's
         # state, so the one replay that follows is the only time the real step runs.  (A mixer that keeps
         # state of its own would otherwise advance it twice on the step that brings a capture about.)
+        # Both overwrite the chosen tokens of the step before, which is why a step that is fed from them
+        # is never the one that brings a capture about.
         self.device_buf.copy_(_all_idle(self.ring.host, self.layout))
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
@@ -201,7 +235,7 @@ class DecodeGraph:
         torch.cuda.synchronize()
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph):
-            self.logits, self.tokens = self._forward()
+            self.logits = self._forward()
 
     def fill(self, entries) -> None:
         """Write the step's descriptor into the pinned buffer.  Raises TableTooWide when a request has
@@ -217,6 +251,8 @@ class DecodeGraph:
                 raise TableTooWide(g, pages)
         tokens = self._view("token_ids")
         tokens[:live] = [e.tokens[0] for e in entries]
+        if self.feeds:
+            self._view("token_src")[:live] = [e.fed_row for e in entries]
         vocab, limit = self.model.spec.vocab_size, self.model.spec.max_positions
         if tokens[:live].min() < 0 or tokens[:live].max() >= vocab:
             raise ConfigError(f"a token id outside the vocabulary of {vocab}")
@@ -226,21 +262,27 @@ class DecodeGraph:
         self._view("state_slots")[:live] = [e.state_slot for e in entries]
         self._idle_rows(live)
 
-    def run(self, entries) -> StepOutput:
+    def run(self, entries, fed: bool = False) -> StepOutput:
+        """``fed``: some entry takes its token from the chosen tokens of the step before.  Raises
+        CannotFeed, before anything is launched, where this step would overwrite them first."""
         live = len(entries)
+        if fed and (not self.feeds or (self.captured and self.graph is None)):
+            raise CannotFeed("this step has to be captured first, which overwrites the chosen tokens")
         self.ring.advance()
         self.fill(entries)
-        if not self.captured:
-            self.device_buf.copy_(self.ring.host, non_blocking=True)
-            self.ring.sent()
-            logits, tokens = self._forward()
-            return StepOutput(logits[:live], tokens[:live])
-        if self.graph is None:
+        if self.captured and self.graph is None:
             self.capture()
         self.device_buf.copy_(self.ring.host, non_blocking=True)
         self.ring.sent()
-        self.graph.replay()
-        return StepOutput(self.logits[:live], self.tokens[:live])
+        if self.captured:
+            self.graph.replay()
+            logits = self.logits
+        else:
+            logits = self._forward()
+        sent, arrived = self.sent[self.ring.at], self.arrived[self.ring.at]
+        sent.copy_(self.tokens, non_blocking=True)
+        arrived.record()
+        return StepOutput(logits[:live], self.tokens[:live], sent[:live], arrived)
 
 
 class ShapeGraph:
@@ -310,6 +352,10 @@ class StepRunner:
         self._shapes: dict = {}          # shape of a step -> ShapeGraph, or None after its first (eager) run
         self.graph_steps = 0
         self.eager_steps = 0
+        # Every decoding step leaves its chosen tokens here, row by row, for a step launched behind it to
+        # take its ids from; ``_feedable`` is how many of them the last step left (0: it was no such step).
+        self._chosen = torch.zeros(GRAPH_MAX_REQUESTS, dtype=torch.int32, device=model.device)
+        self._feedable = 0
 
     def _is_plain_decode(self, entries) -> bool:
         return ((self.use_graphs or self.pads) and 0 < len(entries) <= GRAPH_MAX_REQUESTS
@@ -371,13 +417,22 @@ class StepRunner:
         return [max(len(manager.table(e.seq_id, g)) for e in entries) for g in range(len(self.cache.layout.groups))]
 
     def run(self, entries) -> StepOutput:
+        """Raises CannotFeed, with nothing launched, when an entry is to be fed on the device
+        (``fed_row``) and this step cannot take it so: it is no plain decoding step, the step before was
+        none or had no such row, or its graph has to be captured (again) first."""
         entries = list(entries)
         if not entries:
             raise ConfigError("an empty batch")
+        fed = any(e.fed_row >= 0 for e in entries)
         if not self._is_plain_decode(entries):
+            if fed:
+                raise CannotFeed("only a step of single tokens takes them from the step before")
+            self._feedable = 0
             return self._run_shaped(entries)
         if len({e.seq_id for e in entries}) != len(entries):
             raise ConfigError("a request appears twice in one step")
+        if fed and max(e.fed_row for e in entries) >= self._feedable:
+            raise CannotFeed(f"the step before chose {self._feedable} tokens")
         for e in entries:
             if e.fresh_state and e.state_slot >= 0:
                 self.cache.clear_state_slot(e.state_slot)
@@ -385,17 +440,21 @@ class StepRunner:
         graph = self._graphs.get(cap)
         if graph is not None:
             try:
-                out = graph.run(entries)
+                out = graph.run(entries, fed)
                 self._count(graph)
+                self._feedable = len(entries)
                 return out
             except TableTooWide:
                 pass
+        if fed:
+            raise CannotFeed("a step of this many requests and pages has to be captured first")
         # no graph for this many requests yet, or a request has outgrown the bucket's table
         widths = [_bucket(w + 1, 32) for w in self._widths_needed(entries)]
-        graph = DecodeGraph(self.model, self.cache, cap, widths, captured=self.use_graphs)
+        graph = DecodeGraph(self.model, self.cache, cap, widths, self._chosen, captured=self.use_graphs)
         self._graphs[cap] = graph
         out = graph.run(entries)
         self._count(graph)
+        self._feedable = len(entries)
         return out
 
     def _count(self, graph) -> None:

@@ -28,6 +28,7 @@ def _signatures(lib) -> None:
     lib.pl_abi_version.restype = c_int
     table = {
         "pl_embed": [p, p, i, p, i, i, i, p],
+        "pl_embed_fed": [p, p, p, p, i, p, i, i, i, p],
         "pl_add_rmsnorm": [p, p, p, i, f, p, i, p, i, i, i, p],
         "pl_residual_add": [p, p, i, i, i, p],
         "pl_add_bias": [p, p, i, i, i, i, p],
@@ -107,17 +108,25 @@ def _ptr(t) -> int:
 
 # ---------------------------------------------------------------------------
 
-def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
-    """out[t] = table[ids[t]] as the 32-bit residual stream; a negative id gives zeros."""
+def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = None,
+          src: torch.Tensor | None = None, fed: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t] = table[ids[t]] as the 32-bit residual stream; a negative id gives zeros.  With ``src`` and
+    ``fed`` a row t whose src[t] is not negative takes fed[src[t]] for its id: a token that an earlier
+    kernel left on the device.  (The caller answers for src[t] < len(fed).)"""
     n = ids.numel()
     V, H = table.shape
     _need(ids, "token ids", (n,), torch.int32)
     _need(table, "embedding table")
+    if (src is None) != (fed is None):
+        raise TensorError("rows fed from the device need both their sources and the tokens")
+    if src is not None:
+        _need(src, "sources of the token ids", (n,), torch.int32)
+        _need(fed, "tokens left on the device", None, torch.int32)
     if out is None:
         out = torch.empty((n, H), dtype=torch.float32, device=table.device)
     _need(out, "embedding output", (n, H), torch.float32)
-    _check(library().pl_embed(ids.data_ptr(), table.data_ptr(), _code(table, "embedding table"),
-                              out.data_ptr(), n, H, V, _stream()))
+    _check(library().pl_embed_fed(ids.data_ptr(), _ptr(src), _ptr(fed), table.data_ptr(),
+                                  _code(table, "embedding table"), out.data_ptr(), n, H, V, _stream()))
     return out
 
 

@@ -43,8 +43,10 @@ def _signatures(lib) -> None:
         "plh_sched_set_chunk": ([vp, sz], None), "plh_sched_set_prefix_cache": ([vp, i32], None),
         "plh_sched_submit": ([vp, u64, P(u32), sz, f32, i32, lg, i32, f32, sz, P(u32), sz, u64], lg),
         "plh_sched_plan": ([vp, P(sz)], lg),
-        "plh_sched_plan_read": ([vp, P(u64), P(i32), P(i32), P(i32), P(i32), P(i32), P(u32), P(u64),
+        "plh_sched_plan_read": ([vp, i32, P(u64), P(i32), P(i32), P(i32), P(i32), P(i32), P(i32), P(u32), P(u64),
                                  P(u64), P(i32), P(u64)], None),
+        "plh_sched_launched": ([vp], lg), "plh_sched_plan_ahead": ([vp, P(sz)], lg),
+        "plh_sched_drop_ahead": ([vp], None),
         "plh_sched_commit": ([vp, P(u32), sz, P(sz)], lg),
         "plh_sched_drain_finished": ([vp, P(sz)], lg),
         "plh_sched_outcome_read": ([vp, P(u64), P(u32), P(u64), P(i32), P(u64), P(u64), P(u32)], None),

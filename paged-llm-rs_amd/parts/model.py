@@ -124,6 +124,7 @@ class DecoderModel:
                            and getattr(self.logit_transform, "graph_safe", True))
         # Mixers that hand requests of few tokens to a kernel of their own say from how many tokens on a
         # request counts as a long portion; a step reports the tokens of the shorter ones for each such limit.
+        self.takes_fed_tokens = True      # the embedding reads ``batch.token_src`` / ``batch.fed_tokens``
         self.portion_limits = tuple(sorted({int(limit) for b in self.blocks
                                             for limit in [getattr(getattr(b, "mixer", None), "short_portion", None)]
                                             if limit}))
@@ -143,7 +144,9 @@ class DecoderModel:
                 raise UnsupportedError("named activations are recorded on the 32-bit path only: in bfloat16 "
                                        "most of them are stages inside kernels and never written")
             top = ActivationTrace(trace)
-        resid = kernels.embed(batch.token_ids, self.embed_tokens)
+        fed = getattr(batch, "fed_tokens", None)
+        resid = kernels.embed(batch.token_ids, self.embed_tokens,
+                              src=batch.token_src if fed is not None else None, fed=fed)
         if self.embed_transform is not None:
             resid = self.embed_transform(resid, batch)
         if top is not None:

@@ -340,7 +340,7 @@ def test_the_engines_settings_change_no_token(model_dirs, case):
     name, prompts, max_tokens, settings, sampling = drawn_engine_case(case)
     d = model_dirs(name, "float32")
     roomy = Engine(d, dtype="f32", block_size=16, num_blocks=64 * len(prompts), max_batch=1, chunk=None,
-                   prefix_cache=False, sampler=settings["sampler"])
+                   prefix_cache=False, sampler=settings["sampler"], ahead=False)
     want = roomy.generate(prompts, max_tokens=max_tokens, stop_tokens=[], **sampling)
     engine = Engine(d, dtype="f32", **settings)
     got = engine.generate(prompts, max_tokens=max_tokens, stop_tokens=[], **sampling)
@@ -377,7 +377,7 @@ def test_requests_that_arrive_and_are_cancelled_while_others_run(model_dirs, cas
                     prefix_cache=rng.random() < 0.5, sampler=rng.choice(["device", "host"]))
     d = model_dirs(name, "float32")
     roomy = Engine(d, dtype="f32", block_size=16, num_blocks=64 * len(requests), max_batch=1, chunk=None,
-                   prefix_cache=False, sampler=settings["sampler"])
+                   prefix_cache=False, sampler=settings["sampler"], ahead=False)
     for r in requests:
         i = roomy.submit(r["prompt"], r["max_tokens"], stop_tokens=[], **r["sampling"])
         roomy.run()
@@ -447,3 +447,116 @@ def test_a_long_run_of_arrivals_gives_the_same_tokens_from_graphs_as_kernel_by_k
 
 
 import numpy as np  # noqa: E402
+
+
+# ---------------------------------------------------------------------------
+# Steps queued ahead: the next decoding step is on the device before the tokens of
+# the one before have been read.
+# ---------------------------------------------------------------------------
+
+def _generate_each(engine, prompts, budgets, stop):
+    ids = [engine.submit(p, m, temperature=0.0, stop_tokens=stop) for p, m in zip(prompts, budgets)]
+    engine.run()
+    return [engine.take_result(i) for i in ids]
+
+
+@pytest.mark.parametrize("name,dtype,graphs", [("B", "f32", True), ("C", "f32", True), ("B", "f32", False), ("B", "bf16", True)])
+def test_steps_queued_ahead_change_no_token(model_dirs, name, dtype, graphs):
+    """Requests of different budgets, one of them ended by a stop token in the middle: with the next step
+    queued before a step's tokens are read, every request has the tokens, and the ending, that it has in
+    an engine that reads every step's tokens before it plans the next."""
+    from paged_llm_rs_amd import Engine
+
+    long_name = "float32" if dtype == "f32" else "bfloat16"
+    d = model_dirs(name, long_name)
+    vocab = TINY_INIT[name]["config"]["vocab_size"]
+    prompts = list(ru.make_prompts(vocab, [9, 21, 4, 14, 30], seed=11).values())
+    budgets = [40, 12, 33, 25, 18]
+    settings = dict(dtype=dtype, block_size=8, num_blocks=96, max_batch=8, chunk=64, prefix_cache=False, graphs=graphs)
+    free = _generate_each(Engine(d, ahead=False, **settings), prompts, budgets, [])
+    # a token that a request produces in the middle and not before stops it there (and whomever else it meets)
+    who, at = next((r, i) for r in (2, 0, 3) for i in range(6, len(free[r].tokens) - 2)
+                   if free[r].tokens[i] not in free[r].tokens[:i])
+    mine = free[who].tokens
+    stop = [mine[at]]
+    want = _generate_each(Engine(d, ahead=False, **settings), prompts, budgets, stop)
+    assert want[who].finish == "stop" and want[who].tokens == mine[:at]
+    engine = Engine(d, ahead=True, **settings)
+    got = _generate_each(engine, prompts, budgets, stop)
+    if dtype == "f32":
+        assert [g.tokens for g in got] == [w.tokens for w in want]
+        assert [g.finish for g in got] == [w.finish for w in want]
+    else:
+        # (in bfloat16 the row that runs once more for the stopped request is rounding noise to the others)
+        for prompt, g, budget in zip(prompts, got, budgets):
+            plain_greedy_check(d, prompt, g.tokens, 2e-2)
+            assert g.finish == "stop" or len(g.tokens) == budget
+    m = engine.metrics()
+    assert m["steps_ahead"] >= 20, "hardly a step was queued ahead"
+    assert m["available"] == m["total"]
+    # and a second round on the same engine: whatever was in flight at the end of the first is gone
+    again = _generate_each(engine, prompts, budgets, stop)
+    assert [g.tokens for g in again] == [g.tokens for g in got]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_step_takes_the_tokens_of_the_step_before_on_the_device(model_dirs, dtype):
+    """The step runner alone: decoding steps whose entries name rows of the step before, in another order
+    and fewer of them, give bit for bit the logits of steps that are handed the tokens."""
+    import numpy as np
+
+    from paged_llm_rs_amd.cache import PagedCache
+    from paged_llm_rs_amd.engine.batch import CannotFeed, StepEntry
+    from paged_llm_rs_amd.engine.step import StepRunner, commit_step
+    from paged_llm_rs_amd.parts.model import DTYPES, load_model
+
+    d = model_dirs("B", dtype)
+    _, model = load_model(d, dtype, "cuda:0")
+    vocab = model.spec.vocab_size
+    prompts = ru.make_prompts(vocab, [11, 5, 19, 8], seed=5)
+
+    def play(fed: bool):
+        cache = PagedCache(model.cache_layout, 8, 64, DTYPES[dtype], "cuda:0", max_seqs=8)
+        runner = StepRunner(model, cache)
+        manager = cache.manager
+        ids = {}
+        for i, (name, toks) in enumerate(prompts.items(), start=1):
+            manager.add_sequence(i)
+            assert manager.reserve(i, len(toks))
+            ids[name] = i
+        first = [StepEntry(ids[n], t, 0, [len(t) - 1]) for n, t in prompts.items()]
+        out = runner.run(first)
+        commit_step(cache, first)
+        tokens = dict(zip(ids.values(), out.greedy_on_host()))
+        rows, logits, refused = None, [], 0
+        orders = [[1, 2, 3, 4], [1, 2, 3, 4], [3, 1, 4, 2], [4, 3], [3, 4], [3], [3], [4, 3]]
+        for order in orders:
+            for i in order:
+                assert manager.reserve(i, 1)
+            plain = [StepEntry(i, [tokens[i]], manager.tokens(i), [0]) for i in order]
+            entries = plain
+            if fed and rows is not None and all(i in rows for i in order):
+                entries = [StepEntry(i, [0], manager.tokens(i), [0], fed_row=rows[i]) for i in order]
+            try:
+                out = runner.run(entries)
+            except CannotFeed:
+                refused += 1
+                out = runner.run(plain)
+            commit_step(cache, entries)
+            logits.append(out.logits.cpu().numpy().copy())
+            chosen = out.greedy_on_host()
+            assert chosen == out.logits.argmax(-1).tolist()
+            tokens.update(zip(order, chosen))
+            rows = {i: row for row, i in enumerate(order)}
+        return logits, refused, runner
+
+    handed, _, _ = play(False)
+    taken, refused, runner = play(True)
+    assert refused == 2, "a step that has to be captured first (of 2 requests, of 1) cannot be fed"
+    for step, (a, b) in enumerate(zip(handed, taken)):
+        assert np.array_equal(a, b), f"step {step}"
+    # a row that the step before did not have, and a step of more than single tokens, are refused too
+    with pytest.raises(CannotFeed):
+        runner.run([StepEntry(3, [0], runner.cache.manager.tokens(3), [0], fed_row=2)])
+    with pytest.raises(CannotFeed):
+        runner.run([StepEntry(3, [0, 1], runner.cache.manager.tokens(3), [1], fed_row=0)])

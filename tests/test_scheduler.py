@@ -499,3 +499,168 @@ def test_every_request_finishes_and_every_page_returns_under_random_load(seed):
     assert set(finished) == set(submitted), "a request was lost"
     assert s.manager.available() == blocks and s.manager.live_sequences == 0
     assert all(f.finish in ("stop", "length") for f in finished.values())
+
+
+# ---------------------------------------------------------------------------
+# Decoding a step ahead: the step behind a decoding step is planned, and would be
+# launched, before that step's tokens are known.  (No counterpart in the reference,
+# whose engine reads every step's tokens before it plans the next.)
+# ---------------------------------------------------------------------------
+
+def drive(s, arrivals, token_of, ahead: bool, steps: int = 4000):
+    """Run the scheduler to the end.  ``arrivals``: {iteration: [(id, prompt, max_tokens)]};
+    ``token_of(id, n)`` is the n-th token request id samples.  With ``ahead`` every step that can be is
+    planned before the tokens of the one before are committed, the way the engine does it.  Returns
+    ({id: tokens}, {id: finish}, steps planned ahead)."""
+    out, finish, count, planned_ahead = {}, {}, {}, 0
+    flight = None
+    for it in range(steps):
+        for seq_id, prompt, most in arrivals.get(it, []):
+            s.submit(seq_id, prompt, 0.0, None, None, most, [99], seq_id)
+            out[seq_id], count[seq_id] = [], 0
+        if flight is not None:
+            plan, flight = flight, None
+        else:
+            plan = s.plan()
+            if plan.kind == sched.IDLE:
+                for f in s.drain_finished().finished:
+                    finish[f.id] = f.finish
+                if it > max(arrivals) and not s.running and not s.waiting:
+                    break
+                continue
+        if ahead and plan.kind == sched.DECODE:
+            s.launched()
+            before = {i: s.manager.tokens(i) for i in s.running_ids()}
+            flight = s.plan_ahead()
+            if flight is not None:
+                planned_ahead += 1
+                for e in flight.entries:
+                    assert plan.ids[e.fed_row] == e.seq_id, "a row is fed the token of its own request"
+                    assert e.start == before[e.seq_id] == s.manager.tokens(e.seq_id)
+                    assert e.start + 1 <= s.manager.capacity(e.seq_id)
+        sampled = []
+        for i in plan.ids:
+            sampled.append(token_of(i, count.get(i, 0)))
+            count[i] = count.get(i, 0) + 1
+        outcome = s.commit(sampled)
+        for i, token in outcome.tokens:
+            out[i].append(token)
+        for f in outcome.finished:
+            finish[f.id] = f.finish
+    else:
+        raise AssertionError("the scheduler did not come to an end")
+    return out, finish, planned_ahead
+
+
+def test_a_step_planned_ahead_has_a_row_for_everyone_the_step_before_cannot_end():
+    s = scheduler(64, 4, 4)
+    submit(s, 1, 3, 2)         # its second token is its last
+    submit(s, 2, 5, 10)
+    submit(s, 3, 2, 10)
+    assert step(s)[0].kind == sched.MIXED and not s.waiting     # the prompts: everyone has one token out
+    plan = s.plan()
+    assert plan.kind == sched.DECODE and plan.ids == [1, 2, 3]
+    assert s.plan_ahead() is None, "not before the step is on the device"
+    s.launched()
+    following = s.plan_ahead()
+    assert [e.seq_id for e in following.entries] == [2, 3] and [e.fed_row for e in following.entries] == [1, 2]
+    assert all(e.want == [0] and len(e.tokens) == 1 for e in following.entries)
+    assert [e.start for e in following.entries] == [s.manager.tokens(2), s.manager.tokens(3)]
+    with pytest.raises(Exception, match="planned ahead"):
+        s.plan()
+    outcome = s.commit([7, 7, 7])
+    assert [f.id for f in outcome.finished] == [1]
+    with pytest.raises(Exception, match="planned ahead"):
+        s.plan()               # the step planned ahead is the planned step now
+    outcome = s.commit([8, 8])
+    assert outcome.tokens == [(2, 8), (3, 8)]
+    assert s.plan().ids == [2, 3]
+
+
+def test_a_stop_token_ends_a_request_whose_row_ahead_then_counts_for_nothing():
+    s = scheduler(64, 4, 4)
+    submit(s, 1, 3, 10)
+    submit(s, 2, 3, 10)
+    assert step(s)[0].kind == sched.MIXED and not s.waiting
+    plan = s.plan()
+    s.launched()
+    following = s.plan_ahead()
+    assert [e.seq_id for e in following.entries] == [1, 2]
+    in_use = s.manager.in_use()
+    outcome = s.commit([99, 7])                      # request 1 stops
+    assert [(f.id, f.finish) for f in outcome.finished] == [(1, "stop")]
+    assert s.manager.in_use() < in_use, "its pages are back although its row ahead is still running"
+    outcome = s.commit([5, 6])                       # the step planned ahead: the token of request 1 is dropped
+    assert outcome.tokens == [(2, 6)] and not outcome.finished
+    assert s.plan().ids == [2]
+
+
+def test_nothing_is_planned_ahead_while_a_request_waits_or_pages_are_short():
+    s = scheduler(64, 4, 4)
+    submit(s, 1, 3, 10)
+    assert step(s)[0].kind == sched.MIXED and not s.waiting
+    s.plan()
+    s.launched()
+    submit(s, 2, 3, 10)                              # arrives while the step runs
+    assert s.plan_ahead() is None
+    s.commit([7])
+    assert s.plan().kind == sched.MIXED              # and is admitted by the ordinary planner
+
+    s = scheduler(2, 4, 4)                           # two pages of four tokens
+    submit(s, 1, 3, 100)
+    step(s)                                          # the prompt: 3 tokens
+    for _ in range(3):                               # tokens 4, 5, 6: the second page is taken
+        assert step(s)[0].kind == sched.DECODE
+    s.plan()                                         # token 7
+    s.launched()
+    assert s.plan_ahead() is not None                # token 8 still has a place
+    s.commit([7])
+    s.commit([7])
+    s.plan()                                         # nothing left: alone and out of pages, the request ends
+    s.launched()
+    assert s.plan_ahead() is None
+    s.commit([])
+    assert s.manager.available() == 2
+
+
+def test_a_step_ahead_that_was_not_launched_is_forgotten():
+    s = scheduler(64, 4, 4)
+    submit(s, 1, 3, 10)
+    assert step(s)[0].kind == sched.MIXED and not s.waiting
+    steps = s.metrics()["steps"]
+    s.plan()
+    s.launched()
+    assert s.plan_ahead() is not None
+    s.drop_ahead()
+    assert s.metrics()["steps"] == steps + 1
+    s.commit([7])
+    assert s.plan().ids == [1]                       # the ordinary planner goes on
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_requests_get_the_same_tokens_with_and_without_steps_planned_ahead(seed):
+    rng = random.Random(100 + seed)
+    bs = rng.choice([2, 4, 16])
+    blocks = rng.randrange(10, 40)
+    chunk = rng.choice([None, 8, 32])
+    max_batch = rng.randrange(1, 6)
+    window = rng.choice([0, 0, 3 * bs])
+    arrivals, next_id = {}, 1
+    for it in range(0, 120):
+        if next_id <= 20 and rng.random() < 0.25:
+            n = rng.randrange(1, bs * blocks // 3)
+            arrivals.setdefault(it, []).append((next_id, [rng.randrange(5) for _ in range(n)], rng.randrange(1, 25)))
+            next_id += 1
+    arrivals.setdefault(0, []).append((next_id, [1, 2, 3], 7))
+
+    def token_of(seq_id, n):
+        return 99 if (seq_id * 31 + n * 17) % 23 == 0 else (seq_id + n) % 50
+
+    results = []
+    for ahead in (False, True):
+        s = scheduler(blocks, bs, max_batch, chunk=chunk, window=window)
+        results.append(drive(s, arrivals, token_of, ahead))
+        assert s.manager.available() == blocks and s.manager.live_sequences == 0
+    (plain_out, plain_finish, none), (ahead_out, ahead_finish, some) = results
+    assert none == 0 and some > 0
+    assert ahead_out == plain_out and ahead_finish == plain_finish
