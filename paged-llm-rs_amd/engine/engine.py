@@ -4,8 +4,8 @@ One iteration (reference: crates/pagedllm-server/src/engine.rs:180-250): ask the
 scheduler for a plan, run the step function, choose a token for every request a
 token comes back for, commit.  A failed step fails the requests in it and
 commits nothing; lengths only move once a step is on the device.  While only
-greedy decoding goes on, the step after is queued before this one's tokens are
-read (``Engine._launch_ahead``).
+decoding goes on, the step after is queued before this one's tokens are read
+(``Engine._launch_ahead``).
 """
 
 from __future__ import annotations
@@ -70,8 +70,8 @@ class Engine:
     the budget of a request that names none).  ``num_blocks`` sets the pool
     directly instead of ``cache_mib``.
 
-    ``ahead``: while nothing but greedy decoding is going on, the next step is queued on the device
-    before the tokens of the one before have been read (they are fed to it on the device), so the
+    ``ahead``: while nothing but decoding is going on (and the tokens are chosen on the device: not with
+    ``sampler="host"``), the next step is queued on the device before the tokens of the one before have been read (they are fed to it on the device), so the
     device does not wait for the host between steps.  The tokens a request gets do not depend on it;
     a request that arrives meanwhile is admitted one step later, and the row of a request that a
     stop token has just ended runs once more for nothing.
@@ -165,6 +165,22 @@ class Engine:
 
     # -- the loop ---------------------------------------------------------------------------
 
+    def _draw_on_device(self, ids, logits, out=None) -> torch.Tensor:
+        """One token per row of ``logits`` by the sampling kernel, each with its request's parameters and the
+        next number of the request's generator (a greedy row takes its largest logit and draws nothing)."""
+        how = [self.scheduler.sampling_of(i) for i in ids]
+        params = torch.tensor([[t, float(k), p, u] for t, k, p, u in how], dtype=torch.float32).pin_memory()
+        params = params.to(logits.device, non_blocking=True)
+        return kernels.sample(logits, params[:, 0].contiguous(), params[:, 1].to(torch.int32).contiguous(),
+                              params[:, 2].contiguous(), params[:, 3].contiguous(), out=out)
+
+    def _chooser(self, plan):
+        """What a decoding step of ``plan`` is run with (``StepRunner.run``): nothing where every request
+        takes its largest logit or the host samples; else the sampling kernel, behind the step."""
+        if self.sampler != "device" or all(self._greedy.get(i, True) for i in plan.ids):
+            return None
+        return lambda logits, out: self._draw_on_device(plan.ids, logits, out)
+
     def _choose(self, plan, output) -> list:
         """One token per id of the plan.  On the device (the default) greedy rows are an argmax and
         the others are drawn by the sampling kernel with the next number of the request's generator;
@@ -174,16 +190,10 @@ class Engine:
         logits = output.logits
         if logits.shape[0] != len(plan.ids):
             raise PagedLLMError(f"{logits.shape[0]} rows of logits for {len(plan.ids)} requests")
-        greedy = [self._greedy.get(i, True) for i in plan.ids]
         if self.sampler == "device":
-            if all(greedy):
-                return output.greedy_on_host()
-            how = [self.scheduler.sampling_of(i) for i in plan.ids]     # draws the number of a request that samples
-            params = torch.tensor([[t, float(k), p, u] for t, k, p, u in how], dtype=torch.float32).pin_memory()
-            params = params.to(logits.device, non_blocking=True)
-            picked = kernels.sample(logits, params[:, 0].contiguous(), params[:, 1].to(torch.int32).contiguous(),
-                                    params[:, 2].contiguous(), params[:, 3].contiguous())
-            return picked.cpu().tolist()
+            if output.sent is not None or all(self._greedy.get(i, True) for i in plan.ids):
+                return output.greedy_on_host()     # chosen behind the step already, or largest logits
+            return self._draw_on_device(plan.ids, logits).cpu().tolist()
         host = logits.cpu().numpy()
         return [self.scheduler.sample_on_host(i, host[row]) for row, i in enumerate(plan.ids)]
 
@@ -203,7 +213,7 @@ class Engine:
         if plan.entries:
             try:
                 if output is None:
-                    output = self.runner.run(plan.entries)
+                    output = self.runner.run(plan.entries, self._chooser(plan))
                 self._launch_ahead(plan)
                 sampled = self._choose(plan, output)
             except PagedLLMError:
@@ -224,17 +234,15 @@ class Engine:
 
     def _launch_ahead(self, plan) -> None:
         """With the step of ``plan`` queued on the device: queue the one behind it as well, if it is known
-        without this one's tokens (see ``Scheduler.plan_ahead``) and every request takes its largest logit
-        (a drawn token comes out of a kernel that runs outside the step)."""
-        if not (self.ahead and self.sampler == "device" and plan.kind == sched.DECODE
-                and all(self._greedy.get(i, True) for i in plan.ids)):
+        without this one's tokens (see ``Scheduler.plan_ahead``) and the tokens are chosen on the device."""
+        if not (self.ahead and self.sampler == "device" and plan.kind == sched.DECODE):
             return
         self.scheduler.launched()
         following = self.scheduler.plan_ahead()
         if following is None:
             return
         try:
-            self._flight = (following, self.runner.run(following.entries))
+            self._flight = (following, self.runner.run(following.entries, self._chooser(following)))
             self.steps_ahead += 1
         except CannotFeed:
             self.scheduler.drop_ahead()      # (a graph has to be captured first: the step runs the ordinary way)

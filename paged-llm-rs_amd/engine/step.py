@@ -76,7 +76,9 @@ class StepOutput:
     """What a step left on the device.  The tensors of a captured step are the graph's own: the next step
     of the same kind overwrites them."""
     logits: torch.Tensor                      # [wanted, vocabulary], 32-bit, on the device
-    greedy: Optional[torch.Tensor] = None     # [wanted] int32 on the device, when already computed
+    # [wanted] int32 on the device, when already computed: the largest logit's index of every row, or what
+    # the ``choose`` that the step was run with put in its place
+    greedy: Optional[torch.Tensor] = None
     sent: Optional[torch.Tensor] = None       # the same in pinned memory, once ``arrived`` has passed
     arrived: Optional[torch.cuda.Event] = None
 
@@ -86,8 +88,8 @@ class StepOutput:
         return self.greedy
 
     def greedy_on_host(self) -> list:
-        """The largest logit's index of every wanted row, as a list.  Waits for this step only, where
-        the step sent its tokens to the host itself."""
+        """The chosen token of every wanted row (see ``greedy``), as a list.  Waits for this step only,
+        where the step sent its tokens to the host itself."""
         if self.sent is not None:
             self.arrived.synchronize()
             return self.sent.tolist()
@@ -262,9 +264,11 @@ class DecodeGraph:
         self._view("state_slots")[:live] = [e.state_slot for e in entries]
         self._idle_rows(live)
 
-    def run(self, entries, fed: bool = False) -> StepOutput:
+    def run(self, entries, fed: bool = False, choose=None) -> StepOutput:
         """``fed``: some entry takes its token from the chosen tokens of the step before.  Raises
-        CannotFeed, before anything is launched, where this step would overwrite them first."""
+        CannotFeed, before anything is launched, where this step would overwrite them first.
+        ``choose(logits, out)``: called behind the step to put other tokens than the largest logits'
+        into ``out`` ([live] int32), which is what travels to the host and what a step behind is fed."""
         live = len(entries)
         if fed and (not self.feeds or (self.captured and self.graph is None)):
             raise CannotFeed("this step has to be captured first, which overwrites the chosen tokens")
@@ -279,6 +283,8 @@ class DecodeGraph:
             logits = self.logits
         else:
             logits = self._forward()
+        if choose is not None:
+            choose(logits[:live], self.tokens[:live])
         sent, arrived = self.sent[self.ring.at], self.arrived[self.ring.at]
         sent.copy_(self.tokens, non_blocking=True)
         arrived.record()
@@ -416,10 +422,14 @@ class StepRunner:
         manager = self.cache.manager
         return [max(len(manager.table(e.seq_id, g)) for e in entries) for g in range(len(self.cache.layout.groups))]
 
-    def run(self, entries) -> StepOutput:
+    def run(self, entries, choose=None) -> StepOutput:
         """Raises CannotFeed, with nothing launched, when an entry is to be fed on the device
         (``fed_row``) and this step cannot take it so: it is no plain decoding step, the step before was
-        none or had no such row, or its graph has to be captured (again) first."""
+        none or had no such row, or its graph has to be captured (again) first.
+
+        ``choose(logits, out)``: for a plain decoding step, what picks the tokens instead of the largest
+        logit (``DecodeGraph.run``); it is called only once the step is on the device, and not at all for
+        any other step, whose output then has no chosen tokens."""
         entries = list(entries)
         if not entries:
             raise ConfigError("an empty batch")
@@ -440,7 +450,7 @@ class StepRunner:
         graph = self._graphs.get(cap)
         if graph is not None:
             try:
-                out = graph.run(entries, fed)
+                out = graph.run(entries, fed, choose)
                 self._count(graph)
                 self._feedable = len(entries)
                 return out
@@ -452,7 +462,7 @@ class StepRunner:
         widths = [_bucket(w + 1, 32) for w in self._widths_needed(entries)]
         graph = DecodeGraph(self.model, self.cache, cap, widths, self._chosen, captured=self.use_graphs)
         self._graphs[cap] = graph
-        out = graph.run(entries)
+        out = graph.run(entries, False, choose)
         self._count(graph)
         self._feedable = len(entries)
         return out

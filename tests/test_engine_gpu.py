@@ -454,17 +454,24 @@ import numpy as np  # noqa: E402
 # the one before have been read.
 # ---------------------------------------------------------------------------
 
-def _generate_each(engine, prompts, budgets, stop):
-    ids = [engine.submit(p, m, temperature=0.0, stop_tokens=stop) for p, m in zip(prompts, budgets)]
+def _generate_each(engine, prompts, budgets, stop, drawn=False):
+    how = [dict(temperature=0.0)] * len(prompts)
+    if drawn:        # some draw, some take the largest logit, in one step
+        how = [dict(temperature=0.9, seed=40 + i) if i % 3 else dict(temperature=0.0) for i in range(len(prompts))]
+        how[2] = dict(temperature=1.1, top_k=30, top_p=0.95, seed=7)
+    ids = [engine.submit(p, m, stop_tokens=stop, **h) for p, m, h in zip(prompts, budgets, how)]
     engine.run()
     return [engine.take_result(i) for i in ids]
 
 
-@pytest.mark.parametrize("name,dtype,graphs", [("B", "f32", True), ("C", "f32", True), ("B", "f32", False), ("B", "bf16", True)])
-def test_steps_queued_ahead_change_no_token(model_dirs, name, dtype, graphs):
+@pytest.mark.parametrize("name,dtype,graphs,drawn", [("B", "f32", True, False), ("C", "f32", True, False),
+                                                     ("B", "f32", False, False), ("B", "bf16", True, False),
+                                                     ("B", "f32", True, True), ("C", "f32", False, True)])
+def test_steps_queued_ahead_change_no_token(model_dirs, name, dtype, graphs, drawn):
     """Requests of different budgets, one of them ended by a stop token in the middle: with the next step
     queued before a step's tokens are read, every request has the tokens, and the ending, that it has in
-    an engine that reads every step's tokens before it plans the next."""
+    an engine that reads every step's tokens before it plans the next.  ``drawn``: most requests draw
+    their tokens (with seeds), which the sampling kernel does behind each step."""
     from paged_llm_rs_amd import Engine
 
     long_name = "float32" if dtype == "f32" else "bfloat16"
@@ -473,16 +480,16 @@ def test_steps_queued_ahead_change_no_token(model_dirs, name, dtype, graphs):
     prompts = list(ru.make_prompts(vocab, [9, 21, 4, 14, 30], seed=11).values())
     budgets = [40, 12, 33, 25, 18]
     settings = dict(dtype=dtype, block_size=8, num_blocks=96, max_batch=8, chunk=64, prefix_cache=False, graphs=graphs)
-    free = _generate_each(Engine(d, ahead=False, **settings), prompts, budgets, [])
+    free = _generate_each(Engine(d, ahead=False, **settings), prompts, budgets, [], drawn)
     # a token that a request produces in the middle and not before stops it there (and whomever else it meets)
     who, at = next((r, i) for r in (2, 0, 3) for i in range(6, len(free[r].tokens) - 2)
                    if free[r].tokens[i] not in free[r].tokens[:i])
     mine = free[who].tokens
     stop = [mine[at]]
-    want = _generate_each(Engine(d, ahead=False, **settings), prompts, budgets, stop)
+    want = _generate_each(Engine(d, ahead=False, **settings), prompts, budgets, stop, drawn)
     assert want[who].finish == "stop" and want[who].tokens == mine[:at]
     engine = Engine(d, ahead=True, **settings)
-    got = _generate_each(engine, prompts, budgets, stop)
+    got = _generate_each(engine, prompts, budgets, stop, drawn)
     if dtype == "f32":
         assert [g.tokens for g in got] == [w.tokens for w in want]
         assert [g.finish for g in got] == [w.finish for w in want]
@@ -495,7 +502,7 @@ def test_steps_queued_ahead_change_no_token(model_dirs, name, dtype, graphs):
     assert m["steps_ahead"] >= 20, "hardly a step was queued ahead"
     assert m["available"] == m["total"]
     # and a second round on the same engine: whatever was in flight at the end of the first is gone
-    again = _generate_each(engine, prompts, budgets, stop)
+    again = _generate_each(engine, prompts, budgets, stop, drawn)
     assert [g.tokens for g in again] == [g.tokens for g in got]
 
 
