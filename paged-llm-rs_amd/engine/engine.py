@@ -119,7 +119,8 @@ class Engine:
             self.prefix_cache = "off (asked for; this model's layers keep a window of their keys or state of their own)"
         self.default_max_tokens = max_tokens
         self.sampler = sampler
-        self.ahead = bool(ahead)
+        # (a model class whose embedding does not take ids from the device is never fed a step ahead)
+        self.ahead = bool(ahead) and bool(getattr(self.model, "takes_fed_tokens", False))
         self._flight = None      # (plan, output) of a step that is on the device and not yet committed
         self.steps_ahead = 0     # steps that were launched before the tokens of the one before were read
         self._next_id = 1
