@@ -68,7 +68,19 @@ struct sk_hand_t {
     // to a product of bfloat16 rows that such a product left: their stripes' sums of squares [n, count]
     const float* parts;
     int count;
+    // w holds the weights in strips (see "Weights in strips" below)
+    int strips;
 };
+
+// Weights in strips.  Read as [N][K], a wave's load of a K step fetches 64 bytes from each of 16 rows of w that
+// lie K elements apart; the memory gives a pass of such loads less than it gives one that reads front to back
+// (a 201 MB matrix at 8 rows: 48.7 us against 42.9, a 50 MB one 16.4 against 14.5, an 8 MB one 4.9 against 4.6).
+// So the same weights can be handed over in the order the matrix cores take them: strips of 16 rows of w, a
+// strip a run of K/32 tiles of 1 KB, a tile (rows r = 0..15 of the strip, elements 32 t .. 32 t + 31 of K) stored
+// as [4 groups of 8 elements][16 rows][8 elements], which is lane g*16 + r of a wave loading its 16 bytes of the
+// tile at byte (g*16 + r)*16.  A wave's stretch of K of a strip is then one contiguous stretch of memory.  The
+// rows of w (for act(gate) * up: the columns of y, so that the up rows start a strip) have to be a multiple of 16
+// and K of 32, and the kernel for one tile of 16 rows of x is the one that reads them (sk_strips_apply).
 #define SK_HAND_CHUNK 8      // sums a lane adds up: sixteen lanes a row, so count <= 128 (a stream of 2,048)
 
 __device__ __forceinline__ bf16x8 sk_load8(const bf16_t* p) {
@@ -247,6 +259,12 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
         const bf16_t* wrow[BT];
         wrow[0] = w + static_cast<size_t>(col_ok ? n0 + c : 0) * K;
         if (BT == 2) wrow[BT - 1] = w + static_cast<size_t>(N_out + (col_ok ? n0 + c : 0)) * K;
+        if (!PANEL && hand.strips) {       // the strip of the tile, and the lane's 16 bytes of the strip's first tile
+            wrow[0] = w + static_cast<size_t>(tile) * 16 * K + lane * 8;
+            if (BT == 2) wrow[BT - 1] = w + static_cast<size_t>(N_out / 16 + tile) * 16 * K + lane * 8;
+        }
+        // where the lane's 8 values of K step `at` (its own piece at + g*8) stand from wrow
+        const int wmul = (!PANEL && hand.strips) ? 16 : 1, wadd = (!PANEL && hand.strips) ? 0 : g * 8;
 
         if constexpr (PANEL) {
             // the tile's rows of w, 1 KB (64 pieces of a row) a load, dealt to the waves in turn
@@ -276,8 +294,8 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
             if constexpr (AHEAD) {
 #pragma unroll
                 for (int u = 0; u < UNR; ++u) {
-                    const int at = k0 + u * SK_KSTEP + g * 8;
-                    const int kk = at < kend ? at : 0;
+                    const int at = k0 + u * SK_KSTEP;
+                    const int kk = at + g * 8 < kend ? at * wmul + wadd : 0;
 #pragma unroll
                     for (int b = 0; b < BT; ++b) ahead[b][u] = sk_load8(wrow[b] + kk);
                 }
@@ -326,9 +344,9 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
                 } else {
 #pragma unroll
                     for (int u = 0; u < UNR; ++u) {
-                        const int at = k0 + u * SK_KSTEP + g * 8;
-                        const bool k_ok = at < kend;
-                        const int kk = k_ok ? at : 0;
+                        const int at = k0 + u * SK_KSTEP;
+                        const bool k_ok = at + g * 8 < kend;
+                        const int kk = k_ok ? at * wmul + wadd : 0;
 #pragma unroll
                         for (int b = 0; b < BT; ++b) {
                             const bf16x8 got = sk_load8(wrow[b] + kk);
@@ -451,6 +469,7 @@ template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT>
 static int launch_one(int waves, const void* x, const void* w, void* y, const float* gain, float eps,
                       const int* rows, int n, int N_out, int K, int act, const sk_hand_t& hand, hipStream_t stream) {
     PL_REQUIRE(!hand.parts || (MT == 1 && PRO == PRO_BF16 && EPI != EPI_ADD && WV <= 8), "skinny product: this shape of product takes no handed norm");
+    PL_REQUIRE(!hand.strips || MT == 1, "skinny product: this shape of product reads the weights row by row");
     const int row_tiles = pl_ceil_div(n, 16 * MT);   // more than one where launch_mt deals the rows out
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
     constexpr int UA = (WV == 16 && UNR >= 2) ? UNR / 2 : UNR;   // K steps a round when rounds overlap
@@ -727,6 +746,7 @@ template <int MT, int WV, int STEPS, int PRO, int EPI, typename OUT>
 static int launch_rows(const void* x, const void* w, void* y, const float* gain, float eps,
                        const int* rows, int n, int N_out, int K, int act, const sk_hand_t& hand, hipStream_t stream) {
     PL_REQUIRE(!hand.x, "skinny product: this shape of product hands nothing forward");
+    PL_REQUIRE(!hand.strips, "skinny product: this shape of product reads the weights row by row");
     PL_REQUIRE(!hand.parts || (PRO == PRO_BF16 && EPI != EPI_ADD && WV * 64 >= MT * 256 && (STEPS <= 8 || MT == 4)),
                "skinny product: this shape of product takes no handed norm");
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
@@ -755,6 +775,7 @@ static int launch_panel(const void* x, const void* w, void* y, const float* gain
                         const int* rows, int n, int N_out, int K, int act, const sk_hand_t& hand, hipStream_t stream) {
     PL_REQUIRE(!hand.parts || (MT == 1 && EPI != EPI_ADD), "skinny product: this shape of product takes no handed norm");
     PL_REQUIRE(!hand.x, "skinny product: this shape of product hands nothing forward");
+    PL_REQUIRE(!hand.strips, "skinny product: this shape of product reads the weights row by row");
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
     constexpr int waves = 8;
     const int grid = min(pl_ceil_div(N_out, SK_TILE_N), SK_MAX_GRID);
@@ -843,6 +864,13 @@ static int launch_mt(const void* x, const void* w, void* y, const float* gain, f
             return launch_unr<3, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
         default: return launch_unr<4, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
     }
+}
+
+// Whether a product of this shape can read its weights in strips: the layout is defined, and launch_mt takes the
+// kernel for one tile of rows.  N_out: the columns of y.
+static inline bool sk_strips_apply(int n, int N_out, int K) {
+    if (n <= 0 || n > 64 || N_out <= 0 || N_out % SK_TILE_N || K <= 0 || K % SK_KSTEP) return false;
+    return n <= 16 || pl_ceil_div(N_out, SK_TILE_N) * pl_ceil_div(n, 16) <= SK_ROW_TILES_GRID;
 }
 
 // Which kernel the launchers above take for a product of bfloat16 rows, as far as the handed norm goes:

@@ -70,6 +70,9 @@ class Engine:
     the budget of a request that names none).  ``num_blocks`` sets the pool
     directly instead of ``cache_mib``.
 
+    ``strips``: the weights are kept a second time in the order the products of a decoding step read them
+    fastest (``kernels.weights_in_strips``), which costs their memory again.
+
     ``ahead``: while nothing but decoding is going on (and the tokens are chosen on the device: not with
     ``sampler="host"``), the next step is queued on the device before the tokens of the one before have been read (they are fed to it on the device), so the
     device does not wait for the host between steps.  The tokens a request gets do not depend on it;
@@ -80,7 +83,7 @@ class Engine:
     def __init__(self, model, dtype: str = "auto", block_size: int = 16, cache_mib: int = 3584,
                  num_blocks: Optional[int] = None, max_batch: int = 16, chunk=128, prefix_cache: bool = True,
                  max_tokens: int = 512, device="cuda:0", sampler: str = "device", graphs: bool = True,
-                 ahead: bool = True):
+                 ahead: bool = True, strips: bool = True):
         self.device = require_gpu(device)
         dtype = {"auto": None, "f32": "float32", "bf16": "bfloat16"}.get(dtype, dtype)
         if dtype is None:
@@ -95,7 +98,7 @@ class Engine:
             raise ConfigError(f"sampler {sampler!r}, which is neither device nor host")
         self.dtype = dtype
         self.model_dir = Path(model)
-        self.config, self.model = load_model(model, dtype, self.device)
+        self.config, self.model = load_model(model, dtype, self.device, strips=strips)
         self.generation = GenerationConfig.from_dir(model)
         element = 4 if dtype == "float32" else 2
         layout = self.model.cache_layout

@@ -39,8 +39,9 @@ def _signatures(lib) -> None:
         "pl_paged_attention_prefill_tile": [i, i],
         "pl_argmax": [p, p, p, p, i, i, p],
         "pl_sample": [p, p, p, p, p, p, i, i, p],
-        "pl_gemm_skinny": [p, p, p, p, f, p, i, i, i, i, i, i, p],
-        "pl_gemm_skinny_hand": [p, p, p, i, i, i, i, i, i, p, i, f, p, p, p, p],
+        "pl_gemm_skinny": [p, p, p, p, f, p, i, i, i, i, i, i, i, p],
+        "pl_gemm_skinny_strips_apply": [i, i, i],
+        "pl_gemm_skinny_hand": [p, p, p, i, i, i, i, i, i, p, i, f, p, p, p, i, p],
         "pl_gemm_skinny_hand_applies": [i, i, i, i, i],
         "pl_gemm_tiled": [p, p, p, i, i, i, i, i, p],
         "pl_gemm_tiled_applies": [i, i, i, i],
@@ -687,10 +688,32 @@ def takes_handed_norm(rows: int, columns: int, width: int, swiglu: bool = False)
             and bool(library().pl_gemm_skinny_hand_applies(rows, columns, width, 1 if swiglu else 0, 1)))
 
 
+def weights_in_strips(w: torch.Tensor) -> torch.Tensor | None:
+    """The bfloat16 weights ``w`` [N, K] again, in the order the waves of ``gemm_skinny`` take them: strips of 16
+    rows, a strip a run of K/32 tiles of 1 KB, a tile stored as [4 groups of 8 elements][16 rows][8 elements], so
+    that a wave's stretch of K of a strip is one contiguous stretch of memory, which the memory serves faster
+    than 64 bytes from each of 16 rows that lie K elements apart.  The result has the shape of ``w`` and is
+    read by ``gemm_skinny(..., strips=...)`` only.  None where the layout is not defined: rows that are no
+    multiple of 16, a K that is no multiple of 32."""
+    if w.dim() != 2 or w.dtype != torch.bfloat16 or not w.is_cuda:
+        return None
+    N, K = w.shape
+    if N % 16 or K % 32:
+        return None
+    return w.view(N // 16, 16, K // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(N, K)
+
+
+def strips_apply(rows: int, columns: int, width: int) -> bool:
+    """Whether ``gemm_skinny`` of so many rows, with ``columns`` columns of output over an inner width of ``width``,
+    reads weights in strips (its kernel for one tile of 16 rows does)."""
+    return bool(library().pl_gemm_skinny_strips_apply(rows, columns, width))
+
+
 def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, swiglu: bool = False,
                 norm_gain: torch.Tensor | None = None, eps: float = 0.0, rows: torch.Tensor | None = None,
                 add_into: torch.Tensor | None = None, activation: str = "silu",
-                handed: "HandedNorm | None" = None, hand: "HandedNorm | None" = None) -> torch.Tensor:
+                handed: "HandedNorm | None" = None, hand: "HandedNorm | None" = None,
+                strips: torch.Tensor | None = None) -> torch.Tensor:
     """y = x . w^T for up to 64 rows on the matrix cores, the bfloat16 weights streamed once.
 
     ``x`` is bfloat16 [n, K]; or, with ``norm_gain``, the 32-bit residual stream, whose rows
@@ -701,7 +724,8 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
     tensor is returned.
     ``handed``: a norm that an earlier product left behind; its rows are the input (``x`` is not looked at)
     and its sums of squares scale the result.  ``hand`` (with ``add_into``): the norm that follows the
-    stream is left behind in it."""
+    stream is left behind in it.
+    ``strips``: what ``weights_in_strips`` made of ``w``; read instead of ``w`` where ``strips_apply`` says so."""
     if handed is not None:
         if norm_gain is not None or not handed.filled:
             raise TensorError("a handed norm is the product's input by itself, once a product has written it")
@@ -734,6 +758,10 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
             raise TensorError(f"matrix product output {out_dtype}" + (" after the activation" if swiglu else ""))
         out = torch.empty((n, N_out), dtype=out_dtype, device=x.device)
         epilogue, out_f32 = (1 if swiglu else 0), (1 if out_dtype == torch.float32 else 0)
+    in_strips = 0
+    if strips is not None and library().pl_gemm_skinny_strips_apply(n, N_out, K):
+        _need(strips, "weights in strips", tuple(w.shape), torch.bfloat16)
+        w, in_strips = strips, 1
     if handed is not None or hand is not None:
         if hand is not None:
             if add_into is None:
@@ -748,13 +776,13 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
             _ptr(handed.ssq if handed is not None else None), handed.ssq.shape[1] if handed is not None else 0,
             float(handed.eps if handed is not None else 0.0),
             _ptr(hand.gain if hand is not None else None), _ptr(hand.x if hand is not None else None),
-            _ptr(hand.ssq if hand is not None else None), _stream()))
+            _ptr(hand.ssq if hand is not None else None), in_strips, _stream()))
         if hand is not None:
             hand.filled = True
         return out
     _check(library().pl_gemm_skinny(
         x.data_ptr(), w.data_ptr(), out.data_ptr(), _ptr(norm_gain), float(eps), _ptr(rows), n, N_out, K,
-        epilogue, out_f32, activation_code(activation), _stream()))
+        epilogue, out_f32, activation_code(activation), in_strips, _stream()))
     return out
 
 
@@ -960,9 +988,11 @@ def fused_norm_applies(rows_out: int, width: int, weight: torch.Tensor) -> bool:
             and skinny_wins(rows_out, weight.shape[0], width))
 
 
-def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype,
+                strips: torch.Tensor | None = None) -> torch.Tensor:
     """y = x . w^T for bfloat16 operands with 32-bit accumulation: few rows stream the
-    weights through the hand-written kernel, many rows go to the library's product."""
+    weights through the hand-written kernel, many rows go to the library's product.
+    ``strips``: the weights again as ``weights_in_strips`` lays them out, for the product that reads them so."""
     _need(x, "matrix product input", None, torch.bfloat16)
     _need(w, "weight", None, torch.bfloat16)
     if out_dtype == torch.float32:
@@ -970,12 +1000,12 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> tor
         if stream_wins(x.shape[0], w.shape[0], x.shape[1]):
             return gemm_stream(x, w, torch.float32)
         if skinny_applies(x) and x.shape[1] <= (SKINNY_F32_FEW_K if x.shape[0] <= 16 else SKINNY_SHALLOW_K):
-            return gemm_skinny(x, w, torch.float32)
+            return gemm_skinny(x, w, torch.float32, strips=strips)
         if x.shape[1] % 8 == 0:
             return torch.mm(x, w.t(), out_dtype=torch.float32)
         return gemm_plain(x, w, out_dtype=torch.float32)
     if skinny_applies(x, w):
-        return gemm_skinny(x, w, out_dtype)
+        return gemm_skinny(x, w, out_dtype, strips=strips)
     if stream_wins(x.shape[0], w.shape[0], x.shape[1]):
         return gemm_stream(x, w, out_dtype)
     splits = library_splits(x.shape[0], w.shape[0], x.shape[1])

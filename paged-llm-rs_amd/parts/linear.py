@@ -13,10 +13,16 @@ from .norm import PendingNorm
 
 
 class Linear:
+    # Whether a bfloat16 weight is kept a second time in the order the product of few rows reads fastest
+    # (``kernels.weights_in_strips``): the decoding steps then read that copy, everything else the weight as
+    # stored.  It doubles the memory of the weights; ``load_model(..., strips=False)`` builds a model without.
+    keep_strips = True
+
     def __init__(self, weight: torch.Tensor, bias: torch.Tensor | None = None):
         if weight.dim() != 2:
             raise TensorError(f"a linear weight of shape {tuple(weight.shape)}")
         self.weight = weight.contiguous()
+        self.strips = kernels.weights_in_strips(self.weight) if Linear.keep_strips else None
         self.out_features, self.in_features = weight.shape
         if bias is not None and tuple(bias.shape) != (self.out_features,):
             raise TensorError(f"a bias of shape {tuple(bias.shape)} for {self.out_features} outputs")
@@ -58,12 +64,13 @@ class Linear:
             if (x.handed is not None and add_into is None and self.weight.dtype == torch.bfloat16
                     and kernels.takes_handed_norm(x.num_rows, columns, self.in_features, swiglu)):
                 return kernels.gemm_skinny(None, self.weight, out_dtype or x.out_dtype, swiglu=swiglu,
-                                           activation=activation, handed=x.handed)
+                                           activation=activation, handed=x.handed, strips=self.strips)
             if (getattr(x.norm, "fuses_into_product", False) and add_into is None
                     and kernels.fused_norm_applies(x.num_rows, self.in_features, self.weight)
                     and self.out_features <= kernels.FUSED_NORM_MAX_COLUMNS):
                 return kernels.gemm_skinny(x.resid, self.weight, out_dtype or x.out_dtype, swiglu=swiglu,
-                                           norm_gain=x.norm.gain32, eps=x.norm.eps, rows=x.rows, activation=activation)
+                                           norm_gain=x.norm.gain32, eps=x.norm.eps, rows=x.rows, activation=activation,
+                                           strips=self.strips)
             x = x.materialize()
         if x.dim() != 2 or x.shape[1] != self.in_features:
             raise TensorError(f"a linear of {self.in_features} inputs given {tuple(x.shape)}")
@@ -78,9 +85,10 @@ class Linear:
             if add_into is not None and not swiglu:
                 if hand is not None and not kernels.hands_norm_forward(x.shape[0], self.out_features, self.in_features):
                     hand = None
-                kernels.gemm_skinny(x, self.weight, add_into=add_into, hand=hand)
+                kernels.gemm_skinny(x, self.weight, add_into=add_into, hand=hand, strips=self.strips)
                 return None
-            return kernels.gemm_skinny(x, self.weight, out_dtype, swiglu=swiglu, activation=activation)
+            return kernels.gemm_skinny(x, self.weight, out_dtype, swiglu=swiglu, activation=activation,
+                                       strips=self.strips)
         if kernels.stream_wins(x.shape[0], self.out_features, self.in_features):
             if add_into is not None and not swiglu:
                 kernels.gemm_stream(x, self.weight, add_into=add_into)
@@ -94,5 +102,5 @@ class Linear:
         if swiglu:
             if kernels.tiled_swiglu_wins(x.shape[0], self.out_features // 2, self.in_features):
                 return kernels.gemm_tiled(x, self.weight, swiglu=True, activation=activation)
-            return kernels.swiglu(kernels.linear_bf16(x, self.weight, x.dtype), activation=activation)
-        return kernels.linear_bf16(x, self.weight, out_dtype)
+            return kernels.swiglu(kernels.linear_bf16(x, self.weight, x.dtype, self.strips), activation=activation)
+        return kernels.linear_bf16(x, self.weight, out_dtype, self.strips)

@@ -289,6 +289,65 @@ def test_gemm_skinny_with_the_norm_before_and_the_residual_after(n, N, K):
     assert rel(resid, want) < 1e-5
 
 
+@pytest.mark.parametrize("n", [1, 8, 16, 17, 40, 64])
+@pytest.mark.parametrize("N,K", [(16, 32), (48, 96), (4096, 1024), (1024, 3072), (6144, 1024), (2064, 4128), (160, 16384),
+                                 (32768 + 32, 512)])
+def test_gemm_skinny_over_weights_in_strips(n, N, K):
+    """The weights in the order the waves take them (strips of 16 rows, tiles of 1 KB): where the product reads
+    them so, every variant gives bit for bit what it gives over the rows: plain, with the norm before, with
+    act(gate) * up, added into the stream, with a norm taken and handed forward; one-hot rows pick single
+    weights.  Where it does not read them so (tiles of rows that go to other kernels), it reads the rows and says
+    so; what the layout is not defined for has none."""
+    from paged_llm_rs_amd import kernels
+
+    x = torch.randn(n, K, device=DEV).bfloat16()
+    w = (torch.randn(N, K, device=DEV) / math.sqrt(K)).bfloat16()
+    strips = kernels.weights_in_strips(w)
+    assert strips.shape == w.shape and strips.dtype == w.dtype
+    assert torch.equal(strips.flatten().sort().values, w.flatten().sort().values), "the same numbers in another order"
+    reads_strips = kernels.strips_apply(n, N, K)
+    assert reads_strips == (n <= 16 or (N // 16) * -(-n // 16) <= 512)
+    # with zeros for the rows, the result says which of the two was read
+    blind = kernels.gemm_skinny(x, torch.zeros_like(w), torch.float32, strips=strips)
+    assert torch.equal(blind, kernels.gemm_skinny(x, w, torch.float32) if reads_strips else torch.zeros_like(blind))
+    for out_dtype in (torch.float32, torch.bfloat16):
+        assert torch.equal(kernels.gemm_skinny(x, w, out_dtype, strips=strips), kernels.gemm_skinny(x, w, out_dtype))
+    a, b = torch.randn(n, N, device=DEV), None
+    b = a.clone()
+    kernels.gemm_skinny(x, w, add_into=a, strips=strips)
+    kernels.gemm_skinny(x, w, add_into=b)
+    assert torch.equal(a, b)
+    if N % 32 == 0:
+        assert kernels.strips_apply(n, N // 2, K) == (n <= 16 or (N // 32) * -(-n // 16) <= 512)
+        for act in ("silu", "gelu_tanh"):
+            assert torch.equal(kernels.gemm_skinny(x, w, swiglu=True, activation=act, strips=strips),
+                               kernels.gemm_skinny(x, w, swiglu=True, activation=act))
+    if K <= 4128:
+        stream = torch.randn(n + 2, K, device=DEV) * 2.0
+        gain = 1 + 0.3 * torch.randn(K, device=DEV)
+        rows = torch.tensor([(5 * i + 1) % (n + 2) for i in range(n)], dtype=torch.int32, device=DEV)
+        assert torch.equal(kernels.gemm_skinny(stream, w, norm_gain=gain, eps=1e-6, rows=rows, strips=strips),
+                           kernels.gemm_skinny(stream, w, norm_gain=gain, eps=1e-6, rows=rows))
+    eye, idx = one_hot_rows(min(n, K), K)
+    assert torch.equal(kernels.gemm_skinny(eye, w, strips=strips), w[:, idx].T.contiguous())
+    # a norm handed forward by a product over strips, and taken by one
+    if kernels.hands_norm_forward(n, N, K) and N <= 2048:
+        gain = 1 + 0.3 * torch.randn(N, device=DEV)
+        outs = []
+        for s in (strips, None):
+            hand = kernels.HandedNorm(gain, 1e-6, n, N, DEV)
+            resid = torch.ones(n, N, device=DEV)
+            kernels.gemm_skinny(x, w, add_into=resid, hand=hand, strips=s)
+            outs.append((resid, hand.x.clone(), hand.ssq.clone()))
+        assert all(torch.equal(p, q) for p, q in zip(*outs))
+        w2 = (torch.randn(64, N, device=DEV) / math.sqrt(N)).bfloat16()
+        if kernels.takes_handed_norm(n, 64, N, False):
+            assert torch.equal(kernels.gemm_skinny(None, w2, handed=hand, strips=kernels.weights_in_strips(w2)),
+                               kernels.gemm_skinny(None, w2, handed=hand))
+    assert kernels.weights_in_strips(w[:N - 8]) is None and kernels.weights_in_strips(w[:, :K - 8].contiguous()) is None
+    assert kernels.weights_in_strips(w.float()) is None
+
+
 def one_hot_rows(n, K):
     """Rows that pick single columns of a weight matrix, and the columns they pick."""
     eye = torch.zeros(n, K, device=DEV, dtype=torch.bfloat16)
