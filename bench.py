@@ -305,17 +305,21 @@ def products_table(torch) -> int:
     for name, columns, width in shapes:
         copies = max(2, min(24, int(1.5e9 // (columns * width * 2))))
         weights = [(torch.randn(columns, width, device=device) / math.sqrt(width)).bfloat16() for _ in range(copies)]
+        strips = [kernels.weights_in_strips(w) for w in weights]
         for rows in (8, 16, 32, 64):
             x = torch.randn(rows, width, device=device).bfloat16()
             entry = {"MB": round(columns * width * 2 / 1e6),
                      "library_us": round(microseconds([lambda w=w: torch.mm(x, w.t()) for w in weights]), 1),
                      "stream_us": round(microseconds([lambda w=w: kernels.gemm_stream(x, w) for w in weights]), 1),
                      "skinny_us": round(microseconds([lambda w=w: kernels.gemm_skinny(x, w) for w in weights]), 1),
+                     "skinny_strips_us": (round(microseconds([lambda w=w, s=s: kernels.gemm_skinny(x, w, strips=s)
+                                                              for w, s in zip(weights, strips)]), 1)
+                                          if kernels.strips_apply(rows, columns, width) else None),
                      "taken": "stream" if kernels.stream_wins(rows, columns, width) else
                               ("skinny" if kernels.skinny_wins(rows, columns, width) else "library")}
             table[f"{name}_rows{rows}"] = entry
             print(f"[bench] {name} {rows} rows: {entry}", file=sys.stderr, flush=True)
-        del weights
+        del weights, strips
     print(json.dumps({"metric": "products of few rows over large weights, microseconds", "unit": "us", "dtype": "bf16",
                       "data": "synthetic: random weights from memory", "products": table}))
     return 0

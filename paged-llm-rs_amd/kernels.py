@@ -797,12 +797,21 @@ SKINNY_SHALLOW_K = 2048
 SKINNY_ROW_TILES_GRID = 512  # column tiles times row tiles up to which the rows are dealt to workgroups too ...
 SKINNY_ROW_TILES_BYTES = 16 << 20   # ... for weights up to this size (4,096 x 4,096 at 32 rows: 19.8 us against the library's 14.0)
 SKINNY_F32_FEW_K = 4096     # the widest stream whose projection onto a large vocabulary it wins, up to 16 rows
+# Over weights in strips, up to 8 rows and a K that sixteen waves cover in one round of loads, it also wins larger
+# matrices (24,576 x 4,096 at 8 rows: 42.6 us against the library's 44 to 46; 10,240 x 5,120: 29.8 against 23.4).
+SKINNY_STRIPS_ROWS = 8
+SKINNY_STRIPS_K = 4096
+SKINNY_STRIPS_BYTES = 256 << 20
 
 
-def skinny_wins(rows: int, weight_rows: int, width: int) -> bool:
+def skinny_wins(rows: int, weight_rows: int, width: int, strips: bool = False) -> bool:
+    """``strips``: the weights are there in strips as well (``weights_in_strips``)."""
     if not 0 < rows <= SKINNY_ROWS or width % 8 or stream_wins(rows, weight_rows, width):
         return False
     if rows <= 16:
+        if (strips and rows <= SKINNY_STRIPS_ROWS and width <= SKINNY_STRIPS_K
+                and weight_rows * width * 2 <= SKINNY_STRIPS_BYTES):
+            return True
         return weight_rows * width * 2 <= SKINNY_WEIGHT_BYTES or width >= SKINNY_DEEP * weight_rows
     # ... or a narrow output, whose tiles of 16 rows go to workgroups of their own (the kernel for up to 16 rows)
     return width <= SKINNY_SHALLOW_K or ((weight_rows // 16) * -(-rows // 16) <= SKINNY_ROW_TILES_GRID
@@ -960,12 +969,12 @@ def gemm_split_library(x: torch.Tensor, w: torch.Tensor, splits: int, out_dtype:
     return out
 
 
-def skinny_applies(x: torch.Tensor, w: torch.Tensor | None = None) -> bool:
+def skinny_applies(x: torch.Tensor, w: torch.Tensor | None = None, strips: bool = False) -> bool:
     """Whether the product of ``x`` goes to the hand-written kernel: whether it can, and, given the
-    weight, whether it is the faster of the two."""
+    weight (and whether it is there in strips as well), whether it is the faster of the two."""
     if x.dtype != torch.bfloat16 or x.shape[0] > SKINNY_ROWS or x.shape[1] % 8:
         return False
-    return w is None or skinny_wins(x.shape[0], w.shape[0], x.shape[1])
+    return w is None or skinny_wins(x.shape[0], w.shape[0], x.shape[1], strips)
 
 
 # A product with more columns than this walks its column tiles in a loop; the norm as its first stage

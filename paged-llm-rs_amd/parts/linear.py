@@ -81,7 +81,7 @@ class Linear:
             # the true 32-bit path: vector-unit multiply-add only
             y = kernels.gemm_plain(x, self.weight, out_dtype=torch.float32)
             return kernels.swiglu(y, activation=activation) if swiglu else y
-        if kernels.skinny_applies(x, self.weight):
+        if kernels.skinny_applies(x, self.weight, self.strips is not None):
             if add_into is not None and not swiglu:
                 if hand is not None and not kernels.hands_norm_forward(x.shape[0], self.out_features, self.in_features):
                     hand = None
