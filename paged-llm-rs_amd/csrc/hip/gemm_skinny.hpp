@@ -611,7 +611,17 @@ gemm_skinny_rows_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ 
 
     for (int tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
         const int n0 = tile * SK_TILE_N;
-        {
+        if (hand.strips) {
+            // the tile's strip (for act(gate) * up: the gate's, then the up's) is K/32 tiles of 1 KB one behind the
+            // other, and goes into LDS as it stands: tile t of a strip is where the lanes of a wave read K step t
+            const int tiles_a_strip = K / SK_KSTEP, loads = BT * tiles_a_strip;
+            for (int j = wave; j < loads; j += WV) {
+                const int b = j / tiles_a_strip, t = j - b * tiles_a_strip;
+                const size_t strip = (b ? N_out / SK_TILE_N : 0) + static_cast<size_t>(tile);
+                sk_load_to_lds(w + (strip * 16 * K + static_cast<size_t>(t) * 512 + lane * 8),
+                               panel + static_cast<size_t>(b) * 16 * K + t * 512);
+            }
+        } else {
             const int chunks = K / 512, loads = BT * 16 * chunks;
             for (int j = wave; j < loads; j += WV) {
                 const int prow = j / chunks, chunk = j - prow * chunks;
@@ -657,7 +667,10 @@ gemm_skinny_rows_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ 
                 kk[j] = kbeg + (live ? u0 + j : 0) * SK_KSTEP + g * 8;
 #pragma unroll
                 for (int b = 0; b < BT; ++b) {
-                    const bf16x8 got = sk_load8(panel + static_cast<size_t>(b * 16 + c) * K + (((kk[j] >> 3) ^ c) << 3));
+                    // (in strips: K step kk / 32 of strip b, the lane's 16 bytes of it)
+                    const size_t at = hand.strips ? static_cast<size_t>(b) * 16 * K + (kk[j] - g * 8) * 16 + lane * 8
+                                                  : static_cast<size_t>(b * 16 + c) * K + (((kk[j] >> 3) ^ c) << 3);
+                    const bf16x8 got = sk_load8(panel + at);
                     bw[j][b] = live ? got : sk_zero8();
                 }
             }
@@ -746,7 +759,6 @@ template <int MT, int WV, int STEPS, int PRO, int EPI, typename OUT>
 static int launch_rows(const void* x, const void* w, void* y, const float* gain, float eps,
                        const int* rows, int n, int N_out, int K, int act, const sk_hand_t& hand, hipStream_t stream) {
     PL_REQUIRE(!hand.x, "skinny product: this shape of product hands nothing forward");
-    PL_REQUIRE(!hand.strips, "skinny product: this shape of product reads the weights row by row");
     PL_REQUIRE(!hand.parts || (PRO == PRO_BF16 && EPI != EPI_ADD && WV * 64 >= MT * 256 && (STEPS <= 8 || MT == 4)),
                "skinny product: this shape of product takes no handed norm");
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
@@ -794,6 +806,21 @@ static int launch_panel(const void* x, const void* w, void* y, const float* gain
     return 0;
 }
 
+// Whether a product of MT tiles of rows goes to the rows kernel (launch_unr's choice, also asked by what decides
+// on strips and handed norms): 16 waves in 16 / MT stretches of K, each a whole number of K steps that a wave can
+// hold at once, the panel (and the norm's gains) within LDS.  steps: the K steps a wave then holds (8 or 16).
+static inline bool sk_rows_kernel_takes(int MT, int K, bool two_tiles, bool norm, int* steps = nullptr) {
+    if (MT != 2 && MT != 4) return false;
+    const int NKS = 16 / MT;
+    const size_t panel = static_cast<size_t>(two_tiles ? 2 : 1) * 16 * K * 2 + (norm ? static_cast<size_t>(K) * 4 : 0);
+    if (K % 512 != 0 || K / SK_KSTEP % NKS != 0 || panel > 144 * 1024) return false;
+    const int need = K / SK_KSTEP / NKS;
+    // (the 32-bit stream takes twice the registers a step; 24 steps would fit the registers of 16 waves only with spills)
+    if (need > (norm ? 8 : 16)) return false;
+    if (steps) *steps = need <= 8 ? 8 : 16;
+    return true;
+}
+
 // How many waves, and how many K steps each asks for at once.  What a wave holds in flight has to fit
 // its registers (512 a lane with four waves, 256 with eight, 128 with sixteen); within that, the
 // fewest waves whose one round of loads covers K are taken, so that the whole matrix is asked for at
@@ -812,17 +839,11 @@ static int launch_unr(const void* x, const void* w, void* y, const float* gain, 
                       const int* rows, int n, int N_out, int K, int act, const sk_hand_t& hand, hipStream_t stream) {
     using S = SkShape<MT, PRO, EPI>;
     if constexpr (MT == 2 || MT == 4) {
-        // 16 waves: 16 / MT stretches of K, each a whole number of K steps that a wave can hold at once
-        constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
-        constexpr int NKS = 16 / MT;
-        const size_t panel = static_cast<size_t>(BT) * 16 * K * 2 + (PRO == PRO_NORM ? static_cast<size_t>(K) * 4 : 0);
-        const int need = K / SK_KSTEP / NKS;             // K steps a wave holds at once
-        if (K % 512 == 0 && K / SK_KSTEP % NKS == 0 && panel <= 144 * 1024) {
-            if (need <= 8) return launch_rows<MT, 16, 8, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
-            if constexpr (PRO == PRO_BF16) {             // the 32-bit stream takes twice the registers a step
-                // (24 steps would fit the registers of 16 waves only with spills: such a K goes the way below)
-                if (need <= 16) return launch_rows<MT, 16, 16, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
-            }
+        int steps = 0;
+        if (sk_rows_kernel_takes(MT, K, EPI == EPI_SWIGLU, PRO == PRO_NORM, &steps)) {
+            if (steps == 8) return launch_rows<MT, 16, 8, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
+            if constexpr (PRO == PRO_BF16)
+                return launch_rows<MT, 16, 16, PRO, EPI, OUT>(x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
         }
     }
     if constexpr (MT >= 2) {
@@ -866,11 +887,15 @@ static int launch_mt(const void* x, const void* w, void* y, const float* gain, f
     }
 }
 
-// Whether a product of this shape can read its weights in strips: the layout is defined, and launch_mt takes the
-// kernel for one tile of rows.  N_out: the columns of y.
-static inline bool sk_strips_apply(int n, int N_out, int K) {
+// Whether a product of this shape reads its weights in strips: the layout is defined, and launch_mt takes the
+// kernel for one tile of rows or the rows kernel.  N_out: the columns of y.  norm: the product starts with the
+// norm of the 32-bit stream; taking: it takes a handed norm.
+static inline bool sk_strips_apply(int n, int N_out, int K, int epilogue, bool norm, bool taking) {
     if (n <= 0 || n > 64 || N_out <= 0 || N_out % SK_TILE_N || K <= 0 || K % SK_KSTEP) return false;
-    return n <= 16 || pl_ceil_div(N_out, SK_TILE_N) * pl_ceil_div(n, 16) <= SK_ROW_TILES_GRID;
+    const int row_tiles = pl_ceil_div(n, 16);
+    if (n <= 16 || pl_ceil_div(N_out, SK_TILE_N) * row_tiles <= SK_ROW_TILES_GRID) return true;
+    const int MT = (taking && row_tiles == 3) ? 4 : row_tiles;
+    return sk_rows_kernel_takes(MT, K, epilogue == EPI_SWIGLU, norm);
 }
 
 // Which kernel the launchers above take for a product of bfloat16 rows, as far as the handed norm goes:
@@ -883,13 +908,7 @@ static inline bool sk_hand_applies(int n, int N_out, int K, int epilogue, bool t
     const int row_tiles = pl_ceil_div(n, 16);
     if (n <= 16 || pl_ceil_div(N_out, SK_TILE_N) * row_tiles <= SK_ROW_TILES_GRID) return true;   // the kernel for one tile of rows
     const int MT = (taking && row_tiles == 3) ? 4 : row_tiles;
-    const int BT = epilogue == EPI_SWIGLU ? 2 : 1;
-    bool rows_kernel = false;
-    if (MT == 2 || MT == 4) {
-        const int NKS = 16 / MT;
-        const size_t panel = static_cast<size_t>(BT) * 16 * K * 2;
-        rows_kernel = K % 512 == 0 && K / SK_KSTEP % NKS == 0 && panel <= 144 * 1024 && K / SK_KSTEP / NKS <= 16;
-    }
+    const bool rows_kernel = sk_rows_kernel_takes(MT, K, epilogue == EPI_SWIGLU, false);
     return taking && rows_kernel;        // (an adding product hands forward from the kernel for one tile of rows only)
 }
 
