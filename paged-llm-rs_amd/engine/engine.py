@@ -307,9 +307,12 @@ class Engine:
     def describe(self) -> str:
         """The start-up banner (reference: main.rs:133-158)."""
         chunk = self.scheduler_chunk
+        stored, strips = self.model.matrix_bytes() if hasattr(self.model, "matrix_bytes") else (0, 0)
         return (
             f"paged-llm-rs_amd\n  model    {self.model_dir}\n"
             f"  backend  MI355X (gfx950), dtype {self.dtype}, chunk {chunk if chunk else 'off'}\n"
+            f"  weights  {stored / 2 ** 30:.2f} GiB of matrices"
+            + (f", and {strips / 2 ** 30:.2f} GiB more for their copies in strips (decoding reads those)\n" if strips else "\n") +
             f"  sampling temperature {self.generation.temperature}, top_p {self.generation.top_p}, "
             f"top_k {self.generation.top_k}, from the model's generation config\n"
             f"  stop     {self.generation.eos_token_ids}\n"

@@ -104,3 +104,23 @@ class Linear:
                 return kernels.gemm_tiled(x, self.weight, swiglu=True, activation=activation)
             return kernels.swiglu(kernels.linear_bf16(x, self.weight, x.dtype, self.strips), activation=activation)
         return kernels.linear_bf16(x, self.weight, out_dtype, self.strips)
+
+
+def linears_of(part, seen=None, depth: int = 0):
+    """Every ``Linear`` that ``part`` holds (its members, their members, the members of lists and tuples; a few
+    levels deep): what a model's memory is made of."""
+    import types
+
+    seen = set() if seen is None else seen
+    if id(part) in seen or depth > 8:
+        return
+    seen.add(id(part))
+    if isinstance(part, Linear):
+        yield part
+    elif isinstance(part, (list, tuple)):
+        for member in part:
+            yield from linears_of(member, seen, depth + 1)
+    elif hasattr(part, "__dict__") and not isinstance(part, (torch.Tensor, type, types.ModuleType, types.FunctionType)):
+        for member in vars(part).values():
+            if not isinstance(member, (torch.Tensor, str, int, float, bool, dict, type(None))):
+                yield from linears_of(member, seen, depth + 1)

@@ -17,7 +17,7 @@ from ..config import load_config
 from ..errors import ConfigError, UnsupportedError, WeightError
 from ..weights.loader import ParamDecl, load_weights
 from . import attention, block, mlp, norm  # noqa: F401  (register the built-in parts)
-from .linear import Linear
+from .linear import Linear, linears_of
 from .norm import PendingNorm
 from .registry import BLOCKS, EMBED_TRANSFORMS, LOGIT_TRANSFORMS, NORMS, lookup, prefixed, scoped
 from .trace import ActivationTrace
@@ -128,6 +128,21 @@ class DecoderModel:
         self.portion_limits = tuple(sorted({int(limit) for b in self.blocks
                                             for limit in [getattr(getattr(b, "mixer", None), "short_portion", None)]
                                             if limit}))
+
+    def matrix_bytes(self) -> tuple:
+        """(bytes of the weight matrices as stored, bytes of their second copies in strips)."""
+        stored = strips = 0
+        tensors = set()
+        for linear in linears_of(self):
+            for which, t in (("stored", linear.weight), ("strips", linear.strips)):
+                if t is None or t.data_ptr() in tensors:
+                    continue
+                tensors.add(t.data_ptr())
+                if which == "stored":
+                    stored += t.numel() * t.element_size()
+                else:
+                    strips += t.numel() * t.element_size()
+        return stored, strips
 
     # -- the forward pass of one step -------------------------------------------------
 

@@ -50,6 +50,10 @@ def test_greedy_generation_matches_the_plain_implementation(model_dirs, name, dt
         plain_greedy_check(d, prompt, result["tokens"], 1e-5 if dtype == "f32" else 2e-2)
     m = engine.metrics()
     assert m["available"] == m["total"] and m["tokens"] == 64
+    # (these sizes are whole strips: a bfloat16 model keeps its matrices a second time, and says so)
+    assert ("GiB more for their copies in strips" in engine.describe()) == (dtype == "bf16" and name in "AB")
+    stored, strips = engine.model.matrix_bytes()
+    assert strips == (stored if dtype == "bf16" and name in "AB" else 0)
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
