@@ -46,6 +46,9 @@ def parser() -> argparse.ArgumentParser:
     p.add_argument("--seed", type=int, default=None)
     p.add_argument("--stop-ids", default=None, help="comma-separated token ids that end a generation")
     p.add_argument("--sampler", default="device", choices=["device", "host"])
+    p.add_argument("--strips", default="on", choices=["on", "off"],
+                   help="keep the weight matrices a second time in the order decoding reads them fastest "
+                        "(their memory again); off reads them as stored")
     # the random-weights mode
     p.add_argument("--random-weights", metavar="CONFIG_JSON",
                    help="write a model folder at --model from this config.json and --init-seed, then run it")
@@ -90,7 +93,7 @@ def main(argv=None) -> int:
         kernels.set_attention(args.attention)
         engine = Engine(args.model, dtype=args.dtype, block_size=args.block_size, cache_mib=args.cache_mib,
                         max_batch=args.max_batch, chunk=chunk, prefix_cache=args.prefix_cache == "on",
-                        max_tokens=args.max_tokens, sampler=args.sampler)
+                        max_tokens=args.max_tokens, sampler=args.sampler, strips=args.strips == "on")
         print(engine.describe(), file=sys.stderr, flush=True)
         if not prompts:
             return 0

@@ -192,6 +192,17 @@ def test_the_command_line(model_dirs, tmp_path):
     bad = subprocess.run([sys.executable, str(ROOT / "bin" / "pagedllm"), "--model", str(d), "--chunk", "0"],
                          capture_output=True, text=True, timeout=600)
     assert bad.returncode == 1 and "--chunk 0" in bad.stderr
+    # bfloat16 with and without the second copy of the matrices: the same tokens, and the banner says which
+    b = model_dirs("A", "bfloat16")
+    runs = {}
+    for strips in ("on", "off"):
+        proc = subprocess.run(
+            [sys.executable, str(ROOT / "bin" / "pagedllm"), "--model", str(b), "--max-tokens", "6", "--strips", strips,
+             "--prompt-ids", "3,17,42,8", "--temperature", "0", "--stop-ids", ""], capture_output=True, text=True, timeout=600)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        assert ("copies in strips" in proc.stderr) == (strips == "on")
+        runs[strips] = json.loads(proc.stdout.strip().splitlines()[0])["tokens"]
+    assert runs["on"] == runs["off"] and len(runs["on"]) == 6
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
