@@ -296,6 +296,7 @@ long plh_sched_plan_ahead(void* s, size_t* sizes) {
     });
 }
 void plh_sched_drop_ahead(void* s) { static_cast<Scheduler*>(s)->drop_ahead(); }
+void plh_sched_abandon(void* s) { static_cast<Scheduler*>(s)->abandon(); }
 static void read_outcome_sizes(const Outcome& o, size_t* sizes) {
     sizes[0] = o.tokens.size();
     sizes[1] = o.finished.size();

@@ -304,6 +304,11 @@ void Scheduler::drop_ahead() {
     ahead_.reset();           // (the pages reserved for its rows stay with their requests, whose next step needs them)
 }
 
+void Scheduler::abandon() {
+    drop_ahead();
+    plan_ = Plan{};
+}
+
 // The step ran.  The sampled tokens join their requests' histories and become
 // what the next step feeds; requests that hit a stop token, their budget or the
 // model's last position are retired (scheduler.rs:717-764).  A token for a

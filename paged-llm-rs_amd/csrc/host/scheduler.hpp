@@ -122,6 +122,9 @@ public:
     const Plan* plan_ahead();
     const Plan* ahead() const { return ahead_ ? &*ahead_ : nullptr; }
     void drop_ahead();
+    // The planned step failed and will not be committed (its requests are cancelled by whoever saw it fail):
+    // it is forgotten, and so is a step planned ahead of it.
+    void abandon();
     const Outcome& last_outcome() const { return outcome_; }
     // `sampled` is one token per id of the plan, in the same order.
     const Outcome& commit(const std::vector<uint32_t>& sampled);

@@ -223,7 +223,7 @@ class Engine:
             except PagedLLMError:
                 # A failed step fails every request in it; nothing was committed
                 # (reference: engine.rs:340-348).
-                self.scheduler.drop_ahead()
+                self.scheduler.abandon()
                 self._flight = None
                 for e in plan.entries:
                     self.scheduler.cancel(e.seq_id)

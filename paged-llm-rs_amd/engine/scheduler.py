@@ -128,6 +128,11 @@ class Scheduler:
         """Forget the step planned ahead: it was not launched after all."""
         self._lib.plh_sched_drop_ahead(self._h)
 
+    def abandon(self) -> None:
+        """The planned step failed and will not be committed: forget it and any step planned ahead of it
+        (the caller cancels its requests)."""
+        self._lib.plh_sched_abandon(self._h)
+
     def _read_outcome(self, sizes) -> Outcome:
         n_tok, n_fin = int(sizes[0]), int(sizes[1])
         u64, i32, u32 = ctypes.c_uint64, ctypes.c_int, ctypes.c_uint32

@@ -46,7 +46,7 @@ def _signatures(lib) -> None:
         "plh_sched_plan_read": ([vp, i32, P(u64), P(i32), P(i32), P(i32), P(i32), P(i32), P(i32), P(u32), P(u64),
                                  P(u64), P(i32), P(u64)], None),
         "plh_sched_launched": ([vp], lg), "plh_sched_plan_ahead": ([vp, P(sz)], lg),
-        "plh_sched_drop_ahead": ([vp], None),
+        "plh_sched_drop_ahead": ([vp], None), "plh_sched_abandon": ([vp], None),
         "plh_sched_commit": ([vp, P(u32), sz, P(sz)], lg),
         "plh_sched_drain_finished": ([vp, P(sz)], lg),
         "plh_sched_outcome_read": ([vp, P(u64), P(u32), P(u64), P(i32), P(u64), P(u64), P(u32)], None),

@@ -582,3 +582,43 @@ def test_a_step_takes_the_tokens_of_the_step_before_on_the_device(model_dirs, dt
         runner.run([StepEntry(3, [0], runner.cache.manager.tokens(3), [0], fed_row=2)])
     with pytest.raises(CannotFeed):
         runner.run([StepEntry(3, [0, 1], runner.cache.manager.tokens(3), [1], fed_row=0)])
+
+
+@pytest.mark.parametrize("ahead,fails_in", [(False, "run"), (True, "run"), (True, "read")])
+def test_a_step_that_fails_fails_its_requests_and_nothing_else(model_dirs, ahead, fails_in, monkeypatch):
+    """The step function refuses a step (forced from the host: the runner is replaced by one that raises; or the
+    read of a step's tokens is): the requests of that step end as failed, nothing of them stays in the cache or the
+    scheduler, whether or not a step was queued ahead, and the engine serves the next request as if nothing had
+    been (reference: engine.rs:340-348)."""
+    from paged_llm_rs_amd import Engine
+    from paged_llm_rs_amd.engine.step import StepOutput
+    from paged_llm_rs_amd.errors import PagedLLMError, TensorError
+
+    d = model_dirs("B", "float32")
+    prompts = list(ru.make_prompts(384, [9, 21, 4], seed=2).values())
+    settings = dict(dtype="f32", block_size=8, num_blocks=64, max_batch=4, chunk=64, prefix_cache=False)
+    want = Engine(d, ahead=False, **settings).generate(prompts[:1], max_tokens=10, stop_tokens=[])
+    engine = Engine(d, ahead=ahead, **settings)
+    ids = [engine.submit(p, 30, temperature=0.0, stop_tokens=[]) for p in prompts]
+    for _ in range(5):
+        engine.step()
+    assert engine.open_requests == 3 and (engine.metrics()["steps_ahead"] > 0) == ahead
+
+    def refuse(*args, **kwargs):
+        raise TensorError("the device said no")
+
+    with monkeypatch.context() as patched:
+        if fails_in == "run":
+            patched.setattr(engine.runner, "run", refuse)
+        else:
+            patched.setattr(StepOutput, "greedy_on_host", refuse)
+        with pytest.raises(PagedLLMError, match="said no"):
+            engine.step()
+    assert engine.open_requests == 0
+    for i in ids:
+        done = engine.take_result(i)
+        assert done.finish == "failed" and 1 <= len(done.tokens) < 30
+    m = engine.metrics()
+    assert m["available"] == m["total"] and engine.scheduler.running == 0 and engine.scheduler.waiting == 0
+    again = engine.generate(prompts[:1], max_tokens=10, stop_tokens=[])
+    assert again[0]["tokens"] == want[0]["tokens"] and again[0]["finish"] == "length"

@@ -637,6 +637,25 @@ def test_a_step_ahead_that_was_not_launched_is_forgotten():
     assert s.plan().ids == [1]                       # the ordinary planner goes on
 
 
+def test_a_failed_step_is_abandoned_with_what_was_planned_ahead_of_it():
+    s = scheduler(64, 4, 4)
+    submit(s, 1, 3, 10)
+    submit(s, 2, 3, 10)
+    assert step(s)[0].kind == sched.MIXED and not s.waiting
+    s.plan()
+    s.launched()
+    assert s.plan_ahead() is not None
+    s.commit([7, 7])                                 # the step planned ahead is the planned step now ...
+    s.abandon()                                      # ... and fails: whoever saw that cancels its requests
+    s.cancel(1)
+    assert s.plan().ids == [2]
+    s.launched()
+    assert s.plan_ahead() is not None
+    s.abandon()                                      # a step and the one planned ahead of it
+    s.cancel(2)
+    assert s.plan().kind == sched.IDLE and s.manager.available() == 64
+
+
 @pytest.mark.parametrize("seed", range(6))
 def test_requests_get_the_same_tokens_with_and_without_steps_planned_ahead(seed):
     rng = random.Random(100 + seed)
