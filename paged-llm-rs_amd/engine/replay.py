@@ -19,10 +19,11 @@ class Replayer:
     LIVE_AT_MOST = 4        # requests that a trace holds at a time
 
     def __init__(self, model_dir, dtype: str, max_tokens: int, block_size: int = 16, device="cuda:0",
-                 max_live: int = 64, graphs: bool = True, pages: int | None = None):
-        """``pages`` sets the pool's size by hand instead of deriving it from ``max_tokens``."""
+                 max_live: int = 64, graphs: bool = True, pages: int | None = None, strips: bool = True):
+        """``pages`` sets the pool's size by hand instead of deriving it from ``max_tokens``.  ``strips``: as
+        in ``load_model``."""
         device = require_gpu(device)
-        self.config, self.model = load_model(model_dir, dtype, device)
+        self.config, self.model = load_model(model_dir, dtype, device, strips=strips)
         if max_tokens < 1:
             raise ConfigError(f"--max-tokens {max_tokens}")
         # Each live request's tokens are counted rounded up to 64, so a pool of max_tokens/block_size pages

@@ -184,6 +184,31 @@ def test_a_pool_of_exactly_the_pages_a_trace_needs(setups, name, dtype, block_si
         replay(d, dtype, prompts, steps, max_live=4, block_size=block_size, pages=peak - 1)
 
 
+@pytest.mark.parametrize("name,block_size,seed", [("B", 8, 2), ("D", 16, 5), ("E", 16, 6), ("V", 16, 7)])
+def test_the_weights_in_strips_change_no_bit(setups, name, block_size, seed, monkeypatch):
+    """A model that keeps its matrices a second time in strips (the products of few rows read those) and one
+    that does not give bit for bit the same logits, over a mixed schedule and over tails decoded one by one: the
+    layout is another order of the same numbers, summed in the same order.  (Large matrices that only go to
+    this product when they are there in strips are kept from it here: another product rounds otherwise.)"""
+    from paged_llm_rs_amd import kernels
+    from paged_llm_rs_amd.engine.replay import Replayer
+    from paged_llm_rs_amd.parts.linear import linears_of
+
+    monkeypatch.setattr(kernels, "SKINNY_STRIPS_ROWS", 0)
+
+    d, prompts, _ = setups(name, "bfloat16")
+    for steps, live in ((ru.mixed(prompts, seed=seed, max_live=4), 4), (ru.tail_decoded(prompts, 32), 1)):
+        got = []
+        for strips in (True, False):
+            r = Replayer(d, "bfloat16", max_tokens=ru.pool_tokens(prompts, live), block_size=block_size, strips=strips)
+            kept = [l.strips is not None for l in linears_of(r.model)]
+            assert (any(kept) if strips else not any(kept)) and len(kept) >= 5
+            got.append(ru.collect(r, steps))
+        assert got[0].keys() == got[1].keys()
+        for key in got[0]:
+            assert np.array_equal(got[0][key], got[1][key]), f"{key}: the strips change a logit"
+
+
 def test_schedules_agree_with_each_other_in_32_bit(setups):
     """The logits at a position do not depend on how the tokens were cut, beyond rounding."""
     d, prompts, _ = setups("B", "float32")
