@@ -5,7 +5,7 @@
 int sk_launch_norm(int epilogue, int out_f32, const void* x, const void* w, void* y, const float* gain, float eps, const int* rows, int n, int N_out, int K, int act, int strips, hipStream_t stream);
 
 static int sk_launch_plain(int epilogue, int out_f32, const void* x, const void* w, void* y, const float* gain,
-                           float eps, const int* rows, int n, int N_out, int K, int act, const sk_hand_t& hand,
+                           float eps, const int* rows, int n, int N_out, int K, int act, const sk_extras_t& hand,
                            hipStream_t stream) {
     return sk_launch<PRO_BF16>(epilogue, out_f32, x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
 }
@@ -34,7 +34,7 @@ extern "C" int pl_gemm_skinny(const void* x, const void* w, void* y, const float
     PL_REQUIRE(!strips || sk_strips_apply(n, N_out, K, epilogue, gain != nullptr, false),
                "skinny product: %d rows, %d columns, width %d are not read from weights in strips", n, N_out, K);
     if (gain) return sk_launch_norm(epilogue, out_f32, x, w, y, gain, eps, rows, n, N_out, K, act, strips ? 1 : 0, stream);
-    sk_hand_t with{};
+    sk_extras_t with{};
     with.strips = strips ? 1 : 0;
     return sk_launch_plain(epilogue, out_f32, x, w, y, gain, eps, rows, n, N_out, K, act, with, stream);
 }
@@ -68,6 +68,6 @@ extern "C" int pl_gemm_skinny_hand(const void* x, const void* w, void* y, int n,
     if (n == 0) return 0;
     PL_REQUIRE(!strips || sk_strips_apply(n, N_out, K, epilogue, false, ssq_parts != nullptr),
                "skinny product: %d rows, %d columns, width %d are not read from weights in strips", n, N_out, K);
-    sk_hand_t hand{hand_gain, static_cast<bf16_t*>(hand_x), hand_ssq, ssq_parts, ssq_parts ? parts : 0, strips ? 1 : 0};
+    sk_extras_t hand{hand_gain, static_cast<bf16_t*>(hand_x), hand_ssq, ssq_parts, ssq_parts ? parts : 0, strips ? 1 : 0};
     return sk_launch_plain(epilogue, out_f32, x, w, y, nullptr, eps, nullptr, n, N_out, K, act, hand, stream);
 }

@@ -58,8 +58,9 @@ struct __attribute__((aligned(16))) sk_u32x4 {
     uint32_t v[4];
 };
 
-// What is handed forward (see above).  All null: nothing is.
-struct sk_hand_t {
+// What a launch carries beside its operands: a norm handed forward (see above; all null: none is), and how
+// the weights are laid out.  (The kernels' parameter of this type is still called `hand`.)
+struct sk_extras_t {
     // from a product that adds into the stream: the next norm's gains [N_out]; x [n, N_out] takes
     // bf16(stream * gain) and ssq [n, column tiles] the stripes' sums of squares
     const float* gain;
@@ -122,7 +123,7 @@ template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT, bool PANEL = 
 __global__ void __launch_bounds__(64 * WV)
 gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OUT* __restrict__ y,
                    const float* __restrict__ gain, float eps, const int* __restrict__ rows, int n, int N_out,
-                   int K, int act, sk_hand_t hand) {
+                   int K, int act, sk_extras_t hand) {
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
     // may be handed the sums of squares of its rows (a product that adds into the stream reads a part's output,
     // never a norm's)
@@ -467,7 +468,7 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
 
 template <int MT, int UNR, int WV, int PRO, int EPI, typename OUT>
 static int launch_one(int waves, const void* x, const void* w, void* y, const float* gain, float eps,
-                      const int* rows, int n, int N_out, int K, int act, const sk_hand_t& hand, hipStream_t stream) {
+                      const int* rows, int n, int N_out, int K, int act, const sk_extras_t& hand, hipStream_t stream) {
     PL_REQUIRE(!hand.parts || (MT == 1 && PRO == PRO_BF16 && EPI != EPI_ADD && WV <= 8), "skinny product: this shape of product takes no handed norm");
     PL_REQUIRE(!hand.strips || MT == 1, "skinny product: this shape of product reads the weights row by row");
     const int row_tiles = pl_ceil_div(n, 16 * MT);   // more than one where launch_mt deals the rows out
@@ -530,7 +531,7 @@ template <int MT, int WV, int STEPS, int PRO, int EPI, typename OUT>
 __global__ void __launch_bounds__(64 * WV)
 gemm_skinny_rows_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OUT* __restrict__ y,
                         const float* __restrict__ gain, float eps, const int* __restrict__ rows, int n, int N_out,
-                        int K, int act, sk_hand_t hand) {
+                        int K, int act, sk_extras_t hand) {
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
     // may be handed the sums of squares of its rows (a stream of up to 2,048: eight steps a wave, or sixteen with four tiles of rows)
     constexpr bool TAKES = PRO == PRO_BF16 && EPI != EPI_ADD && WV * 64 >= MT * 256 && (STEPS <= 8 || MT == 4);
@@ -757,7 +758,7 @@ gemm_skinny_rows_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ 
 // The rows variant's launch: WV waves, MT tiles of rows, WV / MT stretches of K of at most STEPS steps.
 template <int MT, int WV, int STEPS, int PRO, int EPI, typename OUT>
 static int launch_rows(const void* x, const void* w, void* y, const float* gain, float eps,
-                       const int* rows, int n, int N_out, int K, int act, const sk_hand_t& hand, hipStream_t stream) {
+                       const int* rows, int n, int N_out, int K, int act, const sk_extras_t& hand, hipStream_t stream) {
     PL_REQUIRE(!hand.x, "skinny product: this shape of product hands nothing forward");
     PL_REQUIRE(!hand.parts || (PRO == PRO_BF16 && EPI != EPI_ADD && WV * 64 >= MT * 256 && (STEPS <= 8 || MT == 4)),
                "skinny product: this shape of product takes no handed norm");
@@ -784,7 +785,7 @@ static int launch_rows(const void* x, const void* w, void* y, const float* gain,
 // The panel variant: 8 waves (256 registers a lane); a wave holds 16 * MT rows of x for UNR K steps.
 template <int MT, int UNR, int PRO, int EPI, typename OUT>
 static int launch_panel(const void* x, const void* w, void* y, const float* gain, float eps,
-                        const int* rows, int n, int N_out, int K, int act, const sk_hand_t& hand, hipStream_t stream) {
+                        const int* rows, int n, int N_out, int K, int act, const sk_extras_t& hand, hipStream_t stream) {
     PL_REQUIRE(!hand.parts || (MT == 1 && EPI != EPI_ADD), "skinny product: this shape of product takes no handed norm");
     PL_REQUIRE(!hand.x, "skinny product: this shape of product hands nothing forward");
     PL_REQUIRE(!hand.strips, "skinny product: this shape of product reads the weights row by row");
@@ -836,7 +837,7 @@ struct SkShape {
 
 template <int MT, int PRO, int EPI, typename OUT>
 static int launch_unr(const void* x, const void* w, void* y, const float* gain, float eps,
-                      const int* rows, int n, int N_out, int K, int act, const sk_hand_t& hand, hipStream_t stream) {
+                      const int* rows, int n, int N_out, int K, int act, const sk_extras_t& hand, hipStream_t stream) {
     using S = SkShape<MT, PRO, EPI>;
     if constexpr (MT == 2 || MT == 4) {
         int steps = 0;
@@ -869,7 +870,7 @@ static int launch_unr(const void* x, const void* w, void* y, const float* gain, 
 
 template <int PRO, int EPI, typename OUT>
 static int launch_mt(const void* x, const void* w, void* y, const float* gain, float eps,
-                     const int* rows, int n, int N_out, int K, int act, const sk_hand_t& hand, hipStream_t stream) {
+                     const int* rows, int n, int N_out, int K, int act, const sk_extras_t& hand, hipStream_t stream) {
     // Few tiles of columns (a narrow output, as of the projections back into the stream): the tiles of 16 rows
     // go to workgroups of their own, the kernel for up to 16 rows on a grid of (column tiles, row tiles), so that
     // the launch has workgroups for every compute unit; each reads its rows of x only, and w comes from L2
@@ -914,7 +915,7 @@ static inline bool sk_hand_applies(int n, int N_out, int K, int epilogue, bool t
 
 template <int PRO>
 static int sk_launch(int epilogue, int out_f32, const void* x, const void* w, void* y, const float* gain,
-                      float eps, const int* rows, int n, int N_out, int K, int act, const sk_hand_t& hand, hipStream_t stream) {
+                      float eps, const int* rows, int n, int N_out, int K, int act, const sk_extras_t& hand, hipStream_t stream) {
     if (epilogue == EPI_STORE)
         return out_f32 ? launch_mt<PRO, EPI_STORE, float>(x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream)
                        : launch_mt<PRO, EPI_STORE, bf16_t>(x, w, y, gain, eps, rows, n, N_out, K, act, hand, stream);
