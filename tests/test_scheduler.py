@@ -683,3 +683,62 @@ def test_requests_get_the_same_tokens_with_and_without_steps_planned_ahead(seed)
     (plain_out, plain_finish, none), (ahead_out, ahead_finish, some) = results
     assert none == 0 and some > 0
     assert ahead_out == plain_out and ahead_finish == plain_finish
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_no_page_is_lost_when_steps_ahead_are_dropped_abandoned_and_cancelled_at_random(seed):
+    """The engine's moves in a random order: plan, launch, plan ahead, and then commit, or drop what was planned
+    ahead, or abandon the step as failed (cancelling its requests), with requests arriving and being cancelled in
+    between.  Pages in use and free always add up, every request ends once, and at the end every page is free."""
+    rng = random.Random(500 + seed)
+    bs = rng.choice([2, 4, 16])
+    blocks = rng.randrange(12, 40)
+    chunk = rng.choice([None, 8, 32])
+    s = scheduler(blocks, bs, rng.randrange(1, 6), chunk=chunk, window=rng.choice([0, 0, 2 * bs]))
+    submitted, ended, cancelled = set(), {}, set()
+    next_id, flight, idle = 1, None, 0
+    for it in range(6000):
+        if next_id <= 40 and rng.random() < 0.2:
+            n = rng.randrange(1, bs * blocks // 3)
+            s.submit(next_id, [rng.randrange(5) for _ in range(n)], 0.0, None, None, rng.randrange(1, 20), [99], next_id)
+            submitted.add(next_id)
+            next_id += 1
+        if submitted - set(ended) - cancelled and rng.random() < 0.03:
+            victim = rng.choice(sorted(submitted - set(ended) - cancelled))
+            s.cancel(victim)
+            cancelled.add(victim)
+        if flight is not None:
+            plan, flight = flight, None
+        else:
+            plan = s.plan()
+            if plan.kind == sched.IDLE:
+                for f in s.drain_finished().finished:
+                    ended[f.id] = ended.get(f.id, 0) + 1
+                idle += 1
+                if next_id > 40 and not s.running and not s.waiting:
+                    break
+                continue
+        move = rng.random()
+        if plan.kind == sched.DECODE and move < 0.8:
+            s.launched()
+            flight = s.plan_ahead()
+            if flight is not None and rng.random() < 0.15:
+                s.drop_ahead()
+                flight = None
+        if move > 0.95:
+            s.abandon()                      # the step failed: whoever saw it cancels its requests
+            flight = None
+            for e in plan.entries:
+                if e.seq_id not in cancelled and e.seq_id not in ended:
+                    s.cancel(e.seq_id)
+                    cancelled.add(e.seq_id)
+        else:
+            tokens = [99 if rng.random() < 0.05 else 7 for _ in plan.ids]
+            for f in s.commit(tokens).finished:
+                ended[f.id] = ended.get(f.id, 0) + 1
+        assert s.manager.in_use() + s.manager.available() == blocks
+    else:
+        raise AssertionError("the scheduler did not come to an end")
+    assert all(count == 1 for count in ended.values()), "a request ended twice"
+    assert set(ended) | cancelled == submitted, "a request was lost"
+    assert s.manager.available() == blocks and s.manager.live_sequences == 0
