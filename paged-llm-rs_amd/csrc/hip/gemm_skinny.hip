@@ -15,9 +15,7 @@ static int sk_launch_plain(int epilogue, int out_f32, const void* x, const void*
 // epilogue 0: y = result, bfloat16 or (out_f32) 32-bit.  1: y = act(gate) * up (act: PL_ACT_*).  2: y, 32-bit, += result.
 // strips: w holds the same weights in strips (gemm_skinny.hpp has the layout; pl_gemm_skinny_strips_apply says for
 // which products that is read).
-extern "C" int pl_gemm_skinny_strips_apply(int n, int N_out, int K, int epilogue, int norm, int taking) {
-    return sk_strips_apply(n, N_out, K, epilogue, norm != 0, taking != 0) ? 1 : 0;
-}
+extern "C" int pl_gemm_skinny_strips_apply(int n, int N_out, int K) { return sk_strips_apply(n, N_out, K) ? 1 : 0; }
 
 extern "C" int pl_gemm_skinny(const void* x, const void* w, void* y, const float* gain, float eps,
                               const int* rows, int n, int N_out, int K, int epilogue, int out_f32, int act,
@@ -31,7 +29,7 @@ extern "C" int pl_gemm_skinny(const void* x, const void* w, void* y, const float
     PL_REQUIRE(!(gain && epilogue == EPI_ADD), "skinny product: a product that reads the residual stream cannot add into it");
     PL_REQUIRE(act >= PL_ACT_SILU && act <= PL_ACT_GELU, "skinny product: activation code %d", act);
     if (n == 0) return 0;
-    PL_REQUIRE(!strips || sk_strips_apply(n, N_out, K, epilogue, gain != nullptr, false),
+    PL_REQUIRE(!strips || sk_strips_apply(n, N_out, K),
                "skinny product: %d rows, %d columns, width %d are not read from weights in strips", n, N_out, K);
     if (gain) return sk_launch_norm(epilogue, out_f32, x, w, y, gain, eps, rows, n, N_out, K, act, strips ? 1 : 0, stream);
     sk_extras_t with{};
@@ -66,7 +64,7 @@ extern "C" int pl_gemm_skinny_hand(const void* x, const void* w, void* y, int n,
     PL_REQUIRE(!hand_x || sk_hand_applies(n, N_out, K, epilogue, false),
                "skinny product: %d rows, %d columns, width %d hand no norm forward", n, N_out, K);
     if (n == 0) return 0;
-    PL_REQUIRE(!strips || sk_strips_apply(n, N_out, K, epilogue, false, ssq_parts != nullptr),
+    PL_REQUIRE(!strips || sk_strips_apply(n, N_out, K),
                "skinny product: %d rows, %d columns, width %d are not read from weights in strips", n, N_out, K);
     sk_extras_t hand{hand_gain, static_cast<bf16_t*>(hand_x), hand_ssq, ssq_parts, ssq_parts ? parts : 0, strips ? 1 : 0};
     return sk_launch_plain(epilogue, out_f32, x, w, y, nullptr, eps, nullptr, n, N_out, K, act, hand, stream);

@@ -612,17 +612,7 @@ gemm_skinny_rows_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ 
 
     for (int tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
         const int n0 = tile * SK_TILE_N;
-        if (hand.strips) {
-            // the tile's strip (for act(gate) * up: the gate's, then the up's) is K/32 tiles of 1 KB one behind the
-            // other, and goes into LDS as it stands: tile t of a strip is where the lanes of a wave read K step t
-            const int tiles_a_strip = K / SK_KSTEP, loads = BT * tiles_a_strip;
-            for (int j = wave; j < loads; j += WV) {
-                const int b = j / tiles_a_strip, t = j - b * tiles_a_strip;
-                const size_t strip = (b ? N_out / SK_TILE_N : 0) + static_cast<size_t>(tile);
-                sk_load_to_lds(w + (strip * 16 * K + static_cast<size_t>(t) * 512 + lane * 8),
-                               panel + static_cast<size_t>(b) * 16 * K + t * 512);
-            }
-        } else {
+        {
             const int chunks = K / 512, loads = BT * 16 * chunks;
             for (int j = wave; j < loads; j += WV) {
                 const int prow = j / chunks, chunk = j - prow * chunks;
@@ -668,10 +658,7 @@ gemm_skinny_rows_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ 
                 kk[j] = kbeg + (live ? u0 + j : 0) * SK_KSTEP + g * 8;
 #pragma unroll
                 for (int b = 0; b < BT; ++b) {
-                    // (in strips: K step kk / 32 of strip b, the lane's 16 bytes of it)
-                    const size_t at = hand.strips ? static_cast<size_t>(b) * 16 * K + (kk[j] - g * 8) * 16 + lane * 8
-                                                  : static_cast<size_t>(b * 16 + c) * K + (((kk[j] >> 3) ^ c) << 3);
-                    const bf16x8 got = sk_load8(panel + at);
+                    const bf16x8 got = sk_load8(panel + static_cast<size_t>(b * 16 + c) * K + (((kk[j] >> 3) ^ c) << 3));
                     bw[j][b] = live ? got : sk_zero8();
                 }
             }
@@ -760,6 +747,7 @@ template <int MT, int WV, int STEPS, int PRO, int EPI, typename OUT>
 static int launch_rows(const void* x, const void* w, void* y, const float* gain, float eps,
                        const int* rows, int n, int N_out, int K, int act, const sk_extras_t& hand, hipStream_t stream) {
     PL_REQUIRE(!hand.x, "skinny product: this shape of product hands nothing forward");
+    PL_REQUIRE(!hand.strips, "skinny product: this shape of product reads the weights row by row");
     PL_REQUIRE(!hand.parts || (PRO == PRO_BF16 && EPI != EPI_ADD && WV * 64 >= MT * 256 && (STEPS <= 8 || MT == 4)),
                "skinny product: this shape of product takes no handed norm");
     constexpr int BT = EPI == EPI_SWIGLU ? 2 : 1;
@@ -889,14 +877,11 @@ static int launch_mt(const void* x, const void* w, void* y, const float* gain, f
 }
 
 // Whether a product of this shape reads its weights in strips: the layout is defined, and launch_mt takes the
-// kernel for one tile of rows or the rows kernel.  N_out: the columns of y.  norm: the product starts with the
-// norm of the 32-bit stream; taking: it takes a handed norm.
-static inline bool sk_strips_apply(int n, int N_out, int K, int epilogue, bool norm, bool taking) {
+// kernel for one tile of rows (the kernels whose weights wait in LDS read the rows: there the strips gained
+// nothing that showed, and cost the deepest shapes registers).  N_out: the columns of y.
+static inline bool sk_strips_apply(int n, int N_out, int K) {
     if (n <= 0 || n > 64 || N_out <= 0 || N_out % SK_TILE_N || K <= 0 || K % SK_KSTEP) return false;
-    const int row_tiles = pl_ceil_div(n, 16);
-    if (n <= 16 || pl_ceil_div(N_out, SK_TILE_N) * row_tiles <= SK_ROW_TILES_GRID) return true;
-    const int MT = (taking && row_tiles == 3) ? 4 : row_tiles;
-    return sk_rows_kernel_takes(MT, K, epilogue == EPI_SWIGLU, norm);
+    return n <= 16 || pl_ceil_div(N_out, SK_TILE_N) * pl_ceil_div(n, 16) <= SK_ROW_TILES_GRID;
 }
 
 // Which kernel the launchers above take for a product of bfloat16 rows, as far as the handed norm goes:

@@ -40,7 +40,7 @@ def _signatures(lib) -> None:
         "pl_argmax": [p, p, p, p, i, i, p],
         "pl_sample": [p, p, p, p, p, p, i, i, p],
         "pl_gemm_skinny": [p, p, p, p, f, p, i, i, i, i, i, i, i, p],
-        "pl_gemm_skinny_strips_apply": [i, i, i, i, i, i],
+        "pl_gemm_skinny_strips_apply": [i, i, i],
         "pl_gemm_skinny_hand": [p, p, p, i, i, i, i, i, i, p, i, f, p, p, p, i, p],
         "pl_gemm_skinny_hand_applies": [i, i, i, i, i],
         "pl_gemm_tiled": [p, p, p, i, i, i, i, i, p],
@@ -703,13 +703,11 @@ def weights_in_strips(w: torch.Tensor) -> torch.Tensor | None:
     return w.view(N // 16, 16, K // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(N, K)
 
 
-def strips_apply(rows: int, columns: int, width: int, swiglu: bool = False, add: bool = False, norm: bool = False,
-                 taking: bool = False) -> bool:
+def strips_apply(rows: int, columns: int, width: int) -> bool:
     """Whether ``gemm_skinny`` of so many rows, with ``columns`` columns of output over an inner width of ``width``,
-    reads weights in strips: its kernel for one tile of 16 rows does, and the one for two or four tiles whose
-    weights wait in LDS.  ``norm``: the product starts with the norm of the stream; ``taking``: it takes a handed one."""
-    return bool(library().pl_gemm_skinny_strips_apply(rows, columns, width, 1 if swiglu else (2 if add else 0),
-                                                      1 if norm else 0, 1 if taking else 0))
+    reads weights in strips: its kernel for one tile of 16 rows does (up to 16 rows, and beyond where the tiles of
+    rows go to workgroups of their own)."""
+    return bool(library().pl_gemm_skinny_strips_apply(rows, columns, width))
 
 
 def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, swiglu: bool = False,
@@ -762,8 +760,7 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
         out = torch.empty((n, N_out), dtype=out_dtype, device=x.device)
         epilogue, out_f32 = (1 if swiglu else 0), (1 if out_dtype == torch.float32 else 0)
     in_strips = 0
-    if strips is not None and library().pl_gemm_skinny_strips_apply(n, N_out, K, epilogue, 1 if norm_gain is not None else 0,
-                                                                    1 if handed is not None else 0):
+    if strips is not None and library().pl_gemm_skinny_strips_apply(n, N_out, K):
         _need(strips, "weights in strips", tuple(w.shape), torch.bfloat16)
         w, in_strips = strips, 1
     if handed is not None or hand is not None:

@@ -305,15 +305,9 @@ def test_gemm_skinny_over_weights_in_strips(n, N, K):
     strips = kernels.weights_in_strips(w)
     assert strips.shape == w.shape and strips.dtype == w.dtype
     assert torch.equal(strips.flatten().sort().values, w.flatten().sort().values), "the same numbers in another order"
-    def expected(columns, two_tiles=False, norm=False):
-        """one tile of rows a workgroup, or the kernel for two or four tiles whose weights wait in LDS"""
-        tiles = -(-n // 16)
-        if n <= 16 or (columns // 16) * tiles <= 512:
-            return True
-        if tiles not in (2, 4) or K % 512 or (K // 32) % (16 // tiles):
-            return False
-        panel = (2 if two_tiles else 1) * 16 * K * 2 + (K * 4 if norm else 0)
-        return panel <= 144 * 1024 and K // 32 // (16 // tiles) <= (8 if norm else 16)
+    def expected(columns):
+        """one tile of rows a workgroup"""
+        return n <= 16 or (columns // 16) * -(-n // 16) <= 512
 
     reads_strips = kernels.strips_apply(n, N, K)
     assert reads_strips == expected(N)
@@ -328,7 +322,7 @@ def test_gemm_skinny_over_weights_in_strips(n, N, K):
     kernels.gemm_skinny(x, w, add_into=b)
     assert torch.equal(a, b)
     if N % 32 == 0:
-        assert kernels.strips_apply(n, N // 2, K, swiglu=True) == expected(N // 2, two_tiles=True)
+        assert kernels.strips_apply(n, N // 2, K) == expected(N // 2)
         for act in ("silu", "gelu_tanh"):
             assert torch.equal(kernels.gemm_skinny(x, w, swiglu=True, activation=act, strips=strips),
                                kernels.gemm_skinny(x, w, swiglu=True, activation=act))
