@@ -517,30 +517,46 @@ __device__ bool sm_few(sm_shared& sm, const float* __restrict__ x, int V, float 
 
 __global__ void __launch_bounds__(SM_THREADS)
 sample_rows_kernel(const float* __restrict__ logits, const float* __restrict__ temperature, const int* __restrict__ top_k,
-                   const float* __restrict__ top_p, const float* __restrict__ uniform, int* __restrict__ out, int V) {
+                   const float* __restrict__ top_p, const float* __restrict__ uniform, int* __restrict__ out, int V,
+                   int out_holds_largest) {
     __shared__ sm_shared sm;
     const int row = blockIdx.x, tid = threadIdx.x;
     const float* x = logits + static_cast<size_t>(row) * V;
     const float temp = temperature[row];
-    // the largest logit and its first index
+    // the largest logit and its first index: already in out[row] where the caller says so (an argmax by the same
+    // rule ran before), unless what stands there is no finite number's place (a row of NaNs has none)
     float bv = -INFINITY;
     int bi = SM_NO_LIMIT;
-    sm_each(x, V, [&](float v, int i) { better(bv, bi, v, i); });
+    bool known = false;
+    if (out_holds_largest) {
+        const int hint = out[row];
+        if (hint >= 0 && hint < V) {
+            const float v = x[hint];
+            if (v > -INFINITY) {                                // (false for a NaN)
+                bv = v;
+                bi = hint;
+                known = true;
+            }
+        }
+    }
+    if (!known) {                                               // (the same in every thread)
+        sm_each(x, V, [&](float v, int i) { better(bv, bi, v, i); });
 #pragma unroll
-    for (int off = PL_WAVE / 2; off > 0; off >>= 1) {
-        const float ov = __shfl_xor(bv, off, PL_WAVE);
-        const int oi = __shfl_xor(bi, off, PL_WAVE);
-        better(bv, bi, ov, oi);
+        for (int off = PL_WAVE / 2; off > 0; off >>= 1) {
+            const float ov = __shfl_xor(bv, off, PL_WAVE);
+            const int oi = __shfl_xor(bi, off, PL_WAVE);
+            better(bv, bi, ov, oi);
+        }
+        if (tid % PL_WAVE == 0) {
+            sm.red_v[tid / PL_WAVE] = bv;
+            sm.red_i[tid / PL_WAVE] = bi;
+        }
+        __syncthreads();
+        bv = sm.red_v[0];
+        bi = sm.red_i[0];
+        for (int w = 1; w < SM_THREADS / PL_WAVE; ++w) better(bv, bi, sm.red_v[w], sm.red_i[w]);
+        __syncthreads();
     }
-    if (tid % PL_WAVE == 0) {
-        sm.red_v[tid / PL_WAVE] = bv;
-        sm.red_i[tid / PL_WAVE] = bi;
-    }
-    __syncthreads();
-    bv = sm.red_v[0];
-    bi = sm.red_i[0];
-    for (int w = 1; w < SM_THREADS / PL_WAVE; ++w) better(bv, bi, sm.red_v[w], sm.red_i[w]);
-    __syncthreads();
     if (!(temp > 0.f) || bi == SM_NO_LIMIT) {                   // greedy, or a row of NaNs
         if (tid == 0) out[row] = bi == SM_NO_LIMIT ? 0 : bi;
         return;
@@ -575,11 +591,14 @@ sample_rows_kernel(const float* __restrict__ logits, const float* __restrict__ t
 
 // One token a row.  temperature <= 0: the largest logit (the first of equals).  top_k <= 0 or >= V and
 // top_p >= 1 switch the cuts off.  uniform: a number in [0, 1) a row, the request's own draw.
+// out_holds_largest: out[row] already is the place of the row's largest logit, as pl_argmax leaves it (the first
+// of equals, NaNs never); the pass over the row that would find it is then left out.
 extern "C" int pl_sample(const float* logits, const float* temperature, const int* top_k, const float* top_p,
-                         const float* uniform, int* out, int m, int V, hipStream_t stream) {
+                         const float* uniform, int* out, int m, int V, int out_holds_largest, hipStream_t stream) {
     PL_REQUIRE(m >= 0 && V > 0, "sampling: rows %d, vocabulary %d", m, V);
     if (m == 0) return 0;
-    sample_rows_kernel<<<m, SM_THREADS, 0, stream>>>(logits, temperature, top_k, top_p, uniform, out, V);
+    sample_rows_kernel<<<m, SM_THREADS, 0, stream>>>(logits, temperature, top_k, top_p, uniform, out, V,
+                                                     out_holds_largest ? 1 : 0);
     PL_CHECK_LAUNCH("sample");
     return 0;
 }

@@ -169,21 +169,24 @@ class Engine:
 
     # -- the loop ---------------------------------------------------------------------------
 
-    def _draw_on_device(self, ids, logits, out=None) -> torch.Tensor:
+    def _draw_on_device(self, ids, logits, out=None, out_holds_largest: bool = False) -> torch.Tensor:
         """One token per row of ``logits`` by the sampling kernel, each with its request's parameters and the
-        next number of the request's generator (a greedy row takes its largest logit and draws nothing)."""
+        next number of the request's generator (a greedy row takes its largest logit and draws nothing).
+        ``out_holds_largest``: ``out`` already holds the rows' largest logits' places (``kernels.sample``)."""
         how = [self.scheduler.sampling_of(i) for i in ids]
         params = torch.tensor([[t, float(k), p, u] for t, k, p, u in how], dtype=torch.float32).pin_memory()
         params = params.to(logits.device, non_blocking=True)
         return kernels.sample(logits, params[:, 0].contiguous(), params[:, 1].to(torch.int32).contiguous(),
-                              params[:, 2].contiguous(), params[:, 3].contiguous(), out=out)
+                              params[:, 2].contiguous(), params[:, 3].contiguous(), out=out,
+                              out_holds_largest=out_holds_largest)
 
     def _chooser(self, plan):
         """What a decoding step of ``plan`` is run with (``StepRunner.run``): nothing where every request
         takes its largest logit or the host samples; else the sampling kernel, behind the step."""
         if self.sampler != "device" or all(self._greedy.get(i, True) for i in plan.ids):
             return None
-        return lambda logits, out: self._draw_on_device(plan.ids, logits, out)
+        # (behind a decoding step the tokens are the largest logits' when the chooser is called)
+        return lambda logits, out: self._draw_on_device(plan.ids, logits, out, out_holds_largest=True)
 
     def _choose(self, plan, output) -> list:
         """One token per id of the plan.  On the device (the default) greedy rows are an argmax and

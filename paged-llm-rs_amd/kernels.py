@@ -38,7 +38,7 @@ def _signatures(lib) -> None:
         "pl_paged_attention_plain": [p, i, p, p, p, p, i, i, p, p, i, i, i, i, f, i, i, p],
         "pl_paged_attention_prefill_tile": [i, i],
         "pl_argmax": [p, p, p, p, i, i, p],
-        "pl_sample": [p, p, p, p, p, p, i, i, p],
+        "pl_sample": [p, p, p, p, p, p, i, i, i, p],
         "pl_gemm_skinny": [p, p, p, p, f, p, i, i, i, i, i, i, i, p],
         "pl_gemm_skinny_strips_apply": [i, i, i],
         "pl_gemm_skinny_hand": [p, p, p, i, i, i, i, i, i, p, i, f, p, p, p, i, p],
@@ -292,11 +292,13 @@ def argmax(logits: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tenso
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-           uniform: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+           uniform: torch.Tensor, out: torch.Tensor | None = None, out_holds_largest: bool = False) -> torch.Tensor:
     """One token a row: logits / temperature, the k most likely, of those the shortest head
     whose mass reaches top_p, and of that the token on which the mass reaches uniform * total,
     all in the order of falling logit and rising index (reference: crates/pagedllm/src/sampler.rs).
-    A row with temperature 0 takes its largest logit.  top_k 0 and top_p 1 cut nothing."""
+    A row with temperature 0 takes its largest logit.  top_k 0 and top_p 1 cut nothing.
+    ``out_holds_largest``: ``out`` comes with what ``argmax`` made of these logits, which saves the kernel
+    its first pass over every row."""
     m, V = logits.shape
     _need(logits, "logits", None, torch.float32)
     _need(temperature, "temperatures", (m,), torch.float32)
@@ -304,10 +306,12 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     _need(top_p, "top_p", (m,), torch.float32)
     _need(uniform, "uniform numbers", (m,), torch.float32)
     if out is None:
+        if out_holds_largest:
+            raise TensorError("no tokens given that could hold the largest logits' places")
         out = torch.empty((m,), dtype=torch.int32, device=logits.device)
     _need(out, "chosen tokens", (m,), torch.int32)
     _check(library().pl_sample(logits.data_ptr(), temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(),
-                               uniform.data_ptr(), out.data_ptr(), m, V, _stream()))
+                               uniform.data_ptr(), out.data_ptr(), m, V, 1 if out_holds_largest else 0, _stream()))
     return out
 
 

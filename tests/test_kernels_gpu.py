@@ -1179,6 +1179,19 @@ def test_sampling_kernel_follows_the_recipe():
     again = kernels.sample(logits, as_f(0), torch.tensor([h[1] for h in how], dtype=torch.int32, device=DEV), as_f(2),
                            as_f(3)).cpu().tolist()
     assert got == again, "a row and a number give the same token on every run"
+    # with the largest logits' places handed in (as behind a decoding step, whose argmax has run), the same tokens;
+    # a place that is none (of a row of NaNs, or nonsense) is not believed
+    spoiled = logits.clone()
+    spoiled[3] = float("nan")
+    hint = kernels.argmax(spoiled)
+    want = kernels.sample(spoiled, as_f(0), torch.tensor([h[1] for h in how], dtype=torch.int32, device=DEV), as_f(2), as_f(3))
+    handed = kernels.sample(spoiled, as_f(0), torch.tensor([h[1] for h in how], dtype=torch.int32, device=DEV), as_f(2),
+                            as_f(3), out=hint.clone(), out_holds_largest=True)
+    assert torch.equal(handed, want) and want.cpu().tolist()[:3] == got[:3] and int(want[3]) == 0
+    nonsense = hint.clone()
+    nonsense[5], nonsense[6] = -7, V + 3
+    assert torch.equal(kernels.sample(spoiled, as_f(0), torch.tensor([h[1] for h in how], dtype=torch.int32, device=DEV),
+                                      as_f(2), as_f(3), out=nonsense, out_holds_largest=True), want)
     same_as_host = 0
     for row, (t, k, p, u) in enumerate(how):
         x = logits[row].cpu().numpy()
