@@ -16,6 +16,7 @@ from dataclasses import dataclass, field
 from pathlib import Path
 from typing import Optional
 
+import numpy as np
 import torch
 
 from .. import kernels
@@ -173,12 +174,16 @@ class Engine:
         """One token per row of ``logits`` by the sampling kernel, each with its request's parameters and the
         next number of the request's generator (a greedy row takes its largest logit and draws nothing).
         ``out_holds_largest``: ``out`` already holds the rows' largest logits' places (``kernels.sample``)."""
-        how = [self.scheduler.sampling_of(i) for i in ids]
-        params = torch.tensor([[t, float(k), p, u] for t, k, p, u in how], dtype=torch.float32).pin_memory()
-        params = params.to(logits.device, non_blocking=True)
-        return kernels.sample(logits, params[:, 0].contiguous(), params[:, 1].to(torch.int32).contiguous(),
-                              params[:, 2].contiguous(), params[:, 3].contiguous(), out=out,
-                              out_holds_largest=out_holds_largest)
+        how = [self.scheduler.sampling_of(i) for i in ids]     # (draws the number of every request that samples)
+        # one transfer: temperatures, top-k, top-p and the drawn numbers as the four rows of one 32-bit array
+        # (the 32-bit floats as their bits), of which the kernel's arguments are views
+        packed = np.empty((4, len(how)), dtype=np.int32)
+        as_float = packed.view(np.float32)
+        for col, (t, k, p, u) in enumerate(how):
+            as_float[0, col], packed[1, col], as_float[2, col], as_float[3, col] = t, k, p, u
+        params = torch.from_numpy(packed).pin_memory().to(logits.device, non_blocking=True)
+        return kernels.sample(logits, params[0].view(torch.float32), params[1], params[2].view(torch.float32),
+                              params[3].view(torch.float32), out=out, out_holds_largest=out_holds_largest)
 
     def _chooser(self, plan):
         """What a decoding step of ``plan`` is run with (``StepRunner.run``): nothing where every request
