@@ -269,29 +269,52 @@ void Scheduler::launched() {
 // which it cannot end but by a stop token, fed the token of its row there.
 const Plan* Scheduler::plan_ahead() {
     if (ahead_) throw Error("a step is planned ahead already");
-    if (plan_.kind != PlanKind::Decode || !plan_.launched || !waiting_.empty()) return nullptr;
-    size_t present = 0;      // (a step that was itself planned ahead may hold rows of requests that have ended since)
-    for (uint64_t id : plan_.ids) present += sequence(id) != nullptr;
-    if (present != running_.size()) return nullptr;              // someone has no row: the planner decides
+    if (plan_.kind != PlanKind::Decode || !plan_.launched || prompt_in_flight()) return nullptr;
+    // Would the planner bring the front of the queue in (or turn it away)?  Then the next step is its to decide.
+    // Whether there is room is asked where the planner asks: before the residents take their pages when prompts
+    // run whole, after them under a token budget.
+    bool stalled = false;
+    auto front_stalls = [&]() -> bool {
+        if (waiting_.empty()) return true;
+        const size_t prompt_len = waiting_.front().pending.size();
+        const bool too_long = max_positions_ > 0 && prompt_len > max_positions_;
+        if (too_long || !cache_->fits_in_total(prompt_len, chunk_ > 0 ? chunk_ : prompt_len)) return false;   // a refusal
+        const bool room = chunk_ > 0 ? cache_->min_available() > 0 : cache_->fits_from_scratch(prompt_len);
+        if (room && cache_->state_slot_available()) return false;
+        stalled = true;
+        return true;
+    };
+    if (chunk_ == 0 && !front_stalls()) return nullptr;
+    // A row for every resident with a token to feed, in the order of arrival, as far as the rows last (as the
+    // planner seats them): the token of its row in the launched step, which is not known yet, or, for a resident
+    // that step had no row for, the token it has been holding.
     Plan next;
     next.kind = PlanKind::Decode;
-    for (size_t row = 0; row < plan_.ids.size(); ++row) {
-        Sequence* s = sequence(plan_.ids[row]);
-        if (!s) continue;
-        if (s->finish != Finish::None || s->pending.size() != 1) return nullptr;
-        if (s->generated + 1 >= s->max_tokens) continue;                                   // its last token
-        if (max_positions_ > 0 && s->history.size() + 1 > max_positions_) continue;        // its last position
-        if (!cache_->reserve(s->id, 1)) return nullptr;
-        next.ids.push_back(s->id);
-        next.advanced.emplace_back(s->id, 1);
-        next.entries.push_back(PlanEntry{s->id, cache_->tokens(s->id), std::vector<uint32_t>(1, 0), true,
-                                         s->state_slot, false});
-        next.fed_rows.push_back(static_cast<int>(row));
+    for (Sequence& s : running_) {
+        if (next.entries.size() == max_batch_) break;
+        if (s.finish != Finish::None) continue;                  // (leaves at the commit)
+        if (s.pending.size() != 1) return nullptr;
+        const auto at = std::find(plan_.ids.begin(), plan_.ids.end(), s.id);
+        const int fed = at == plan_.ids.end() ? -1 : static_cast<int>(at - plan_.ids.begin());
+        if (fed >= 0) {
+            if (s.generated + 1 >= s.max_tokens) continue;                                 // its last token
+            if (max_positions_ > 0 && s.history.size() + 1 > max_positions_) continue;     // its last position
+        }
+        if (!cache_->reserve(s.id, 1)) return nullptr;           // who gives way is the planner's decision
+        const size_t first = cache_->tokens(s.id);
+        next.ids.push_back(s.id);
+        next.advanced.emplace_back(s.id, 1);
+        next.entries.push_back(PlanEntry{s.id, first, std::vector<uint32_t>(1, fed >= 0 ? 0u : s.history[first]), true,
+                                         s.state_slot, false});
+        next.fed_rows.push_back(fed);
     }
     if (next.entries.empty()) return nullptr;
+    if (chunk_ > 0 && !front_stalls()) return nullptr;
+    if (stalled) metrics_.admission_stalls += 1;
     metrics_.steps += 1;
     metrics_.decode_steps += 1;
     metrics_.decode_rows += next.entries.size();
+    next.stalled = stalled;
     ahead_ = std::move(next);
     return &*ahead_;
 }
@@ -301,6 +324,7 @@ void Scheduler::drop_ahead() {
     metrics_.steps -= 1;
     metrics_.decode_steps -= 1;
     metrics_.decode_rows -= ahead_->entries.size();
+    if (ahead_->stalled) metrics_.admission_stalls -= 1;
     ahead_.reset();           // (the pages reserved for its rows stay with their requests, whose next step needs them)
 }
 

@@ -60,6 +60,7 @@ struct Plan {
     // A step planned ahead (see plan_ahead): for every entry the row of the step before whose token it is
     // fed; the entry's own token is a placeholder.  Empty for every other step.
     std::vector<int> fed_rows;
+    bool stalled = false;                               // planning it counted a stall of the queue's front (drop_ahead takes it back)
     bool launched = false;                              // the lengths in the cache have moved for it
 };
 
@@ -111,11 +112,13 @@ public:
     // `launched` says that the planned step is queued on the device: its tokens are as good as written
     // for everything queued behind it, so the lengths in the cache move now (commit does this itself
     // where nobody has).  `plan_ahead` gives the step behind a launched decoding step, or nothing when
-    // that step is not known yet: a request waits or is part-way through its prompt, a resident was left
-    // without a row, or the pools have no page for a row (then the ordinary planner decides who gives
-    // way, after the commit).  Requests that the launched step ends by their budget or the model's last
-    // position have no row in it; one that a stop token ends has, and that row's token is dropped when
-    // it is committed.  After the commit of the step before, the step planned ahead is the planned
+    // that step is not known yet: the planner would bring the front of the queue in or turn it away, a
+    // request is part-way through its prompt, or the pools have no page for a row (then the ordinary
+    // planner decides who gives way, after the commit).  Otherwise it is a decoding step again: rows for
+    // the residents in their order as far as the rows last, as the planner seats them.  Requests that the
+    // launched step ends by their budget or the model's last position have no row in it; one that a stop
+    // token ends has, and that row's token is dropped when it is committed (a resident that would have
+    // had its row gets one a step later).  After the commit of the step before, the step planned ahead is the planned
     // step, and `plan` may not be asked until it is committed too.  `drop_ahead` forgets a step planned
     // ahead that was not launched after all.
     void launched();

@@ -114,11 +114,14 @@ class Scheduler:
         native.check(self._lib.plh_sched_launched(self._h))
 
     def plan_ahead(self):
-        """The step behind a launched decoding step, before that step's tokens are known: a row for every
-        request of it that it can only end by a stop token, each fed on the device the token of its row
-        there (``StepEntry.fed_row``).  None when the next step is not known yet (a request waits, pages
-        have run out, a resident has no row).  Once the step before is committed, the step planned ahead
-        is the planned step: it is committed next, and ``plan`` may not be asked before."""
+        """The step behind a launched decoding step, before that step's tokens are known: rows for the
+        residents as the planner would seat them.  A request with a row in the launched step, which that
+        step can only end by a stop token, is fed the token of its row there on the device
+        (``StepEntry.fed_row``); one without (there were more residents than rows) brings the token it
+        holds.  None when the next step is not known yet: the front of the queue can come in or is to be
+        turned away, a prompt is part-way in, or pages have run out.  Once the step before is committed,
+        the step planned ahead is the planned step: it is committed next, and ``plan`` may not be asked
+        before."""
         sizes = (ctypes.c_size_t * 4)()
         if not native.check(self._lib.plh_sched_plan_ahead(self._h, sizes)):
             return None

@@ -521,6 +521,30 @@ def test_steps_queued_ahead_change_no_token(model_dirs, name, dtype, graphs, dra
     assert [g.tokens for g in again] == [g.tokens for g in got]
 
 
+@pytest.mark.parametrize("name,chunk,drawn", [("B", 64, False), ("C", None, False), ("B", None, True)])
+def test_steps_are_queued_ahead_in_a_crowded_engine(model_dirs, name, chunk, drawn):
+    """More requests than rows and than the pages hold at once: some wait in the queue, some residents have no
+    row in a step.  Steps are queued ahead all the same while the queue cannot move, rows of requests that had
+    none in the step before bring their own token beside rows that are fed on the device, and every request has
+    the tokens and the ending of an engine that reads every step's tokens first."""
+    from paged_llm_rs_amd import Engine
+
+    d = model_dirs(name, "float32")
+    vocab = TINY_INIT[name]["config"]["vocab_size"]
+    prompts = list(ru.make_prompts(vocab, [9, 21, 4, 14, 30, 7, 12], seed=23).values())
+    budgets = [30, 9, 26, 17, 12, 21, 5]
+    settings = dict(dtype="f32", block_size=8, num_blocks=16, max_batch=3, chunk=chunk, prefix_cache=False)
+    want = _generate_each(Engine(d, ahead=False, **settings), prompts, budgets, [], drawn)
+    engine = Engine(d, ahead=True, **settings)
+    got = _generate_each(engine, prompts, budgets, [], drawn)
+    assert [g.tokens for g in got] == [w.tokens for w in want]
+    assert [g.finish for g in got] == [w.finish for w in want]
+    m = engine.metrics()
+    assert m["steps_ahead"] >= 0.5 * m["decode_steps"], (m["steps_ahead"], m["decode_steps"])
+    assert m["admission_stalls"] > 0 and m["preemptions"] > 0, "the engine was not crowded"
+    assert m["available"] == m["total"]
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_step_takes_the_tokens_of_the_step_before_on_the_device(model_dirs, dtype):
     """The step runner alone: decoding steps whose entries name rows of the step before, in another order

@@ -511,8 +511,8 @@ def drive(s, arrivals, token_of, ahead: bool, steps: int = 4000):
     """Run the scheduler to the end.  ``arrivals``: {iteration: [(id, prompt, max_tokens)]};
     ``token_of(id, n)`` is the n-th token request id samples.  With ``ahead`` every step that can be is
     planned before the tokens of the one before are committed, the way the engine does it.  Returns
-    ({id: tokens}, {id: finish}, steps planned ahead)."""
-    out, finish, count, planned_ahead = {}, {}, {}, 0
+    ({id: tokens}, {id: finish}, (steps planned ahead, steps of single tokens))."""
+    out, finish, count, planned_ahead, decoding = {}, {}, {}, 0, 0
     flight = None
     for it in range(steps):
         for seq_id, prompt, most in arrivals.get(it, []):
@@ -528,6 +528,7 @@ def drive(s, arrivals, token_of, ahead: bool, steps: int = 4000):
                 if it > max(arrivals) and not s.running and not s.waiting:
                     break
                 continue
+        decoding += plan.kind == sched.DECODE
         if ahead and plan.kind == sched.DECODE:
             s.launched()
             before = {i: s.manager.tokens(i) for i in s.running_ids()}
@@ -535,7 +536,11 @@ def drive(s, arrivals, token_of, ahead: bool, steps: int = 4000):
             if flight is not None:
                 planned_ahead += 1
                 for e in flight.entries:
-                    assert plan.ids[e.fed_row] == e.seq_id, "a row is fed the token of its own request"
+                    if e.fed_row >= 0:
+                        assert plan.ids[e.fed_row] == e.seq_id, "a row is fed the token of its own request"
+                    else:
+                        assert e.seq_id not in plan.ids and e.tokens == out[e.seq_id][-1:], \
+                            "a request without a row in the step before brings its last token itself"
                     assert e.start == before[e.seq_id] == s.manager.tokens(e.seq_id)
                     assert e.start + 1 <= s.manager.capacity(e.seq_id)
         sampled = []
@@ -549,7 +554,7 @@ def drive(s, arrivals, token_of, ahead: bool, steps: int = 4000):
             finish[f.id] = f.finish
     else:
         raise AssertionError("the scheduler did not come to an end")
-    return out, finish, planned_ahead
+    return out, finish, (planned_ahead, decoding)
 
 
 def test_a_step_planned_ahead_has_a_row_for_everyone_the_step_before_cannot_end():
@@ -623,6 +628,101 @@ def test_nothing_is_planned_ahead_while_a_request_waits_or_pages_are_short():
     assert s.manager.available() == 2
 
 
+def test_steps_are_planned_ahead_while_the_queue_cannot_move():
+    """Serving at its limit: more residents than rows, and a front of the queue that no page or slot can
+    take yet.  The planner would decode, so the step is planned ahead; when the front can come in, it is not."""
+    s = scheduler(64, 4, 2, chunk=16)                # two rows
+    for seq_id in (1, 2, 3):
+        submit(s, seq_id, 3, 10)
+    step(s)
+    assert step(s)[0].kind == sched.MIXED and s.running == 3 and not s.waiting   # the third prompt beside two rows
+    plan = s.plan()
+    assert plan.kind == sched.DECODE and plan.ids == [1, 2]
+    s.launched()
+    following = s.plan_ahead()
+    assert [(e.seq_id, e.fed_row) for e in following.entries] == [(1, 0), (2, 1)], "the rows the planner would give"
+    s.commit([7, 7])
+    s.commit([7, 7])
+    # request 1 has one token left: the step behind its last has a row for request 3, which brings its own token
+    s = scheduler(64, 4, 2, chunk=16)
+    submit(s, 1, 3, 3)
+    submit(s, 2, 3, 10)
+    submit(s, 3, 3, 10)
+    step(s)
+    step(s)
+    assert s.plan().ids == [1, 2]
+    s.launched()
+    following = s.plan_ahead()
+    assert [(e.seq_id, e.fed_row, e.tokens) for e in following.entries] == [(2, 1, [0]), (3, -1, [7])]
+    assert following.entries[1].start == s.manager.tokens(3)
+    outcome = s.commit([8, 8])
+    assert [f.id for f in outcome.finished] == [1]
+    assert s.commit([5, 6]).tokens == [(2, 5), (3, 6)]
+
+    # a queue that waits for a state slot, and one that waits for pages
+    s = scheduler(64, 4, 4, chunk=16, state_slots=1)
+    submit(s, 1, 3, 10)
+    submit(s, 2, 3, 10)
+    step(s)
+    assert s.running == 1 and s.waiting == 1
+    assert s.plan().kind == sched.DECODE
+    stalls = s.metrics()["admission_stalls"]
+    s.launched()
+    assert s.plan_ahead() is not None
+    assert s.metrics()["admission_stalls"] == stalls + 1, "the stall is counted as the planner counts it"
+    s.drop_ahead()
+    assert s.metrics()["admission_stalls"] == stalls
+    s.commit([7])
+
+    s = scheduler(4, 4, 4, chunk=None)               # prompts run whole: the front needs all its pages at once
+    submit(s, 1, 9, 10)                              # three of the four pages
+    step(s)
+    submit(s, 2, 0, 10, prompt=[2] * 6)              # two pages: waits
+    assert s.plan().kind == sched.DECODE
+    s.launched()
+    following = s.plan_ahead()
+    assert following is not None and following.ids == [1]
+    s.commit([7])
+    s.commit([7])
+    s.cancel(1)
+    assert s.plan().kind == sched.PREFILL            # and comes in by the planner once the pages are back
+
+    s = scheduler(4, 4, 4, chunk=None)               # a front that can never be served is the planner's to turn away
+    submit(s, 1, 9, 10)
+    step(s)
+    assert s.plan().kind == sched.DECODE
+    s.launched()
+    submit(s, 2, 1000, 1)
+    assert s.plan_ahead() is None
+    s.commit([7])
+    assert s.plan().kind == sched.REFUSED
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_a_crowded_scheduler_plans_most_decoding_steps_ahead(seed):
+    """Many more requests than rows and pages, all at once: the same tokens and endings as without planning
+    ahead, and most decoding steps are planned ahead although the queue is never empty."""
+    rng = random.Random(900 + seed)
+    bs, blocks, max_batch = 4, 24, 3
+    chunk = [None, 16][seed % 2]
+    arrivals = {0: [(i, [rng.randrange(5) for _ in range(rng.randrange(2, 14))], rng.randrange(8, 30))
+                    for i in range(1, 13)]}
+
+    def token_of(seq_id, n):
+        return 99 if (seq_id * 13 + n * 7) % 41 == 0 else (seq_id + n) % 50
+
+    results = []
+    for ahead in (False, True):
+        s = scheduler(blocks, bs, max_batch, chunk=chunk)
+        results.append(drive(s, arrivals, token_of, ahead))
+        assert s.manager.available() == blocks and s.manager.live_sequences == 0
+    (plain_out, plain_finish, _), (ahead_out, ahead_finish, (planned_ahead, decoding)) = results
+    assert ahead_out == plain_out and ahead_finish == plain_finish
+    # (the steps of single tokens that are not planned ahead: the first behind a prompt, and those behind which
+    # the front of the queue comes in)
+    assert planned_ahead > 0.6 * decoding, (planned_ahead, decoding)
+
+
 def test_a_step_ahead_that_was_not_launched_is_forgotten():
     s = scheduler(64, 4, 4)
     submit(s, 1, 3, 10)
@@ -680,7 +780,7 @@ def test_requests_get_the_same_tokens_with_and_without_steps_planned_ahead(seed)
         s = scheduler(blocks, bs, max_batch, chunk=chunk, window=window)
         results.append(drive(s, arrivals, token_of, ahead))
         assert s.manager.available() == blocks and s.manager.live_sequences == 0
-    (plain_out, plain_finish, none), (ahead_out, ahead_finish, some) = results
+    (plain_out, plain_finish, (none, _)), (ahead_out, ahead_finish, (some, _)) = results
     assert none == 0 and some > 0
     assert ahead_out == plain_out and ahead_finish == plain_finish
 
