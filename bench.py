@@ -341,9 +341,12 @@ def main() -> int:
                         help="leave out the points of the 8b shape (a mixed step) and the 32b shape (decode at batch 64)")
     parser.add_argument("--prefill-eager", action="store_true",
                         help="launch the prefill step kernel by kernel every time (a prompt length seen once)")
+    parser.add_argument("--ahead", choices=["on", "off"], default="on",
+                        help="--only engine: whether the engine queues a decoding step before it has read the tokens "
+                             "of the one before")
     parser.add_argument("--only", choices=["decode", "prefill", "engine", "mixed", "serving", "products"], default=None,
                         help="run one part alone: the decode steps at --batch, the prefill, or (not part of the "
-                             "default line) the whole engine on 1/4/16/32/64 requests at once, 16 prompt tokens and "
+                             "default line) the whole engine on 1/4/16/32/64/128 requests at once, 16 prompt tokens and "
                              "128 generated each, as the reference's own table of clients does; mixed: one step of a "
                              "512-token slice of a prompt beside 63 decoded tokens; serving: the reference's two other "
                              "tables, first tokens behind a shared preamble with the prefix cache off and on, and the "
@@ -462,10 +465,12 @@ def main() -> int:
         from paged_llm_rs_amd.engine.engine import Engine
 
         del runner, cache
-        engine = Engine(folder, dtype="bf16", block_size=BLOCK_SIZE, num_blocks=64 * 12 + 64, max_batch=64, chunk=128)
+        engine = Engine(folder, dtype="bf16", block_size=BLOCK_SIZE, num_blocks=64 * 12 + 64, max_batch=64, chunk=128,
+                        ahead=args.ahead == "on")
         rng = random.Random(7)
         result = {}
-        for clients in (1, 4, 16, 32, 64):
+        # (128 requests are more than the engine has rows and pages for at once: some wait in the queue)
+        for clients in (1, 4, 16, 32, 64, 128):
             prompts = [[rng.randrange(cfg["vocab_size"]) for _ in range(16)] for _ in range(clients)]
             for timed_run in (False, False, True):      # a shape of step is captured when it comes the second time
                 torch.cuda.synchronize()
