@@ -89,6 +89,11 @@ class LayerContext:
 
 
 class DecoderModel:
+    # The embedding takes a row's id from ``batch.fed_tokens[batch.token_src[t]]`` where ``batch.token_src[t]`` names
+    # a row of the step before: the runner and the engine may then queue a decoding step before the host has read
+    # the tokens of the one before.  (A model class without the attribute, or with False, is stepped the ordinary way.)
+    takes_fed_tokens = True
+
     def __init__(self, spec, params: dict, dtype: torch.dtype, device):
         self.spec = spec
         self.dtype = dtype
@@ -124,7 +129,6 @@ class DecoderModel:
                            and getattr(self.logit_transform, "graph_safe", True))
         # Mixers that hand requests of few tokens to a kernel of their own say from how many tokens on a
         # request counts as a long portion; a step reports the tokens of the shorter ones for each such limit.
-        self.takes_fed_tokens = True      # the embedding reads ``batch.token_src`` / ``batch.fed_tokens``
         self.portion_limits = tuple(sorted({int(limit) for b in self.blocks
                                             for limit in [getattr(getattr(b, "mixer", None), "short_portion", None)]
                                             if limit}))

@@ -545,6 +545,28 @@ def test_steps_are_queued_ahead_in_a_crowded_engine(model_dirs, name, chunk, dra
     assert m["available"] == m["total"]
 
 
+def test_an_engine_whose_model_takes_no_ids_from_the_device_plans_nothing_ahead(model_dirs, monkeypatch):
+    """Taking a row's id from the step before on the device is something a model offers (``takes_fed_tokens``).  One
+    that does not is driven the ordinary way, every step's tokens read before the next is planned: its decode
+    graphs have no piece that names rows of the step before, and it generates what the model that offers it does."""
+    from paged_llm_rs_amd import Engine
+    from paged_llm_rs_amd.parts.model import DecoderModel
+
+    d = model_dirs("B", "float32")
+    vocab = TINY_INIT["B"]["config"]["vocab_size"]
+    prompts = list(ru.make_prompts(vocab, [9, 21, 4], seed=5).values())
+    settings = dict(dtype="f32", block_size=8, num_blocks=64, max_batch=4, chunk=64, prefix_cache=False)
+    want = Engine(d, **settings).generate(prompts, max_tokens=20, stop_tokens=[])
+    monkeypatch.setattr(DecoderModel, "takes_fed_tokens", False)
+    engine = Engine(d, **settings)
+    assert not engine.ahead
+    got = engine.generate(prompts, max_tokens=20, stop_tokens=[])
+    assert [g["tokens"] for g in got] == [w["tokens"] for w in want]
+    assert engine.metrics()["steps_ahead"] == 0
+    graphs = [g for g in engine.runner._graphs.values()]
+    assert graphs and all(g.batch.token_src is None for g in graphs)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_step_takes_the_tokens_of_the_step_before_on_the_device(model_dirs, dtype):
     """The step runner alone: decoding steps whose entries name rows of the step before, in another order
