@@ -319,6 +319,12 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
         within -= low * block_size;
         blk = table[bi];
     };
+    // UP: the page of key j (of the last key, past it), through the scalar unit: the entry's place as a 32-bit
+    // count of bytes behind the table's row, which one scalar load takes as it stands
+    auto page_of = [&](int j) {
+        const uint32_t at = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(min(j, last_pos) >> log2_bs)) << 2;
+        return *reinterpret_cast<const int*>(reinterpret_cast<const char*>(table) + at);
+    };
     auto lookup = [&](int k0) {
 #pragma unroll
         for (int i = 0; i < KI; ++i) {
@@ -328,7 +334,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
                 const int j0 = k0 + (64 * wave_id + i * NT) / CP;
                 kj0[i] = j0;
                 kwithin[i] = j0 & (block_size - 1);
-                kblk[i] = table[__builtin_amdgcn_readfirstlane(min(j0, last_pos) >> log2_bs)];
+                kblk[i] = page_of(j0);
             } else {
                 locate(k0 + ((tid + i * NT) / CP) % AP_BN, kblk[i], kwithin[i], kin[i]);
             }
@@ -344,7 +350,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
                 const int j0 = k0 + (64 * wave_id + i * NT) / CP;
                 ahead_j0[i] = j0;
                 ahead_within[i] = j0 & (block_size - 1);
-                ahead_blk[i] = table[__builtin_amdgcn_readfirstlane(min(j0, last_pos) >> log2_bs)];
+                ahead_blk[i] = page_of(j0);
             }
         }
     };
@@ -430,16 +436,22 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
             place_v[odd] = (lane / CP) * row_bytes + piece_v[odd];
         }
     }
+    // (The scalar unit, which the waves of a compute unit share, does the addresses: a page's first byte as one
+    // product of two 32-bit numbers, and one comparison a tile for whether any of its rows needs the redirection
+    // below; with both done a load at a time the addresses took a sixth of the kernel's time.)
+    const uint32_t page_bytes = static_cast<uint32_t>(block_size) * row_bytes;
     auto ask = [&]() {               // pages from kblk/kwithin, looked up before
         if constexpr (DIRECT) {
+            const int tile_first = k_first + asked * AP_BN;
+            const bool at_an_edge = tile_first + AP_BN - 1 > last_pos || tile_first < first_pos;
 #pragma unroll
             for (int i = 0; i < KI; ++i) {
                 const int first_row = (64 * wave_id + i * NT) / CP;
-                const int page = __builtin_amdgcn_readfirstlane(max(kblk[i], 0));
-                const size_t base = (static_cast<size_t>(page) * block_size + kwithin[i]) * row_bytes;
+                const uint32_t page = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(max(kblk[i], 0)));
+                const size_t base = static_cast<size_t>(page) * page_bytes + static_cast<uint32_t>(kwithin[i]) * row_bytes;
                 const char* gk = reinterpret_cast<const char*>(k_pool) + base + place_k[ROWS_ALTERNATE ? i & 1 : 0];
                 const char* gv = reinterpret_cast<const char*>(v_pool) + base + place_v[ROWS_ALTERNATE ? i & 1 : 0];
-                if (kj0[i] + 64 / CP - 1 > last_pos || kj0[i] < first_pos) {   // (the same for the wave)
+                if (at_an_edge && (kj0[i] + 64 / CP - 1 > last_pos || kj0[i] < first_pos)) {   // (the same for the wave)
                     const int j = kj0[i] + lane / CP;
                     if (j > last_pos || j < first_pos)
                         gv = reinterpret_cast<const char*>(v_pool) + last_base + piece_v[ROWS_ALTERNATE ? i & 1 : 0];
@@ -1010,6 +1022,8 @@ extern "C" int pl_paged_attention_prefill(const void* q, int q_stride, void* out
     PL_REQUIRE((nkv * d) % 8 == 0, "prefill attention: a cache row of %d elements is not read 16 bytes at a time", nkv * d);
     if (num_seqs <= 0 || max_q_len <= 0) return 0;
     PL_REQUIRE(total_rows >= max_q_len, "prefill attention: %d rows for a portion of %d", total_rows, max_q_len);
+    PL_REQUIRE(static_cast<unsigned long long>(block_size) * nkv * d * 2 < (1ull << 32),
+               "prefill attention: a page of %d tokens of %d heads of %d takes more bytes than 32 bits count", block_size, nkv, d);
     const int dt = pl_ceil_div(d, 32);
     // few tokens a request: 64-token tiles give twice the workgroups
 #ifdef AP_FORCE_SMALL
