@@ -925,6 +925,55 @@ def test_paged_attention_of_portions(nq, nkv, d, bs, requests, window, splits):
         assert err < 1e-2, f"token {i} (request {s}, position {p}): {err:.3e}"
 
 
+def test_paged_attention_over_pages_beyond_four_gib_of_a_pool():
+    """The byte offset of a page is a 64-bit number: a request whose pages lie behind the first 4 GiB of the
+    pools (each 4.5 GiB here, untouched but for those pages) gets what it gets from the same pages at the
+    pools' start, from the tiled kernel (a portion of 48 tokens) and from the single-token kernel."""
+    from paged_llm_rs_amd import kernels
+
+    dtype = torch.bfloat16
+    nq, nkv, d, bs = 4, 2, 128, 16
+    requests = [(210, 48), (77, 1)]
+    ctx_lens = [c for c, _ in requests]
+    bt, k_small, v_small, keys, values = build_paged(nkv, d, bs, ctx_lens, dtype, seed=3)
+    small_pages = k_small.shape[0] // bs
+    page_bytes = bs * nkv * d * 2
+    far = (4 << 30) // page_bytes + 11                       # the first page behind 4 GiB, and a few more
+    big_pages = far + small_pages
+    k_pool = torch.empty(big_pages * bs, nkv * d, dtype=dtype, device=DEV)
+    v_pool = torch.empty(big_pages * bs, nkv * d, dtype=dtype, device=DEV)
+    k_pool[far * bs:] = k_small
+    v_pool[far * bs:] = v_small
+    k_pool[:small_pages * bs] = poison_rows(small_pages * bs, nkv * d, dtype).to(DEV)   # what an offset cut to 32 bits would read
+    v_pool[:small_pages * bs] = poison_rows(small_pages * bs, nkv * d, dtype).to(DEV)
+    bt_far = torch.where(bt >= 0, bt + far, bt)
+    n = sum(c for _, c in requests)
+    stride = (nq + 2 * nkv) * d
+    q = torch.randn(n, stride, device=DEV).to(dtype)
+    q_start, q_len, positions, seq_of = [], [], [], []
+    for s_, (ctx, count) in enumerate(requests):
+        q_start.append(len(positions))
+        q_len.append(count)
+        positions += list(range(ctx - count, ctx))
+        seq_of += [s_] * count
+    as_i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    scale = 1 / math.sqrt(d)
+    out = torch.zeros((n, nq * d), dtype=dtype, device=DEV)
+    limit = kernels.SHORT_PORTION
+    kernels.paged_attention_prefill(q, stride, out, as_i32(q_start), as_i32(q_len), as_i32(ctx_lens), max(q_len), bt_far, bs,
+                                    k_pool, v_pool, nq, nkv, d, scale, 0, short_limit=limit, splits=1)
+    kernels.paged_attention_decode(q, stride, out, as_i32(positions), as_i32(seq_of), bt_far, bs, k_pool, v_pool, nq, nkv, d,
+                                   scale, 0, splits=2, q_len=as_i32(q_len), short_limit=limit)
+    g = nq // nkv
+    for i in range(n):
+        s_, pos = seq_of[i], positions[i]
+        want = attention_ref(q[i, :nq * d].double().cpu().reshape(nq, d), keys[s_], values[s_], pos, g, scale, 0)
+        err = rel(out[i].reshape(nq, d), want)
+        assert err < 1e-2, f"token {i} (request {s_}, position {pos}): {err:.3e}"
+    del k_pool, v_pool
+    torch.cuda.empty_cache()
+
+
 GROUPED_CASES = [
     # nq, nkv, d, block size, [(context length after the step, tokens of the step)], window
     (32, 8, 128, 16, [(513, 1), (40, 1), (2100, 1), (1, 1)], 0),
