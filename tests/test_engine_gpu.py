@@ -545,6 +545,41 @@ def test_steps_are_queued_ahead_in_a_crowded_engine(model_dirs, name, chunk, dra
     assert m["available"] == m["total"]
 
 
+@pytest.mark.parametrize("case", range(8))
+def test_steps_queued_ahead_change_no_token_under_drawn_loads(model_dirs, case):
+    """Drawn loads on drawn engines, most of them crowded (few rows, few pages, stop tokens that end requests in the
+    middle, some requests drawing their tokens): every request has the tokens and the ending it has in an engine
+    that reads every step's tokens before it plans the next, and every page comes back."""
+    import random
+
+    from paged_llm_rs_amd import Engine
+
+    rng = random.Random(1000 + case)
+    name = rng.choice("ABC")
+    d = model_dirs(name, "float32")
+    vocab = TINY_INIT[name]["config"]["vocab_size"]
+    n = rng.randint(3, 24)
+    prompts = [[rng.randrange(vocab) for _ in range(rng.choice([rng.randint(1, 12), rng.randint(20, 60)]))] for _ in range(n)]
+    budgets = [rng.randint(1, 40) for _ in range(n)]
+    bs = rng.choice([4, 8, 16])
+    need_one = -(-max(len(p) + b for p, b in zip(prompts, budgets)) // bs)
+    settings = dict(dtype="f32", block_size=bs, num_blocks=rng.choice([need_one + 1, need_one * 2, need_one * 3, 8 * need_one]),
+                    max_batch=rng.choice([1, 2, 3, 5, 8, 40]), chunk=rng.choice([None, 4, 16, 64]), prefix_cache=False,
+                    graphs=rng.random() < 0.7)
+    drawn = rng.random() < 0.4
+    stops = [rng.randrange(vocab) for _ in range(rng.choice([0, 0, 3, 12]))]
+    results = {}
+    for ahead in (False, True):
+        engine = Engine(d, ahead=ahead, **settings)
+        ids = [engine.submit(p, b, stop_tokens=stops, **(dict(temperature=0.9, seed=50 + i) if drawn and i % 2 else dict(temperature=0.0)))
+               for i, (p, b) in enumerate(zip(prompts, budgets))]
+        engine.run()
+        results[ahead] = [engine.take_result(i) for i in ids]
+        m = engine.metrics()
+        assert m["available"] == m["total"], "pages were lost"
+    assert [(r.tokens, r.finish) for r in results[True]] == [(r.tokens, r.finish) for r in results[False]], settings
+
+
 def test_an_engine_whose_model_takes_no_ids_from_the_device_plans_nothing_ahead(model_dirs, monkeypatch):
     """Taking a row's id from the step before on the device is something a model offers (``takes_fed_tokens``).  One
     that does not is driven the ordinary way, every step's tokens read before the next is planned: its decode
