@@ -297,8 +297,14 @@ const Plan* Scheduler::plan_ahead() {
         const auto at = std::find(plan_.ids.begin(), plan_.ids.end(), s.id);
         const int fed = at == plan_.ids.end() ? -1 : static_cast<int>(at - plan_.ids.begin());
         if (fed >= 0) {
-            if (s.generated + 1 >= s.max_tokens) continue;                                 // its last token
-            if (max_positions_ > 0 && s.history.size() + 1 > max_positions_) continue;     // its last position
+            const bool last_token = s.generated + 1 >= s.max_tokens;
+            const bool last_position = max_positions_ > 0 && s.history.size() + 1 > max_positions_;
+            if (last_token || last_position) {
+                // It leaves at the commit and its pages with it: a queue that stalls now may not stall then, and
+                // bringing the front in is the planner's step.
+                if (!waiting_.empty()) return nullptr;
+                continue;
+            }
         }
         if (!cache_->reserve(s.id, 1)) return nullptr;           // who gives way is the planner's decision
         const size_t first = cache_->tokens(s.id);

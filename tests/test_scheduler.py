@@ -507,7 +507,7 @@ def test_every_request_finishes_and_every_page_returns_under_random_load(seed):
 # whose engine reads every step's tokens before it plans the next.)
 # ---------------------------------------------------------------------------
 
-def drive(s, arrivals, token_of, ahead: bool, steps: int = 4000):
+def drive(s, arrivals, token_of, ahead: bool, steps: int = 4000, log=None):
     """Run the scheduler to the end.  ``arrivals``: {iteration: [(id, prompt, max_tokens)]};
     ``token_of(id, n)`` is the n-th token request id samples.  With ``ahead`` every step that can be is
     planned before the tokens of the one before are committed, the way the engine does it.  Returns
@@ -529,6 +529,8 @@ def drive(s, arrivals, token_of, ahead: bool, steps: int = 4000):
                     break
                 continue
         decoding += plan.kind == sched.DECODE
+        if log is not None:
+            log.append((plan.kind, tuple(plan.ids), tuple((e.seq_id, e.start, len(e.tokens)) for e in plan.entries)))
         if ahead and plan.kind == sched.DECODE:
             s.launched()
             before = {i: s.manager.tokens(i) for i in s.running_ids()}
@@ -783,6 +785,38 @@ def test_requests_get_the_same_tokens_with_and_without_steps_planned_ahead(seed)
     (plain_out, plain_finish, (none, _)), (ahead_out, ahead_finish, (some, _)) = results
     assert none == 0 and some > 0
     assert ahead_out == plain_out and ahead_finish == plain_finish
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_without_stop_tokens_planning_ahead_changes_no_step(seed):
+    """Where no stop token ends a request, nothing a step's tokens say changes the step behind it: with steps planned
+    ahead the scheduler runs the very same steps, row for row, as without (a queue that stalls, requests that give
+    way and come back, more residents than rows).  Where the step's own end changes what the planner would do (a
+    request at its budget leaves, and the front of the queue may come in) nothing is planned ahead."""
+    rng = random.Random(300 + seed)
+    bs = rng.choice([2, 4, 16])
+    blocks = rng.randrange(8, 30)
+    chunk = rng.choice([None, 4, 8, 32])
+    max_batch = rng.randrange(1, 6)
+    window = rng.choice([0, 0, 3 * bs])
+    # (all requests are there from the start: one that arrives while a step planned ahead is queued comes in a step
+    # later than it would otherwise, which is the one difference that planning ahead makes by design)
+    arrivals = {0: [(i, [rng.randrange(5) for _ in range(rng.randrange(1, bs * blocks // 3))], rng.randrange(1, 25))
+                    for i in range(1, rng.randrange(3, 26))]}
+
+    def token_of(seq_id, n):
+        return (seq_id + n) % 50          # never the stop token (99)
+
+    logs = []
+    for ahead in (False, True):
+        s = scheduler(blocks, bs, max_batch, chunk=chunk, window=window)
+        # (no shared prefixes: a page that holds a token fed on the device gets its name a commit later, so a
+        # newcomer may find a page less to share than it would otherwise)
+        s.manager.set_prefix_cache(False)
+        log = []
+        drive(s, arrivals, token_of, ahead, log=log)
+        logs.append(log)
+    assert logs[0] == logs[1]
 
 
 @pytest.mark.parametrize("seed", range(8))
