@@ -71,7 +71,15 @@ struct sk_extras_t {
     int count;
     // w holds the weights in strips (see "Weights in strips" below)
     int strips;
+    // the K steps a wave of the launch takes (ceil(steps / waves): the launch knows both, and a division by a number
+    // the kernel learns only when it runs is some thirty instructions in front of its first loads); 0: not said
+    int steps_a_wave;
 };
+
+static inline sk_extras_t sk_with_steps(sk_extras_t extras, int K, int waves) {
+    extras.steps_a_wave = pl_ceil_div(pl_ceil_div(K, 32), waves);
+    return extras;
+}
 
 // Weights in strips.  Read as [N][K], a wave's load of a K step fetches 64 bytes from each of 16 rows of w that
 // lie K elements apart; the memory gives a pass of such loads less than it gives one that reads front to back
@@ -144,7 +152,7 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
 
     // K is cut into one stretch of whole steps a wave.
     const int steps = (K + SK_KSTEP - 1) / SK_KSTEP;
-    const int per_wave = (steps + nwaves - 1) / nwaves;
+    const int per_wave = hand.steps_a_wave > 0 ? hand.steps_a_wave : (steps + nwaves - 1) / nwaves;
     const int kbeg = wave * per_wave * SK_KSTEP;
     const int kend = min(K, (wave + 1) * per_wave * SK_KSTEP);
     const bool one_round = per_wave <= UNR;
@@ -214,6 +222,9 @@ gemm_skinny_kernel(const void* __restrict__ x_, const bf16_t* __restrict__ w, OU
 
 #pragma unroll
     for (int m = 0; m < MT; ++m) ssq[m] = 0.f;
+    // (x before the weights although those come from furthest away: loads are waited for in the order in which they
+    // were asked for, and what is done with x, the norm's arithmetic among it, is done while the weights are on
+    // their way.)
     bool x_asked = one_round && kbeg < kend;
     if (x_asked) ask_x(kbeg);
 
@@ -501,20 +512,20 @@ static int launch_one(int waves, const void* x, const void* w, void* y, const fl
             const size_t lds_h = static_cast<size_t>(wh) * (BT * MT * 256 + MT * 16) * sizeof(float);
             if (pl_ceil_div(steps, wh) > UH)
                 gemm_skinny_kernel<MT, UHA, WV, PRO, EPI, OUT, false, true, true><<<grid3, 64 * wh, lds_h, stream>>>(
-                    x, wb, yo, gain, eps, rows, n, N_out, K, act, hand);
+                    x, wb, yo, gain, eps, rows, n, N_out, K, act, sk_with_steps(hand, K, wh));
             else
                 gemm_skinny_kernel<MT, UH, WV, PRO, EPI, OUT, false, false, true><<<grid3, 64 * wh, lds_h, stream>>>(
-                    x, wb, yo, gain, eps, rows, n, N_out, K, act, hand);
+                    x, wb, yo, gain, eps, rows, n, N_out, K, act, sk_with_steps(hand, K, wh));
             PL_CHECK_LAUNCH("gemm_skinny");
             return 0;
         }
     }
     if (several)
         gemm_skinny_kernel<MT, UA, WV, PRO, EPI, OUT, false, true><<<grid3, 64 * waves, lds_bytes, stream>>>(
-            x, wb, yo, gain, eps, rows, n, N_out, K, act, hand);
+            x, wb, yo, gain, eps, rows, n, N_out, K, act, sk_with_steps(hand, K, waves));
     else
         gemm_skinny_kernel<MT, UNR, WV, PRO, EPI, OUT><<<grid3, 64 * waves, lds_bytes, stream>>>(
-            x, wb, yo, gain, eps, rows, n, N_out, K, act, hand);
+            x, wb, yo, gain, eps, rows, n, N_out, K, act, sk_with_steps(hand, K, waves));
     PL_CHECK_LAUNCH("gemm_skinny");
     return 0;
 }
@@ -790,7 +801,7 @@ static int launch_panel(const void* x, const void* w, void* y, const float* gain
         PL_REQUIRE(e == hipSuccess, "skinny product: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
     }
     kernel<<<grid, 64 * waves, lds_bytes, stream>>>(x, static_cast<const bf16_t*>(w), static_cast<OUT*>(y), gain, eps,
-                                                   rows, n, N_out, K, act, hand);
+                                                   rows, n, N_out, K, act, sk_with_steps(hand, K, waves));
     PL_CHECK_LAUNCH("gemm_skinny");
     return 0;
 }
