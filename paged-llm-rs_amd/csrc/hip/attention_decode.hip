@@ -208,7 +208,8 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
                               const int* __restrict__ q_len, int short_limit, int num_seqs,
                               const int* __restrict__ block_table, int max_blocks, int block_size,
                               bf16_t* __restrict__ k_pool, bf16_t* __restrict__ v_pool, int nq,
-                              int nkv, int d, float scale_log2e, int window, int splits, int tiles, ad_fuse_t fuse) {
+                              int nkv, int d, float scale_log2e, int window, int splits, int tiles, int g,
+                              uint32_t splits_magic, ad_fuse_t fuse) {
     constexpr int KPW = PL_WAVE / LPK;  // keys a wave handles with one load
     constexpr int ROUND = WV * KPW * U;
     extern __shared__ float lds[];      // [AD_PAGES_LDS] page numbers, then [WV][GT][2] running max and sum, [WV][GT][d] accumulators
@@ -223,9 +224,10 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
     const int seq = seq_of[t];
     if (q_len && q_len[seq] >= short_limit) return;  // a long portion: the tiled kernel's
 
-    const int g = nq / nkv;
-    const int kvh = blockIdx.x / tiles;
-    const int tile = blockIdx.x % tiles;
+    // (g = nq / nkv and splits_magic = ceil(2^32 / splits) come from the launch: a division by a number that the
+    // kernel learns only when it runs is some thirty instructions, and these stood in front of its first loads)
+    const int kvh = tiles == 1 ? static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x) / tiles;
+    const int tile = tiles == 1 ? 0 : static_cast<int>(blockIdx.x) % tiles;
     const int h0 = kvh * g + tile * GT;               // first query head of this workgroup
     const int heads = min(GT, g - tile * GT);         // how many of the GT are real
     const int split = blockIdx.z;
@@ -241,7 +243,9 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
     const int first = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
     const int limit = fuse.mode == 2 ? pos : pos + 1;   // the token's own key is not in the cache yet
     const int total = max(limit - first, 0);
-    const int per_split = pl_ceil_div(pl_ceil_div(total, splits), ROUND) * ROUND;
+    // ceil(total / splits): the high half of (total + splits - 1) * ceil(2^32 / splits), exact below 2^32 / splits
+    const int share = splits == 1 ? total : static_cast<int>(__umulhi(static_cast<uint32_t>(total + splits - 1), splits_magic));
+    const int per_split = pl_ceil_div(share, ROUND) * ROUND;
     const int s_begin = first + split * per_split;
     const int s_end = min(limit, s_begin + per_split);
     const int rounds = s_end > s_begin ? pl_ceil_div(s_end - s_begin, ROUND) : 0;
@@ -535,13 +539,15 @@ paged_attention_merge_kernel(const float* __restrict__ part_acc, const float* __
         rest = blockIdx.x * blockDim.x + threadIdx.x;
         inside = rest < per_token;
         rest = min(rest, per_token - 1);
-    } else {
-        const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-        t = min(idx / per_token, n - 1);
-        rest = idx - t * per_token;
-        inside = idx < n * per_token;
+    } else {                 // blockIdx.y is the token
+        t = blockIdx.y;
+        rest = blockIdx.x * blockDim.x + threadIdx.x;
+        inside = rest < per_token;
+        rest = min(rest, per_token - 1);
     }
-    const int h = rest / d, dd = rest - h * d;
+    // (a head size that is a power of two spares the kernel a division in front of its loads)
+    const int h = (d & (d - 1)) == 0 ? rest >> (31 - __builtin_clz(static_cast<unsigned>(d))) : rest / d;
+    const int dd = rest - h * d;
     const size_t base = (static_cast<size_t>(t) * nq + h) * splits;
     const int pos = positions[t];
     const int len = q_len ? q_len[seq_of[t]] : 0;
@@ -592,10 +598,11 @@ static int launch_decode_keys(const void* q, int q_stride, void* out, float* par
     paged_attention_decode_kernel<LPK, GT, U, WV><<<grid, 64 * WV, lds_bytes, stream>>>(
         static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), part_acc, part_ml, positions, seq_of,
         q_len, short_limit, compact ? num_seqs : 0, block_table, max_blocks, block_size, static_cast<bf16_t*>(k_pool),
-        static_cast<bf16_t*>(v_pool), nq, nkv, d, scale * 1.4426950408889634f, window, splits, tiles, fuse);
+        static_cast<bf16_t*>(v_pool), nq, nkv, d, scale * 1.4426950408889634f, window, splits, tiles, g,
+        static_cast<uint32_t>((0x100000000ull + splits - 1) / static_cast<unsigned>(splits)), fuse);
     PL_CHECK_LAUNCH("paged_attention_decode");
     if (splits > 1) {
-        const dim3 mgrid = compact ? dim3(pl_ceil_div(nq * d, 256), short_rows) : dim3(pl_ceil_div(n * nq * d, 256));
+        const dim3 mgrid = dim3(pl_ceil_div(nq * d, 256), compact ? short_rows : n);
 #define AD_MERGE(SP)                                                                                              \
     paged_attention_merge_kernel<SP><<<mgrid, 256, 0, stream>>>(part_acc, part_ml, static_cast<bf16_t*>(out),     \
                                                                 positions, seq_of, q_len, short_limit, nq, d,     \
