@@ -754,6 +754,38 @@ def test_paged_attention_of_single_tokens(kernel, nq, nkv, d, bs, ctx_lens, wind
     assert bool((out[-1] == 7.0).all()), "a padding row is not written"
 
 
+@pytest.mark.parametrize("splits", [1, 2])
+@pytest.mark.parametrize("bs,ctx,window", [(1, 2600, 0), (2, 5001, 0), (1, 2600, 2300)])
+def test_single_tokens_over_more_pages_than_the_kernel_keeps_at_hand(bs, ctx, window, splits):
+    """The single-token kernel copies the page numbers of a workgroup's stretch of keys into LDS, 2,048 of them
+    at most; a longer stretch (small pages, one share) looks each page up in the table.  Both ways, beside each
+    other in one launch (the second request is short), against 64-bit arithmetic; one key far back carries
+    nearly all the weight of the long request's last token, so that a page looked up wrongly shows."""
+    from paged_llm_rs_amd import kernels
+
+    nq, nkv, d = 4, 2, 64
+    dtype = torch.bfloat16
+    bt, k_pool, v_pool, keys, values = build_paged(nkv, d, bs, [ctx, 37], dtype, seed=ctx + bs)
+    toks = [(0, ctx - 1), (0, ctx // 2), (0, 2047 * bs), (0, 2048 * bs), (1, 36), (1, 0)]
+    stride = (nq + 2 * nkv) * d
+    q = torch.randn(len(toks), stride, device=DEV).to(dtype)
+    target = ctx - 2200                      # (inside the window where there is one)
+    slot = int(bt[0, target // bs]) * bs + target % bs
+    for kvh in range(nkv):
+        k_pool[slot, kvh * d:(kvh + 1) * d] = (q[0, kvh * 2 * d: kvh * 2 * d + d].float() * 4).to(dtype)
+        keys[0][target, kvh] = k_pool[slot, kvh * d:(kvh + 1) * d].double().cpu()
+    positions = torch.tensor([p for _, p in toks], dtype=torch.int32, device=DEV)
+    seq_of = torch.tensor([s for s, _ in toks], dtype=torch.int32, device=DEV)
+    scale = 1 / math.sqrt(d)
+    out = torch.zeros(len(toks), nq * d, dtype=dtype, device=DEV)
+    kernels.paged_attention_decode(q, stride, out, positions, seq_of, bt, bs, k_pool, v_pool, nq, nkv, d, scale, window,
+                                   splits=splits)
+    for i, (s, p) in enumerate(toks):
+        want = attention_ref(q[i, :nq * d].double().cpu().reshape(nq, d), keys[s], values[s], p, nq // nkv, scale, window)
+        assert rel(out[i].reshape(nq, d), want) < 1e-2, f"token {i} (request {s}, position {p})"
+    assert rel(out[0].reshape(nq, d)[0], values[0][target, 0]) < 0.2, "the far key's value is the answer"
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("nq,nkv,d,bs,ctx_lens,window", [(3, 1, 24, 4, [37, 5], 0), (4, 2, 10, 8, [70], 0),
                                                           (2, 2, 100, 16, [130, 20], 33), (5, 5, 1, 2, [9], 0)])
@@ -815,7 +847,8 @@ def test_a_far_key_among_hundreds_is_found(kernel):
 
 @pytest.mark.parametrize("nq,nkv,d,bs,ctx_lens,window,rot,norm", [
     (16, 8, 128, 16, [513, 40, 1], 0, 128, True), (6, 1, 32, 8, [70, 9], 0, 32, True), (6, 2, 48, 16, [100, 17, 64], 0, 32, False),
-    (4, 2, 64, 16, [300, 31], 48, 64, True), (32, 2, 128, 16, [300], 0, 128, True), (3, 3, 80, 2, [37, 12], 0, 0, True)])
+    (4, 2, 64, 16, [300, 31], 48, 64, True), (32, 2, 128, 16, [300], 0, 128, True), (3, 3, 80, 2, [37, 12], 0, 0, True),
+    (4, 2, 64, 1, [2300, 5], 0, 64, True)])     # (more pages than the kernel copies into LDS: looked up in the table)
 @pytest.mark.parametrize("splits", [1, 3])
 def test_decode_attention_that_prepares_its_own_queries_and_keys(nq, nkv, d, bs, ctx_lens, window, rot, norm, splits):
     """One token a request: the norm, the rotation and the cache write inside the attention kernel give what
