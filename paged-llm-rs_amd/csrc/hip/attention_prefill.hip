@@ -1078,6 +1078,8 @@ extern "C" int pl_paged_attention_grouped(const void* q, int q_stride, void* out
                "grouped attention: %d blocks a row, query stride %d, window %d", max_blocks, q_stride, window);
     if (num_seqs <= 0 || max_q_len <= 0) return 0;
     PL_REQUIRE(total_rows >= max_q_len, "grouped attention: %d rows for portions of %d", total_rows, max_q_len);
+    PL_REQUIRE(static_cast<unsigned long long>(block_size) * nkv * d * 2 < (1ull << 32),
+               "grouped attention: a page of %d tokens of %d heads of %d takes more bytes than 32 bits count", block_size, nkv, d);
     if (d == 64)
         return launch_prefill<2, 1, 2, 2, true>(q, q_stride, out, q_start, q_len, ctx_len, short_limit, num_seqs, max_q_len,
                                                 block_table, max_blocks, block_size, k_pool, v_pool, nq, nkv, d, scale,
