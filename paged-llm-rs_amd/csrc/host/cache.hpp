@@ -122,6 +122,8 @@ public:
     size_t capacity(uint64_t id) const;
     // Pages still needed, in the hungriest group, to hold `count` more tokens.
     size_t blocks_needed(uint64_t id, size_t count) const;
+    // The same in one group.
+    size_t blocks_needed_in(uint64_t id, size_t group, size_t count) const { return needed_in_group(table(id), group, count); }
     // Take pages until `count` more tokens fit; nothing is taken when any pool
     // cannot supply its share.
     bool reserve(uint64_t id, size_t count);

@@ -273,13 +273,26 @@ const Plan* Scheduler::plan_ahead() {
     // Would the planner bring the front of the queue in (or turn it away)?  Then the next step is its to decide.
     // Whether there is room is asked where the planner asks: before the residents take their pages when prompts
     // run whole, after them under a token budget.
+    // Nothing is taken from the pools before the step is known to stand: a plan given up half way would leave
+    // its pages with the residents a step early, and the planner would then find less room for the queue's front
+    // than it finds without steps planned ahead.
+    const size_t groups = cache_->num_groups();
+    std::vector<size_t> need(groups, 0);                          // pages the rows seated so far take, a group
+    auto room_left = [&]() -> size_t {                            // (what min_available() will say once they have them)
+        size_t least = SIZE_MAX;
+        for (size_t g = 0; g < groups; ++g) {
+            const size_t free_now = cache_->pool(g).available();
+            least = std::min(least, free_now > need[g] ? free_now - need[g] : 0);
+        }
+        return least;
+    };
     bool stalled = false;
     auto front_stalls = [&]() -> bool {
         if (waiting_.empty()) return true;
         const size_t prompt_len = waiting_.front().pending.size();
         const bool too_long = max_positions_ > 0 && prompt_len > max_positions_;
         if (too_long || !cache_->fits_in_total(prompt_len, chunk_ > 0 ? chunk_ : prompt_len)) return false;   // a refusal
-        const bool room = chunk_ > 0 ? cache_->min_available() > 0 : cache_->fits_from_scratch(prompt_len);
+        const bool room = chunk_ > 0 ? room_left() > 0 : cache_->fits_from_scratch(prompt_len);
         if (room && cache_->state_slot_available()) return false;
         stalled = true;
         return true;
@@ -288,10 +301,9 @@ const Plan* Scheduler::plan_ahead() {
     // A row for every resident with a token to feed, in the order of arrival, as far as the rows last (as the
     // planner seats them): the token of its row in the launched step, which is not known yet, or, for a resident
     // that step had no row for, the token it has been holding.
-    Plan next;
-    next.kind = PlanKind::Decode;
+    std::vector<std::pair<Sequence*, int>> seated;
     for (Sequence& s : running_) {
-        if (next.entries.size() == max_batch_) break;
+        if (seated.size() == max_batch_) break;
         if (s.finish != Finish::None) continue;                  // (leaves at the commit)
         if (s.pending.size() != 1) return nullptr;
         const auto at = std::find(plan_.ids.begin(), plan_.ids.end(), s.id);
@@ -306,7 +318,19 @@ const Plan* Scheduler::plan_ahead() {
                 continue;
             }
         }
-        if (!cache_->reserve(s.id, 1)) return nullptr;           // who gives way is the planner's decision
+        for (size_t g = 0; g < groups; ++g) {
+            need[g] += cache_->blocks_needed_in(s.id, g, 1);
+            if (need[g] > cache_->pool(g).available()) return nullptr;   // who gives way is the planner's decision
+        }
+        seated.emplace_back(&s, fed);
+    }
+    if (seated.empty()) return nullptr;
+    if (chunk_ > 0 && !front_stalls()) return nullptr;
+    Plan next;
+    next.kind = PlanKind::Decode;
+    for (const auto& [seq, fed] : seated) {
+        Sequence& s = *seq;
+        if (!cache_->reserve(s.id, 1)) throw Error("a step planned ahead found no page where it had counted one");
         const size_t first = cache_->tokens(s.id);
         next.ids.push_back(s.id);
         next.advanced.emplace_back(s.id, 1);
@@ -314,8 +338,6 @@ const Plan* Scheduler::plan_ahead() {
                                          s.state_slot, false});
         next.fed_rows.push_back(fed);
     }
-    if (next.entries.empty()) return nullptr;
-    if (chunk_ > 0 && !front_stalls()) return nullptr;
     if (stalled) metrics_.admission_stalls += 1;
     metrics_.steps += 1;
     metrics_.decode_steps += 1;

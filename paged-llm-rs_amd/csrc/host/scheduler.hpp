@@ -115,7 +115,9 @@ public:
     // that step is not known yet: the planner would bring the front of the queue in or turn it away, a
     // request is part-way through its prompt, the pools have no page for a row (then the ordinary
     // planner decides who gives way, after the commit), or a request waits while the launched step is some
-    // resident's last by its budget or position (its pages come back at the commit, and the front may come in).  Otherwise it is a decoding step again: rows for
+    // resident's last by its budget or position (its pages come back at the commit, and the front may come in).
+    // When it gives nothing it has taken nothing: the pages of its rows are counted first and taken only once the
+    // step stands, so that the planner finds the pools as it would without steps ahead.  Otherwise it is a decoding step again: rows for
     // the residents in their order as far as the rows last, as the planner seats them.  Requests that the
     // launched step ends by their budget or the model's last position have no row in it; one that a stop
     // token ends has, and that row's token is dropped when it is committed (a resident that would have

@@ -630,6 +630,26 @@ def test_nothing_is_planned_ahead_while_a_request_waits_or_pages_are_short():
     assert s.manager.available() == 2
 
 
+def test_a_step_ahead_that_cannot_stand_takes_no_page():
+    """Two of three residents need a new page for the step ahead and one page is free: the step is the planner's
+    (someone gives way), and the resident that could have had the page does not hold it a step early, where it
+    would stand between the planner and the queue's front."""
+    s = scheduler(7, 2, 4)                           # seven pages of two tokens
+    submit(s, 1, 1, 100, prompt=[1])
+    submit(s, 2, 2, 100, prompt=[2, 2])
+    submit(s, 3, 2, 100, prompt=[3, 3])
+    assert step(s)[0].kind == sched.MIXED            # the prompts: a page each
+    assert step(s)[0].kind == sched.DECODE           # positions 1, 2, 2: requests 2 and 3 take their second page
+    plan = s.plan()                                  # positions 2, 3, 3: request 1 takes its second page
+    assert plan.kind == sched.DECODE and s.manager.available() == 1
+    s.launched()
+    assert s.plan_ahead() is None                    # positions 3, 4, 4 would take two pages
+    assert s.manager.available() == 1
+    s.commit([7, 7, 7])
+    plan = s.plan()                                  # the planner's step: one of the two gives way
+    assert plan.kind == sched.DECODE and len(plan.ids) == 2 and plan.ids[0] == 1 and s.metrics()["preemptions"] == 1
+
+
 def test_steps_are_planned_ahead_while_the_queue_cannot_move():
     """Serving at its limit: more residents than rows, and a front of the queue that no page or slot can
     take yet.  The planner would decode, so the step is planned ahead; when the front can come in, it is not."""
@@ -787,7 +807,7 @@ def test_requests_get_the_same_tokens_with_and_without_steps_planned_ahead(seed)
     assert ahead_out == plain_out and ahead_finish == plain_finish
 
 
-@pytest.mark.parametrize("seed", range(10))
+@pytest.mark.parametrize("seed", list(range(10)) + [1051, 1052, 1102, 1148, 1173])
 def test_without_stop_tokens_planning_ahead_changes_no_step(seed):
     """Where no stop token ends a request, nothing a step's tokens say changes the step behind it: with steps planned
     ahead the scheduler runs the very same steps, row for row, as without (a queue that stalls, requests that give
