@@ -46,20 +46,30 @@ class SafetensorsFile:
             header = json.loads(self._file.read(length))
         except (json.JSONDecodeError, UnicodeDecodeError) as e:
             raise WeightError(f"{self.path}: header is not JSON: {e}") from e
+        if not isinstance(header, dict):
+            raise WeightError(f"{self.path}: header is not a JSON object")
         self.metadata = header.pop("__metadata__", {})
         self.entries = header
         self._base = 8 + length
         self._map = mmap.mmap(self._file.fileno(), 0, access=mmap.ACCESS_READ) if size else None
         for name, e in self.entries.items():
-            if e.get("dtype") not in _DTYPES:
-                raise WeightError(f"{self.path}: {name} has dtype {e.get('dtype')!r}, which is not read here")
-            begin, end = e["data_offsets"]
+            # (a file that was cut, or written by something else, is a wrong weight file and said to be one)
+            whole = (lambda v: isinstance(v, int) and not isinstance(v, bool) and v >= 0)
+            offsets = e.get("data_offsets") if isinstance(e, dict) else None
+            if not (isinstance(e, dict) and isinstance(e.get("shape"), list) and all(whole(n) for n in e["shape"])
+                    and isinstance(offsets, list) and len(offsets) == 2 and all(whole(n) for n in offsets)
+                    and isinstance(e.get("dtype"), str)):
+                raise WeightError(f"{self.path}: the entry of {name!r} is not a dtype, a shape and two data offsets")
+            if e["dtype"] not in _DTYPES:
+                raise WeightError(f"{self.path}: {name} has dtype {e['dtype']!r}, which is not read here")
+            begin, end = offsets
             count = 1
-            for s in e["shape"]:
-                count *= s
+            for n in e["shape"]:
+                count *= n
             width = torch.empty((), dtype=_DTYPES[e["dtype"]]).element_size()
-            if end - begin != count * width or self._base + end > size:
-                raise WeightError(f"{self.path}: {name} has {end - begin} bytes for shape {e['shape']}")
+            if end < begin or end - begin != count * width or self._base + end > size:
+                raise WeightError(f"{self.path}: {name} has the bytes {begin} to {end} for shape {e['shape']}, in a file "
+                                  f"with {size - self._base} bytes of data")
 
     def names(self):
         return list(self.entries)

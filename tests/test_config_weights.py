@@ -131,6 +131,65 @@ def test_own_reader_agrees_with_the_library_reader(tmp_path):
         assert torch.equal(back[k], v)
 
 
+def test_a_damaged_weight_file_is_a_weight_error_and_nothing_else(tmp_path):
+    """A header that is cut, is no object, or describes a tensor wrongly (no offsets, a negative or broken shape,
+    bytes that do not match the shape or lie outside the file) is refused as a wrong weight file: whatever is
+    done to the header's bytes, the reader either reads what the library reader reads or raises WeightError."""
+    import random
+    import struct
+
+    good = {"a": torch.randn(3, 5), "b": torch.arange(6, dtype=torch.int32)}
+    write_safetensors(tmp_path / "good.safetensors", good)
+    raw = (tmp_path / "good.safetensors").read_bytes()
+    (length,) = struct.unpack("<Q", raw[:8])
+    header, data = json.loads(raw[8:8 + length]), raw[8 + length:]
+
+    def rewritten(head) -> bytes:
+        blob = json.dumps(head).encode()
+        return struct.pack("<Q", len(blob)) + blob + data
+
+    entry = dict(header["a"])
+    cases = {
+        "no object": rewritten([1, 2]),
+        "no entry": rewritten({"a": 5}),
+        "no offsets": rewritten({"a": {k: v for k, v in entry.items() if k != "data_offsets"}}),
+        "no shape": rewritten({"a": {k: v for k, v in entry.items() if k != "shape"}}),
+        "a negative size": rewritten({"a": {**entry, "shape": [-3, -5]}}),
+        "a broken size": rewritten({"a": {**entry, "shape": [3.0, "5"]}}),
+        "offsets backwards": rewritten({"a": {**entry, "data_offsets": [60, 0]}}),
+        "a negative offset": rewritten({"a": {**entry, "data_offsets": [-60, 0]}}),
+        "bytes past the end": rewritten({"a": {**entry, "data_offsets": [1 << 40, (1 << 40) + 60]}}),
+        "too few bytes": rewritten({"a": {**entry, "data_offsets": [0, 56]}}),
+        "an unknown dtype": rewritten({"a": {**entry, "dtype": "F8_E4M3"}}),
+        "a dtype that is no name": rewritten({"a": {**entry, "dtype": 32}}),
+        "a cut file": raw[:8 + length + 10],
+        "a cut header": raw[:8 + length // 2],
+        "a header longer than the file": struct.pack("<Q", 1 << 50) + raw[8:],
+        "four bytes": raw[:4],
+    }
+    for what, blob in cases.items():
+        (tmp_path / "bad.safetensors").write_bytes(blob)
+        with pytest.raises(WeightError):
+            SafetensorsFile(tmp_path / "bad.safetensors")
+            raise AssertionError(f"{what} was read")
+
+    rng = random.Random(0)
+    read, refused = 0, 0
+    for _ in range(300):                                     # bytes of the header overwritten at random
+        blob = bytearray(raw)
+        for _ in range(rng.randrange(1, 4)):
+            blob[rng.randrange(0, 8 + length)] = rng.choice(b'0123456789[]{}",:-eE \\x00\xff')
+        (tmp_path / "bad.safetensors").write_bytes(bytes(blob))
+        try:
+            f = SafetensorsFile(tmp_path / "bad.safetensors")
+            for name in f.names():
+                assert f.tensor(name).numel() == f.tensor(name).reshape(-1).shape[0]
+            read += 1
+        except WeightError:
+            refused += 1
+    assert read + refused == 300 and refused > 100
+
+
 def test_random_model_is_seeded_and_complete(tmp_path):
     a = write_random_model(tmp_path / "a", TINY_A, seed=0, std=0.02, gain_std=0.1, dtype="float32")
     b = write_random_model(tmp_path / "b", TINY_A, seed=0, std=0.02, gain_std=0.1, dtype="float32")
