@@ -37,10 +37,13 @@ class GenerationConfig:
             generation = read_json(directory / "generation_config.json")
         except PagedLLMError:
             generation = None
+        if not isinstance(generation, dict):                 # (absent, or a file that holds no object)
+            generation = None
         eos = _token_ids(generation.get("eos_token_id")) if generation else None
         if eos is None:
             try:
-                eos = _token_ids(read_json(directory / "config.json").get("eos_token_id"))
+                config = read_json(directory / "config.json")
+                eos = _token_ids(config.get("eos_token_id")) if isinstance(config, dict) else None
             except PagedLLMError:
                 eos = None
 

@@ -77,6 +77,8 @@ class Qwen3Config:
         if d.get("rope_scaling") is not None:
             raise refuse("rope_scaling, the rotary table here is unscaled")
         nested = d.get("rope_parameters")
+        if nested is not None and not isinstance(nested, dict):
+            raise ConfigError(f"rope_parameters {nested!r}, which has to be an object")
         if nested is not None and nested.get("rope_type") not in (None, "default"):
             raise refuse(f"rope_type {nested.get('rope_type')!r}, the rotary table here is unscaled")
         if d.get("rope_theta") is not None:

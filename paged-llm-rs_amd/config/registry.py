@@ -27,10 +27,12 @@ def architectures() -> list:
 
 
 def config_class_for(d: dict):
+    if not isinstance(d, dict):
+        raise ConfigError("config.json does not hold an object")
     names = d.get("architectures")
     if isinstance(names, list) and names:
         name = names[0]
-        if name in _ARCHITECTURES:
+        if isinstance(name, str) and name in _ARCHITECTURES:
             return _ARCHITECTURES[name]
         raise UnsupportedError(
             f"architecture {name!r}, the registry knows {', '.join(architectures())}"
@@ -38,7 +40,7 @@ def config_class_for(d: dict):
     model_type = d.get("model_type")
     if model_type is None:
         raise ConfigError("config.json names neither architectures nor model_type")
-    if model_type in _MODEL_TYPES:
+    if isinstance(model_type, str) and model_type in _MODEL_TYPES:
         return _MODEL_TYPES[model_type]
     raise UnsupportedError(
         f"model_type {model_type!r}, the registry knows {', '.join(sorted(_MODEL_TYPES))}"

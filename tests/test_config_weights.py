@@ -73,6 +73,46 @@ def test_missing_keys_and_bad_values_are_config_errors():
         load_config(d)
 
 
+def test_values_of_the_wrong_kind_are_config_errors(tmp_path):
+    """Whatever stands where a key's value should (a list for a name, a number for the rotary base's object, a
+    file that holds no object, a file cut short), the configuration is refused with one of the engine's own
+    errors and nothing else; the generation defaults of such a folder are none."""
+    import random
+
+    from paged_llm_rs_amd.errors import PagedLLMError
+
+    for key, value in [("model_type", [1, 2]), ("model_type", {"a": 1}), ("rope_parameters", 5), ("rope_parameters", "x"),
+                       ("architectures", [["Qwen3ForCausalLM"]]), ("architectures", [7])]:
+        d = qwen3_06b()
+        d[key] = value
+        with pytest.raises(PagedLLMError):
+            load_config(d)
+    (tmp_path / "config.json").write_text("[1, 2]")
+    with pytest.raises(ConfigError):
+        load_config(tmp_path)
+    (tmp_path / "generation_config.json").write_text("[3]")
+    assert GenerationConfig.from_dir(tmp_path) == GenerationConfig()
+
+    rng = random.Random(0)
+    values = [None, 0, -1, 1.5, "x", [], {}, True, 1 << 40, [1, 2], {"rope_theta": "a"}, 1e308, ""]
+    for _ in range(500):
+        d = qwen3_06b()
+        d["architectures"] = ["Qwen3ForCausalLM"]
+        for _ in range(rng.randrange(1, 3)):
+            key = rng.choice(list(d) + ["rope_parameters", "rope_scaling", "layer_types", "eos_token_id"])
+            if rng.random() < 0.2:
+                d.pop(key, None)
+            else:
+                d[key] = rng.choice(values)
+        text = json.dumps(d)
+        (tmp_path / "config.json").write_text(text[:rng.randrange(len(text))] if rng.random() < 0.1 else text)
+        try:
+            load_config(tmp_path)
+        except PagedLLMError:
+            pass
+        GenerationConfig.from_dir(tmp_path)
+
+
 def test_registry_chooses_by_architecture_then_model_type():
     assert "Qwen3ForCausalLM" in architectures()
     d = qwen3_06b()
