@@ -14,7 +14,7 @@ import json
 import sys
 from pathlib import Path
 
-from .errors import ConfigError, PagedLLMError
+from .errors import ConfigError, IoError, PagedLLMError
 
 
 def parser() -> argparse.ArgumentParser:
@@ -60,9 +60,20 @@ def parser() -> argparse.ArgumentParser:
 
 def parse_ids(text: str) -> list:
     text = text.strip()
-    if text.startswith("["):
-        return [int(t) for t in json.loads(text)]
-    return [int(t) for t in text.replace(",", " ").split()]
+    try:
+        if text.startswith("["):
+            return [int(t) for t in json.loads(text)]
+        return [int(t) for t in text.replace(",", " ").split()]
+    except (ValueError, TypeError):
+        shown = text if len(text) <= 60 else text[:57] + "..."
+        raise ConfigError(f"token ids are whole numbers, separated by commas or spaces or as a JSON list: {shown!r}") from None
+
+
+def read_text(path, what: str) -> str:
+    try:
+        return Path(path).read_text()
+    except OSError as e:
+        raise IoError(f"reading {what} {path}: {e}") from e
 
 
 def main(argv=None) -> int:
@@ -80,13 +91,16 @@ def main(argv=None) -> int:
         if args.random_weights:
             from .weights import write_random_model
 
-            config = json.loads(Path(args.random_weights).read_text())
+            try:
+                config = json.loads(read_text(args.random_weights, "--random-weights"))
+            except json.JSONDecodeError as e:
+                raise ConfigError(f"--random-weights {args.random_weights} is not JSON: {e}") from None
             write_random_model(args.model, config, seed=args.init_seed, std=args.init_std,
                                gain_std=args.init_gain_std,
                                dtype="float32" if args.dtype == "f32" else "bfloat16")
         prompts = [parse_ids(p) for p in args.prompt_ids]
         if args.prompt_file:
-            prompts += [parse_ids(line) for line in Path(args.prompt_file).read_text().splitlines() if line.strip()]
+            prompts += [parse_ids(line) for line in read_text(args.prompt_file, "--prompt-file").splitlines() if line.strip()]
         from . import kernels
         from .engine import Engine
 

@@ -153,6 +153,23 @@ def test_generation_config(tmp_path):
     assert GenerationConfig.from_dir(tmp_path).top_k is None
 
 
+def test_the_command_line_says_what_is_wrong_with_its_arguments(tmp_path, capsys):
+    """Prompts that are no numbers and files that are not there end the command line with one line and the
+    status 1, before anything is loaded (cli.py; the reference's main.rs reports its errors the same way)."""
+    from paged_llm_rs_amd.cli import main
+
+    for args, says in [(["--prompt-ids", "a,b"], "token ids are whole numbers"),
+                       (["--prompt-ids", "[1,[2]]"], "token ids are whole numbers"),
+                       (["--prompt-file", str(tmp_path / "none.txt")], "--prompt-file"),
+                       (["--random-weights", str(tmp_path / "none.json")], "--random-weights"),
+                       (["--chunk", "some", "--prompt-ids", "1"], "--chunk")]:
+        assert main(["--model", str(tmp_path / "model")] + args) == 1
+        assert says in capsys.readouterr().err
+    (tmp_path / "cut.json").write_text('{"hidden_size": ')
+    assert main(["--model", str(tmp_path / "model"), "--random-weights", str(tmp_path / "cut.json")]) == 1
+    assert "is not JSON" in capsys.readouterr().err
+
+
 # --- safetensors and weights ----------------------------------------------------------------
 
 def test_own_reader_agrees_with_the_library_reader(tmp_path):

@@ -219,6 +219,26 @@ def test_schedules_agree_with_each_other_in_32_bit(setups):
     assert worst <= 2e-6, f"{worst:.3e}"
 
 
+def test_trace_run_names_the_line_it_cannot_take(setups, tmp_path):
+    """A line that is no step, a token outside the vocabulary and a trace that outgrows --max-tokens each end the
+    program with the status 1 and one line that names the input's line; the steps before it are done."""
+    d, prompts, _ = setups("A", "float32")
+    vocab = TINY_INIT["A"]["config"]["vocab_size"]
+    good = {"step": 0, "entries": [{"id": "a", "tokens": [1, 2, 3], "want": [2]}], "end": []}
+    for bad, says in [("{\"step\": 1, \"entries\": [", "line 2"), ("[1, 2]", "line 2"),
+                      (json.dumps({"step": 1, "entries": [{"id": "a", "tokens": [vocab], "want": []}], "end": []}), "vocabulary"),
+                      (json.dumps({"step": 1, "entries": [{"id": "a", "want": []}], "end": []}), "line 2"),
+                      (json.dumps({"step": 1, "entries": [{"id": "b", "tokens": [1] * 200, "want": []}], "end": []}), "--max-tokens")]:
+        proc = subprocess.run(
+            [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(d), "--dtype", "float32",
+             "--out", str(tmp_path / "out"), "--max-tokens", "128"],
+            input=json.dumps(good) + "\n" + bad + "\n", capture_output=True, text=True, timeout=600)
+        assert proc.returncode == 1, proc.stderr[-2000:]
+        assert proc.stdout.split("\n")[0] == "done 0" and "done 1" not in proc.stdout
+        last = proc.stderr.strip().split("\n")[-1]
+        assert last.startswith("[trace_run] error") and says in last, last
+
+
 def test_trace_run_program(setups, tmp_path):
     """The program itself: JSON lines in, <step>.f32 out, a ``done`` line after each step."""
     d, prompts, want = setups("A", "float32")
